@@ -1,0 +1,346 @@
+"""ctypes front end of the CPU oracle (``libtenmo_oracle.so``).
+
+TEST INFRASTRUCTURE ONLY: imported by ``tests/``, by ``__graft_entry__.smoke()`` and by the
+``cpu_baseline`` leg of ``bench.py`` as the checker / reported baseline.  The product package
+never imports it.
+
+A view is ``(storage, offset, shape, strides)`` in elements, the reference's NDBuffer layout
+(tenmo/ndbuffer.mojo).  ``View.of(ndarray)`` takes any fp32 numpy view (transposed, sliced,
+``as_strided``) and describes it relative to its own first element.
+"""
+from __future__ import annotations
+
+import ctypes as C
+import os
+import subprocess
+from typing import Optional, Sequence, Tuple
+
+import numpy as np
+
+MAX_RANK = 8
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(_HERE, "libtenmo_oracle.so")
+
+DOT, VM, MV, MM, INVALID = 0, 1, 2, 3, -1
+
+
+class _CView(C.Structure):
+    _fields_ = [
+        ("data", C.c_void_p),
+        ("offset", C.c_int64),
+        ("rank", C.c_int32),
+        ("shape", C.c_int64 * MAX_RANK),
+        ("strides", C.c_int64 * MAX_RANK),
+    ]
+
+
+class OracleError(RuntimeError):
+    """Raised where the reference panics (shape mismatch, incompatible broadcast ...)."""
+
+
+def build(force: bool = False) -> str:
+    """Compile the oracle with its Makefile (g++, OpenMP)."""
+    if force or not os.path.exists(_LIB_PATH):
+        subprocess.check_call(["make", "-C", _HERE, "-j8"] + (["-B"] if force else []),
+                              stdout=subprocess.DEVNULL)
+    return _LIB_PATH
+
+
+_lib = None
+
+
+def lib():
+    global _lib
+    if _lib is None:
+        if not os.path.exists(_LIB_PATH):
+            build()
+        L = C.CDLL(_LIB_PATH)
+        vp = C.POINTER(_CView)
+        i64p, i32p, fp, dp = C.POINTER(C.c_int64), C.POINTER(C.c_int32), C.c_void_p, C.c_void_p
+        L.oracle_last_error.restype = C.c_char_p
+        L.oracle_simd_width.restype = C.c_int
+        L.oracle_force_simd_width.argtypes = [C.c_int]
+        L.oracle_num_physical_cores.restype = C.c_int
+        L.oracle_is_contiguous.argtypes = [C.c_int32, i64p, i64p]
+        L.oracle_classify_matmul.argtypes = [C.c_int32, i64p, C.c_int32, i64p]
+        L.oracle_mm2d_f32.argtypes = [vp, vp, fp, C.c_int, C.POINTER(C.c_int), C.POINTER(C.c_int)]
+        L.oracle_mmnd_f32.argtypes = [vp, vp, fp, C.c_int, i64p, i32p, C.c_int64]
+        L.oracle_result_shape.argtypes = [C.c_int, vp, vp, i64p, i32p]
+        L.oracle_result_shape.restype = C.c_int64
+        L.oracle_mv_f32.argtypes = [vp, vp, fp]
+        L.oracle_vm_f32.argtypes = [vp, vp, fp]
+        L.oracle_mv_backward_f32.argtypes = [vp, vp, fp, fp, fp]
+        L.oracle_vm_backward_f32.argtypes = [vp, vp, fp, fp, fp]
+        L.oracle_dot_f32.argtypes = [vp, vp, fp]
+        L.oracle_sum_over_broadcasted_axes_f32.argtypes = [fp, C.c_int32, i64p, C.c_int32, i64p, fp]
+        L.oracle_mmnd_f64acc.argtypes = [vp, vp, dp, C.c_int]
+        L.oracle_mv_f64acc.argtypes = [vp, vp, dp]
+        L.oracle_vm_f64acc.argtypes = [vp, vp, dp]
+        L.oracle_mlp_create.argtypes = [C.c_int, i64p, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int64]
+        L.oracle_mlp_create.restype = C.c_void_p
+        L.oracle_mlp_destroy.argtypes = [C.c_void_p]
+        L.oracle_mlp_step.argtypes = [C.c_void_p, fp, C.c_void_p, C.c_int64, C.c_float, C.c_int]
+        L.oracle_mlp_step.restype = C.c_float
+        L.oracle_mlp_forward.argtypes = [C.c_void_p, fp, C.c_int64, fp, C.c_int]
+        L.oracle_mlp_get_params.argtypes = [C.c_void_p, C.c_int, fp, fp]
+        L.oracle_mlp_get_grads.argtypes = [C.c_void_p, C.c_int, fp, fp]
+        _lib = L
+    return _lib
+
+
+def _check(rc: int):
+    if rc < 0:
+        raise OracleError(lib().oracle_last_error().decode())
+
+
+def _i64(seq: Sequence[int]):
+    return (C.c_int64 * max(1, len(seq)))(*[int(x) for x in seq])
+
+
+class View:
+    """(storage, offset, shape, strides) in elements over an fp32 numpy buffer."""
+
+    def __init__(self, storage: np.ndarray, offset: int, shape: Sequence[int], strides: Sequence[int]):
+        assert storage.dtype == np.float32 and storage.flags["C_CONTIGUOUS"]
+        assert len(shape) == len(strides) <= MAX_RANK
+        self.storage = storage
+        self.offset = int(offset)
+        self.shape = tuple(int(s) for s in shape)
+        self.strides = tuple(int(s) for s in strides)
+
+    @staticmethod
+    def of(a: np.ndarray) -> "View":
+        a = np.asarray(a)
+        assert a.dtype == np.float32
+        for s in a.strides:
+            assert s % 4 == 0
+        v = View.__new__(View)
+        v.storage = a  # keeps the memory alive; pointer already includes the view's own offset
+        v.offset = 0
+        v.shape = tuple(a.shape)
+        v.strides = tuple(s // 4 for s in a.strides)
+        return v
+
+    @property
+    def rank(self) -> int:
+        return len(self.shape)
+
+    def transpose_last2(self) -> "View":
+        """Swap the two trailing dims as a view (NDBuffer.transpose, tenmo/ndbuffer.mojo:1040-1062)."""
+        v = View.__new__(View)
+        v.storage, v.offset = self.storage, self.offset
+        sh, st = list(self.shape), list(self.strides)
+        sh[-1], sh[-2] = sh[-2], sh[-1]
+        st[-1], st[-2] = st[-2], st[-1]
+        v.shape, v.strides = tuple(sh), tuple(st)
+        return v
+
+    def c(self) -> _CView:
+        cv = _CView()
+        cv.data = self.storage.ctypes.data
+        cv.offset = self.offset
+        cv.rank = self.rank
+        for i, (s, t) in enumerate(zip(self.shape, self.strides)):
+            cv.shape[i] = s
+            cv.strides[i] = t
+        return cv
+
+    def numpy(self) -> np.ndarray:
+        """Materialise the view (test helper)."""
+        base = self.storage.reshape(-1)[self.offset:] if self.offset else self.storage
+        return np.lib.stride_tricks.as_strided(base, self.shape, tuple(4 * s for s in self.strides))
+
+
+def _as_view(x) -> View:
+    return x if isinstance(x, View) else View.of(x)
+
+
+def simd_width() -> int:
+    return lib().oracle_simd_width()
+
+
+def force_simd_width(w: int) -> None:
+    lib().oracle_force_simd_width(int(w))
+
+
+def num_physical_cores() -> int:
+    return lib().oracle_num_physical_cores()
+
+
+def is_contiguous(shape: Sequence[int], strides: Sequence[int]) -> bool:
+    return bool(lib().oracle_is_contiguous(len(shape), _i64(shape), _i64(strides)))
+
+
+def classify_matmul(shape_a: Sequence[int], shape_b: Sequence[int]) -> int:
+    return lib().oracle_classify_matmul(len(shape_a), _i64(shape_a), len(shape_b), _i64(shape_b))
+
+
+def result_shape(mode: int, A, B) -> Tuple[int, ...]:
+    A, B = _as_view(A), _as_view(B)
+    out = (C.c_int64 * (MAX_RANK + 2))()
+    r = C.c_int32()
+    _check(lib().oracle_result_shape(mode, C.byref(A.c()), C.byref(B.c()), out, C.byref(r)))
+    return tuple(out[i] for i in range(r.value))
+
+
+def mm2d(A, B, nthreads: int = 0, info: Optional[dict] = None) -> np.ndarray:
+    """MmCpu2d.tiled_matmul (tenmo/matmul_cpu.mojo:80-135)."""
+    A, B = _as_view(A), _as_view(B)
+    if A.rank != 2 or B.rank != 2 or A.shape[1] != B.shape[0]:
+        out = np.zeros((1,), np.float32)
+    else:
+        out = np.empty((A.shape[0], B.shape[1]), np.float32)
+    path, tiles = C.c_int(), (C.c_int * 3)()
+    _check(lib().oracle_mm2d_f32(C.byref(A.c()), C.byref(B.c()), out.ctypes.data, nthreads, C.byref(path), tiles))
+    if info is not None:
+        info["path"] = path.value
+        info["tiles"] = tuple(tiles)
+    return out
+
+
+def mmnd(A, B, nthreads: int = 0, work_item_limit: int = 0, out: Optional[np.ndarray] = None) -> np.ndarray:
+    """MmCpuNd.tiled_matmul (tenmo/matmul_cpu.mojo:568-625)."""
+    A, B = _as_view(A), _as_view(B)
+    shape = result_shape(MM, A, B)
+    if out is None:
+        out = np.empty(shape, np.float32)
+    _check(lib().oracle_mmnd_f32(C.byref(A.c()), C.byref(B.c()), out.ctypes.data, nthreads, None, None, work_item_limit))
+    return out
+
+
+def matmul(A, B, nthreads: int = 0) -> np.ndarray:
+    """NDBuffer-level dispatch of MatmulNd.forward: rank-2 x rank-2 goes to the 2-D kernel
+    (tenmo/matmul.mojo:151-152), anything else to the batched one."""
+    A, B = _as_view(A), _as_view(B)
+    if A.rank == 2 and B.rank == 2:
+        return mm2d(A, B, nthreads)
+    return mmnd(A, B, nthreads)
+
+
+def mm_f64(A, B, nthreads: int = 0) -> np.ndarray:
+    A, B = _as_view(A), _as_view(B)
+    shape = result_shape(MM, A, B)
+    out = np.empty(shape, np.float64)
+    _check(lib().oracle_mmnd_f64acc(C.byref(A.c()), C.byref(B.c()), out.ctypes.data, nthreads))
+    return out
+
+
+def mv(M, v) -> np.ndarray:
+    M, v = _as_view(M), _as_view(v)
+    if M.rank < 2 or v.rank < 1:
+        _check(lib().oracle_mv_f32(C.byref(M.c()), C.byref(v.c()), None))
+    out = np.empty(result_shape(MV, M, v), np.float32)
+    _check(lib().oracle_mv_f32(C.byref(M.c()), C.byref(v.c()), out.ctypes.data))
+    return out
+
+
+def vm(v, M) -> np.ndarray:
+    v, M = _as_view(v), _as_view(M)
+    if M.rank < 2 or v.rank < 1:
+        _check(lib().oracle_vm_f32(C.byref(v.c()), C.byref(M.c()), None))
+    out = np.empty(result_shape(VM, v, M), np.float32)
+    _check(lib().oracle_vm_f32(C.byref(v.c()), C.byref(M.c()), out.ctypes.data))
+    return out
+
+
+def mv_f64(M, v) -> np.ndarray:
+    M, v = _as_view(M), _as_view(v)
+    out = np.empty(result_shape(MV, M, v), np.float64)
+    _check(lib().oracle_mv_f64acc(C.byref(M.c()), C.byref(v.c()), out.ctypes.data))
+    return out
+
+
+def vm_f64(v, M) -> np.ndarray:
+    v, M = _as_view(v), _as_view(M)
+    out = np.empty(result_shape(VM, v, M), np.float64)
+    _check(lib().oracle_vm_f64acc(C.byref(v.c()), C.byref(M.c()), out.ctypes.data))
+    return out
+
+
+def mv_backward(M, v, dy: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
+    """(dM, dv) at the parents' shapes (tenmo/matrixvector.mojo:19-201)."""
+    M, v = _as_view(M), _as_view(v)
+    dy = np.ascontiguousarray(dy, np.float32)
+    dM, dv = np.empty(M.shape, np.float32), np.empty(v.shape, np.float32)
+    _check(lib().oracle_mv_backward_f32(C.byref(M.c()), C.byref(v.c()), dy.ctypes.data, dM.ctypes.data, dv.ctypes.data))
+    return dM, dv
+
+
+def vm_backward(v, M, dy: np.ndarray) -> Tuple[np.ndarray, np.ndarray]:
+    """(dv, dM) at the parents' shapes (tenmo/vectormatrix.mojo:18-206)."""
+    v, M = _as_view(v), _as_view(M)
+    dy = np.ascontiguousarray(dy, np.float32)
+    dv, dM = np.empty(v.shape, np.float32), np.empty(M.shape, np.float32)
+    _check(lib().oracle_vm_backward_f32(C.byref(v.c()), C.byref(M.c()), dy.ctypes.data, dv.ctypes.data, dM.ctypes.data))
+    return dv, dM
+
+
+def dot(a, b) -> np.float32:
+    a, b = _as_view(a), _as_view(b)
+    out = np.zeros((), np.float32)
+    _check(lib().oracle_dot_f32(C.byref(a.c()), C.byref(b.c()), out.ctypes.data))
+    return out[()]
+
+
+def sum_over_broadcasted_axes(src: np.ndarray, target_shape: Sequence[int]) -> np.ndarray:
+    src = np.ascontiguousarray(src, np.float32)
+    dst = np.empty(tuple(target_shape), np.float32)
+    _check(lib().oracle_sum_over_broadcasted_axes_f32(src.ctypes.data, src.ndim, _i64(src.shape),
+                                                      len(target_shape), _i64(target_shape), dst.ctypes.data))
+    return dst
+
+
+def matmul_backward(A, B, dC: np.ndarray, nthreads: int = 0) -> Tuple[np.ndarray, np.ndarray]:
+    """Matmul2dBackward / MatmulNdBackward (tenmo/matmul.mojo:22-54, :99-137): the two gradient
+    GEMMs on transposed views, then the reduction to each parent's shape."""
+    A, B = _as_view(A), _as_view(B)
+    dCv = View.of(np.ascontiguousarray(dC, np.float32))
+    gA = matmul(dCv, B.transpose_last2(), nthreads)
+    gB = matmul(A.transpose_last2(), dCv, nthreads)
+    if gA.shape != A.shape:
+        gA = sum_over_broadcasted_axes(gA, A.shape)
+    if gB.shape != B.shape:
+        gB = sum_over_broadcasted_axes(gB, B.shape)
+    return gA, gB
+
+
+class MLP:
+    """The 4-layer MLP training step of the MNIST example, restated on the oracle's own matmul."""
+
+    def __init__(self, dims: Sequence[int], weights, biases, max_batch: int):
+        self.dims = [int(d) for d in dims]
+        L = len(dims) - 1
+        self._W = [np.ascontiguousarray(w, np.float32) for w in weights]
+        self._b = [np.ascontiguousarray(b, np.float32) for b in biases]
+        Wp = (C.c_void_p * L)(*[w.ctypes.data for w in self._W])
+        bp = (C.c_void_p * L)(*[b.ctypes.data for b in self._b])
+        self._h = lib().oracle_mlp_create(L, _i64(self.dims), Wp, bp, max_batch)
+        self.L = L
+
+    def __del__(self):
+        if getattr(self, "_h", None):
+            lib().oracle_mlp_destroy(self._h)
+            self._h = None
+
+    def step(self, x: np.ndarray, y: np.ndarray, lr: float, nthreads: int = 0) -> float:
+        x = np.ascontiguousarray(x, np.float32)
+        y = np.ascontiguousarray(y, np.int32)
+        return float(lib().oracle_mlp_step(self._h, x.ctypes.data, y.ctypes.data, x.shape[0], lr, nthreads))
+
+    def forward(self, x: np.ndarray, nthreads: int = 0) -> np.ndarray:
+        x = np.ascontiguousarray(x, np.float32)
+        out = np.empty((x.shape[0], self.dims[-1]), np.float32)
+        _check(lib().oracle_mlp_forward(self._h, x.ctypes.data, x.shape[0], out.ctypes.data, nthreads))
+        return out
+
+    def params(self, layer: int):
+        W = np.empty((self.dims[layer], self.dims[layer + 1]), np.float32)
+        b = np.empty((self.dims[layer + 1],), np.float32)
+        _check(lib().oracle_mlp_get_params(self._h, layer, W.ctypes.data, b.ctypes.data))
+        return W, b
+
+    def grads(self, layer: int):
+        W = np.empty((self.dims[layer], self.dims[layer + 1]), np.float32)
+        b = np.empty((self.dims[layer + 1],), np.float32)
+        _check(lib().oracle_mlp_get_grads(self._h, layer, W.ctypes.data, b.ctypes.data))
+        return W, b
