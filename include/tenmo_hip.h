@@ -1,0 +1,192 @@
+/*
+ * libtenmo_hip.so — MI355X (gfx950) implementation of Tenmo's fp32 matrix-product path.
+ *
+ * C ABI only: plain pointers and sizes, no C++ or framework types.  Every pointer named
+ * "device" is HIP device memory on the GPU selected by tenmo_hip_init(); every size, offset
+ * and stride is in ELEMENTS (fp32), never bytes.  An operand is a view
+ *     element(i, j) = base[offset + sum_d batch_coord[d]*batch_stride[d] + i*row_stride + j*col_stride]
+ * which is the reference's NDBuffer (shape, strides, offset over shared storage).  Strides may
+ * be swapped (transposed view), padded, zero (broadcast) or overlapping; inputs are never written.
+ *
+ * Calls are enqueued on one library stream and return without waiting unless `sync` is
+ * non-zero (the reference enqueues on its DeviceContext and synchronises on demand,
+ * tenmo/kernels/matmul_kernel.mojo:259-277).  All functions return 0 on success or a
+ * negative tenmo_status; they never abort and never throw.  The message of the last failure on
+ * the calling thread is returned by tenmo_hip_last_error() — the text a Mojo caller would put
+ * into `raise Error(msg)`.
+ *
+ * Single caller thread per process is assumed (as in the reference); calls issued from one
+ * thread execute in issue order.
+ */
+#ifndef TENMO_HIP_H
+#define TENMO_HIP_H
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define TENMO_MAX_RANK 8 /* tenmo/mnemonics.mojo:45 (max_rank) */
+
+typedef enum {
+    TENMO_OK = 0,
+    TENMO_ERR_NOT_INITIALIZED = -1,
+    TENMO_ERR_INVALID_SHAPE = -2,   /* where the reference panics / raises on shapes */
+    TENMO_ERR_INVALID_ARGUMENT = -3,
+    TENMO_ERR_HIP = -4,             /* a HIP runtime call failed; message carries hipGetErrorString */
+    TENMO_ERR_UNSUPPORTED = -5
+} tenmo_status;
+
+/* opcodes of tenmo/mnemonics.mojo:26-30 as returned by tenmo_hip_classify_matmul */
+enum { TENMO_OP_DOT = 0, TENMO_OP_VM = 1, TENMO_OP_MV = 2, TENMO_OP_MM = 3, TENMO_OP_INVALID = -1 };
+
+/* NDBuffer as seen by the device code: tenmo/ndbuffer.mojo (shape, strides, offset, storage). */
+typedef struct {
+    const float* data;  /* device pointer to the first element of the STORAGE */
+    int64_t offset;     /* elements */
+    int32_t rank;       /* <= TENMO_MAX_RANK */
+    int64_t shape[TENMO_MAX_RANK];
+    int64_t strides[TENMO_MAX_RANK];
+} tenmo_view;
+
+/* ---- lifetime, stream, errors ------------------------------------------------------------ */
+
+/* Selects the GPU, creates the library stream and its scratch.  Idempotent.
+ * Replaces: DeviceContext(device_id) in tenmo/device.mojo:87-90. */
+int tenmo_hip_init(int device_id);
+int tenmo_hip_shutdown(void);
+/* == DeviceContext.synchronize(), tenmo/kernels/matmul_kernel.mojo:277 */
+int tenmo_hip_sync(void);
+const char* tenmo_hip_last_error(void);
+/* The hipStream_t all work is enqueued on (as void*), and a way to make the library use the
+ * caller's stream instead (NULL restores the library's own). */
+void* tenmo_hip_get_stream(void);
+int tenmo_hip_set_stream(void* hip_stream);
+/* Device facts the caller may want for reporting: number of compute units, name. */
+int tenmo_hip_device_info(int* compute_units, char* name, int name_len);
+/* Overrides of the automatic kernel selection, for measurement: "gemm_tile" (0: 256x128, 1: 128x128,
+ * 2: 64x64 workgroup tile; -1 automatic) and "gemm_splitk" (number of K slices; -1 automatic).  The
+ * environment variables TENMO_HIP_GEMM_TILE / TENMO_HIP_GEMM_SPLITK set the same at init.
+ * No counterpart in the reference, whose tile size is the compile-time TILE_SIZE=32
+ * (tenmo/ndbuffer.mojo:63). */
+int tenmo_hip_set_tuning(const char* name, int value);
+/* Stopwatch on the stream the kernels run on: begin records a HIP event, end records a second
+ * one, waits for it and returns the milliseconds between them (the reference times with
+ * perf_counter_ns around sync=True calls, profile_gpu.mojo:161-258). */
+int tenmo_hip_timer_begin(void);
+int tenmo_hip_timer_end(float* elapsed_ms);
+
+/* ---- kernel-level entry points ------------------------------------------------------------ */
+
+/* C[batch..., M, N] (dense, row-major, caller-allocated: the reference allocates the result with
+ * enqueue_create_buffer, tenmo/kernels/matmul_kernel.mojo:223) = A[.., M, K] . B[.., K, N].
+ * batch_shape is the broadcast result batch shape (rank <= 6); a_/b_batch_strides hold 0 where
+ * that operand's dim is 1 or missing (tenmo/kernels/matmul_kernel.mojo:196-214,
+ * tenmo/matmul_cpu.mojo:710-724).  Offsets ARE applied (CPU semantics, matmul_cpu.mojo:191,197).
+ * accumulate: 0 -> C = A.B (reference semantics); 1 -> C += A.B (fused Gradbox accumulation,
+ * tenmo/gradbox.mojo:1358-1364).
+ * Replaces: matmul_2d_tiled + MatmulNdGpu.launch, tenmo/kernels/matmul_kernel.mojo:38-120,:128-283. */
+int tenmo_hip_gemm_f32(const float* A, int64_t a_off, int64_t a_rs, int64_t a_cs,
+                       const float* B, int64_t b_off, int64_t b_rs, int64_t b_cs,
+                       float* C, int64_t M, int64_t N, int64_t K,
+                       int32_t batch_rank, const int64_t* batch_shape,
+                       const int64_t* a_batch_strides, const int64_t* b_batch_strides,
+                       int32_t accumulate, int32_t sync);
+
+/* out[batch..., m] = Mx[.., m, k] . v[.., k]
+ * Replaces: matrix_vector_nd + MatrixVectorNdGpu.launch, tenmo/kernels/matrixvector_kernel.mojo:13-171
+ * (which assumes dense inner dims; this entry point honours the strides and offset). */
+int tenmo_hip_mv_f32(const float* Mx, int64_t m_off, int64_t m_rs, int64_t m_cs,
+                     const float* v, int64_t v_off, int64_t v_s,
+                     float* out, int64_t m, int64_t k,
+                     int32_t batch_rank, const int64_t* batch_shape,
+                     const int64_t* m_batch_strides, const int64_t* v_batch_strides,
+                     int32_t accumulate, int32_t sync);
+
+/* out[batch..., n] = v[.., k] . Mx[.., k, n]
+ * Replaces: vector_matmul_nd + VectorMatmulNdGpu.launch, tenmo/kernels/vectormatrix_kernel.mojo:13-170. */
+int tenmo_hip_vm_f32(const float* v, int64_t v_off, int64_t v_s,
+                     const float* Mx, int64_t m_off, int64_t m_rs, int64_t m_cs,
+                     float* out, int64_t k, int64_t n,
+                     int32_t batch_rank, const int64_t* batch_shape,
+                     const int64_t* v_batch_strides, const int64_t* m_batch_strides,
+                     int32_t accumulate, int32_t sync);
+
+/* out[0] = sum_i a[i]*b[i]   (a stride of 0 broadcasts a one-element operand,
+ * tenmo/dotproduct.mojo:67-74).  Replaces: DotproductKernel.launch,
+ * tenmo/kernels/dotproduct_kernel.mojo:19-110. */
+int tenmo_hip_dot_f32(const float* a, int64_t a_off, int64_t a_s,
+                      const float* b, int64_t b_off, int64_t b_s,
+                      int64_t n, float* out, int32_t sync);
+
+/* ---- view-level entry points: the bodies of the reference's launch functions -------------- */
+
+/* tenmo/matmul.mojo:258-272 */
+int tenmo_hip_classify_matmul(int32_t rank_a, const int64_t* shape_a, int32_t rank_b, const int64_t* shape_b);
+
+/* Shape of the result of op (TENMO_OP_MM / _MV / _VM) with the reference's validation
+ * (tenmo/kernels/matmul_kernel.mojo:146-177, matrixvector.mojo:213-233, vectormatrix.mojo:218-238);
+ * returns the element count (an empty batch product counts as 1 for MM), or a negative status. */
+int64_t tenmo_hip_result_shape(int32_t op, const tenmo_view* A, const tenmo_view* B,
+                               int64_t* out_shape, int32_t* out_rank);
+
+/* MatmulNdGpu.launch(A, B, sync) — tenmo/kernels/matmul_kernel.mojo:128-283 — with the result
+ * buffer supplied by the caller (dense, tenmo_hip_result_shape elements). */
+int tenmo_hip_matmul_nd(const tenmo_view* A, const tenmo_view* B, float* C, int32_t sync);
+/* MatrixVectorNdGpu.launch — tenmo/kernels/matrixvector_kernel.mojo:80-171 */
+int tenmo_hip_matrix_vector_nd(const tenmo_view* Mx, const tenmo_view* v, float* out, int32_t sync);
+/* VectorMatmulNdGpu.launch — tenmo/kernels/vectormatrix_kernel.mojo:80-170 */
+int tenmo_hip_vector_matmul_nd(const tenmo_view* v, const tenmo_view* Mx, float* out, int32_t sync);
+
+/* Matmul2dBackward / MatmulNdBackward — tenmo/matmul.mojo:22-54, :99-137.
+ * dC is the dense upstream gradient at the result shape.  For each non-NULL grad pointer the
+ * gradient  dA = dC . B^T(view)  /  dB = A^T(view) . dC  is reduced over broadcast batch axes to
+ * that parent's own shape (sum_over_broadcasted_axes, tenmo/sum_mean_reduction.mojo:185-211) and
+ * ADDED into the dense buffer grad_A / grad_B (Ancestor.update_grad(AddTensor),
+ * tenmo/ancestry.mojo:72-105).  Pass NULL for a parent that does not require grad (:34, :45). */
+int tenmo_hip_matmul_backward(const tenmo_view* A, const tenmo_view* B, const float* dC,
+                              float* grad_A, float* grad_B, int32_t sync);
+/* MatrixVectorMulNdBackward — tenmo/matrixvector.mojo:19-201 (CPU-only in the reference):
+ * grad_M += outer(dy, v), grad_v += M^T . dy, both dense at the parents' shapes. */
+int tenmo_hip_mv_backward(const tenmo_view* Mx, const tenmo_view* v, const float* dy,
+                          float* grad_M, float* grad_v, int32_t sync);
+/* VectorMatmulNdBackward — tenmo/vectormatrix.mojo:18-206: grad_v += M . dy, grad_M += outer(v, dy). */
+int tenmo_hip_vm_backward(const tenmo_view* v, const tenmo_view* Mx, const float* dy,
+                          float* grad_v, float* grad_M, int32_t sync);
+
+/* ---- the reference's existing plugin ABI --------------------------------------------------- */
+
+/* Exact CBLAS prototype the reference binds with
+ *   get_function[CBLAS_SGEMM_FN]("cblas_sgemm")      tenmo/blashandle.mojo:136-151, :231, :655
+ * HOST pointers: operands are staged to the GPU, multiplied there, and C is copied back before
+ * the call returns, so `mojo -D BLAS_PATH=/path/libtenmo_hip.so` makes LinearBLAS /
+ * SequentialBLAS / BLASMatmul2dBackward run on the GPU unchanged.  Row- and column-major,
+ * all four transpose cases, alpha/beta honoured.  Initialises device 0 on first use. */
+void cblas_sgemm(int order, int trans_a, int trans_b, int M, int N, int K, float alpha,
+                 const float* A, int lda, const float* B, int ldb, float beta, float* C, int ldc);
+
+/* ---- MLP training-step harness (callers of the path) -------------------------------------- */
+
+/* Linear(x.W + b) -> ReLU -> ... -> Linear -> CrossEntropy(mean) -> backward -> SGD(lr), the step
+ * of examples/mnist.mojo:150-162 over tenmo/net.mojo:179-216, relu.mojo:99-141,
+ * crossentropy.mojo:285-432,:775-793, optim.mojo:93-120.  All GEMMs go through
+ * tenmo_hip_gemm_f32; the element-wise stages are small fused kernels on the same stream.
+ * dims[0..n_layers] are the layer widths; W[l] is [dims[l], dims[l+1]] row-major (the reference
+ * stores weights [in, out], net.mojo:91-97), b[l] is [dims[l+1]]; both HOST arrays, copied in. */
+typedef struct tenmo_mlp tenmo_mlp;
+tenmo_mlp* tenmo_hip_mlp_create(int32_t n_layers, const int64_t* dims,
+                                const float* const* W_host, const float* const* b_host, int64_t max_batch);
+void tenmo_hip_mlp_destroy(tenmo_mlp*);
+/* x: device [batch, dims[0]] dense; y: device int32 [batch].  The mean loss of this step is
+ * written to loss_out[0] (device).  No host synchronisation unless sync != 0. */
+int tenmo_hip_mlp_step(tenmo_mlp*, const float* x, const int32_t* y, int64_t batch, float lr,
+                       float* loss_out, int32_t sync);
+int tenmo_hip_mlp_forward(tenmo_mlp*, const float* x, int64_t batch, float* logits_out, int32_t sync);
+/* copy a layer's parameters / last gradients to HOST arrays (synchronises) */
+int tenmo_hip_mlp_get_params(tenmo_mlp*, int32_t layer, float* W_host, float* b_host);
+int tenmo_hip_mlp_get_grads(tenmo_mlp*, int32_t layer, float* dW_host, float* db_host);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* TENMO_HIP_H */

@@ -1,0 +1,150 @@
+// Small element-wise / reduction kernels around the matrix products: the reduction of a batched
+// gradient to a broadcast parent's shape, outer-product gradients of mv/vm, and the stages of the
+// MLP training-step harness (bias add + ReLU, cross-entropy forward/backward, bias gradient, SGD).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "gemm_mfma.hpp"
+
+namespace tenmo {
+
+// ---- sum_over_broadcasted_axes (tenmo/sum_mean_reduction.mojo:185-211) fused with the
+// Gradbox "+=" (tenmo/gradbox.mojo:1358-1364): dst[parent shape] += sum over the batch dims that
+// the parent broadcast.  src is dense [batch_shape..., inner]; dst is dense at the parent's shape.
+struct BroadcastReduceArgs {
+    const float* src;
+    float* dst;
+    int64_t inner;           // elements of the trailing (non-batch) dims
+    int64_t dst_batch;       // product of the parent's own batch dims
+    int32_t rank;            // result batch rank
+    int64_t shape[MAX_BATCH_RANK];     // result batch shape
+    int64_t src_str[MAX_BATCH_RANK];   // dense strides of src batch dims (in units of `inner`)
+    int32_t kept[MAX_BATCH_RANK];      // 1 where the parent has this dim with size > 1
+    int64_t reduced_total;   // product of the reduced dims
+};
+
+__global__ void broadcast_reduce_add_kernel(const BroadcastReduceArgs g) {
+    const int64_t total = g.dst_batch * g.inner;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t in = idx % g.inner;
+        int64_t pb = idx / g.inner;
+        // kept coordinates -> base offset in src
+        int64_t base = 0;
+        for (int d = g.rank - 1; d >= 0; --d) {
+            if (g.kept[d]) { base += (pb % g.shape[d]) * g.src_str[d]; pb /= g.shape[d]; }
+        }
+        float acc = 0.f;
+        for (int64_t r = 0; r < g.reduced_total; ++r) {
+            int64_t rr = r, off = base;
+            for (int d = g.rank - 1; d >= 0; --d) {
+                if (!g.kept[d]) { off += (rr % g.shape[d]) * g.src_str[d]; rr /= g.shape[d]; }
+            }
+            acc += g.src[off * g.inner + in];
+        }
+        g.dst[idx] += acc;
+    }
+}
+
+// ---- outer-product gradients of mv / vm -------------------------------------------------------
+// grad[b_parent][i][j] += sum over broadcast batches of  p[b][i] * q[b][j]
+// (tenmo/matrixvector.mojo:87-139, tenmo/vectormatrix.mojo:145-201).  One thread per grad element;
+// the loop over batches that map to the same parent element keeps the sum deterministic.
+struct OuterArgs {
+    const float* p; int64_t p_s;   // left factor, element stride; advanced by its offset
+    const float* q; int64_t q_s;   // right factor
+    float* grad;                   // dense [parent batch..., I, J]
+    int64_t I, J;
+    int64_t parent_batch;          // product of the parent's own batch dims
+    int32_t rank;
+    int64_t shape[MAX_BATCH_RANK];
+    int64_t p_str[MAX_BATCH_RANK]; // batch strides of p, q (0 where broadcast)
+    int64_t q_str[MAX_BATCH_RANK];
+    int32_t kept[MAX_BATCH_RANK];  // 1 where the gradient's parent has this batch dim (> 1)
+    int64_t reduced_total;
+};
+
+__global__ void outer_add_kernel(const OuterArgs g) {
+    const int64_t total = g.parent_batch * g.I * g.J;
+    for (int64_t idx = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total; idx += (int64_t)gridDim.x * blockDim.x) {
+        const int64_t j = idx % g.J, i = (idx / g.J) % g.I;
+        int64_t pb = idx / (g.J * g.I);
+        int64_t pbase = 0, qbase = 0;
+        for (int d = g.rank - 1; d >= 0; --d) {
+            if (g.kept[d]) { const int64_t c = pb % g.shape[d]; pb /= g.shape[d]; pbase += c * g.p_str[d]; qbase += c * g.q_str[d]; }
+        }
+        float acc = 0.f;
+        for (int64_t r = 0; r < g.reduced_total; ++r) {
+            int64_t rr = r, po = pbase, qo = qbase;
+            for (int d = g.rank - 1; d >= 0; --d) {
+                if (!g.kept[d]) { const int64_t c = rr % g.shape[d]; rr /= g.shape[d]; po += c * g.p_str[d]; qo += c * g.q_str[d]; }
+            }
+            acc += g.p[po + i * g.p_s] * g.q[qo + j * g.q_s];
+        }
+        g.grad[idx] += acc;
+    }
+}
+
+__global__ void fill_kernel(float* p, int64_t n, float value) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = value;
+}
+
+// ---- MLP harness stages -----------------------------------------------------------------------
+// z[r][c] += b[c]; if relu: z = max(z, 0)   (tenmo/net.mojo:198-201, tenmo/relu.mojo:99-141)
+__global__ void bias_act_kernel(float* __restrict z, const float* __restrict b, int64_t rows, int64_t cols, int relu) {
+    const int64_t total = rows * cols;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        float x = z[i] + b[i % cols];
+        z[i] = (relu && !(x > 0.f)) ? 0.f : x;
+    }
+}
+
+// g[i] = (h[i] > 0) ? g[i] : 0     ReLU backward with the mask recomputed from the activation
+// (mask = x > 0 in tenmo/relu.mojo:120-123; h > 0 exactly when x > 0)
+__global__ void relu_backward_kernel(float* __restrict g, const float* __restrict h, int64_t n) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
+        if (!(h[i] > 0.f)) g[i] = 0.f;
+}
+
+// Fused class-index cross-entropy, mean reduction (tenmo/crossentropy.mojo:285-432) and its
+// gradient (softmax - onehot) / valid_count (:775-793, :451-481).  One thread per row (C is tiny in
+// the harness); per-row losses go to row_loss for the ordered sum below.
+__global__ void cross_entropy_kernel(const float* __restrict logits, const int32_t* __restrict y, int64_t rows, int64_t C,
+                                     float* __restrict dz, float* __restrict row_loss) {
+    const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (r >= rows) return;
+    const float* x = logits + r * C;
+    float mx = -3.402823466e+38f;
+    for (int64_t c = 0; c < C; ++c) mx = fmaxf(mx, x[c]);
+    float sum_exp = 0.f;
+    for (int64_t c = 0; c < C; ++c) sum_exp += expf(x[c] - mx);
+    const float lse = logf(fmaxf(sum_exp, 1e-7f));
+    const int32_t t = y[r];
+    row_loss[r] = -(x[t] - mx - lse);
+    const float inv = 1.f / sum_exp, scale = 1.f / (float)rows;
+    for (int64_t c = 0; c < C; ++c) dz[r * C + c] = (expf(x[c] - mx) * inv - (c == t ? 1.f : 0.f)) * scale;
+}
+
+// loss = (sum of row losses in row order) / rows — the order of the reference's scalar loop
+__global__ void ordered_mean_kernel(const float* __restrict row_loss, int64_t rows, float* __restrict out) {
+    if (blockIdx.x == 0 && threadIdx.x == 0) {
+        float s = 0.f;
+        for (int64_t r = 0; r < rows; ++r) s += row_loss[r];
+        *out = s / (float)rows;
+    }
+}
+
+// db[c] = sum_r g[r][c], rows ascending (tenmo/broadcast.mojo:81-87)
+__global__ void column_sum_kernel(const float* __restrict g, int64_t rows, int64_t cols, float* __restrict db) {
+    const int64_t c = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (c >= cols) return;
+    float s = 0.f;
+    for (int64_t r = 0; r < rows; ++r) s += g[r * cols + c];
+    db[c] = s;
+}
+
+// p -= lr * g   (tenmo/optim.mojo:93-120, no momentum, no weight decay)
+__global__ void sgd_kernel(float* __restrict p, const float* __restrict g, int64_t n, float lr) {
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = p[i] - lr * g[i];
+}
+
+} // namespace tenmo

@@ -1,0 +1,242 @@
+// Memory-bound products for gfx950: matrix x vector, (few rows) x matrix, dot.
+// Every kernel streams the matrix exactly once with 16-byte-per-lane loads and reduces inside the
+// wavefront; none of them can use the matrix cores profitably (<= 8 flop per byte of HBM traffic).
+//
+// Replaces matrix_vector_nd (tenmo/kernels/matrixvector_kernel.mojo:13-77), vector_matmul_nd
+// (tenmo/kernels/vectormatrix_kernel.mojo:13-77) and dot_product (tenmo/kernels/dotproduct_kernel.mojo:19-110).
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "gemm_mfma.hpp"
+
+namespace tenmo {
+
+__device__ __forceinline__ float wave_sum(float x) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) x += __shfl_down(x, off, 64);
+    return x;
+}
+
+struct GemvArgs {
+    const float* Mx;  // advanced by the view offset
+    const float* v;
+    float* out;
+    int64_t m_rs, m_cs, v_s;
+    int64_t rows, k;       // row kernel: out has `rows` entries per batch, k = reduction length
+    int32_t accumulate;
+    BatchDesc batch;       // a_str: matrix batch strides, b_str: vector batch strides
+};
+
+// ---- rows kernel: unit stride along the reduction (row-major matrix . vector) ----------------
+// One wavefront owns R consecutive rows; its 64 lanes walk k in 16-byte steps, so every global
+// load instruction of a row is one contiguous 1 KiB burst.  R rows share each vector load.
+constexpr int MV_WAVES = 4;
+template <int R, int UNROLL>
+__global__ __launch_bounds__(64 * MV_WAVES) void mv_rows_kernel(const GemvArgs g) {
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int64_t row0 = ((int64_t)blockIdx.x * MV_WAVES + wave) * R;
+    if (row0 >= g.rows) return;
+    int64_t m_off, v_off;
+    batch_offsets(g.batch, blockIdx.y, m_off, v_off);
+    const float* __restrict Mb = g.Mx + m_off;
+    const float* __restrict vb = g.v + v_off;
+
+    const float* rowp[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) rowp[r] = Mb + min(row0 + r, g.rows - 1) * g.m_rs; // clamped rows are discarded below
+
+    float acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = 0.f;
+
+    const int64_t k = g.k;
+    const bool v_unit = (g.v_s == 1);
+    constexpr int STEP = 64 * 4;
+    int64_t kk = (int64_t)lane * 4;
+    // main loop: UNROLL independent 16-byte loads per row in flight
+    for (; kk + (int64_t)(UNROLL - 1) * STEP + 3 < k; kk += (int64_t)UNROLL * STEP) {
+        f32x4 mv[UNROLL][R], vv[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) {
+            const int64_t kx = kk + (int64_t)u * STEP;
+#pragma unroll
+            for (int r = 0; r < R; ++r) mv[u][r] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(rowp[r] + kx));
+            if (v_unit) vv[u] = *reinterpret_cast<const f32x4_u*>(vb + kx);
+            else vv[u] = f32x4{vb[kx * g.v_s], vb[(kx + 1) * g.v_s], vb[(kx + 2) * g.v_s], vb[(kx + 3) * g.v_s]};
+        }
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u)
+#pragma unroll
+            for (int r = 0; r < R; ++r) {
+                acc[r] = fmaf(mv[u][r].x, vv[u].x, acc[r]);
+                acc[r] = fmaf(mv[u][r].y, vv[u].y, acc[r]);
+                acc[r] = fmaf(mv[u][r].z, vv[u].z, acc[r]);
+                acc[r] = fmaf(mv[u][r].w, vv[u].w, acc[r]);
+            }
+    }
+    for (; kk < k; kk += STEP) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            if (kk + e < k) {
+                const float x = vb[(kk + e) * g.v_s];
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[r] = fmaf(rowp[r][kk + e], x, acc[r]);
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        const float s = wave_sum(acc[r]);
+        if (lane == 0 && row0 + r < g.rows) {
+            float* o = g.out + (int64_t)blockIdx.y * g.rows + row0 + r;
+            *o = g.accumulate ? *o + s : s;
+        }
+    }
+}
+
+// ---- columns kernel: unit stride across the outputs ((R x k) . (k x n), R <= 8) ---------------
+// out[r][j] = sum_k X[r][k] * Mx[k][j].  A workgroup owns 1024 consecutive columns (one 16-byte
+// load per lane per k row: 1 KiB bursts per wavefront) and one slice of k; the R x slice block of
+// X is staged in LDS and broadcast.  Partial sums of the k slices go to `partial` and are added by
+// colsplit_reduce_kernel, so the result does not depend on scheduling.
+struct ColsArgs {
+    const float* X;   // (R x k) left operand: vector(s); element (r,k) = X[r*x_rs + k*x_ks]
+    const float* Mx;  // (k x n) right operand, unit stride along n, row pitch m_rs
+    float* out;       // dense [batch][R][n]  (or partial [splits][batch][R][n])
+    int64_t x_rs, x_ks, m_rs;
+    int64_t k, n;
+    int32_t rows;     // actual row count (<= R)
+    int32_t accumulate;
+    int32_t k_splits;
+    int64_t k_per_split;
+    BatchDesc batch;  // a_str: X batch strides, b_str: Mx batch strides
+};
+
+constexpr int COLS_THREADS = 256;
+constexpr int COLS_KCHUNK = 128; // k rows staged per LDS refill
+
+template <int R>
+__global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
+    __shared__ float xs[R][COLS_KCHUNK];
+    const int t = threadIdx.x;
+    const int64_t col = ((int64_t)blockIdx.x * COLS_THREADS + t) * 4;
+    const int64_t batch = blockIdx.z;
+    int64_t x_off, m_off;
+    batch_offsets(g.batch, batch, x_off, m_off);
+    const float* __restrict Xb = g.X + x_off;
+    const float* __restrict Mb = g.Mx + m_off;
+
+    const int64_t k_begin = (int64_t)blockIdx.y * g.k_per_split;
+    const int64_t k_end = min(g.k, k_begin + g.k_per_split);
+    const bool full = (col + 3 < g.n);
+    const bool any = (col < g.n);
+
+    f32x4 acc[R];
+#pragma unroll
+    for (int r = 0; r < R; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    for (int64_t kc = k_begin; kc < k_end; kc += COLS_KCHUNK) {
+        const int len = (int)min((int64_t)COLS_KCHUNK, k_end - kc);
+        __syncthreads();
+        for (int idx = t; idx < R * COLS_KCHUNK; idx += COLS_THREADS) {
+            const int r = idx / COLS_KCHUNK, kk = idx % COLS_KCHUNK;
+            xs[r][kk] = (r < g.rows && kk < len) ? Xb[(int64_t)r * g.x_rs + (kc + kk) * g.x_ks] : 0.f;
+        }
+        __syncthreads();
+        if (full) {
+            const float* __restrict p = Mb + kc * g.m_rs + col;
+            int kk = 0;
+            for (; kk + 4 <= len; kk += 4) {
+                f32x4 m0 = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(p + (int64_t)(kk + 0) * g.m_rs));
+                f32x4 m1 = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(p + (int64_t)(kk + 1) * g.m_rs));
+                f32x4 m2 = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(p + (int64_t)(kk + 2) * g.m_rs));
+                f32x4 m3 = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(p + (int64_t)(kk + 3) * g.m_rs));
+#pragma unroll
+                for (int r = 0; r < R; ++r) {
+                    acc[r] += m0 * xs[r][kk + 0];
+                    acc[r] += m1 * xs[r][kk + 1];
+                    acc[r] += m2 * xs[r][kk + 2];
+                    acc[r] += m3 * xs[r][kk + 3];
+                }
+            }
+            for (; kk < len; ++kk) {
+                f32x4 m0 = *reinterpret_cast<const f32x4_u*>(p + (int64_t)kk * g.m_rs);
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[r] += m0 * xs[r][kk];
+            }
+        } else if (any) {
+            for (int kk = 0; kk < len; ++kk) {
+                const float* p = Mb + (kc + kk) * g.m_rs + col;
+                f32x4 m0 = {0.f, 0.f, 0.f, 0.f};
+                m0.x = p[0];
+                if (col + 1 < g.n) m0.y = p[1];
+                if (col + 2 < g.n) m0.z = p[2];
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[r] += m0 * xs[r][kk];
+            }
+        }
+    }
+    if (!any) return;
+    const bool to_partial = g.k_splits > 1;
+    float* __restrict ob = g.out + ((to_partial ? (int64_t)blockIdx.y * gridDim.z : 0) + batch) * g.rows * g.n;
+    const bool accumulate = g.accumulate && !to_partial;
+#pragma unroll
+    for (int r = 0; r < R; ++r) {
+        if (r >= g.rows) break;
+        float* o = ob + (int64_t)r * g.n + col;
+        if (full) {
+            f32x4 v = acc[r];
+            if (accumulate) v += *reinterpret_cast<const f32x4_u*>(o);
+            *reinterpret_cast<f32x4_u*>(o) = v;
+        } else {
+            const float a[4] = {acc[r].x, acc[r].y, acc[r].z, acc[r].w};
+            for (int e = 0; e < 4; ++e)
+                if (col + e < g.n) o[e] = accumulate ? o[e] + a[e] : a[e];
+        }
+    }
+}
+
+// ---- generic kernel: any strides, one thread per output (correct, not fast) -------------------
+__global__ void mv_generic_kernel(const GemvArgs g) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= g.rows) return;
+    int64_t m_off, v_off;
+    batch_offsets(g.batch, blockIdx.y, m_off, v_off);
+    const float* Mb = g.Mx + m_off + i * g.m_rs;
+    const float* vb = g.v + v_off;
+    float acc = 0.f;
+    for (int64_t j = 0; j < g.k; ++j) acc = fmaf(Mb[j * g.m_cs], vb[j * g.v_s], acc);
+    float* o = g.out + (int64_t)blockIdx.y * g.rows + i;
+    *o = g.accumulate ? *o + acc : acc;
+}
+
+// ---- dot ---------------------------------------------------------------------------------------
+constexpr int DOT_THREADS = 256;
+__device__ __forceinline__ float block_sum(float x) {
+    __shared__ float part[DOT_THREADS / 64];
+    x = wave_sum(x);
+    if ((threadIdx.x & 63) == 0) part[threadIdx.x >> 6] = x;
+    __syncthreads();
+    float s = 0.f;
+    if (threadIdx.x == 0)
+        for (int w = 0; w < DOT_THREADS / 64; ++w) s += part[w];
+    return s; // valid on thread 0
+}
+
+__global__ __launch_bounds__(DOT_THREADS) void dot_partial_kernel(const float* __restrict a, int64_t a_s, const float* __restrict b, int64_t b_s,
+                                                                  int64_t n, float* __restrict partial) {
+    float acc = 0.f;
+    const int64_t stride = (int64_t)gridDim.x * DOT_THREADS;
+    for (int64_t i = (int64_t)blockIdx.x * DOT_THREADS + threadIdx.x; i < n; i += stride) acc = fmaf(a[i * a_s], b[i * b_s], acc);
+    const float s = block_sum(acc);
+    if (threadIdx.x == 0) partial[blockIdx.x] = s;
+}
+
+__global__ __launch_bounds__(DOT_THREADS) void dot_final_kernel(const float* __restrict partial, int nparts, float* __restrict out) {
+    float acc = 0.f;
+    for (int i = threadIdx.x; i < nparts; i += DOT_THREADS) acc += partial[i];
+    const float s = block_sum(acc);
+    if (threadIdx.x == 0) *out = s;
+}
+
+} // namespace tenmo

@@ -1,0 +1,1040 @@
+// libtenmo_hip.so — host side of the C ABI declared in include/tenmo_hip.h.
+//
+// Shape validation, broadcast-batch resolution and kernel selection happen here; the arithmetic is
+// in gemm_mfma.hpp (matrix cores), gemv.hpp (HBM-bound products) and elementwise.hpp.
+// This file is what the bodies of the reference's launch functions become:
+//   MatmulNdGpu.launch          tenmo/kernels/matmul_kernel.mojo:128-283
+//   MatrixVectorNdGpu.launch    tenmo/kernels/matrixvector_kernel.mojo:80-171
+//   VectorMatmulNdGpu.launch    tenmo/kernels/vectormatrix_kernel.mojo:80-170
+// plus the backward entries that the reference runs through the same launches
+// (tenmo/matmul.mojo:22-54, :99-137) and the CBLAS prototype it already binds
+// (tenmo/blashandle.mojo:136-151).
+#include <hip/hip_runtime.h>
+
+#include <algorithm>
+#include <cstdarg>
+#include <cstdio>
+#include <cstdlib>
+#include <cstring>
+#include <mutex>
+#include <string>
+#include <vector>
+
+#include "../../include/tenmo_hip.h"
+#include "elementwise.hpp"
+#include "gemm_mfma.hpp"
+#include "gemv.hpp"
+
+using namespace tenmo;
+
+namespace {
+
+thread_local std::string t_err;
+
+int fail(int code, const char* fmt, ...) {
+    char buf[1024];
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(buf, sizeof buf, fmt, ap);
+    va_end(ap);
+    t_err = buf;
+    return code;
+}
+
+#define HIP_TRY(expr)                                                                              \
+    do {                                                                                           \
+        hipError_t e_ = (expr);                                                                    \
+        if (e_ != hipSuccess) return fail(TENMO_ERR_HIP, "%s failed: %s", #expr, hipGetErrorString(e_)); \
+    } while (0)
+
+struct State {
+    bool ready = false;
+    int device = -1;
+    int cus = 0;
+    std::string name;
+    hipStream_t own_stream = nullptr;
+    hipStream_t stream = nullptr;
+    // grow-only device scratch: split-K / column-split partials, batched gradients before reduction
+    float* ws = nullptr;
+    size_t ws_bytes = 0;
+    // second scratch, for results that must outlive a kernel which itself uses `ws`
+    float* ws2 = nullptr;
+    size_t ws2_bytes = 0;
+    // staging buffers of the host-pointer CBLAS entry point
+    float* stage[3] = {nullptr, nullptr, nullptr};
+    size_t stage_bytes[3] = {0, 0, 0};
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    // tuning overrides (environment, read once): -1 = automatic
+    int force_tile = -1;
+    int force_splitk = -1;
+};
+State S;
+std::mutex S_mu;
+
+int env_int(const char* name, int dflt) {
+    const char* v = getenv(name);
+    return v && *v ? atoi(v) : dflt;
+}
+
+int ensure_ready() {
+    if (!S.ready) return fail(TENMO_ERR_NOT_INITIALIZED, "tenmo_hip: not initialised, call tenmo_hip_init(device_id) first");
+    return 0;
+}
+
+int workspace(size_t bytes, float** out) {
+    if (bytes > S.ws_bytes) {
+        if (S.ws) {
+            HIP_TRY(hipStreamSynchronize(S.stream));
+            HIP_TRY(hipFree(S.ws));
+            S.ws = nullptr; S.ws_bytes = 0;
+        }
+        size_t want = std::max(bytes, (size_t)64 << 20);
+        HIP_TRY(hipMalloc(&S.ws, want));
+        S.ws_bytes = want;
+    }
+    *out = S.ws;
+    return 0;
+}
+
+int workspace2(size_t bytes, float** out) {
+    if (bytes > S.ws2_bytes) {
+        if (S.ws2) {
+            HIP_TRY(hipStreamSynchronize(S.stream));
+            HIP_TRY(hipFree(S.ws2));
+            S.ws2 = nullptr; S.ws2_bytes = 0;
+        }
+        HIP_TRY(hipMalloc(&S.ws2, bytes));
+        S.ws2_bytes = bytes;
+    }
+    *out = S.ws2;
+    return 0;
+}
+
+int finish(int32_t sync) {
+    HIP_TRY(hipGetLastError());
+    if (sync) HIP_TRY(hipStreamSynchronize(S.stream));
+    return 0;
+}
+
+std::string shape_str(const int64_t* s, int r) {
+    std::string o = "(";
+    for (int i = 0; i < r; ++i) o += (i ? ", " : "") + std::to_string(s[i]);
+    return o + ")";
+}
+
+int64_t product(const int64_t* s, int r) {
+    int64_t p = 1;
+    for (int i = 0; i < r; ++i) p *= s[i];
+    return p;
+}
+
+int fill_batch(BatchDesc& bd, int32_t rank, const int64_t* shape, const int64_t* a_str, const int64_t* b_str, int64_t* count) {
+    if (rank < 0 || rank > MAX_BATCH_RANK) return fail(TENMO_ERR_INVALID_ARGUMENT, "batch rank %d outside 0..%d", rank, MAX_BATCH_RANK);
+    if (rank > 0 && (!shape || !a_str || !b_str)) return fail(TENMO_ERR_INVALID_ARGUMENT, "batch_rank > 0 needs batch_shape and both batch stride arrays");
+    bd.rank = rank;
+    int64_t n = 1;
+    for (int d = 0; d < MAX_BATCH_RANK; ++d) {
+        bd.shape[d] = d < rank ? shape[d] : 1;
+        bd.a_str[d] = d < rank ? a_str[d] : 0;
+        bd.b_str[d] = d < rank ? b_str[d] : 0;
+        if (d < rank) {
+            if (shape[d] < 0) return fail(TENMO_ERR_INVALID_SHAPE, "negative batch dim");
+            n *= shape[d];
+        }
+    }
+    *count = n;
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// GEMM dispatch
+// ------------------------------------------------------------------------------------------------
+
+int operand_mode(int64_t row_stride, int64_t k_stride, int64_t rows, int64_t K) {
+    if (k_stride == 1) return KMAJOR_VEC;
+    if (row_stride == 1) return MNMAJOR_VEC;
+    if (K == 1) return KMAJOR_VEC;     // the k stride is never used
+    if (rows == 1) return MNMAJOR_VEC; // the row stride is never used
+    return KMAJOR_GEN;
+}
+
+template <int BM, int BN, int AM, int BMo>
+void launch_gemm_variant(const GemmArgs& g, dim3 grid) {
+    hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, AM, BMo>), grid, dim3(GEMM_THREADS), 0, S.stream, g);
+}
+
+template <int BM, int BN>
+int launch_gemm_tile(const GemmArgs& g, dim3 grid, int am, int bm) {
+#define TENMO_CASE(A_, B_) if (am == A_ && bm == B_) { launch_gemm_variant<BM, BN, A_, B_>(g, grid); return 0; }
+    TENMO_CASE(KMAJOR_VEC, KMAJOR_VEC) TENMO_CASE(KMAJOR_VEC, MNMAJOR_VEC) TENMO_CASE(KMAJOR_VEC, KMAJOR_GEN)
+    TENMO_CASE(MNMAJOR_VEC, KMAJOR_VEC) TENMO_CASE(MNMAJOR_VEC, MNMAJOR_VEC) TENMO_CASE(MNMAJOR_VEC, KMAJOR_GEN)
+    TENMO_CASE(KMAJOR_GEN, KMAJOR_VEC) TENMO_CASE(KMAJOR_GEN, MNMAJOR_VEC) TENMO_CASE(KMAJOR_GEN, KMAJOR_GEN)
+#undef TENMO_CASE
+    return fail(TENMO_ERR_UNSUPPORTED, "no GEMM variant for operand modes %d/%d", am, bm);
+}
+
+struct TileShape { int bm, bn; };
+const TileShape kTiles[3] = {{256, 128}, {128, 128}, {64, 64}};
+
+int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, int64_t b_rs, int64_t b_cs, float* C,
+                  int64_t M, int64_t N, int64_t K, const BatchDesc& bd, int64_t batch_count, int accumulate) {
+    if (M == 0 || N == 0 || batch_count == 0) return 0;
+    if (K == 0) { // empty reduction: the reference's zero-initialised result
+        if (!accumulate) {
+            const int64_t n = batch_count * M * N;
+            hipLaunchKernelGGL(fill_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 65535)), dim3(256), 0, S.stream, C, n, 0.f);
+        }
+        return 0;
+    }
+    GemmArgs g{};
+    g.A = A; g.B = B; g.C = C;
+    g.a_rs = a_rs; g.a_cs = a_cs; g.b_rs = b_rs; g.b_cs = b_cs;
+    g.M = M; g.N = N; g.K = K;
+    g.accumulate = accumulate;
+    g.batch = bd;
+    g.batch_count = batch_count;
+    const int am = operand_mode(a_rs, a_cs, M, K);
+    const int bm = operand_mode(b_cs, b_rs, N, K);
+
+    // tile: the largest whose grid still fills the chip
+    auto blocks = [&](int t) { return ((M + kTiles[t].bm - 1) / kTiles[t].bm) * ((N + kTiles[t].bn - 1) / kTiles[t].bn) * batch_count; };
+    int tile = 2;
+    if (blocks(0) >= (int64_t)S.cus * 3 / 2) tile = 0;
+    else if (blocks(1) >= (int64_t)S.cus) tile = 1;
+    if (S.force_tile >= 0 && S.force_tile < 3) tile = S.force_tile;
+
+    // split K when even the chosen tile leaves most of the chip idle and K is long
+    int splits = 1;
+    const int64_t nb = blocks(tile);
+    if (nb < S.cus && K >= 1024) {
+        splits = (int)std::min<int64_t>({(2 * (int64_t)S.cus + nb - 1) / nb, K / 256, (int64_t)32});
+        if (splits < 1) splits = 1;
+    }
+    if (S.force_splitk > 0) splits = S.force_splitk;
+    g.k_splits = splits;
+    g.k_per_split = K;
+    if (splits > 1) {
+        int64_t per = (K + splits - 1) / splits;
+        per = (per + GEMM_BK - 1) / GEMM_BK * GEMM_BK;
+        g.k_per_split = per;
+        splits = (int)((K + per - 1) / per);
+        g.k_splits = splits;
+    }
+    if (splits > 1) {
+        float* ws;
+        if (int rc = workspace((size_t)splits * batch_count * M * N * sizeof(float), &ws)) return rc;
+        g.partial = ws;
+    }
+    g.tiles_m = (int32_t)((M + kTiles[tile].bm - 1) / kTiles[tile].bm);
+    g.tiles_n = (int32_t)((N + kTiles[tile].bn - 1) / kTiles[tile].bn);
+    if (nb > 0x7fffffffLL) return fail(TENMO_ERR_UNSUPPORTED, "grid too large");
+    dim3 grid((unsigned)nb, (unsigned)splits, 1);
+    int rc = 0;
+    switch (tile) {
+        case 0: rc = launch_gemm_tile<256, 128>(g, grid, am, bm); break;
+        case 1: rc = launch_gemm_tile<128, 128>(g, grid, am, bm); break;
+        default: rc = launch_gemm_tile<64, 64>(g, grid, am, bm); break;
+    }
+    if (rc) return rc;
+    if (splits > 1) {
+        const int64_t n = batch_count * M * N;
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
+                           g.partial, C, n, splits, accumulate);
+    }
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// mv / vm dispatch.  Both reduce to two streaming kernels chosen by which matrix dim has unit stride:
+//   rows kernel : unit stride along the reduction  -> one wavefront per few outputs
+//   cols kernel : unit stride along the outputs    -> one lane per four outputs, k split over blocks
+// ------------------------------------------------------------------------------------------------
+
+// out[b][i] = sum_j Mat[b](i, j) * vec[b](j), i < n_out, j < n_red;  Mat(i,j) = Mx[i*out_s + j*red_s]
+int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* vec, int64_t v_s, float* out,
+                    int64_t n_out, int64_t n_red, const BatchDesc& bd_mat_vec, int64_t batch_count, int accumulate) {
+    if (n_out == 0 || batch_count == 0) return 0;
+    if (batch_count > 65535) return fail(TENMO_ERR_UNSUPPORTED, "more than 65535 batches in mv/vm");
+    if (n_red == 0) {
+        if (!accumulate) {
+            const int64_t n = batch_count * n_out;
+            hipLaunchKernelGGL(fill_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 65535)), dim3(256), 0, S.stream, out, n, 0.f);
+        }
+        return 0;
+    }
+    if (red_s == 1 || n_red == 1) {
+        GemvArgs g{};
+        g.Mx = Mx; g.v = vec; g.out = out;
+        g.m_rs = out_s; g.m_cs = 1; g.v_s = v_s; g.rows = n_out; g.k = n_red; g.accumulate = accumulate; g.batch = bd_mat_vec;
+        if (n_red == 1 && red_s != 1) { // degenerate: a single product per output
+            g.m_cs = red_s;
+            hipLaunchKernelGGL(mv_generic_kernel, dim3((unsigned)((n_out + 255) / 256), (unsigned)batch_count), dim3(256), 0, S.stream, g);
+            return 0;
+        }
+        // fewer rows per wavefront when the matrix is short, so the grid still covers the chip
+        const int64_t waves4 = (n_out + 3) / 4;
+        if (waves4 >= (int64_t)S.cus * 8) {
+            hipLaunchKernelGGL((mv_rows_kernel<4, 2>), dim3((unsigned)((n_out + 4 * MV_WAVES - 1) / (4 * MV_WAVES)), (unsigned)batch_count), dim3(64 * MV_WAVES), 0, S.stream, g);
+        } else if (n_out >= (int64_t)S.cus * 8) {
+            hipLaunchKernelGGL((mv_rows_kernel<2, 4>), dim3((unsigned)((n_out + 2 * MV_WAVES - 1) / (2 * MV_WAVES)), (unsigned)batch_count), dim3(64 * MV_WAVES), 0, S.stream, g);
+        } else {
+            hipLaunchKernelGGL((mv_rows_kernel<1, 4>), dim3((unsigned)((n_out + MV_WAVES - 1) / MV_WAVES), (unsigned)batch_count), dim3(64 * MV_WAVES), 0, S.stream, g);
+        }
+        return 0;
+    }
+    if (out_s == 1 || n_out == 1) {
+        if (n_out == 1 && out_s != 1) {
+            GemvArgs g{};
+            g.Mx = Mx; g.v = vec; g.out = out;
+            g.m_rs = out_s; g.m_cs = red_s; g.v_s = v_s; g.rows = n_out; g.k = n_red; g.accumulate = accumulate; g.batch = bd_mat_vec;
+            hipLaunchKernelGGL(mv_generic_kernel, dim3(1, (unsigned)batch_count), dim3(256), 0, S.stream, g);
+            return 0;
+        }
+        ColsArgs c{};
+        c.X = vec; c.Mx = Mx; c.out = out;
+        c.x_rs = 0; c.x_ks = v_s; c.m_rs = red_s; c.k = n_red; c.n = n_out; c.rows = 1; c.accumulate = accumulate;
+        // in ColsArgs the X operand uses a_str and the matrix b_str: swap relative to (matrix, vector)
+        c.batch = bd_mat_vec;
+        for (int d = 0; d < MAX_BATCH_RANK; ++d) std::swap(c.batch.a_str[d], c.batch.b_str[d]);
+        const int64_t col_blocks = (n_out + COLS_THREADS * 4 - 1) / (COLS_THREADS * 4);
+        int64_t splits = 1;
+        const int64_t want = (int64_t)S.cus * 8;
+        if (col_blocks * batch_count < want) splits = std::min<int64_t>((want + col_blocks * batch_count - 1) / (col_blocks * batch_count), (n_red + COLS_KCHUNK - 1) / COLS_KCHUNK);
+        splits = std::max<int64_t>(1, std::min<int64_t>(splits, 65535));
+        int64_t per = (n_red + splits - 1) / splits;
+        per = (per + COLS_KCHUNK - 1) / COLS_KCHUNK * COLS_KCHUNK;
+        splits = (n_red + per - 1) / per;
+        c.k_splits = (int32_t)splits; c.k_per_split = per;
+        float* target = out;
+        if (splits > 1) {
+            float* ws;
+            if (int rc = workspace((size_t)splits * batch_count * n_out * sizeof(float), &ws)) return rc;
+            target = ws;
+        }
+        c.out = target;
+        hipLaunchKernelGGL((cols_kernel<1>), dim3((unsigned)col_blocks, (unsigned)splits, (unsigned)batch_count), dim3(COLS_THREADS), 0, S.stream, c);
+        if (splits > 1) {
+            const int64_t n = batch_count * n_out;
+            hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
+                               target, out, n, (int)splits, accumulate);
+        }
+        return 0;
+    }
+    GemvArgs g{};
+    g.Mx = Mx; g.v = vec; g.out = out;
+    g.m_rs = out_s; g.m_cs = red_s; g.v_s = v_s; g.rows = n_out; g.k = n_red; g.accumulate = accumulate; g.batch = bd_mat_vec;
+    hipLaunchKernelGGL(mv_generic_kernel, dim3((unsigned)((n_out + 255) / 256), (unsigned)batch_count), dim3(256), 0, S.stream, g);
+    return 0;
+}
+
+// skinny GEMM: M <= 8 rows against a row-major B — the matrix is streamed once, like vm
+template <int R>
+void launch_cols(const ColsArgs& c, dim3 grid) { hipLaunchKernelGGL((cols_kernel<R>), grid, dim3(COLS_THREADS), 0, S.stream, c); }
+
+int skinny_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, int64_t b_rs, float* C,
+                    int64_t M, int64_t N, int64_t K, const BatchDesc& bd, int64_t batch_count, int accumulate) {
+    ColsArgs c{};
+    c.X = A; c.Mx = B; c.x_rs = a_rs; c.x_ks = a_cs; c.m_rs = b_rs; c.k = K; c.n = N; c.rows = (int32_t)M; c.accumulate = accumulate;
+    c.batch = bd;
+    const int64_t col_blocks = (N + COLS_THREADS * 4 - 1) / (COLS_THREADS * 4);
+    int64_t splits = 1;
+    const int64_t want = (int64_t)S.cus * 8;
+    if (col_blocks * batch_count < want) splits = std::min<int64_t>((want + col_blocks * batch_count - 1) / (col_blocks * batch_count), (K + COLS_KCHUNK - 1) / COLS_KCHUNK);
+    splits = std::max<int64_t>(1, std::min<int64_t>(splits, 65535));
+    int64_t per = (K + splits - 1) / splits;
+    per = (per + COLS_KCHUNK - 1) / COLS_KCHUNK * COLS_KCHUNK;
+    splits = (K + per - 1) / per;
+    c.k_splits = (int32_t)splits; c.k_per_split = per;
+    float* target = C;
+    if (splits > 1) {
+        float* ws;
+        if (int rc = workspace((size_t)splits * batch_count * M * N * sizeof(float), &ws)) return rc;
+        target = ws;
+    }
+    c.out = target;
+    dim3 grid((unsigned)col_blocks, (unsigned)splits, (unsigned)batch_count);
+    if (M <= 1) launch_cols<1>(c, grid);
+    else if (M <= 2) launch_cols<2>(c, grid);
+    else if (M <= 4) launch_cols<4>(c, grid);
+    else launch_cols<8>(c, grid);
+    if (splits > 1) {
+        const int64_t n = batch_count * M * N;
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
+                           target, C, n, (int)splits, accumulate);
+    }
+    return 0;
+}
+
+// ------------------------------------------------------------------------------------------------
+// view helpers
+// ------------------------------------------------------------------------------------------------
+
+int check_view(const tenmo_view* v, const char* who) {
+    if (!v) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: null view", who);
+    if (v->rank < 0 || v->rank > TENMO_MAX_RANK) return fail(TENMO_ERR_INVALID_SHAPE, "%s: rank %d exceeds max_rank %d", who, v->rank, TENMO_MAX_RANK);
+    for (int d = 0; d < v->rank; ++d)
+        if (v->shape[d] < 0) return fail(TENMO_ERR_INVALID_SHAPE, "%s: negative dimension", who);
+    return 0;
+}
+
+// right-aligned broadcast (tenmo/broadcasthelper.mojo:33-62)
+bool broadcast_batch(const int64_t* sa, int ra, const int64_t* sb, int rb, int64_t* out, int* rout) {
+    const int r = std::max(ra, rb);
+    for (int d = 0; d < r; ++d) {
+        const int ia = d - (r - ra), ib = d - (r - rb);
+        const int64_t da = ia >= 0 ? sa[ia] : 1, db = ib >= 0 ? sb[ib] : 1;
+        if (da == db) out[d] = da;
+        else if (da == 1) out[d] = db;
+        else if (db == 1) out[d] = da;
+        else return false;
+    }
+    *rout = r;
+    return true;
+}
+
+// strides an operand contributes to the result batch dims: 0 where its dim is 1 or missing
+void batch_strides_of(const tenmo_view* v, int own_batch_rank, int result_batch_rank, int64_t* out) {
+    for (int d = 0; d < result_batch_rank; ++d) {
+        const int od = d - (result_batch_rank - own_batch_rank);
+        out[d] = (od >= 0 && v->shape[od] > 1) ? v->strides[od] : 0;
+    }
+}
+
+struct Geometry {
+    int64_t oshape[TENMO_MAX_RANK + 2];
+    int32_t orank;
+    int batch_rank;
+    int64_t batch_count;
+};
+
+// trailing dims: MM (2,2), MV (2,1), VM (1,2)
+int resolve(int op, const tenmo_view* A, const tenmo_view* B, Geometry* g, const char* who) {
+    if (int rc = check_view(A, who)) return rc;
+    if (int rc = check_view(B, who)) return rc;
+    const int ta = op == TENMO_OP_VM ? 1 : 2, tb = op == TENMO_OP_MV ? 1 : 2;
+    if (op == TENMO_OP_MM) {
+        if (A->rank < 2) return fail(TENMO_ERR_INVALID_SHAPE, "MatmulNdGpu: A must have rank >= 2");
+        if (B->rank < 2) return fail(TENMO_ERR_INVALID_SHAPE, "MatmulNdGpu: B must have rank >= 2");
+    } else if (op == TENMO_OP_MV) {
+        if (A->rank < 2) return fail(TENMO_ERR_INVALID_SHAPE, "MatrixVectorMulNd: matrix must have at least 2 dimensions");
+        if (B->rank < 1) return fail(TENMO_ERR_INVALID_SHAPE, "MatrixVectorMulNd: vector must have at least 1 dimension");
+    } else if (op == TENMO_OP_VM) {
+        if (A->rank < 1) return fail(TENMO_ERR_INVALID_SHAPE, "VectorMatmulNd: vector must have rank >= 1");
+        if (B->rank < 2) return fail(TENMO_ERR_INVALID_SHAPE, "VectorMatmulNd: matrix must have rank >= 2");
+    } else {
+        return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: unknown op %d", who, op);
+    }
+    const int64_t ka = A->shape[A->rank - 1], kb = B->shape[B->rank - tb];
+    if (ka != kb) {
+        if (op == TENMO_OP_MM) return fail(TENMO_ERR_INVALID_SHAPE, "MatmulNdGpu: inner dims must match, got %lld and %lld", (long long)ka, (long long)kb);
+        if (op == TENMO_OP_MV) return fail(TENMO_ERR_INVALID_SHAPE, "MatrixVectorMulNd: inner dimensions must match");
+        return fail(TENMO_ERR_INVALID_SHAPE, "VectorMatmulNd: inner dimensions must match");
+    }
+    int br = 0;
+    if (!broadcast_batch(A->shape, A->rank - ta, B->shape, B->rank - tb, g->oshape, &br))
+        return fail(TENMO_ERR_INVALID_SHAPE, "ShapeBroadcaster -> broadcast_shape - cannot broadcast shapes: %s, %s",
+                    shape_str(A->shape, A->rank - ta).c_str(), shape_str(B->shape, B->rank - tb).c_str());
+    if (br > MAX_BATCH_RANK) return fail(TENMO_ERR_INVALID_SHAPE, "%s: result rank exceeds max_rank %d", who, TENMO_MAX_RANK);
+    g->batch_rank = br;
+    g->batch_count = product(g->oshape, br);
+    if (op != TENMO_OP_VM) g->oshape[br++] = A->shape[A->rank - 2];
+    if (op != TENMO_OP_MV) g->oshape[br++] = B->shape[B->rank - 1];
+    g->orank = br;
+    return 0;
+}
+
+BatchDesc make_batch(const Geometry& g, const tenmo_view* A, int ta, const tenmo_view* B, int tb) {
+    BatchDesc bd{};
+    bd.rank = g.batch_rank;
+    int64_t as[MAX_BATCH_RANK] = {0}, bs[MAX_BATCH_RANK] = {0};
+    batch_strides_of(A, A->rank - ta, g.batch_rank, as);
+    batch_strides_of(B, B->rank - tb, g.batch_rank, bs);
+    for (int d = 0; d < MAX_BATCH_RANK; ++d) {
+        bd.shape[d] = d < g.batch_rank ? g.oshape[d] : 1;
+        bd.a_str[d] = d < g.batch_rank ? as[d] : 0;
+        bd.b_str[d] = d < g.batch_rank ? bs[d] : 0;
+    }
+    return bd;
+}
+
+tenmo_view transposed_last2(const tenmo_view* v) {
+    tenmo_view t = *v;
+    std::swap(t.shape[t.rank - 1], t.shape[t.rank - 2]);
+    std::swap(t.strides[t.rank - 1], t.strides[t.rank - 2]);
+    return t;
+}
+
+tenmo_view dense_view(const float* p, const int64_t* shape, int rank) {
+    tenmo_view v{};
+    v.data = p; v.offset = 0; v.rank = rank;
+    int64_t acc = 1;
+    for (int d = rank - 1; d >= 0; --d) { v.shape[d] = shape[d]; v.strides[d] = acc; acc *= shape[d]; }
+    return v;
+}
+
+int matmul_views(const tenmo_view* A, const tenmo_view* B, float* C, int accumulate, const char* who) {
+    Geometry g;
+    if (int rc = resolve(TENMO_OP_MM, A, B, &g, who)) return rc;
+    int64_t batch_count = g.batch_count;
+    if (batch_count == 0) return 0; // no output elements (the reference only widens the loop count, matmul_cpu.mojo:666-667)
+    const BatchDesc bd = make_batch(g, A, 2, B, 2);
+    const int64_t M = A->shape[A->rank - 2], K = A->shape[A->rank - 1], N = B->shape[B->rank - 1];
+    const float* Ap = A->data + A->offset;
+    const float* Bp = B->data + B->offset;
+    const int64_t a_rs = A->strides[A->rank - 2], a_cs = A->strides[A->rank - 1];
+    const int64_t b_rs = B->strides[B->rank - 2], b_cs = B->strides[B->rank - 1];
+    if (M <= 8 && (b_cs == 1 || N == 1) && N >= 2048 && K > 0)
+        return skinny_dispatch(Ap, a_rs, a_cs, Bp, b_rs, C, M, N, K, bd, batch_count, accumulate);
+    return gemm_dispatch(Ap, a_rs, a_cs, Bp, b_rs, b_cs, C, M, N, K, bd, batch_count, accumulate);
+}
+
+// dst (dense, parent's shape) += sum over the batch dims of `full` that the parent broadcast
+int reduce_to_parent(const float* full, const Geometry& g, const tenmo_view* parent, int trailing, float* dst) {
+    BroadcastReduceArgs r{};
+    r.src = full; r.dst = dst;
+    r.inner = 1;
+    for (int d = g.batch_rank; d < g.orank; ++d) r.inner *= g.oshape[d];
+    r.rank = g.batch_rank;
+    const int own = parent->rank - trailing;
+    int64_t acc = 1, kept_total = 1, red_total = 1;
+    for (int d = g.batch_rank - 1; d >= 0; --d) {
+        r.shape[d] = g.oshape[d];
+        r.src_str[d] = acc;
+        acc *= g.oshape[d];
+        const int od = d - (g.batch_rank - own);
+        r.kept[d] = (od >= 0 && parent->shape[od] > 1) ? 1 : 0;
+        if (r.kept[d]) kept_total *= g.oshape[d]; else red_total *= g.oshape[d];
+    }
+    r.dst_batch = kept_total;
+    r.reduced_total = red_total;
+    const int64_t total = kept_total * r.inner;
+    if (total == 0) return 0;
+    hipLaunchKernelGGL(broadcast_reduce_add_kernel, dim3((unsigned)std::min<int64_t>((total + 255) / 256, 65535)), dim3(256), 0, S.stream, r);
+    return 0;
+}
+
+bool same_batch(const Geometry& g, const tenmo_view* parent, int trailing) {
+    const int own = parent->rank - trailing;
+    if (own != g.batch_rank) {
+        // missing leading dims are fine only if the result's are all 1
+        for (int d = 0; d < g.batch_rank - own; ++d) if (g.oshape[d] != 1) return false;
+    }
+    for (int d = std::max(0, g.batch_rank - own); d < g.batch_rank; ++d)
+        if (parent->shape[d - (g.batch_rank - own)] != g.oshape[d]) return false;
+    return true;
+}
+
+} // namespace
+
+// ================================================================================================
+// C ABI
+// ================================================================================================
+extern "C" {
+
+const char* tenmo_hip_last_error(void) { return t_err.c_str(); }
+
+int tenmo_hip_init(int device_id) {
+    std::lock_guard<std::mutex> lock(S_mu);
+    if (S.ready) {
+        if (S.device == device_id) return 0;
+        return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_init: already initialised on device %d", S.device);
+    }
+    int count = 0;
+    HIP_TRY(hipGetDeviceCount(&count));
+    if (device_id < 0 || device_id >= count) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_init: device %d not present (%d visible)", device_id, count);
+    HIP_TRY(hipSetDevice(device_id));
+    hipDeviceProp_t prop;
+    HIP_TRY(hipGetDeviceProperties(&prop, device_id));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0)
+        return fail(TENMO_ERR_UNSUPPORTED, "tenmo_hip_init: device %d is %s; this library is built for gfx950 only", device_id, prop.gcnArchName);
+    S.device = device_id;
+    S.cus = prop.multiProcessorCount;
+    S.name = prop.name;
+    HIP_TRY(hipStreamCreate(&S.own_stream));
+    S.stream = S.own_stream;
+    HIP_TRY(hipEventCreate(&S.ev0));
+    HIP_TRY(hipEventCreate(&S.ev1));
+    S.force_tile = env_int("TENMO_HIP_GEMM_TILE", -1);
+    S.force_splitk = env_int("TENMO_HIP_GEMM_SPLITK", -1);
+    S.ready = true;
+    return 0;
+}
+
+int tenmo_hip_shutdown(void) {
+    std::lock_guard<std::mutex> lock(S_mu);
+    if (!S.ready) return 0;
+    hipStreamSynchronize(S.stream);
+    if (S.ws) hipFree(S.ws);
+    if (S.ws2) hipFree(S.ws2);
+    for (int i = 0; i < 3; ++i) if (S.stage[i]) hipFree(S.stage[i]);
+    hipEventDestroy(S.ev0);
+    hipEventDestroy(S.ev1);
+    hipStreamDestroy(S.own_stream);
+    S = State();
+    return 0;
+}
+
+int tenmo_hip_sync(void) {
+    if (int rc = ensure_ready()) return rc;
+    HIP_TRY(hipStreamSynchronize(S.stream));
+    return 0;
+}
+
+void* tenmo_hip_get_stream(void) { return S.ready ? (void*)S.stream : nullptr; }
+
+int tenmo_hip_set_stream(void* s) {
+    if (int rc = ensure_ready()) return rc;
+    HIP_TRY(hipStreamSynchronize(S.stream));
+    S.stream = s ? (hipStream_t)s : S.own_stream;
+    return 0;
+}
+
+int tenmo_hip_device_info(int* cus, char* name, int name_len) {
+    if (int rc = ensure_ready()) return rc;
+    if (cus) *cus = S.cus;
+    if (name && name_len > 0) { strncpy(name, S.name.c_str(), name_len - 1); name[name_len - 1] = 0; }
+    return 0;
+}
+
+int tenmo_hip_set_tuning(const char* name, int value) {
+    if (!name) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: null name");
+    if (!strcmp(name, "gemm_tile")) { S.force_tile = value; return 0; }
+    if (!strcmp(name, "gemm_splitk")) { S.force_splitk = value; return 0; }
+    return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: unknown knob '%s'", name);
+}
+
+int tenmo_hip_timer_begin(void) {
+    if (int rc = ensure_ready()) return rc;
+    HIP_TRY(hipEventRecord(S.ev0, S.stream));
+    return 0;
+}
+
+int tenmo_hip_timer_end(float* ms) {
+    if (int rc = ensure_ready()) return rc;
+    HIP_TRY(hipEventRecord(S.ev1, S.stream));
+    HIP_TRY(hipEventSynchronize(S.ev1));
+    HIP_TRY(hipEventElapsedTime(ms, S.ev0, S.ev1));
+    return 0;
+}
+
+int tenmo_hip_gemm_f32(const float* A, int64_t a_off, int64_t a_rs, int64_t a_cs,
+                       const float* B, int64_t b_off, int64_t b_rs, int64_t b_cs,
+                       float* C, int64_t M, int64_t N, int64_t K,
+                       int32_t batch_rank, const int64_t* batch_shape,
+                       const int64_t* a_batch_strides, const int64_t* b_batch_strides,
+                       int32_t accumulate, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    if (M < 0 || N < 0 || K < 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_gemm_f32: negative dimension");
+    if ((!A || !B || !C) && M * N > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_gemm_f32: null pointer");
+    BatchDesc bd{};
+    int64_t count = 1;
+    if (int rc = fill_batch(bd, batch_rank, batch_shape, a_batch_strides, b_batch_strides, &count)) return rc;
+    if (int rc = gemm_dispatch(A + a_off, a_rs, a_cs, B + b_off, b_rs, b_cs, C, M, N, K, bd, count, accumulate)) return rc;
+    return finish(sync);
+}
+
+int tenmo_hip_mv_f32(const float* Mx, int64_t m_off, int64_t m_rs, int64_t m_cs,
+                     const float* v, int64_t v_off, int64_t v_s,
+                     float* out, int64_t m, int64_t k,
+                     int32_t batch_rank, const int64_t* batch_shape,
+                     const int64_t* m_batch_strides, const int64_t* v_batch_strides,
+                     int32_t accumulate, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    if (m < 0 || k < 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_mv_f32: negative dimension");
+    BatchDesc bd{};
+    int64_t count = 1;
+    if (int rc = fill_batch(bd, batch_rank, batch_shape, m_batch_strides, v_batch_strides, &count)) return rc;
+    if (int rc = matvec_dispatch(Mx + m_off, m_rs, m_cs, v + v_off, v_s, out, m, k, bd, count, accumulate)) return rc;
+    return finish(sync);
+}
+
+int tenmo_hip_vm_f32(const float* v, int64_t v_off, int64_t v_s,
+                     const float* Mx, int64_t m_off, int64_t m_rs, int64_t m_cs,
+                     float* out, int64_t k, int64_t n,
+                     int32_t batch_rank, const int64_t* batch_shape,
+                     const int64_t* v_batch_strides, const int64_t* m_batch_strides,
+                     int32_t accumulate, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    if (n < 0 || k < 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_vm_f32: negative dimension");
+    BatchDesc bd{};
+    int64_t count = 1;
+    // matvec_dispatch wants (matrix, vector) order in the batch descriptor
+    if (int rc = fill_batch(bd, batch_rank, batch_shape, m_batch_strides, v_batch_strides, &count)) return rc;
+    // out[j] = sum_i Mx(i, j) v(i): outputs walk the matrix columns, the reduction walks its rows
+    if (int rc = matvec_dispatch(Mx + m_off, m_cs, m_rs, v + v_off, v_s, out, n, k, bd, count, accumulate)) return rc;
+    return finish(sync);
+}
+
+int tenmo_hip_dot_f32(const float* a, int64_t a_off, int64_t a_s, const float* b, int64_t b_off, int64_t b_s,
+                      int64_t n, float* out, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    if (n < 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_dot_f32: negative length");
+    const int parts = (int)std::max<int64_t>(1, std::min<int64_t>((n + DOT_THREADS * 8 - 1) / (DOT_THREADS * 8), 1024));
+    float* ws;
+    if (int rc = workspace(parts * sizeof(float), &ws)) return rc;
+    hipLaunchKernelGGL(dot_partial_kernel, dim3(parts), dim3(DOT_THREADS), 0, S.stream, a + a_off, a_s, b + b_off, b_s, n, ws);
+    hipLaunchKernelGGL(dot_final_kernel, dim3(1), dim3(DOT_THREADS), 0, S.stream, ws, parts, out);
+    return finish(sync);
+}
+
+int tenmo_hip_classify_matmul(int32_t ra, const int64_t* a, int32_t rb, const int64_t* b) {
+    if (ra <= 1 && rb <= 1) return TENMO_OP_DOT;
+    if (ra == 1 && rb >= 2) return TENMO_OP_VM;
+    if (ra >= 2 && rb == 1) return TENMO_OP_MV;
+    if (ra >= 2 && rb >= 2) return a[ra - 1] == b[rb - 2] ? TENMO_OP_MM : TENMO_OP_INVALID;
+    return TENMO_OP_INVALID;
+}
+
+int64_t tenmo_hip_result_shape(int32_t op, const tenmo_view* A, const tenmo_view* B, int64_t* out_shape, int32_t* out_rank) {
+    Geometry g;
+    if (int rc = resolve(op, A, B, &g, "tenmo_hip_result_shape")) return rc;
+    if (out_shape) std::copy(g.oshape, g.oshape + g.orank, out_shape);
+    if (out_rank) *out_rank = g.orank;
+    return product(g.oshape, g.orank);
+}
+
+int tenmo_hip_matmul_nd(const tenmo_view* A, const tenmo_view* B, float* C, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    if (int rc = matmul_views(A, B, C, 0, "tenmo_hip_matmul_nd")) return rc;
+    return finish(sync);
+}
+
+int tenmo_hip_matrix_vector_nd(const tenmo_view* Mx, const tenmo_view* v, float* out, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    Geometry g;
+    if (int rc = resolve(TENMO_OP_MV, Mx, v, &g, "tenmo_hip_matrix_vector_nd")) return rc;
+    const BatchDesc bd = make_batch(g, Mx, 2, v, 1);
+    const int64_t m = Mx->shape[Mx->rank - 2], k = Mx->shape[Mx->rank - 1];
+    if (int rc = matvec_dispatch(Mx->data + Mx->offset, Mx->strides[Mx->rank - 2], Mx->strides[Mx->rank - 1],
+                                 v->data + v->offset, v->strides[v->rank - 1], out, m, k, bd, g.batch_count, 0)) return rc;
+    return finish(sync);
+}
+
+int tenmo_hip_vector_matmul_nd(const tenmo_view* v, const tenmo_view* Mx, float* out, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    Geometry g;
+    if (int rc = resolve(TENMO_OP_VM, v, Mx, &g, "tenmo_hip_vector_matmul_nd")) return rc;
+    const BatchDesc bd = make_batch(g, Mx, 2, v, 1); // (matrix, vector) order
+    const int64_t k = Mx->shape[Mx->rank - 2], n = Mx->shape[Mx->rank - 1];
+    if (int rc = matvec_dispatch(Mx->data + Mx->offset, Mx->strides[Mx->rank - 1], Mx->strides[Mx->rank - 2],
+                                 v->data + v->offset, v->strides[v->rank - 1], out, n, k, bd, g.batch_count, 0)) return rc;
+    return finish(sync);
+}
+
+int tenmo_hip_matmul_backward(const tenmo_view* A, const tenmo_view* B, const float* dC,
+                              float* grad_A, float* grad_B, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    Geometry g;
+    if (int rc = resolve(TENMO_OP_MM, A, B, &g, "tenmo_hip_matmul_backward")) return rc;
+    if (g.batch_count == 0) return 0;
+    const tenmo_view dCv = dense_view(dC, g.oshape, g.orank);
+    if (grad_A) { // dA = dC . B^T(view)   (tenmo/matmul.mojo:36-38, :116-121)
+        const tenmo_view Bt = transposed_last2(B);
+        if (same_batch(g, A, 2)) {
+            if (int rc = matmul_views(&dCv, &Bt, grad_A, 1, "tenmo_hip_matmul_backward")) return rc;
+        } else {
+            Geometry gg;
+            if (int rc = resolve(TENMO_OP_MM, &dCv, &Bt, &gg, "tenmo_hip_matmul_backward")) return rc;
+            // the GEMM may itself use the first scratch for split-K: the batched gradient lives in the second
+            float* full = nullptr;
+            if (int rc = workspace2((size_t)product(gg.oshape, gg.orank) * sizeof(float), &full)) return rc;
+            if (int rc = matmul_views(&dCv, &Bt, full, 0, "tenmo_hip_matmul_backward")) return rc;
+            if (int rc = reduce_to_parent(full, gg, A, 2, grad_A)) return rc;
+        }
+    }
+    if (grad_B) { // dB = A^T(view) . dC   (tenmo/matmul.mojo:46-48, :127-132)
+        const tenmo_view At = transposed_last2(A);
+        if (same_batch(g, B, 2)) {
+            if (int rc = matmul_views(&At, &dCv, grad_B, 1, "tenmo_hip_matmul_backward")) return rc;
+        } else {
+            Geometry gg;
+            if (int rc = resolve(TENMO_OP_MM, &At, &dCv, &gg, "tenmo_hip_matmul_backward")) return rc;
+            float* full = nullptr;
+            if (int rc = workspace2((size_t)product(gg.oshape, gg.orank) * sizeof(float), &full)) return rc;
+            if (int rc = matmul_views(&At, &dCv, full, 0, "tenmo_hip_matmul_backward")) return rc;
+            if (int rc = reduce_to_parent(full, gg, B, 2, grad_B)) return rc;
+        }
+    }
+    return finish(sync);
+}
+
+static int outer_grad(const float* p, int64_t p_s, const int64_t* p_bstr, const float* q, int64_t q_s, const int64_t* q_bstr,
+                      float* grad, int64_t I, int64_t J, const Geometry& g, const tenmo_view* parent) {
+    OuterArgs o{};
+    o.p = p; o.p_s = p_s; o.q = q; o.q_s = q_s; o.grad = grad; o.I = I; o.J = J;
+    o.rank = g.batch_rank;
+    const int own = parent->rank - 2;
+    int64_t kept_total = 1, red_total = 1;
+    for (int d = 0; d < g.batch_rank; ++d) {
+        o.shape[d] = g.oshape[d];
+        o.p_str[d] = p_bstr[d];
+        o.q_str[d] = q_bstr[d];
+        const int od = d - (g.batch_rank - own);
+        o.kept[d] = (od >= 0 && parent->shape[od] > 1) ? 1 : 0;
+        if (o.kept[d]) kept_total *= g.oshape[d]; else red_total *= g.oshape[d];
+    }
+    o.parent_batch = kept_total;
+    o.reduced_total = red_total;
+    const int64_t total = kept_total * I * J;
+    if (total == 0) return 0;
+    hipLaunchKernelGGL(outer_add_kernel, dim3((unsigned)std::min<int64_t>((total + 255) / 256, 65535)), dim3(256), 0, S.stream, o);
+    return 0;
+}
+
+int tenmo_hip_mv_backward(const tenmo_view* Mx, const tenmo_view* v, const float* dy,
+                          float* grad_M, float* grad_v, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    Geometry g;
+    if (int rc = resolve(TENMO_OP_MV, Mx, v, &g, "tenmo_hip_mv_backward")) return rc;
+    if (g.batch_count == 0) return 0;
+    const int64_t m = Mx->shape[Mx->rank - 2], k = Mx->shape[Mx->rank - 1];
+    int64_t dy_bstr[MAX_BATCH_RANK] = {0}, v_bstr[MAX_BATCH_RANK] = {0}, m_bstr[MAX_BATCH_RANK] = {0};
+    { int64_t acc = m; for (int d = g.batch_rank - 1; d >= 0; --d) { dy_bstr[d] = acc; acc *= g.oshape[d]; } }
+    batch_strides_of(v, v->rank - 1, g.batch_rank, v_bstr);
+    batch_strides_of(Mx, Mx->rank - 2, g.batch_rank, m_bstr);
+    if (grad_M) // dM[i][j] += dy[i] * v[j]   (tenmo/matrixvector.mojo:87-139)
+        if (int rc = outer_grad(dy, 1, dy_bstr, v->data + v->offset, v->strides[v->rank - 1], v_bstr, grad_M, m, k, g, Mx)) return rc;
+    if (grad_v) { // dv = M^T . dy  (:162-196), reduced over the batches v broadcast
+        // as a batched vector x matrix: dy[.., m] . M[.., m, k] -> [.., k]
+        BatchDesc bd{};
+        bd.rank = g.batch_rank;
+        for (int d = 0; d < MAX_BATCH_RANK; ++d) {
+            bd.shape[d] = d < g.batch_rank ? g.oshape[d] : 1;
+            bd.a_str[d] = d < g.batch_rank ? m_bstr[d] : 0;  // matrix
+            bd.b_str[d] = d < g.batch_rank ? dy_bstr[d] : 0; // vector
+        }
+        Geometry gg = g;
+        gg.oshape[g.batch_rank] = k; gg.orank = g.batch_rank + 1;
+        const bool direct = same_batch(g, v, 1);
+        float* target = grad_v;
+        float* full = nullptr;
+        if (!direct) {
+            if (int rc = workspace2((size_t)g.batch_count * k * sizeof(float), &full)) return rc;
+            target = full;
+        }
+        if (int rc = matvec_dispatch(Mx->data + Mx->offset, Mx->strides[Mx->rank - 1], Mx->strides[Mx->rank - 2], dy, 1, target, k, m, bd, g.batch_count, direct ? 1 : 0)) return rc;
+        if (!direct) if (int rc = reduce_to_parent(full, gg, v, 1, grad_v)) return rc;
+    }
+    return finish(sync);
+}
+
+int tenmo_hip_vm_backward(const tenmo_view* v, const tenmo_view* Mx, const float* dy,
+                          float* grad_v, float* grad_M, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    Geometry g;
+    if (int rc = resolve(TENMO_OP_VM, v, Mx, &g, "tenmo_hip_vm_backward")) return rc;
+    if (g.batch_count == 0) return 0;
+    const int64_t k = Mx->shape[Mx->rank - 2], n = Mx->shape[Mx->rank - 1];
+    int64_t dy_bstr[MAX_BATCH_RANK] = {0}, v_bstr[MAX_BATCH_RANK] = {0}, m_bstr[MAX_BATCH_RANK] = {0};
+    { int64_t acc = n; for (int d = g.batch_rank - 1; d >= 0; --d) { dy_bstr[d] = acc; acc *= g.oshape[d]; } }
+    batch_strides_of(v, v->rank - 1, g.batch_rank, v_bstr);
+    batch_strides_of(Mx, Mx->rank - 2, g.batch_rank, m_bstr);
+    if (grad_M) // dM[i][j] += v[i] * dy[j]   (tenmo/vectormatrix.mojo:145-201)
+        if (int rc = outer_grad(v->data + v->offset, v->strides[v->rank - 1], v_bstr, dy, 1, dy_bstr, grad_M, k, n, g, Mx)) return rc;
+    if (grad_v) { // dv[i] = sum_j dy[j] M[i][j]  (:65-100): a matrix x vector with M as is
+        BatchDesc bd{};
+        bd.rank = g.batch_rank;
+        for (int d = 0; d < MAX_BATCH_RANK; ++d) {
+            bd.shape[d] = d < g.batch_rank ? g.oshape[d] : 1;
+            bd.a_str[d] = d < g.batch_rank ? m_bstr[d] : 0;
+            bd.b_str[d] = d < g.batch_rank ? dy_bstr[d] : 0;
+        }
+        Geometry gg = g;
+        gg.oshape[g.batch_rank] = k; gg.orank = g.batch_rank + 1;
+        const bool direct = same_batch(g, v, 1);
+        float* target = grad_v;
+        float* full = nullptr;
+        if (!direct) {
+            if (int rc = workspace2((size_t)g.batch_count * k * sizeof(float), &full)) return rc;
+            target = full;
+        }
+        if (int rc = matvec_dispatch(Mx->data + Mx->offset, Mx->strides[Mx->rank - 2], Mx->strides[Mx->rank - 1], dy, 1, target, k, n, bd, g.batch_count, direct ? 1 : 0)) return rc;
+        if (!direct) if (int rc = reduce_to_parent(full, gg, v, 1, grad_v)) return rc;
+    }
+    return finish(sync);
+}
+
+// ---- CBLAS-compatible host-pointer entry point --------------------------------------------------
+
+static int stage_buffer(int i, size_t bytes, float** out) {
+    if (bytes > S.stage_bytes[i]) {
+        if (S.stage[i]) { HIP_TRY(hipStreamSynchronize(S.stream)); HIP_TRY(hipFree(S.stage[i])); S.stage[i] = nullptr; S.stage_bytes[i] = 0; }
+        HIP_TRY(hipMalloc(&S.stage[i], bytes));
+        S.stage_bytes[i] = bytes;
+    }
+    *out = S.stage[i];
+    return 0;
+}
+
+static int sgemm_impl(int order, int ta, int tb, int M, int N, int K, float alpha, const float* A, int lda,
+                      const float* B, int ldb, float beta, float* C, int ldc) {
+    if (!S.ready) { if (int rc = tenmo_hip_init(0)) return rc; }
+    const bool row = (order == 101);
+    if (!row && order != 102) return fail(TENMO_ERR_INVALID_ARGUMENT, "cblas_sgemm: order must be 101 (RowMajor) or 102 (ColMajor)");
+    auto is_t = [](int t) { return t == 112 || t == 113; };
+    if ((ta != 111 && !is_t(ta)) || (tb != 111 && !is_t(tb))) return fail(TENMO_ERR_INVALID_ARGUMENT, "cblas_sgemm: bad transpose flag");
+    if (M < 0 || N < 0 || K < 0) return fail(TENMO_ERR_INVALID_SHAPE, "cblas_sgemm: negative dimension");
+    if (M == 0 || N == 0) return 0;
+    // stored extents of A and B in their own storage order
+    const int a_r = row ? (is_t(ta) ? K : M) : (is_t(ta) ? M : K); // number of ld-strided lines of A
+    const int a_c = row ? (is_t(ta) ? M : K) : (is_t(ta) ? K : M); // contiguous extent
+    const int b_r = row ? (is_t(tb) ? N : K) : (is_t(tb) ? K : N);
+    const int b_c = row ? (is_t(tb) ? K : N) : (is_t(tb) ? N : K);
+    const int c_r = row ? M : N, c_c = row ? N : M;
+    if (lda < std::max(1, a_c) || ldb < std::max(1, b_c) || ldc < std::max(1, c_c)) return fail(TENMO_ERR_INVALID_ARGUMENT, "cblas_sgemm: leading dimension too small");
+    float *dA, *dB, *dC;
+    if (int rc = stage_buffer(0, std::max<size_t>(1, (size_t)a_r * a_c) * sizeof(float), &dA)) return rc;
+    if (int rc = stage_buffer(1, std::max<size_t>(1, (size_t)b_r * b_c) * sizeof(float), &dB)) return rc;
+    if (int rc = stage_buffer(2, (size_t)M * N * sizeof(float), &dC)) return rc;
+    if (K > 0) {
+        HIP_TRY(hipMemcpy2DAsync(dA, (size_t)a_c * 4, A, (size_t)lda * 4, (size_t)a_c * 4, a_r, hipMemcpyHostToDevice, S.stream));
+        HIP_TRY(hipMemcpy2DAsync(dB, (size_t)b_c * 4, B, (size_t)ldb * 4, (size_t)b_c * 4, b_r, hipMemcpyHostToDevice, S.stream));
+    }
+    // logical (M x K) and (K x N) operands as strided views of the staged dense copies
+    int64_t a_rs, a_cs, b_rs, b_cs;
+    if (row) {
+        a_rs = is_t(ta) ? 1 : a_c; a_cs = is_t(ta) ? a_c : 1;
+        b_rs = is_t(tb) ? 1 : b_c; b_cs = is_t(tb) ? b_c : 1;
+    } else { // column-major storage: element (i,j) of the stored matrix at i + j*ld
+        a_rs = is_t(ta) ? a_c : 1; a_cs = is_t(ta) ? 1 : a_c;
+        b_rs = is_t(tb) ? b_c : 1; b_cs = is_t(tb) ? 1 : b_c;
+    }
+    BatchDesc bd{};
+    for (int d = 0; d < MAX_BATCH_RANK; ++d) bd.shape[d] = 1;
+    int rc;
+    if (row) rc = gemm_dispatch(dA, a_rs, a_cs, dB, b_rs, b_cs, dC, M, N, K, bd, 1, 0);
+    else     rc = gemm_dispatch(dB, b_cs, b_rs, dA, a_cs, a_rs, dC, N, M, K, bd, 1, 0); // C^T = B^T . A^T, dense [N][M] == column-major C
+    if (rc) return rc;
+    HIP_TRY(hipGetLastError());
+    std::vector<float> host((size_t)M * N);
+    HIP_TRY(hipMemcpyAsync(host.data(), dC, (size_t)M * N * sizeof(float), hipMemcpyDeviceToHost, S.stream));
+    HIP_TRY(hipStreamSynchronize(S.stream));
+    for (int r = 0; r < c_r; ++r) {
+        float* crow = C + (size_t)r * ldc;
+        const float* hrow = host.data() + (size_t)r * c_c;
+        if (beta == 0.f) for (int c = 0; c < c_c; ++c) crow[c] = alpha * hrow[c];
+        else for (int c = 0; c < c_c; ++c) crow[c] = alpha * hrow[c] + beta * crow[c];
+    }
+    return 0;
+}
+
+void cblas_sgemm(int order, int ta, int tb, int M, int N, int K, float alpha, const float* A, int lda,
+                 const float* B, int ldb, float beta, float* C, int ldc) {
+    // the CBLAS prototype has no error channel; failures are left in tenmo_hip_last_error() and
+    // reported on stderr, as a BLAS would do through xerbla
+    if (int rc = sgemm_impl(order, ta, tb, M, N, K, alpha, A, lda, B, ldb, beta, C, ldc))
+        fprintf(stderr, "libtenmo_hip cblas_sgemm: error %d: %s\n", rc, t_err.c_str());
+}
+
+// ---- MLP training-step harness --------------------------------------------------------------------
+
+struct tenmo_mlp {
+    int L = 0;
+    std::vector<int64_t> dims;
+    int64_t max_batch = 0;
+    std::vector<float*> W, b, dW, db, act, grad; // act[l]: output of layer l ([B, dims[l+1]]); grad[l]: its gradient
+    float* row_loss = nullptr;
+};
+
+static unsigned grid_for(int64_t n) { return (unsigned)std::max<int64_t>(1, std::min<int64_t>((n + 255) / 256, 4096)); }
+
+tenmo_mlp* tenmo_hip_mlp_create(int32_t L, const int64_t* dims, const float* const* Wh, const float* const* bh, int64_t max_batch) {
+    if (ensure_ready()) return nullptr;
+    if (L < 1 || !dims || !Wh || !bh || max_batch < 1) { fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_mlp_create: bad arguments"); return nullptr; }
+    auto* m = new tenmo_mlp();
+    m->L = L; m->dims.assign(dims, dims + L + 1); m->max_batch = max_batch;
+    m->W.assign(L, nullptr); m->b.assign(L, nullptr); m->dW.assign(L, nullptr); m->db.assign(L, nullptr);
+    m->act.assign(L, nullptr); m->grad.assign(L, nullptr);
+    bool ok = true;
+    for (int l = 0; l < L && ok; ++l) {
+        const size_t wn = (size_t)dims[l] * dims[l + 1], bn = (size_t)dims[l + 1], an = (size_t)max_batch * dims[l + 1];
+        ok = ok && hipMalloc(&m->W[l], wn * 4) == hipSuccess && hipMalloc(&m->dW[l], wn * 4) == hipSuccess;
+        ok = ok && hipMalloc(&m->b[l], bn * 4) == hipSuccess && hipMalloc(&m->db[l], bn * 4) == hipSuccess;
+        ok = ok && hipMalloc(&m->act[l], an * 4) == hipSuccess && hipMalloc(&m->grad[l], an * 4) == hipSuccess;
+        ok = ok && hipMemcpy(m->W[l], Wh[l], wn * 4, hipMemcpyHostToDevice) == hipSuccess;
+        ok = ok && hipMemcpy(m->b[l], bh[l], bn * 4, hipMemcpyHostToDevice) == hipSuccess;
+    }
+    ok = ok && hipMalloc(&m->row_loss, (size_t)max_batch * 4) == hipSuccess;
+    if (!ok) { fail(TENMO_ERR_HIP, "tenmo_hip_mlp_create: device allocation or upload failed"); tenmo_hip_mlp_destroy(m); return nullptr; }
+    return m;
+}
+
+void tenmo_hip_mlp_destroy(tenmo_mlp* m) {
+    if (!m) return;
+    if (S.ready) hipStreamSynchronize(S.stream);
+    for (auto* v : {&m->W, &m->b, &m->dW, &m->db, &m->act, &m->grad})
+        for (float* p : *v) if (p) hipFree(p);
+    if (m->row_loss) hipFree(m->row_loss);
+    delete m;
+}
+
+static int mlp_forward(tenmo_mlp* m, const float* x, int64_t B) {
+    BatchDesc bd{};
+    for (int d = 0; d < MAX_BATCH_RANK; ++d) bd.shape[d] = 1;
+    const float* in = x;
+    for (int l = 0; l < m->L; ++l) {
+        const int64_t I = m->dims[l], O = m->dims[l + 1];
+        if (int rc = gemm_dispatch(in, I, 1, m->W[l], O, 1, m->act[l], B, O, I, bd, 1, 0)) return rc;
+        hipLaunchKernelGGL(bias_act_kernel, dim3(grid_for(B * O)), dim3(256), 0, S.stream, m->act[l], m->b[l], B, O, l + 1 < m->L ? 1 : 0);
+        in = m->act[l];
+    }
+    return 0;
+}
+
+int tenmo_hip_mlp_forward(tenmo_mlp* m, const float* x, int64_t B, float* logits_out, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    if (!m || B < 1 || B > m->max_batch) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_mlp_forward: batch outside 1..max_batch");
+    if (int rc = mlp_forward(m, x, B)) return rc;
+    HIP_TRY(hipMemcpyAsync(logits_out, m->act[m->L - 1], (size_t)B * m->dims[m->L] * 4, hipMemcpyDeviceToDevice, S.stream));
+    return finish(sync);
+}
+
+int tenmo_hip_mlp_step(tenmo_mlp* m, const float* x, const int32_t* y, int64_t B, float lr, float* loss_out, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    if (!m || B < 1 || B > m->max_batch) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_mlp_step: batch outside 1..max_batch");
+    if (int rc = mlp_forward(m, x, B)) return rc;
+    const int L = m->L;
+    const int64_t C = m->dims[L];
+    hipLaunchKernelGGL(cross_entropy_kernel, dim3((unsigned)((B + 63) / 64)), dim3(64), 0, S.stream, m->act[L - 1], y, B, C, m->grad[L - 1], m->row_loss);
+    hipLaunchKernelGGL(ordered_mean_kernel, dim3(1), dim3(64), 0, S.stream, m->row_loss, B, loss_out);
+    BatchDesc bd{};
+    for (int d = 0; d < MAX_BATCH_RANK; ++d) bd.shape[d] = 1;
+    for (int l = L - 1; l >= 0; --l) {
+        const int64_t I = m->dims[l], O = m->dims[l + 1];
+        const float* in = l == 0 ? x : m->act[l - 1];
+        const float* gl = m->grad[l];
+        hipLaunchKernelGGL(column_sum_kernel, dim3((unsigned)((O + 63) / 64)), dim3(64), 0, S.stream, gl, B, O, m->db[l]);
+        // dW = in^T(view) . g        (tenmo/matmul.mojo:46-48)
+        if (int rc = gemm_dispatch(in, 1, I, gl, O, 1, m->dW[l], I, O, B, bd, 1, 0)) return rc;
+        if (l > 0) { // dX = g . W^T(view)  (tenmo/matmul.mojo:36-38); the network input needs no gradient (:34)
+            if (int rc = gemm_dispatch(gl, O, 1, m->W[l], 1, O, m->grad[l - 1], B, I, O, bd, 1, 0)) return rc;
+            hipLaunchKernelGGL(relu_backward_kernel, dim3(grid_for(B * I)), dim3(256), 0, S.stream, m->grad[l - 1], m->act[l - 1], B * I);
+        }
+    }
+    for (int l = 0; l < L; ++l) {
+        const int64_t wn = m->dims[l] * m->dims[l + 1], bn = m->dims[l + 1];
+        hipLaunchKernelGGL(sgd_kernel, dim3(grid_for(wn)), dim3(256), 0, S.stream, m->W[l], m->dW[l], wn, lr);
+        hipLaunchKernelGGL(sgd_kernel, dim3(grid_for(bn)), dim3(256), 0, S.stream, m->b[l], m->db[l], bn, lr);
+    }
+    return finish(sync);
+}
+
+int tenmo_hip_mlp_get_params(tenmo_mlp* m, int32_t l, float* Wh, float* bh) {
+    if (int rc = ensure_ready()) return rc;
+    if (!m || l < 0 || l >= m->L) return fail(TENMO_ERR_INVALID_ARGUMENT, "layer out of range");
+    HIP_TRY(hipStreamSynchronize(S.stream));
+    if (Wh) HIP_TRY(hipMemcpy(Wh, m->W[l], (size_t)m->dims[l] * m->dims[l + 1] * 4, hipMemcpyDeviceToHost));
+    if (bh) HIP_TRY(hipMemcpy(bh, m->b[l], (size_t)m->dims[l + 1] * 4, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+int tenmo_hip_mlp_get_grads(tenmo_mlp* m, int32_t l, float* Wh, float* bh) {
+    if (int rc = ensure_ready()) return rc;
+    if (!m || l < 0 || l >= m->L) return fail(TENMO_ERR_INVALID_ARGUMENT, "layer out of range");
+    HIP_TRY(hipStreamSynchronize(S.stream));
+    if (Wh) HIP_TRY(hipMemcpy(Wh, m->dW[l], (size_t)m->dims[l] * m->dims[l + 1] * 4, hipMemcpyDeviceToHost));
+    if (bh) HIP_TRY(hipMemcpy(bh, m->db[l], (size_t)m->dims[l + 1] * 4, hipMemcpyDeviceToHost));
+    return 0;
+}
+
+} // extern "C"
