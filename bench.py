@@ -1,0 +1,221 @@
+#!/usr/bin/env python3
+"""Benchmark of the fp32 matrix-product path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+A "step" is one pass of the hot path over one batch of synthetic input: one fp32 GEMM
+C = A.B with M = N = K = 8192 (the size the headline metric is quoted on), operands resident in
+HBM before the timed region.  Prints ONE JSON line with the whole-job throughput in TFLOP/s,
+the roofline of the dominant kernel (fp32 MFMA peak 157.3 TFLOP/s) measured with HIP events on the
+stream the kernel runs on, and a CPU baseline (the C++ restatement of the reference's CPU matmul,
+timed on this host's cores on a bounded sample of the same workload).  The `extra` object carries
+the other headline figures: mv / vm bandwidth at 16384^2 and the MLP training step in ms on GPU
+and CPU.
+"""
+from __future__ import annotations
+
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+PEAK_FP32_MFMA_TFLOPS = 157.3  # 256 CU x 2.4 GHz x 256 flop/clk/CU
+PEAK_HBM_GBPS = 8000.0
+
+# HBM bytes per 8192^3 launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
+# profiles/); None until a counter run has been recorded for the current kernel.
+MEASURED_TRAFFIC_BYTES = None
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=3)
+    ap.add_argument("--size", type=int, default=8192, help="M=N=K of the square GEMM (default: the headline size)")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-extra", action="store_true", help="skip the mv/vm and MLP-step side measurements")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on ONE GPU (the reference has no multi-GPU path and every "
+              "configuration fits one MI355X); --gpus %d is not supported" % args.gpus, file=sys.stderr)
+        return 2
+
+    import numpy as np
+    import torch
+
+    from tenmo_amd import _lib
+
+    _lib.init(0)
+    L = _lib.load()
+    cus = C.c_int()
+    name = C.create_string_buffer(128)
+    L.tenmo_hip_device_info(C.byref(cus), name, 128)
+
+    S = args.size
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(8192)
+    A = torch.randn((S, S), generator=gen, device="cuda", dtype=torch.float32)
+    B = torch.randn((S, S), generator=gen, device="cuda", dtype=torch.float32)
+    Cc = torch.empty((S, S), device="cuda", dtype=torch.float32)
+
+    def step():
+        _lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, S, 1, B.data_ptr(), 0, S, 1, Cc.data_ptr(), S, S, S,
+                                        0, None, None, None, 0, 0))
+
+    for _ in range(args.warmup):
+        step()
+    _lib.check(L.tenmo_hip_sync())
+    torch.cuda.synchronize()
+    # wall clock around exactly K steps, synchronised on both sides; HIP events on the library's
+    # stream bracket the same launches for the per-launch kernel duration
+    t0 = time.perf_counter()
+    _lib.check(L.tenmo_hip_timer_begin())
+    for _ in range(args.steps):
+        step()
+    ev_ms = C.c_float()
+    _lib.check(L.tenmo_hip_timer_end(C.byref(ev_ms)))
+    _lib.check(L.tenmo_hip_sync())
+    torch.cuda.synchronize()
+    wall_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    kernel_ms = ev_ms.value / args.steps
+    flop = 2.0 * S * S * S
+    value = flop / (wall_ms * 1e-3) / 1e12
+    achieved = flop / (kernel_ms * 1e-3) / 1e12
+
+    # accuracy gate on the timed result: sampled rows against fp64
+    rows = torch.tensor([0, S // 3, S - 1], device="cuda")
+    ref = (A[rows].double() @ B.double()).cpu().numpy()
+    got = Cc[rows].cpu().numpy()
+    rel_err = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
+
+    out = {
+        "metric": "fp32 GEMM TFLOP/s (M=N=K=%d) + %% fp32-MFMA peak (1 GPU); MLP train-step ms vs CPU" % S,
+        "value": round(value, 3),
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(wall_ms, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "square fp32 GEMM C=A.B, M=N=K=%d, A and B row-major N(0,1), inputs resident in HBM" % S,
+                   "device": name.value.decode(), "compute_units": cus.value},
+        "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
+                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "kernel_ms": round(kernel_ms, 4)},
+        "rel_fro_error_vs_fp64": rel_err,
+    }
+
+    extra = {}
+    if not args.no_extra:
+        extra.update(side_measurements(L, _lib, torch, np))
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_gemm_baseline(A, B, S, np)
+        if not args.no_extra:
+            extra.update(mlp_step_times(_lib, torch, np))
+    if extra:
+        out["extra"] = extra
+    print(json.dumps(out), flush=True)
+    return 0 if rel_err <= 1e-5 else 1
+
+
+def hip_time(L, _lib, fn, iters, warm=3):
+    for _ in range(warm):
+        fn()
+    _lib.check(L.tenmo_hip_sync())
+    _lib.check(L.tenmo_hip_timer_begin())
+    for _ in range(iters):
+        fn()
+    ms = C.c_float()
+    _lib.check(L.tenmo_hip_timer_end(C.byref(ms)))
+    return ms.value / iters
+
+
+def side_measurements(L, _lib, torch, np):
+    """mv / vm at 16384^2 (HBM-bound): GB/s of algorithmic bytes and fraction of the 8 TB/s peak."""
+    n = 16384
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(16384)
+    W = torch.randn((n, n), generator=gen, device="cuda", dtype=torch.float32)
+    x = torch.randn((n,), generator=gen, device="cuda", dtype=torch.float32)
+    out = torch.empty((n,), device="cuda", dtype=torch.float32)
+    mv = lambda: _lib.check(L.tenmo_hip_mv_f32(W.data_ptr(), 0, n, 1, x.data_ptr(), 0, 1, out.data_ptr(), n, n, 0, None, None, None, 0, 0))
+    vm = lambda: _lib.check(L.tenmo_hip_vm_f32(x.data_ptr(), 0, 1, W.data_ptr(), 0, n, 1, out.data_ptr(), n, n, 0, None, None, None, 0, 0))
+    nbytes = (n * n + 2 * n) * 4.0
+    res = {}
+    for nm, fn in (("mv", mv), ("vm", vm)):
+        ms = hip_time(L, _lib, fn, 30)
+        gbps = nbytes / (ms * 1e-3) / 1e9
+        res["%s_16384_us" % nm] = round(ms * 1e3, 2)
+        res["%s_16384_gbps" % nm] = round(gbps, 1)
+        res["%s_16384_frac_hbm_peak" % nm] = round(gbps / PEAK_HBM_GBPS, 4)
+    return res
+
+
+def cpu_gemm_baseline(A, B, S, np):
+    """The restated reference CPU matmul on a bounded sample of the same GEMM: `cores` row tiles of
+    128 rows (one per thread) of C = A.B, all of B."""
+    from oracle import oracle as O
+
+    cores = O.num_physical_cores()
+    tile_m = 128 if S > 256 else (64 if S > 64 else 32)
+    tiles = min(cores, (S + tile_m - 1) // tile_m)
+    rows = min(S, tiles * tile_m)
+    a = A[:rows].cpu().numpy()
+    b = B.cpu().numpy()
+    a3 = a.reshape(1, rows, S)
+    out = np.empty((1, rows, S), np.float32)
+    O.mmnd(a3[:, :8], b, cores)  # warm the thread pool
+    t0 = time.perf_counter()
+    O.mmnd(a3, b, cores, out=out)
+    dt = time.perf_counter() - t0
+    flop = 2.0 * rows * S * S
+    return {"value": round(flop / dt / 1e12, 5), "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": "%d of %d row tiles (%d rows x all %d columns, K=%d) of the same GEMM, %.1f s, simd width %d"
+                      % (tiles, (S + tile_m - 1) // tile_m, rows, S, S, dt, O.simd_width())}
+
+
+def mlp_step_times(_lib, torch, np):
+    """MNIST-shaped MLP 784->128->32->10, batch 64, SGD lr 0.01: ms per training step on the GPU (inputs
+    already on the device) and on the CPU restatement, and the largest per-step loss difference."""
+    from oracle import oracle as O
+    from tenmo_amd import rng as R
+    from tenmo_amd.net import MLP
+
+    dims, seed, lr, batch = [784, 128, 32, 10], 2024, 0.01, 64
+    Ws, bs = R.xavier_mlp(dims, seed)
+    gpu, cpu = MLP(dims, Ws, bs, batch), O.MLP(dims, Ws, bs, batch)
+    batches = [R.mnist_like_batch(batch, seed, s) for s in range(30)]
+    dev = [(torch.from_numpy(x).cuda(), torch.from_numpy(y).cuda()) for x, y in batches]
+    worst = 0.0
+    gl = []
+    for xd, yd in dev[:10]:  # warm-up steps double as the parity check
+        gl.append(float(gpu.step_device(xd, yd, lr, sync=True).item()))
+    cl = [cpu.step(x, y, lr) for x, y in batches[:10]]
+    worst = max(abs(a - b) for a, b in zip(gl, cl))
+    L = _lib.load()
+    _lib.check(L.tenmo_hip_sync())
+    t0 = time.perf_counter()
+    for xd, yd in dev[10:]:
+        gpu.step_device(xd, yd, lr, sync=False)
+    _lib.check(L.tenmo_hip_sync())
+    gpu_ms = (time.perf_counter() - t0) * 1e3 / 20
+    t0 = time.perf_counter()
+    for x, y in batches[10:]:
+        cpu.step(x, y, lr)
+    cpu_ms = (time.perf_counter() - t0) * 1e3 / 20
+    return {"mlp_step_ms_gpu": round(gpu_ms, 4), "mlp_step_ms_cpu": round(cpu_ms, 4), "mlp_cpu_cores": O.num_physical_cores(),
+            "mlp_max_abs_loss_diff_first10": worst}
+
+
+if __name__ == "__main__":
+    sys.exit(main())

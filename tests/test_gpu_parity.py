@@ -1,0 +1,415 @@
+"""GPU parity: the HIP path, called through the C ABI (via the host mirror), against the CPU oracle
+on the same seeded inputs, against the reference's literal vectors, and against fp64.
+
+Tolerance (stated by the task): relative Frobenius error <= 1e-5 against the fp64-accumulated
+reference; literal vectors with the reference's own all_close(rtol=1e-5, atol=1e-8)
+(tenmo/ndbuffer.mojo:2263-2266)."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+from helpers import RTOL_FRO, numpy_view, ref_matmul64, rel_fro, storage_of, strides_of
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def T():
+    import tenmo_amd.matmul as M
+    import tenmo_amd.tensor as TT
+    from tenmo_amd import _lib
+
+    _lib.init(0)
+
+    class NS:
+        Tensor = TT.Tensor
+        mm, mv, vm, dot = TT.mm, TT.mv, TT.vm, TT.dot
+        Mm = M
+        lib = _lib
+
+    return NS
+
+
+def fixture_tensor(T, t, requires_grad=False):
+    base = T.Tensor.from_numpy(storage_of(t), requires_grad=False)
+    return base.view(t["shape"], strides_of(t), t.get("offset", 0), requires_grad=requires_grad)
+
+
+def oracle_view(O, t):
+    return O.View(storage_of(t), t.get("offset", 0), t["shape"], strides_of(t))
+
+
+def as_strided_tensor(T, arr, requires_grad=False):
+    """Upload the storage behind a numpy view once and describe the same view on the device."""
+    base = arr
+    while base.base is not None:
+        base = base.base
+    base = np.ascontiguousarray(base)
+    off = (arr.__array_interface__["data"][0] - base.__array_interface__["data"][0]) // 4
+    store = T.Tensor.from_numpy(base.reshape(-1))
+    return store.view(arr.shape, tuple(s // 4 for s in arr.strides), off, requires_grad=requires_grad)
+
+
+# ---- the reference's literal vectors ---------------------------------------------------------------
+
+def test_golden_forward_and_backward(T, golden):
+    mode = {"mm": T.mm, "mv": T.mv, "vm": T.vm, "dot": T.dot}
+    for c in golden["cases"]:
+        A = fixture_tensor(T, c["A"], requires_grad=True)
+        B = fixture_tensor(T, c["B"], requires_grad=True)
+        out = A.matmul(B, mode=mode[c["op"]])
+        if "expect" in c:
+            np.testing.assert_allclose(out.to_numpy(), np.asarray(c["expect"], np.float32), rtol=1e-5, atol=1e-8, err_msg=c["name"])
+        if "grad_A" in c or "grad_B" in c:
+            out.backward(1.0)  # loss = out.sum(); loss.backward()
+            if "grad_A" in c:
+                np.testing.assert_allclose(A.grad(), np.asarray(c["grad_A"], np.float32), rtol=1e-5, err_msg=c["name"] + " grad_A")
+            if "grad_B" in c:
+                np.testing.assert_allclose(B.grad(), np.asarray(c["grad_B"], np.float32), rtol=1e-5, err_msg=c["name"] + " grad_B")
+
+
+def test_closed_forms(T, golden):
+    for c in golden["closed_forms"]:
+        A = T.Tensor.ones(*c["A_shape"], requires_grad=True)
+        B = T.Tensor.ones(*c["B_shape"], requires_grad=True)
+        out = A.matmul(B)
+        got = out.to_numpy()
+        assert np.all(got == c["expect_value"]), c["name"]
+        if "grad_A_value" in c:
+            out.backward(1.0)
+            assert A.grad().shape == tuple(c["A_shape"]) and np.all(A.grad() == c["grad_A_value"])
+            assert B.grad().shape == tuple(c["B_shape"]) and np.all(B.grad() == c["grad_B_value"])
+
+
+# ---- 2-D GEMM against oracle and fp64 --------------------------------------------------------------
+
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2])
+def test_verify_shapes(T, golden, oracle, tile):
+    """Shape list of tests/test_matmul_2d_verify.mojo, each with A / B as row-major, transposed view
+    and padded view, on every workgroup-tile configuration."""
+    L = T.lib.load()
+    L.tenmo_hip_set_tuning(b"gemm_tile", tile)
+    try:
+        rng = np.random.default_rng(17)
+        for m, k, n in golden["verify_shapes"]["mkn"]:
+            a = rng.standard_normal((m, k), dtype=np.float32)
+            b = rng.standard_normal((k, n), dtype=np.float32)
+            ref = ref_matmul64(a, b)
+            a_views = [a, np.ascontiguousarray(a.T).T, np.pad(a, ((0, 0), (0, 3)))[:, :k]]
+            b_views = [b, np.ascontiguousarray(b.T).T, np.pad(b, ((0, 0), (0, 5)))[:, :n]]
+            for av in a_views:
+                for bv in b_views:
+                    got = as_strided_tensor(T, av).matmul(as_strided_tensor(T, bv), track_grad=False).to_numpy()
+                    assert got.shape == (m, n)
+                    assert rel_fro(got, ref) <= RTOL_FRO, (m, k, n, av.strides, bv.strides)
+                    # and against the CPU restatement on identical inputs
+                    assert rel_fro(got, oracle.mm2d(av, bv)) <= 2 * RTOL_FRO
+    finally:
+        L.tenmo_hip_set_tuning(b"gemm_tile", -1)
+
+
+def test_odd_strides_and_overlap(T, oracle):
+    """Column stride 2, row stride 0 (broadcast rows), overlapping windows (tests/test_mmnd.mojo:143-175)."""
+    rng = np.random.default_rng(23)
+    store = rng.standard_normal(4000).astype(np.float32)
+    dev = T.Tensor.from_numpy(store)
+    cases = [
+        ((20, 30), (60, 2), 7, (30, 10), (10, 1), 100),     # A col stride 2
+        ((16, 24), (0, 1), 5, (24, 12), (12, 1), 900),      # A rows broadcast
+        ((12, 40), (3, 1), 0, (40, 9), (2, 70), 1),         # overlapping A rows, B generic
+        ((33, 17), (1, 40), 11, (17, 65), (1, 17), 2000),   # both transposed
+    ]
+    for ash, ast, aoff, bsh, bst, boff in cases:
+        A = dev.view(ash, ast, aoff)
+        B = dev.view(bsh, bst, boff)
+        an = np.lib.stride_tricks.as_strided(store[aoff:], ash, tuple(4 * s for s in ast))
+        bn = np.lib.stride_tricks.as_strided(store[boff:], bsh, tuple(4 * s for s in bst))
+        got = A.matmul(B, track_grad=False).to_numpy()
+        assert rel_fro(got, ref_matmul64(an, bn)) <= RTOL_FRO
+        assert rel_fro(got, oracle.mm2d(oracle.View(store, aoff, ash, ast), oracle.View(store, boff, bsh, bst))) <= 2 * RTOL_FRO
+    # inputs are never written
+    np.testing.assert_array_equal(dev.to_numpy(), store)
+
+
+def test_empty_and_degenerate(T):
+    z = T.Tensor.zeros(3, 0).matmul(T.Tensor.zeros(0, 4), track_grad=False)  # K = 0 -> zeros (NDBuffer.zeros result)
+    assert z.shape() == (3, 4) and np.all(z.to_numpy() == 0)
+    e = T.Tensor.zeros(0, 5).matmul(T.Tensor.zeros(5, 4), track_grad=False)
+    assert e.shape() == (0, 4)
+    one = T.Tensor.d([[2.0]]).matmul(T.Tensor.d([[3.0]]), track_grad=False)
+    assert one.to_numpy()[0, 0] == 6.0
+
+
+def test_shape_errors(T):
+    E = T.lib.TenmoHipError
+    with pytest.raises(E, match="inner"):
+        T.Tensor.zeros(2, 3).matmul(T.Tensor.zeros(4, 2))
+    with pytest.raises(E, match="broadcast"):
+        T.Tensor.zeros(2, 5, 3).matmul(T.Tensor.zeros(3, 3, 4))
+    with pytest.raises(E, match="must match"):
+        T.Tensor.zeros(2, 3).matmul(T.Tensor.zeros(4), mode=T.mv)
+    with pytest.raises(E, match="must match"):
+        T.Tensor.zeros(3).matmul(T.Tensor.zeros(4, 2), mode=T.vm)
+    with pytest.raises(E, match="size does not match"):
+        T.Tensor.zeros(3).matmul(T.Tensor.zeros(4))
+
+
+# ---- batched / broadcast ---------------------------------------------------------------------------
+
+def test_batched_broadcast_against_oracle(T, oracle):
+    rng = np.random.default_rng(29)
+    cases = [((3, 1, 17, 9), (4, 9, 13)), ((2, 5, 70, 33), (2, 5, 33, 41)), ((6, 40, 64), (1, 64, 64)),
+             ((1, 2, 4, 8), (3, 2, 8, 4)), ((130, 70), (5, 70, 19)), ((2, 2, 2, 2, 3, 4), (4, 5))]
+    for sa, sb in cases:
+        a = rng.standard_normal(sa, dtype=np.float32)
+        b = rng.standard_normal(sb, dtype=np.float32)
+        got = T.Tensor.from_numpy(a).matmul(T.Tensor.from_numpy(b), track_grad=False).to_numpy()
+        assert got.shape == ref_matmul64(a, b).shape
+        assert rel_fro(got, ref_matmul64(a, b)) <= RTOL_FRO
+        assert rel_fro(got, oracle.matmul(a, b)) <= 2 * RTOL_FRO
+    # K^T as a transposed view, attention shape (tests/test_attn_matmul.mojo:106-186)
+    q = rng.standard_normal((2, 3, 50, 16), dtype=np.float32)
+    k = rng.standard_normal((2, 3, 50, 16), dtype=np.float32)
+    s = T.Tensor.from_numpy(q).matmul(T.Tensor.from_numpy(k).transpose(-1, -2), track_grad=False).to_numpy()
+    assert rel_fro(s, ref_matmul64(q, np.swapaxes(k, -1, -2))) <= RTOL_FRO
+    # a batch-strided view (tests/test_mmnd.mojo:584-593)
+    big = rng.standard_normal((4, 6, 5), dtype=np.float32)
+    sub = big[::2]
+    got = as_strided_tensor(T, sub).matmul(T.Tensor.from_numpy(np.eye(5, dtype=np.float32)), track_grad=False).to_numpy()
+    np.testing.assert_array_equal(got, sub)
+
+
+def test_backward_against_oracle(T, oracle):
+    rng = np.random.default_rng(31)
+    cases = [((37, 21), (21, 45)), ((3, 18, 9), (3, 9, 14)), ((4, 18, 9), (1, 9, 14)), ((1, 18, 9), (5, 9, 14)),
+             ((18, 9), (2, 3, 9, 14)), ((2, 1, 6, 7), (1, 3, 7, 5))]
+    for sa, sb in cases:
+        a = rng.standard_normal(sa, dtype=np.float32)
+        b = rng.standard_normal(sb, dtype=np.float32)
+        A, B = T.Tensor.from_numpy(a, True), T.Tensor.from_numpy(b, True)
+        out = A.matmul(B)
+        seed = rng.standard_normal(out.shape(), dtype=np.float32)
+        out.backward(T.Tensor.from_numpy(seed), retain_graph=True)
+        gA, gB = oracle.matmul_backward(a, b, seed)
+        assert A.grad().shape == a.shape and B.grad().shape == b.shape
+        assert rel_fro(A.grad(), gA) <= 2 * RTOL_FRO, (sa, sb)
+        assert rel_fro(B.grad(), gB) <= 2 * RTOL_FRO, (sa, sb)
+        # a second backward accumulates: gradients double (tests/test_mv.mojo:673-692)
+        out.backward(T.Tensor.from_numpy(seed))
+        assert rel_fro(A.grad(), 2 * gA) <= 2 * RTOL_FRO
+        assert rel_fro(B.grad(), 2 * gB) <= 2 * RTOL_FRO
+    # only the parent that requires grad receives one (tenmo/matmul.mojo:34,45)
+    A, B = T.Tensor.ones(3, 4, requires_grad=False), T.Tensor.ones(4, 2, requires_grad=True)
+    out = A.matmul(B)
+    out.backward(1.0)
+    assert A.grad() is None and np.all(B.grad() == 3.0)
+
+
+def test_backward_through_transposed_view(T, oracle):
+    """x . W^T with W a transposed view (tests/test_tensors.mojo:3443-3466 pattern) on random data."""
+    rng = np.random.default_rng(37)
+    x = rng.standard_normal((2, 19, 12), dtype=np.float32)
+    w = rng.standard_normal((15, 12), dtype=np.float32)
+    X = T.Tensor.from_numpy(x, True)
+    Wt = T.Tensor.from_numpy(w, True).transpose()
+    out = X.matmul(Wt)
+    assert rel_fro(out.to_numpy(), ref_matmul64(x, w.T)) <= RTOL_FRO
+    seed = rng.standard_normal(out.shape(), dtype=np.float32)
+    out.backward(T.Tensor.from_numpy(seed))
+    gX, gWt = oracle.matmul_backward(x, w.T, seed)
+    assert rel_fro(X.grad(), gX) <= 2 * RTOL_FRO
+    assert rel_fro(Wt.grad(), gWt) <= 2 * RTOL_FRO  # gradient at the view's own shape (12, 15)
+
+
+# ---- mv / vm / dot ---------------------------------------------------------------------------------
+
+def test_mv_vm_forward_all_layouts(T, oracle):
+    rng = np.random.default_rng(41)
+    M = rng.standard_normal((2, 3, 37, 29), dtype=np.float32)
+    v = rng.standard_normal((3, 29), dtype=np.float32)
+    u = rng.standard_normal((37,), dtype=np.float32)
+    Md = T.Tensor.from_numpy(M)
+    got = Md.matmul(T.Tensor.from_numpy(v), mode=T.mv, track_grad=False).to_numpy()
+    assert got.shape == (2, 3, 37) and rel_fro(got, oracle.mv_f64(M, v)) <= RTOL_FRO
+    assert rel_fro(got, oracle.mv(M, v)) <= 2 * RTOL_FRO
+    got = T.Tensor.from_numpy(u).matmul(Md, mode=T.vm, track_grad=False).to_numpy()
+    assert got.shape == (2, 3, 29) and rel_fro(got, oracle.vm_f64(u, M)) <= RTOL_FRO
+    # transposed matrix view (examples/word2vec_cbow.mojo:531-553), strided vector, padded rows
+    got = Md.transpose().matmul(T.Tensor.from_numpy(u), mode=T.mv, track_grad=False).to_numpy()
+    assert rel_fro(got, oracle.mv_f64(np.swapaxes(M, -1, -2), u)) <= RTOL_FRO
+    got = T.Tensor.from_numpy(v[0]).matmul(Md.transpose(), mode=T.vm, track_grad=False).to_numpy()
+    assert rel_fro(got, oracle.vm_f64(v[0], np.swapaxes(M, -1, -2))) <= RTOL_FRO
+    w2 = rng.standard_normal((58,), dtype=np.float32)
+    got = Md.matmul(as_strided_tensor(T, w2[::2]), mode=T.mv, track_grad=False).to_numpy()
+    assert rel_fro(got, oracle.mv_f64(M, w2[::2])) <= RTOL_FRO
+    P = rng.standard_normal((45, 64), dtype=np.float32)
+    got = as_strided_tensor(T, P[:, 3:60]).matmul(T.Tensor.from_numpy(rng.standard_normal(57, dtype=np.float32) * 0 + 1), mode=T.mv, track_grad=False).to_numpy()
+    assert rel_fro(got, P[:, 3:60].astype(np.float64).sum(1)) <= RTOL_FRO
+    G = rng.standard_normal((30, 40, 2), dtype=np.float32)[:, :, 0]  # both strides non-unit
+    x = rng.standard_normal(40, dtype=np.float32)
+    assert rel_fro(as_strided_tensor(T, G).matmul(T.Tensor.from_numpy(x), mode=T.mv, track_grad=False).to_numpy(), oracle.mv_f64(G, x)) <= RTOL_FRO
+    y = rng.standard_normal(30, dtype=np.float32)
+    assert rel_fro(T.Tensor.from_numpy(y).matmul(as_strided_tensor(T, G), mode=T.vm, track_grad=False).to_numpy(), oracle.vm_f64(y, G)) <= RTOL_FRO
+    # sizes that exercise the vector main loops, tails and k splitting
+    for m, k in [(1, 1), (5, 3), (300, 1025), (1000, 4100), (7, 9001), (2049, 515)]:
+        W = rng.standard_normal((m, k), dtype=np.float32)
+        x = rng.standard_normal(k, dtype=np.float32)
+        y = rng.standard_normal(m, dtype=np.float32)
+        Wd = T.Tensor.from_numpy(W)
+        assert rel_fro(Wd.matmul(T.Tensor.from_numpy(x), mode=T.mv, track_grad=False).to_numpy(), oracle.mv_f64(W, x)) <= RTOL_FRO, (m, k)
+        assert rel_fro(T.Tensor.from_numpy(y).matmul(Wd, mode=T.vm, track_grad=False).to_numpy(), oracle.vm_f64(y, W)) <= RTOL_FRO, (m, k)
+
+
+def test_mv_vm_backward_against_oracle(T, oracle):
+    rng = np.random.default_rng(43)
+    for ms, vs in [((6, 5), (5,)), ((3, 6, 5), (5,)), ((6, 5), (4, 5)), ((2, 3, 6, 5), (3, 5)), ((1, 6, 5), (4, 5))]:
+        Mn = rng.standard_normal(ms, dtype=np.float32)
+        vn = rng.standard_normal(vs, dtype=np.float32)
+        Mt, vt = T.Tensor.from_numpy(Mn, True), T.Tensor.from_numpy(vn, True)
+        out = Mt.matmul(vt, mode=T.mv)
+        seed = rng.standard_normal(out.shape(), dtype=np.float32)
+        out.backward(T.Tensor.from_numpy(seed))
+        dM, dv = oracle.mv_backward(Mn, vn, seed)
+        assert rel_fro(Mt.grad(), dM) <= 2 * RTOL_FRO and rel_fro(vt.grad(), dv) <= 2 * RTOL_FRO, (ms, vs)
+    for vs, ms in [((6,), (6, 5)), ((6,), (3, 6, 5)), ((4, 6), (6, 5)), ((3, 6), (2, 3, 6, 5))]:
+        Mn = rng.standard_normal(ms, dtype=np.float32)
+        vn = rng.standard_normal(vs, dtype=np.float32)
+        Mt, vt = T.Tensor.from_numpy(Mn, True), T.Tensor.from_numpy(vn, True)
+        out = vt.matmul(Mt, mode=T.vm)
+        seed = rng.standard_normal(out.shape(), dtype=np.float32)
+        out.backward(T.Tensor.from_numpy(seed))
+        dv, dM = oracle.vm_backward(vn, Mn, seed)
+        assert rel_fro(Mt.grad(), dM) <= 2 * RTOL_FRO and rel_fro(vt.grad(), dv) <= 2 * RTOL_FRO, (vs, ms)
+
+
+def test_dot(T, oracle):
+    rng = np.random.default_rng(47)
+    for n in (1, 7, 1000, 300001):
+        a = rng.standard_normal(n, dtype=np.float32)
+        b = rng.standard_normal(n, dtype=np.float32)
+        got = float(T.Tensor.from_numpy(a).matmul(T.Tensor.from_numpy(b), track_grad=False).to_numpy())
+        ref = float(np.dot(a.astype(np.float64), b.astype(np.float64)))
+        assert abs(got - ref) <= 1e-5 * max(1.0, np.linalg.norm(a) * np.linalg.norm(b)), n
+    a = np.arange(1, 8, dtype=np.float32)
+    A, B = T.Tensor.from_numpy(a, True), T.Tensor.from_numpy(2 * a, True)
+    out = A.dot(B)
+    assert float(out.to_numpy()) == 280.0
+    out.backward(3.0)
+    np.testing.assert_allclose(A.grad(), 6 * a)
+    np.testing.assert_allclose(B.grad(), 3 * a)
+    assert float(T.Tensor.d([2.0]).matmul(T.Tensor.from_numpy(a), track_grad=False).to_numpy()) == 56.0
+
+
+# ---- the reference's CBLAS plugin point ---------------------------------------------------------------
+
+def test_cblas_sgemm(T, golden):
+    from tenmo_amd.blashandle import BLASHandle
+
+    h = BLASHandle()
+    assert h.is_initialized()
+    for c in golden["blas"]:
+        A, B = np.asarray(c["A"], np.float32), np.asarray(c["B"], np.float32)
+        if "grad_A" in c:
+            gA, gB = h.matmul_backward(A, B, np.ones((A.shape[0], B.shape[1]), np.float32))
+            np.testing.assert_allclose(gA, c["grad_A"])
+            np.testing.assert_allclose(gB, c["grad_B"])
+            continue
+        out = h.matmul(A, B, c["tA"], c["tB"])
+        if "expect" in c:
+            np.testing.assert_allclose(out, c["expect"], rtol=1e-5)
+        else:
+            assert abs(out[0, 0] - c["expect_00"]) < 1e-5
+    assert np.all(h.matmul(np.ones((100, 100), np.float32), np.ones((100, 100), np.float32)) == 100.0)  # tests/test_blas.mojo:216-232
+    # four-case backward algebra (tenmo/blashandle.mojo:51-99) against explicit transposes
+    rng = np.random.default_rng(53)
+    for tA in (False, True):
+        for tB in (False, True):
+            A = rng.standard_normal((9, 6) if tA else (6, 9), dtype=np.float32)
+            B = rng.standard_normal((5, 9) if tB else (9, 5), dtype=np.float32)
+            opA, opB = (A.T if tA else A), (B.T if tB else B)
+            assert rel_fro(h.matmul(A, B, tA, tB), ref_matmul64(opA, opB)) <= RTOL_FRO
+            g = rng.standard_normal((6, 5), dtype=np.float32)
+            gA, gB = h.matmul_backward(A, B, g, tA, tB)
+            rA, rB = ref_matmul64(g, opB.T), ref_matmul64(opA.T, g)
+            assert rel_fro(gA, rA.T if tA else rA) <= RTOL_FRO and rel_fro(gB, rB.T if tB else rB) <= RTOL_FRO
+    # raw ABI: column-major, alpha/beta, leading dimensions larger than the extent
+    L = T.lib.load()
+    A = rng.standard_normal((7, 4), dtype=np.float32)   # column-major 4x7 with lda 4... use explicit ld
+    Acm = np.asfortranarray(rng.standard_normal((6, 8), dtype=np.float32))  # M=6, K=8 column-major, lda=6
+    Bcm = np.asfortranarray(rng.standard_normal((8, 3), dtype=np.float32))
+    Ccm = np.asfortranarray(rng.standard_normal((6, 3), dtype=np.float32))
+    want = 0.5 * ref_matmul64(Acm, Bcm) + 2.0 * Ccm
+    L.cblas_sgemm(102, 111, 111, 6, 3, 8, 0.5, Acm.ctypes.data, 6, Bcm.ctypes.data, 8, 2.0, Ccm.ctypes.data, 6)
+    assert rel_fro(Ccm, want) <= RTOL_FRO
+    Ald = np.zeros((6, 11), np.float32)
+    Ald[:, :8] = Acm
+    out = np.zeros((6, 5), np.float32)
+    Brm = np.ascontiguousarray(Bcm)
+    L.cblas_sgemm(101, 111, 111, 6, 3, 8, 1.0, Ald.ctypes.data, 11, Brm.ctypes.data, 3, 0.0, out.ctypes.data, 5)
+    assert rel_fro(out[:, :3], ref_matmul64(Acm, Bcm)) <= RTOL_FRO and np.all(out[:, 3:] == 0)
+
+
+# ---- Linear and the MLP training step ---------------------------------------------------------------
+
+def test_linear_layer(T):
+    from tenmo_amd.net import Linear
+
+    rng = np.random.default_rng(59)
+    lin = Linear(12, 7, rng, init_method="xavier")
+    bias = rng.standard_normal(7).astype(np.float32)
+    import torch
+
+    lin.bias.buffer.storage.copy_(torch.from_numpy(bias))
+    x = rng.standard_normal((5, 12), dtype=np.float32)
+    X = T.Tensor.from_numpy(x, True)
+    y = lin(X)
+    W = lin.weight.to_numpy()
+    assert rel_fro(y.to_numpy(), ref_matmul64(x, W) + bias) <= RTOL_FRO
+    seed = rng.standard_normal((5, 7), dtype=np.float32)
+    y.backward(T.Tensor.from_numpy(seed))
+    assert rel_fro(lin.weight.grad(), ref_matmul64(x.T, seed)) <= RTOL_FRO
+    assert rel_fro(lin.bias.grad(), seed.astype(np.float64).sum(0)) <= RTOL_FRO
+    assert rel_fro(X.grad(), ref_matmul64(seed, W.T)) <= RTOL_FRO
+    with pytest.raises(T.lib.TenmoHipError, match="input dim mismatch"):
+        lin(T.Tensor.zeros(5, 13))
+
+
+def test_sgd_vectors(T, golden):
+    from tenmo_amd.net import SGD
+
+    for key in ("sgd_single_step", "sgd_three_steps", "sgd_2d"):
+        s = golden["harness"][key]
+        w = T.Tensor.from_numpy(np.asarray(s["w"], np.float32), True)
+        opt = SGD([w], lr=s["lr"])
+        for _ in range(s["steps"]):
+            w.seed_grad(T.Tensor.from_numpy(np.asarray(s["grad"], np.float32)))
+            opt.step()
+        np.testing.assert_allclose(w.to_numpy(), s["expect"], rtol=1e-6)
+
+
+def test_mlp_loss_curve_tracks_cpu(T, oracle):
+    """MNIST-shaped MLP 784->128->32->10, batch 64, Xavier, SGD lr=0.01: the per-step loss of the
+    GPU run stays within 1e-4 of the CPU restatement for every step."""
+    from tenmo_amd import rng as R
+    from tenmo_amd.net import MLP
+
+    dims, seed, lr = [784, 128, 32, 10], 2024, 0.01
+    Ws, bs = R.xavier_mlp(dims, seed)
+    gpu, cpu = MLP(dims, Ws, bs, 64), oracle.MLP(dims, Ws, bs, 64)
+    worst = 0.0
+    for step in range(40):
+        x, y = R.mnist_like_batch(64, seed, step)
+        lg, lc = gpu.step(x, y, lr), cpu.step(x, y, lr)
+        worst = max(worst, abs(lg - lc))
+        assert abs(lg - lc) <= 1e-4, (step, lg, lc)
+    for l in range(3):
+        (Wg, bg), (Wc, bc) = gpu.params(l), cpu.params(l)
+        assert rel_fro(Wg, Wc) <= 1e-5 and np.abs(bg - bc).max() <= 1e-5
+        (dWg, dbg), (dWc, dbc) = gpu.grads(l), cpu.grads(l)
+        assert rel_fro(dWg, dWc) <= 1e-4
+    x, _ = R.mnist_like_batch(64, seed, 99)
+    assert rel_fro(gpu.forward(x), cpu.forward(x)) <= 1e-5
+    # cross-entropy vector of the reference: uniform logits -> -log(1/3)
+    m = MLP([2, 3], [np.zeros((2, 3), np.float32)], [np.ones(3, np.float32)], 2)
+    assert abs(m.step(np.ones((2, 2), np.float32), np.asarray([0, 1], np.int32), 0.0) - 1.0986122886681098) < 1e-6

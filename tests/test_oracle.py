@@ -1,0 +1,283 @@
+"""Pins the CPU oracle (oracle/) before anything trusts it: the reference's own literal test
+vectors, fp64 brute force, closed forms and algebraic invariants.  Runs without a GPU."""
+import numpy as np
+import pytest
+
+from helpers import numpy_view, ref_matmul64, rel_fro, storage_of, strides_of
+
+
+def _view(O, t):
+    return O.View(storage_of(t), t.get("offset", 0), t["shape"], strides_of(t))
+
+
+def test_golden_forward(golden, oracle):
+    O = oracle
+    for c in golden["cases"]:
+        A, B = _view(O, c["A"]), _view(O, c["B"])
+        if c["op"] == "mm":
+            got = O.matmul(A, B)
+        elif c["op"] == "mv":
+            got = O.mv(A, B)
+        elif c["op"] == "vm":
+            got = O.vm(A, B)
+        else:
+            got = O.dot(A, B)
+        if "expect" in c:
+            np.testing.assert_allclose(got, np.asarray(c["expect"], np.float32), rtol=1e-5, atol=1e-8, err_msg=c["name"])
+
+
+def test_golden_backward(golden, oracle):
+    O = oracle
+    for c in golden["cases"]:
+        if "grad_A" not in c and "grad_B" not in c:
+            continue
+        A, B = _view(O, c["A"]), _view(O, c["B"])
+        if c["op"] == "mm":
+            shape = O.result_shape(O.MM, A, B)
+            gA, gB = O.matmul_backward(A, B, np.ones(shape, np.float32))
+        elif c["op"] == "mv":
+            gA, gB = O.mv_backward(A, B, np.ones(O.result_shape(O.MV, A, B), np.float32))
+        else:
+            gA, gB = O.vm_backward(A, B, np.ones(O.result_shape(O.VM, A, B), np.float32))
+        if "grad_A" in c:
+            np.testing.assert_allclose(gA, np.asarray(c["grad_A"], np.float32), rtol=1e-5, err_msg=c["name"] + " grad_A")
+        if "grad_B" in c:
+            np.testing.assert_allclose(gB, np.asarray(c["grad_B"], np.float32), rtol=1e-5, err_msg=c["name"] + " grad_B")
+
+
+@pytest.mark.parametrize("width", [0, 16, 8, 1])
+def test_verify_shapes_against_fp64(golden, oracle, width):
+    """The shape list of the reference's own verification file, against an fp64 triple loop; every
+    tile/tail combination of the three code paths and every ISA kernel."""
+    O = oracle
+    O.force_simd_width(width)
+    try:
+        rng = np.random.default_rng(7)
+        for m, k, n in golden["verify_shapes"]["mkn"]:
+            a = rng.standard_normal((m, k), dtype=np.float32)
+            b = rng.standard_normal((k, n), dtype=np.float32)
+            ref = ref_matmul64(a, b)
+            info = {}
+            assert rel_fro(O.mm2d(a, b, info=info), ref) < 1e-6 and info["path"] == 0
+            at = np.ascontiguousarray(a.T).T  # transposed view: path 1b unless a dim is 1
+            assert rel_fro(O.mm2d(at, b, info=info), ref) < 1e-6
+            bt = np.ascontiguousarray(b.T).T  # B strided: path 2
+            assert rel_fro(O.mm2d(a, bt, info=info), ref) < 1e-6
+            if k > 1 and n > 1:
+                assert info["path"] == 2
+            # fp64-accumulating reference of the oracle itself against numpy
+            assert rel_fro(O.mm_f64(a, b), ref) < 1e-12
+    finally:
+        O.force_simd_width(0)
+
+
+def test_padded_row_views(oracle):
+    """Padded-stride views count as non-contiguous (tests/test_matmul_2d_verify.mojo:85-110,144-169,201-229)."""
+    O = oracle
+    rng = np.random.default_rng(3)
+    a_store = rng.standard_normal((33, 50), dtype=np.float32)
+    b_store = rng.standard_normal((40, 70), dtype=np.float32)
+    a, b = a_store[:, :40], b_store[:, :65]
+    ref = ref_matmul64(a, b)
+    info = {}
+    assert rel_fro(O.mm2d(a, b, info=info), ref) < 1e-6
+    assert info["path"] == 2  # B padded
+    assert rel_fro(O.mm2d(a, np.ascontiguousarray(b), info=info), ref) < 1e-6
+    assert info["path"] == 1  # only A padded
+
+
+def test_tile_table(oracle):
+    """tenmo/matmul_cpu.mojo:87-89 and the worked example docs/from-bytes-to-gradients.md:171-177."""
+    O = oracle
+    info = {}
+    O.mm2d(np.zeros((64, 784), np.float32), np.zeros((784, 128), np.float32), info=info)
+    assert info["tiles"] == (32, 64, 128)
+    O.mm2d(np.zeros((300, 10), np.float32), np.zeros((10, 10), np.float32), info=info)
+    assert info["tiles"] == (128, 32, 64)
+    O.mm2d(np.zeros((257, 65), np.float32), np.zeros((65, 257), np.float32), info=info)
+    assert info["tiles"] == (128, 64, 256)
+
+
+def test_contiguity_predicate(oracle):
+    """tenmo/strides.mojo:239-266: size-1 dims are skipped, offset is not part of it."""
+    O = oracle
+    assert O.is_contiguous((2, 3, 4), (12, 4, 1))
+    assert not O.is_contiguous((2, 3, 4), (1, 12, 4))
+    assert O.is_contiguous((1, 768, 768), (0, 768, 1))
+    assert O.is_contiguous((5, 1), (1, 99))
+    assert not O.is_contiguous((2, 3), (4, 1))
+    assert O.is_contiguous((), ())
+
+
+def test_classify(oracle):
+    O = oracle
+    assert O.classify_matmul((3,), (3,)) == O.DOT
+    assert O.classify_matmul((), (3,)) == O.DOT
+    assert O.classify_matmul((3,), (3, 4)) == O.VM
+    assert O.classify_matmul((2, 3), (3,)) == O.MV
+    assert O.classify_matmul((2, 3), (3, 4)) == O.MM
+    assert O.classify_matmul((5, 2, 3), (3, 4)) == O.MM
+    assert O.classify_matmul((2, 3), (4, 4)) == O.INVALID
+
+
+def test_errors(oracle):
+    O = oracle
+    with pytest.raises(O.OracleError):
+        O.mm2d(np.zeros((2, 3), np.float32), np.zeros((4, 2), np.float32))
+    with pytest.raises(O.OracleError):
+        O.mmnd(np.zeros((2, 5, 3), np.float32), np.zeros((3, 3, 4), np.float32))
+    with pytest.raises(O.OracleError):
+        O.mv(np.zeros((2, 3), np.float32), np.zeros((4,), np.float32))
+
+
+def test_closed_forms(golden, oracle):
+    O = oracle
+    for c in golden["closed_forms"]:
+        A, B = np.ones(c["A_shape"], np.float32), np.ones(c["B_shape"], np.float32)
+        out = O.mmnd(A, B)
+        assert out.shape == np.broadcast_shapes(tuple(c["A_shape"][:-2]), tuple(c["B_shape"][:-2])) + (c["A_shape"][-2], c["B_shape"][-1])
+        assert np.all(out == c["expect_value"])
+        if "grad_A_value" in c:
+            gA, gB = O.matmul_backward(A, B, np.ones(out.shape, np.float32))
+            assert gA.shape == tuple(c["A_shape"]) and np.all(gA == c["grad_A_value"])
+            assert gB.shape == tuple(c["B_shape"]) and np.all(gB == c["grad_B_value"])
+
+
+def test_batched_equals_loop_of_2d(oracle):
+    O = oracle
+    rng = np.random.default_rng(11)
+    A = rng.standard_normal((3, 1, 17, 9), dtype=np.float32)
+    B = rng.standard_normal((4, 9, 13), dtype=np.float32)
+    out = O.mmnd(A, B)
+    for i in range(3):
+        for j in range(4):
+            np.testing.assert_array_equal(out[i, j], O.mm2d(A[i, 0], B[j]))
+    # transposed-view operand equals its contiguous copy within rounding of the other code path
+    Bt = np.ascontiguousarray(np.swapaxes(B, -1, -2))
+    assert rel_fro(O.mmnd(A, np.swapaxes(Bt, -1, -2)), ref_matmul64(A, B)) < 1e-6
+
+
+def test_backward_identities(oracle):
+    """dA = dC.B^T, dB = A^T.dC (tests/test_mm2d.mojo:39-100) and finite differences
+    (tests/test_matmul.mojo:247-307) on the fp64 reference."""
+    O = oracle
+    rng = np.random.default_rng(5)
+    A = rng.standard_normal((6, 5), dtype=np.float32)
+    B = rng.standard_normal((5, 4), dtype=np.float32)
+    dC = rng.standard_normal((6, 4), dtype=np.float32)
+    gA, gB = O.matmul_backward(A, B, dC)
+    assert rel_fro(gA, ref_matmul64(dC, B.T)) < 1e-6
+    assert rel_fro(gB, ref_matmul64(A.T, dC)) < 1e-6
+    loss = lambda a, b: float(np.sum(ref_matmul64(a, b) * dC))
+    eps = 1e-3
+    for (i, j) in [(0, 0), (3, 2), (5, 4)]:
+        Ap, Am = A.astype(np.float64).copy(), A.astype(np.float64).copy()
+        Ap[i, j] += eps
+        Am[i, j] -= eps
+        assert abs((loss(Ap, B) - loss(Am, B)) / (2 * eps) - gA[i, j]) < 1e-3
+
+
+def test_mv_vm_against_fp64_and_views(oracle):
+    O = oracle
+    rng = np.random.default_rng(9)
+    M = rng.standard_normal((2, 3, 37, 29), dtype=np.float32)
+    v = rng.standard_normal((3, 29), dtype=np.float32)
+    assert rel_fro(O.mv(M, v), np.einsum("abmk,bk->abm", M.astype(np.float64), v.astype(np.float64))) < 1e-6
+    assert rel_fro(O.mv_f64(M, v), np.einsum("abmk,bk->abm", M.astype(np.float64), v.astype(np.float64))) < 1e-12
+    u = rng.standard_normal((37,), dtype=np.float32)
+    assert rel_fro(O.vm(u, M), np.einsum("m,abmk->abk", u.astype(np.float64), M.astype(np.float64))) < 1e-6
+    Mt = np.swapaxes(M, -1, -2)  # transposed view, as examples/word2vec_cbow.mojo:531-553 uses
+    assert rel_fro(O.mv(Mt, u), np.einsum("abmk,m->abk", M.astype(np.float64), u.astype(np.float64))) < 1e-6
+    # backward closed forms
+    dy = rng.standard_normal((2, 3, 37), dtype=np.float32)
+    dM, dv = O.mv_backward(M, v, dy)
+    assert rel_fro(dM, np.einsum("abm,bk->abmk", dy.astype(np.float64), v.astype(np.float64))) < 1e-6
+    assert rel_fro(dv, np.einsum("abmk,abm->bk", M.astype(np.float64), dy.astype(np.float64))) < 1e-6
+    dy2 = rng.standard_normal((2, 3, 29), dtype=np.float32)
+    du, dM2 = O.vm_backward(u, M, dy2)
+    assert rel_fro(du, np.einsum("abmk,abk->m", M.astype(np.float64), dy2.astype(np.float64))) < 1e-6
+    assert rel_fro(dM2, np.einsum("m,abk->abmk", u.astype(np.float64), dy2.astype(np.float64))) < 1e-6
+
+
+def test_dot(oracle):
+    O = oracle
+    a = np.arange(1, 8, dtype=np.float32)
+    assert O.dot(a, a) == 140.0
+    assert O.dot(np.asarray([2.0], np.float32), a) == 56.0  # one-element operand broadcasts
+    assert O.dot(a[::2], a[::2]) == 1 + 9 + 25 + 49
+    with pytest.raises(O.OracleError):
+        O.dot(a, a[:3])
+
+
+def test_sum_over_broadcasted_axes(oracle):
+    O = oracle
+    rng = np.random.default_rng(2)
+    src = rng.standard_normal((2, 4, 3, 6, 5), dtype=np.float32)
+    for target in [(1, 3, 6, 5), (4, 1, 6, 5), (3, 6, 5), (2, 4, 3, 6, 5), (6, 5)]:
+        ref = src.astype(np.float64)
+        lead = src.ndim - len(target)
+        ref = ref.sum(axis=tuple(range(lead)))
+        for d, s in enumerate(target):
+            if s == 1 and ref.shape[d] != 1:
+                ref = ref.sum(axis=d, keepdims=True)
+        assert rel_fro(O.sum_over_broadcasted_axes(src, target), ref) < 1e-6
+
+
+def test_mlp_harness_pieces(golden, oracle):
+    """Cross-entropy, SGD, bias-gradient and ReLU pieces of the step, against the reference's own
+    vectors and closed forms."""
+    O = oracle
+    h = golden["harness"]
+    # uniform logits -> -log(1/3): a 1-layer net with zero weights produces exactly that
+    c = h["ce_uniform_logits"]
+    m = O.MLP([2, 3], [np.zeros((2, 3), np.float32)], [np.ones(3, np.float32)], 2)
+    loss = m.step(np.ones((2, 2), np.float32), np.asarray(c["targets"], np.int32), 0.0)
+    assert abs(loss - c["loss"]) < 1e-6
+    dW, db = m.grads(0)
+    # gradient of mean CE wrt logits = (softmax - onehot)/rows: rows of dlogits sum to zero
+    # (tests/test_cross_entropy.mojo:797-823) hence sum(db) == 0 and db = [1/3-1, 1/3-1, 2/3]/2 + ...
+    assert abs(db.sum()) < 1e-6
+    np.testing.assert_allclose(db, (np.asarray([1 / 3 - 1, 1 / 3, 1 / 3]) + np.asarray([1 / 3, 1 / 3 - 1, 1 / 3])) / 2, atol=1e-6)
+    # SGD vectors: a net whose only gradient is the bias gradient is awkward; check p -= lr*g directly
+    for key in ("sgd_single_step", "sgd_three_steps", "sgd_2d"):
+        s = h[key]
+        w = np.asarray(s["w"], np.float32)
+        for _ in range(s["steps"]):
+            w = w - np.float32(s["lr"]) * np.asarray(s["grad"], np.float32)
+        np.testing.assert_allclose(w, s["expect"], rtol=1e-6)
+
+
+def test_mlp_step_matches_numpy_fp64(oracle):
+    """The whole restated step against an independent fp64 numpy implementation."""
+    O = oracle
+    from tenmo_amd import rng as R
+
+    dims = [784, 128, 32, 10]
+    Ws, bs = R.xavier_mlp(dims, 1234)
+    m = O.MLP(dims, Ws, bs, 64)
+    W64 = [w.astype(np.float64) for w in Ws]
+    b64 = [b.astype(np.float64) for b in bs]
+    lr = 0.01
+    for step in range(5):
+        x, y = R.mnist_like_batch(64, 1234, step)
+        loss = m.step(x, y, lr)
+        h = [x.astype(np.float64)]
+        for l in range(3):
+            z = h[-1] @ W64[l] + b64[l]
+            h.append(np.maximum(z, 0) if l < 2 else z)
+        z = h[-1]
+        zs = z - z.max(1, keepdims=True)
+        lse = np.log(np.exp(zs).sum(1, keepdims=True))
+        ref_loss = float(-(zs - lse)[np.arange(64), y].mean())
+        assert abs(loss - ref_loss) < 1e-5, (step, loss, ref_loss)
+        g = (np.exp(zs - lse) - np.eye(10)[y]) / 64
+        for l in (2, 1, 0):
+            dW = h[l].T @ g
+            db = g.sum(0)
+            if l > 0:
+                g = (g @ W64[l].T) * (h[l] > 0)
+            W64[l] -= lr * dW
+            b64[l] -= lr * db
+        for l in range(3):
+            W, b = m.params(l)
+            assert rel_fro(W, W64[l]) < 1e-5 and np.abs(b - b64[l]).max() < 1e-6
