@@ -37,7 +37,7 @@ def _finish_backward(output: Tensor, retain_graph: bool) -> None:
 class Matmul2dBackward:
     @staticmethod
     def backward(output: Tensor, retain_graph: bool = False) -> List[Tensor]:
-        A, B = output.ancestors
+        A, B = output.ancestors[:2]  # a Linear appends its bias as a third parent
         check(_lib.load().tenmo_hip_matmul_backward(C.byref(A.buffer.c_view()), C.byref(B.buffer.c_view()),
                                                     output.gradbox.data_ptr(), _ptr_or_null(A), _ptr_or_null(B), 0))
         _finish_backward(output, retain_graph)
