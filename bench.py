@@ -40,6 +40,8 @@ def main() -> int:
     ap.add_argument("--size", type=int, default=8192, help="M=N=K of the square GEMM (default: the headline size)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the mv/vm and MLP-step side measurements")
+    ap.add_argument("--pmc-calibration", action="store_true",
+                    help="also run one plain 1 GiB device copy, the known-size kernel against which FETCH_SIZE/WRITE_SIZE are scaled")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the reference has no multi-GPU path and every "
@@ -56,6 +58,13 @@ def main() -> int:
     cus = C.c_int()
     name = C.create_string_buffer(128)
     L.tenmo_hip_device_info(C.byref(cus), name, 128)
+
+    if args.pmc_calibration:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     S = args.size
     gen = torch.Generator(device="cuda")

@@ -3,16 +3,24 @@
 // C[b][M,N] (dense) (+)= A[b][M,K] . B[b][K,N] where A and B are arbitrary strided views.
 // Replaces matmul_2d_tiled + MatmulNdGpu.launch (tenmo/kernels/matmul_kernel.mojo:38-120,:128-283).
 //
-// Workgroup: 256 threads = 4 wavefronts (2x2), one BM x BN tile of C, K walked in steps of BK=16
-// through a double-buffered LDS stage (one barrier per step; the next step's global loads are in
-// flight in registers while the current one feeds the matrix cores).
+// Workgroup: 256 threads = 4 wavefronts (2x2), one BM x BN tile of C, K walked in steps of BK=16.
+// Two workgroups share a CU (<= 256 VGPRs per lane, <= 72 KiB LDS each), so every SIMD holds two
+// wavefronts that cover each other's barrier and LDS latencies.
 //
 // Each operand is staged in the LDS layout that matches its memory order, so the global->LDS copy
 // is always a straight 16-byte-per-lane copy and a transposed view costs nothing extra:
-//   K-major  (unit stride along K: row-major A, transposed-view B):  tile[row][k], row pitch BK+4
+//   K-major  (unit stride along K: row-major A, transposed-view B): tile[row][16 k], the four
+//            16-byte chunks of a row XOR-swizzled by (row>>2)&3 so that both the row-wise copy-in
+//            and the column-wise operand fetch are free of bank conflicts without padding
 //   MN-major (unit stride along M/N: transposed-view A, row-major B): tile[k][row]
 // Any other striding (both strides non-unit, zero or overlapping) takes the element-wise
 // "generic" loader into the K-major layout.
+//
+// Interior tiles run a three-stage LDS ring filled by direct global->LDS loads
+// (global_load_lds_dwordx4: no staging registers, two K steps in flight), with the operand fetch
+// of the next half step issued before the MFMAs of the current one and carried across the
+// workgroup barrier, so the matrix pipe does not drain at the barrier.  Edge tiles and the K tail
+// use register-staged, bounds-checked loads into two stages of the same ring.
 //
 // MFMA operand order.  v_mfma_f32_32x32x2 consumes, per lane l, A[i=l%32][k=l/32] and
 // B[k=l/32][j=l%32].  The sum over k is order-free, so within every 8-wide k chunk the kernel
@@ -35,7 +43,6 @@ typedef float f32x2_u __attribute__((ext_vector_type(2), aligned(4)));
 typedef float f32x4_u __attribute__((ext_vector_type(4), aligned(4)));
 
 constexpr int GEMM_BK = 16;
-constexpr int GEMM_LDK = GEMM_BK + 4; // K-major row pitch: conflict-free 16-byte reads
 constexpr int GEMM_THREADS = 256;
 constexpr int MAX_BATCH_RANK = 6;
 
@@ -73,59 +80,93 @@ __device__ __forceinline__ void batch_offsets(const BatchDesc& bd, int64_t b, in
     }
 }
 
-// ---- global -> registers -> LDS for one operand tile of ROWS x BK ----------------------------
+// float offset of 16-byte chunk q (0..3) of `row` in a K-major tile
+__device__ __forceinline__ int kmajor_off(int row, int q) { return 4 * (4 * row + (q ^ ((row >> 2) & 3))); }
+
+// ---- one operand tile of ROWS x BK: global -> LDS ---------------------------------------------
 // `row` indexes M for A and N for B; element(row, k) = base[row*rs + k*ks].
 template <int ROWS, int MODE>
 struct TileLoader {
-    static constexpr int NCH = ROWS / 64; // 16-byte chunks per thread
-    f32x4 r[NCH];
+    static constexpr int NCH = ROWS / 64; // 16-byte chunks per thread == direct loads per wavefront
+    static constexpr int QPR = ROWS / 4;  // MN-major: chunks per k row
+    static constexpr int KROWS_PER_WAVELOAD = 256 / ROWS > 0 ? 256 / ROWS : 1;
+    f32x4 r[NCH];        // staging registers of the checked path
+    const float* d0;     // direct path: this lane's source of wave-load 0 at the first K step
+    int64_t dstep;       // direct path: source step between consecutive wave-loads
+    int64_t kstep;       // source step per unit k
 
-    __device__ __forceinline__ void load(const float* __restrict base, int64_t rs, int64_t ks,
-                                         int64_t row0, int64_t k0, int64_t R, int64_t K, bool interior, int t) {
+    __device__ __forceinline__ void init_direct(const float* __restrict base, int64_t rs, int64_t ks, int64_t row0, int64_t k_begin, int t) {
+        const int lane = t & 63, wave = t >> 6;
+        if constexpr (MODE == MNMAJOR_VEC) {
+            const int kk = wave * NCH * KROWS_PER_WAVELOAD + (4 * lane) / ROWS;
+            d0 = base + (k_begin + kk) * ks + row0 + (4 * lane) % ROWS;
+            dstep = KROWS_PER_WAVELOAD * ks;
+            kstep = ks;
+        } else {
+            const int q = (lane & 3) ^ ((lane >> 4) & 3);
+            d0 = base + (row0 + wave * NCH * 16 + (lane >> 2)) * rs + k_begin + 4 * q;
+            dstep = 16 * rs;
+            kstep = 1;
+        }
+    }
+
+    // tile at K offset koff -> LDS tile `lds` (wave-uniform), straight from global memory.
+    // Lane L of a wave-load writes bytes [16L, 16L+16) of that load's 1 KiB LDS block (M0 holds the
+    // block's LDS address).  Issued through inline assembly on purpose: the compiler's wait-count
+    // pass otherwise drains every outstanding direct load before any later LDS read, which would
+    // serialise the ring.  The callers wait for these loads explicitly with s_waitcnt vmcnt(n).
+    __device__ __forceinline__ void load_direct(float* lds, int64_t koff, int t) const {
+        static_assert(MODE != KMAJOR_GEN, "the generic loader has no direct path");
+        const int wave = t >> 6;
+        const float* p = d0 + koff * kstep;
+        const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + (wave * NCH + j) * 1024);
+            const float* src = p + j * dstep;
+            asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src) : "memory");
+        }
+    }
+
+    // register-staged loads with every element checked against the extents (edge tiles, K tail,
+    // generic strides)
+    __device__ __forceinline__ void load_checked(const float* __restrict base, int64_t rs, int64_t ks,
+                                                 int64_t row0, int64_t k0, int64_t R, int64_t K, int t) {
         if constexpr (MODE == KMAJOR_VEC) {
             const int kq = t & 3;
 #pragma unroll
             for (int i = 0; i < NCH; ++i) {
                 const int64_t row = row0 + (t >> 2) + 64 * i;
                 const int64_t k = k0 + 4 * kq;
-                if (interior) {
-                    r[i] = *reinterpret_cast<const f32x4_u*>(base + row * rs + k);
-                } else {
-                    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-                    if (row < R) {
-                        const float* p = base + row * rs + k;
-                        if (k + 3 < K) v = *reinterpret_cast<const f32x4_u*>(p);
-                        else {
-                            if (k + 0 < K) v.x = p[0];
-                            if (k + 1 < K) v.y = p[1];
-                            if (k + 2 < K) v.z = p[2];
-                        }
+                f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                if (row < R) {
+                    const float* p = base + row * rs + k;
+                    if (k + 3 < K) v = *reinterpret_cast<const f32x4_u*>(p);
+                    else {
+                        if (k + 0 < K) v.x = p[0];
+                        if (k + 1 < K) v.y = p[1];
+                        if (k + 2 < K) v.z = p[2];
                     }
-                    r[i] = v;
                 }
+                r[i] = v;
             }
         } else if constexpr (MODE == MNMAJOR_VEC) {
-            constexpr int QPR = ROWS / 4; // chunks per k row
 #pragma unroll
             for (int i = 0; i < NCH; ++i) {
                 const int c = t + GEMM_THREADS * i;
                 const int64_t k = k0 + c / QPR;
                 const int64_t row = row0 + 4 * (c % QPR);
-                if (interior) {
-                    r[i] = *reinterpret_cast<const f32x4_u*>(base + k * ks + row);
-                } else {
-                    f32x4 v = {0.f, 0.f, 0.f, 0.f};
-                    if (k < K) {
-                        const float* p = base + k * ks + row;
-                        if (row + 3 < R) v = *reinterpret_cast<const f32x4_u*>(p);
-                        else {
-                            if (row + 0 < R) v.x = p[0];
-                            if (row + 1 < R) v.y = p[1];
-                            if (row + 2 < R) v.z = p[2];
-                        }
+                f32x4 v = {0.f, 0.f, 0.f, 0.f};
+                if (k < K) {
+                    const float* p = base + k * ks + row;
+                    if (row + 3 < R) v = *reinterpret_cast<const f32x4_u*>(p);
+                    else {
+                        if (row + 0 < R) v.x = p[0];
+                        if (row + 1 < R) v.y = p[1];
+                        if (row + 2 < R) v.z = p[2];
                     }
-                    r[i] = v;
                 }
+                r[i] = v;
             }
         } else { // KMAJOR_GEN: element loads, any strides
             const int kq = t & 3;
@@ -148,7 +189,6 @@ struct TileLoader {
 
     __device__ __forceinline__ void store(float* __restrict lds, int t) const {
         if constexpr (MODE == MNMAJOR_VEC) {
-            constexpr int QPR = ROWS / 4;
 #pragma unroll
             for (int i = 0; i < NCH; ++i) {
                 const int c = t + GEMM_THREADS * i;
@@ -157,13 +197,10 @@ struct TileLoader {
         } else {
 #pragma unroll
             for (int i = 0; i < NCH; ++i)
-                *reinterpret_cast<f32x4*>(lds + ((t >> 2) + 64 * i) * GEMM_LDK + 4 * (t & 3)) = r[i];
+                *reinterpret_cast<f32x4*>(lds + kmajor_off((t >> 2) + 64 * i, t & 3)) = r[i];
         }
     }
 };
-
-template <int ROWS, int MODE>
-constexpr int lds_floats() { return MODE == MNMAJOR_VEC ? GEMM_BK * ROWS : ROWS * GEMM_LDK; }
 
 // ---- LDS -> MFMA operand registers for one 8-wide k chunk ------------------------------------
 // f[b][s]: operand of block b at MFMA step s.  `wave_row0` is the wave's first row in the tile.
@@ -187,7 +224,7 @@ __device__ __forceinline__ void load_fragments(const float* __restrict lds, int 
     } else {
 #pragma unroll
         for (int b = 0; b < NBLK; ++b) {
-            f32x4 v = *reinterpret_cast<const f32x4*>(lds + (wave_row0 + 32 * b + i) * GEMM_LDK + kc * 8 + 4 * h);
+            f32x4 v = *reinterpret_cast<const f32x4*>(lds + kmajor_off(wave_row0 + 32 * b + i, 2 * kc + h));
             f[b][0] = v.x; f[b][1] = v.y; f[b][2] = v.z; f[b][3] = v.w;
         }
     }
@@ -209,13 +246,29 @@ __device__ __forceinline__ int64_t xcd_remap(int64_t pid, int64_t n) {
     return base + local;
 }
 
+// s_waitcnt vmcnt(n) only (expcnt / lgkmcnt left unconstrained), gfx9 encoding
+__device__ __forceinline__ constexpr int vmcnt_imm(int n) { return (n & 0xF) | (0x7 << 4) | (0xF << 8) | ((n >> 4) << 14); }
+
+// workgroup barrier without the memory fence of __syncthreads(): the callers order their LDS
+// traffic themselves (the direct loads are waited for with vmcnt, the reads happen after it)
+__device__ __forceinline__ void bare_barrier() {
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+}
+
 template <int BM, int BN, int AMODE, int BMODE>
 __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmArgs g) {
     constexpr int TM = BM / 2, TN = BN / 2;     // wave tile (2x2 waves)
     constexpr int MB = TM / 32, NB = TN / 32;   // 32x32 MFMA blocks per wave tile
-    constexpr int A_FLOATS = lds_floats<BM, AMODE>();
-    constexpr int B_FLOATS = lds_floats<BN, BMODE>();
-    __shared__ __attribute__((aligned(16))) float lds[2 * (A_FLOATS + B_FLOATS)];
+    constexpr int A_FLOATS = BM * GEMM_BK;
+    constexpr int STAGE_FLOATS = (BM + BN) * GEMM_BK;
+    constexpr bool DIRECT = (AMODE != KMAJOR_GEN) && (BMODE != KMAJOR_GEN);
+    // three separate objects: the compiler can then tell that a direct load into one stage does
+    // not alias the operand fetch from another
+    __shared__ __attribute__((aligned(1024))) float stage0[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage2[DIRECT ? STAGE_FLOATS : 4];
 
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int wm = wave >> 1, wn = wave & 1;
@@ -261,45 +314,104 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     TileLoader<BM, AMODE> la;
     TileLoader<BN, BMODE> lb;
 
-    if (nk > 0) {
-        const bool in0 = rows_interior && (k_begin + GEMM_BK <= k_end);
-        la.load(Ab, a_row_s, a_k_s, m0, k_begin, g.M, k_end, in0, t);
-        lb.load(Bb, b_row_s, b_k_s, n0, k_begin, g.N, k_end, in0, t);
-        la.store(lds, t);
-        lb.store(lds + A_FLOATS, t);
-    }
-    __syncthreads();
-
-    for (int64_t it = 0; it < nk; ++it) {
-        const int cur = (int)(it & 1);
-        const float* __restrict As = lds + cur * (A_FLOATS + B_FLOATS);
-        const float* __restrict Bs = As + A_FLOATS;
-        const bool more = (it + 1 < nk);
-        if (more) {
-            const int64_t k0 = k_begin + (it + 1) * GEMM_BK;
-            const bool interior = rows_interior && (k0 + GEMM_BK <= k_end);
-            la.load(Ab, a_row_s, a_k_s, m0, k0, g.M, k_end, interior, t);
-            lb.load(Bb, b_row_s, b_k_s, n0, k0, g.N, k_end, interior, t);
-        }
+    auto mfma_chunk = [&](const float (&fa)[MB][4], const float (&fb)[NB][4]) {
+#pragma unroll
+        for (int s = 0; s < 4; ++s)
+#pragma unroll
+            for (int i = 0; i < MB; ++i)
+#pragma unroll
+                for (int j = 0; j < NB; ++j)
+                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+    };
+    auto compute = [&](const float* __restrict st) {
 #pragma unroll
         for (int kc = 0; kc < GEMM_BK / 8; ++kc) {
             float fa[MB][4], fb[NB][4];
-            load_fragments<BM, AMODE, MB>(As, wm * TM, kc, lane, fa);
-            load_fragments<BN, BMODE, NB>(Bs, wn * TN, kc, lane, fb);
-#pragma unroll
-            for (int s = 0; s < 4; ++s)
-#pragma unroll
-                for (int i = 0; i < MB; ++i)
-#pragma unroll
-                    for (int j = 0; j < NB; ++j)
-                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+            load_fragments<BM, AMODE, MB>(st, wm * TM, kc, lane, fa);
+            load_fragments<BN, BMODE, NB>(st + A_FLOATS, wn * TN, kc, lane, fb);
+            mfma_chunk(fa, fb);
         }
-        if (more) {
-            float* nxt = lds + (cur ^ 1) * (A_FLOATS + B_FLOATS);
-            la.store(nxt, t);
-            lb.store(nxt + A_FLOATS, t);
+    };
+
+    int64_t done = 0; // K steps finished by the direct pipeline
+    if constexpr (DIRECT) {
+        // ---- interior tiles: three-stage direct-to-LDS ring ----
+        const int64_t nfast = rows_interior ? (k_end - k_begin) / GEMM_BK : 0;
+        if (nfast > 0) {
+            constexpr int NL = TileLoader<BM, AMODE>::NCH + TileLoader<BN, BMODE>::NCH; // direct loads per wave per K step
+            la.init_direct(Ab, a_row_s, a_k_s, m0, k_begin, t);
+            lb.init_direct(Bb, b_row_s, b_k_s, n0, k_begin, t);
+            auto issue = [&](float* st, int64_t it) {
+                la.load_direct(st, it * GEMM_BK, t);
+                lb.load_direct(st + A_FLOATS, it * GEMM_BK, t);
+            };
+            float fa0[MB][4], fb0[NB][4], fa1[MB][4], fb1[NB][4];
+            issue(stage0, 0);
+            if (nfast > 1) {
+                issue(stage1, 1);
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(NL));
+            } else {
+                __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+            }
+            bare_barrier();
+            load_fragments<BM, AMODE, MB>(stage0, wm * TM, 0, lane, fa0);
+            load_fragments<BN, BMODE, NB>(stage0 + A_FLOATS, wn * TN, 0, lane, fb0);
+
+            // one K step: `cur` holds step it, `nxt` step it+1 (in flight), `ld` receives step it+2
+            auto step = [&](float* cur, float* nxt, float* ld, int64_t it) {
+                const bool have_ld = it + 2 < nfast, have_next = it + 1 < nfast;
+                if (have_ld) issue(ld, it + 2);
+                load_fragments<BM, AMODE, MB>(cur, wm * TM, 1, lane, fa1);
+                load_fragments<BN, BMODE, NB>(cur + A_FLOATS, wn * TN, 1, lane, fb1);
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_chunk(fa0, fb0);
+                __builtin_amdgcn_sched_barrier(0);
+                if (have_next) {
+                    if (have_ld) __builtin_amdgcn_s_waitcnt(vmcnt_imm(NL));
+                    else __builtin_amdgcn_s_waitcnt(vmcnt_imm(0));
+                    bare_barrier();
+                    load_fragments<BM, AMODE, MB>(nxt, wm * TM, 0, lane, fa0);
+                    load_fragments<BN, BMODE, NB>(nxt + A_FLOATS, wn * TN, 0, lane, fb0);
+                }
+                __builtin_amdgcn_sched_barrier(0);
+                mfma_chunk(fa1, fb1);
+                __builtin_amdgcn_sched_barrier(0);
+            };
+            for (int64_t it = 0; it < nfast; it += 3) {
+                step(stage0, stage1, stage2, it);
+                if (it + 1 >= nfast) break;
+                step(stage1, stage2, stage0, it + 1);
+                if (it + 2 >= nfast) break;
+                step(stage2, stage0, stage1, it + 2);
+            }
+            done = nfast;
+            __syncthreads(); // every wave has left the ring before the tail reuses stage0/stage1
         }
+    }
+
+    // ---- edge tiles, the K tail, generic strides: register-staged checked loads, two stages ----
+    if (done < nk) {
+        la.load_checked(Ab, a_row_s, a_k_s, m0, k_begin + done * GEMM_BK, g.M, k_end, t);
+        lb.load_checked(Bb, b_row_s, b_k_s, n0, k_begin + done * GEMM_BK, g.N, k_end, t);
+        la.store(stage0, t);
+        lb.store(stage0 + A_FLOATS, t);
         __syncthreads();
+        for (int64_t it = done; it < nk; ++it) {
+            float* cur = ((it - done) & 1) ? stage1 : stage0;
+            float* nxt = ((it - done) & 1) ? stage0 : stage1;
+            const bool more = (it + 1 < nk);
+            if (more) {
+                const int64_t k0 = k_begin + (it + 1) * GEMM_BK;
+                la.load_checked(Ab, a_row_s, a_k_s, m0, k0, g.M, k_end, t);
+                lb.load_checked(Bb, b_row_s, b_k_s, n0, k0, g.N, k_end, t);
+            }
+            compute(cur);
+            if (more) {
+                la.store(nxt, t);
+                lb.store(nxt + A_FLOATS, t);
+            }
+            __syncthreads();
+        }
     }
 
     // ---- epilogue ----
