@@ -11,7 +11,8 @@ from typing import Sequence
 
 MAX_RANK = 8
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(_HERE, "libtenmo_hip.so")
+# TENMO_HIP_LIBRARY plays the role of the reference's BLAS_PATH define (tenmo/blashandle.mojo:108-110)
+LIB_PATH = os.environ.get("TENMO_HIP_LIBRARY") or os.path.join(_HERE, "libtenmo_hip.so")
 
 OP_DOT, OP_VM, OP_MV, OP_MM, OP_INVALID = 0, 1, 2, 3, -1
 

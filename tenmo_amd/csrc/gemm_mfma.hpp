@@ -42,6 +42,15 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x2_u __attribute__((ext_vector_type(2), aligned(4)));
 typedef float f32x4_u __attribute__((ext_vector_type(4), aligned(4)));
 
+#ifndef TENMO_EXP_SETPRIO
+#define TENMO_EXP_SETPRIO 1
+#endif
+#ifndef TENMO_EXP_GROUP_M
+#define TENMO_EXP_GROUP_M 8
+#endif
+#ifndef TENMO_EXP_XCD
+#define TENMO_EXP_XCD 0
+#endif
 constexpr int GEMM_BK = 16;
 constexpr int GEMM_THREADS = 256;
 constexpr int MAX_BATCH_RANK = 6;
@@ -275,10 +284,10 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
 
     // ---- which tile ----
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-    int64_t pid = xcd_remap(blockIdx.x, gridDim.x);
+    int64_t pid = TENMO_EXP_XCD ? xcd_remap(blockIdx.x, gridDim.x) : (int64_t)blockIdx.x;
     const int64_t batch = pid / tiles;
     const int64_t tid = pid % tiles;
-    constexpr int GROUP_M = 8;
+    constexpr int GROUP_M = TENMO_EXP_GROUP_M;
     const int64_t per_group = (int64_t)GROUP_M * g.tiles_n;
     const int64_t first_m = (tid / per_group) * GROUP_M;
     const int64_t gsz = min((int64_t)g.tiles_m - first_m, (int64_t)GROUP_M);
@@ -315,6 +324,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     TileLoader<BN, BMODE> lb;
 
     auto mfma_chunk = [&](const float (&fa)[MB][4], const float (&fb)[NB][4]) {
+        if (TENMO_EXP_SETPRIO == 1) __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
@@ -322,6 +332,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
 #pragma unroll
                 for (int j = 0; j < NB; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+        if (TENMO_EXP_SETPRIO == 1) __builtin_amdgcn_s_setprio(0);
     };
     auto compute = [&](const float* __restrict st) {
 #pragma unroll

@@ -146,18 +146,16 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
         if (full) {
             const float* __restrict p = Mb + kc * g.m_rs + col;
             int kk = 0;
-            for (; kk + 4 <= len; kk += 4) {
-                f32x4 m0 = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(p + (int64_t)(kk + 0) * g.m_rs));
-                f32x4 m1 = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(p + (int64_t)(kk + 1) * g.m_rs));
-                f32x4 m2 = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(p + (int64_t)(kk + 2) * g.m_rs));
-                f32x4 m3 = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(p + (int64_t)(kk + 3) * g.m_rs));
+            constexpr int U = 8; // independent 16-byte loads in flight per lane
+            for (; kk + U <= len; kk += U) {
+                f32x4 m[U];
 #pragma unroll
-                for (int r = 0; r < R; ++r) {
-                    acc[r] += m0 * xs[r][kk + 0];
-                    acc[r] += m1 * xs[r][kk + 1];
-                    acc[r] += m2 * xs[r][kk + 2];
-                    acc[r] += m3 * xs[r][kk + 3];
-                }
+                for (int u = 0; u < U; ++u)
+                    m[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(p + (int64_t)(kk + u) * g.m_rs));
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+#pragma unroll
+                    for (int r = 0; r < R; ++r) acc[r] += m[u] * xs[r][kk + u];
             }
             for (; kk < len; ++kk) {
                 f32x4 m0 = *reinterpret_cast<const f32x4_u*>(p + (int64_t)kk * g.m_rs);

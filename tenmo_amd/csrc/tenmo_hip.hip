@@ -67,6 +67,7 @@ struct State {
     // tuning overrides (environment, read once): -1 = automatic
     int force_tile = -1;
     int force_splitk = -1;
+    int cols_waves_per_cu = 8; // target workgroups per CU of the column-streaming kernels
 };
 State S;
 std::mutex S_mu;
@@ -298,7 +299,7 @@ int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* 
         for (int d = 0; d < MAX_BATCH_RANK; ++d) std::swap(c.batch.a_str[d], c.batch.b_str[d]);
         const int64_t col_blocks = (n_out + COLS_THREADS * 4 - 1) / (COLS_THREADS * 4);
         int64_t splits = 1;
-        const int64_t want = (int64_t)S.cus * 8;
+        const int64_t want = (int64_t)S.cus * S.cols_waves_per_cu;
         if (col_blocks * batch_count < want) splits = std::min<int64_t>((want + col_blocks * batch_count - 1) / (col_blocks * batch_count), (n_red + COLS_KCHUNK - 1) / COLS_KCHUNK);
         splits = std::max<int64_t>(1, std::min<int64_t>(splits, 65535));
         int64_t per = (n_red + splits - 1) / splits;
@@ -338,7 +339,7 @@ int skinny_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, 
     c.batch = bd;
     const int64_t col_blocks = (N + COLS_THREADS * 4 - 1) / (COLS_THREADS * 4);
     int64_t splits = 1;
-    const int64_t want = (int64_t)S.cus * 8;
+    const int64_t want = (int64_t)S.cus * S.cols_waves_per_cu;
     if (col_blocks * batch_count < want) splits = std::min<int64_t>((want + col_blocks * batch_count - 1) / (col_blocks * batch_count), (K + COLS_KCHUNK - 1) / COLS_KCHUNK);
     splits = std::max<int64_t>(1, std::min<int64_t>(splits, 65535));
     int64_t per = (K + splits - 1) / splits;
@@ -600,6 +601,7 @@ int tenmo_hip_set_tuning(const char* name, int value) {
     if (!name) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: null name");
     if (!strcmp(name, "gemm_tile")) { S.force_tile = value; return 0; }
     if (!strcmp(name, "gemm_splitk")) { S.force_splitk = value; return 0; }
+    if (!strcmp(name, "cols_wg_per_cu")) { S.cols_waves_per_cu = value > 0 ? value : 8; return 0; }
     return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: unknown knob '%s'", name);
 }
 
