@@ -27,9 +27,10 @@ sys.path.insert(0, ROOT)
 PEAK_FP32_MFMA_TFLOPS = 157.3  # 256 CU x 2.4 GHz x 256 flop/clk/CU
 PEAK_HBM_GBPS = 8000.0
 
-# HBM bytes per 8192^3 launch measured with rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE (see
-# profiles/); None until a counter run has been recorded for the current kernel.
-MEASURED_TRAFFIC_BYTES = None
+# Bytes moved between L2 and the memory fabric per 8192^3 launch, from two rocprofv3 --pmc runs
+# (FETCH_SIZE 4.328e6 KiB scaled by 2.0, WRITE_SIZE 2.621e5 KiB scaled by 1.0; the scale factors are
+# what the same counters read for a plain 1 GiB copy).  Only valid for the default size.
+MEASURED_TRAFFIC_BYTES = 9.13e9
 
 
 def main() -> int:
@@ -119,7 +120,7 @@ def main() -> int:
         "config": {"workload": "square fp32 GEMM C=A.B, M=N=K=%d, A and B row-major N(0,1), inputs resident in HBM" % S,
                    "device": name.value.decode(), "compute_units": cus.value},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES,
+                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES if S == 8192 else None,
                      "kernel_ms": round(kernel_ms, 4)},
         "rel_fro_error_vs_fp64": rel_err,
     }
