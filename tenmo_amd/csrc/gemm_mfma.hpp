@@ -471,13 +471,22 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     }
 }
 
-// Sums the k_splits partial results into C (plain or accumulating).
+// Sums the k_splits partial results into C (plain or accumulating), slices in a fixed order.
+// One thread per output; eight slice loads in flight per thread.
 __global__ void splitk_reduce_kernel(const float* __restrict partial, float* __restrict C, int64_t n, int splits, int accumulate) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (; i < n; i += stride) {
         float s = accumulate ? C[i] : 0.f;
-        for (int p = 0; p < splits; ++p) s += partial[(int64_t)p * n + i];
+        int p = 0;
+        for (; p + 8 <= splits; p += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = partial[(int64_t)(p + u) * n + i];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += v[u];
+        }
+        for (; p < splits; ++p) s += partial[(int64_t)p * n + i];
         C[i] = s;
     }
 }

@@ -67,7 +67,7 @@ struct State {
     // tuning overrides (environment, read once): -1 = automatic
     int force_tile = -1;
     int force_splitk = -1;
-    int cols_waves_per_cu = 8; // target workgroups per CU of the column-streaming kernels
+    int cols_waves_per_cu = 2; // target workgroups per CU of the column-streaming kernels (long K slices stream best)
 };
 State S;
 std::mutex S_mu;
@@ -601,7 +601,7 @@ int tenmo_hip_set_tuning(const char* name, int value) {
     if (!name) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: null name");
     if (!strcmp(name, "gemm_tile")) { S.force_tile = value; return 0; }
     if (!strcmp(name, "gemm_splitk")) { S.force_splitk = value; return 0; }
-    if (!strcmp(name, "cols_wg_per_cu")) { S.cols_waves_per_cu = value > 0 ? value : 8; return 0; }
+    if (!strcmp(name, "cols_wg_per_cu")) { S.cols_waves_per_cu = value > 0 ? value : 2; return 0; }
     return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: unknown knob '%s'", name);
 }
 
