@@ -42,15 +42,6 @@ typedef float f32x16 __attribute__((ext_vector_type(16)));
 typedef float f32x2_u __attribute__((ext_vector_type(2), aligned(4)));
 typedef float f32x4_u __attribute__((ext_vector_type(4), aligned(4)));
 
-#ifndef TENMO_EXP_SETPRIO
-#define TENMO_EXP_SETPRIO 1
-#endif
-#ifndef TENMO_EXP_GROUP_M
-#define TENMO_EXP_GROUP_M 8
-#endif
-#ifndef TENMO_EXP_XCD
-#define TENMO_EXP_XCD 0
-#endif
 constexpr int GEMM_BK = 16;
 constexpr int GEMM_THREADS = 256;
 constexpr int MAX_BATCH_RANK = 6;
@@ -100,21 +91,29 @@ struct TileLoader {
     static constexpr int QPR = ROWS / 4;  // MN-major: chunks per k row
     static constexpr int KROWS_PER_WAVELOAD = 256 / ROWS > 0 ? 256 / ROWS : 1;
     f32x4 r[NCH];        // staging registers of the checked path
-    const float* d0;     // direct path: this lane's source of wave-load 0 at the first K step
-    int64_t dstep;       // direct path: source step between consecutive wave-loads
+    const float* d[NCH]; // direct path: this lane's source of wave-load j at the first K step
     int64_t kstep;       // source step per unit k
 
-    __device__ __forceinline__ void init_direct(const float* __restrict base, int64_t rs, int64_t ks, int64_t row0, int64_t k_begin, int t) {
+    // Rows at or beyond the extent R are clamped onto valid rows: their products are never stored,
+    // they only have to be readable.  (An MN-major operand moves 4 rows per 16-byte chunk, so a
+    // ragged extent there needs R % 4 == 0; the caller checks.)
+    __device__ __forceinline__ void init_direct(const float* __restrict base, int64_t rs, int64_t ks, int64_t row0, int64_t k_begin, int64_t R, int t) {
         const int lane = t & 63, wave = t >> 6;
         if constexpr (MODE == MNMAJOR_VEC) {
-            const int kk = wave * NCH * KROWS_PER_WAVELOAD + (4 * lane) / ROWS;
-            d0 = base + (k_begin + kk) * ks + row0 + (4 * lane) % ROWS;
-            dstep = KROWS_PER_WAVELOAD * ks;
+            const int64_t row = min(row0 + (4 * lane) % ROWS, R - 4);
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+                const int kk = (wave * NCH + j) * KROWS_PER_WAVELOAD + (4 * lane) / ROWS;
+                d[j] = base + (k_begin + kk) * ks + row;
+            }
             kstep = ks;
         } else {
             const int q = (lane & 3) ^ ((lane >> 4) & 3);
-            d0 = base + (row0 + wave * NCH * 16 + (lane >> 2)) * rs + k_begin + 4 * q;
-            dstep = 16 * rs;
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+                const int64_t row = min(row0 + (wave * NCH + j) * 16 + (lane >> 2), R - 1);
+                d[j] = base + row * rs + k_begin + 4 * q;
+            }
             kstep = 1;
         }
     }
@@ -127,12 +126,12 @@ struct TileLoader {
     __device__ __forceinline__ void load_direct(float* lds, int64_t koff, int t) const {
         static_assert(MODE != KMAJOR_GEN, "the generic loader has no direct path");
         const int wave = t >> 6;
-        const float* p = d0 + koff * kstep;
+        const int64_t step = koff * kstep;
         const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
 #pragma unroll
         for (int j = 0; j < NCH; ++j) {
             const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + (wave * NCH + j) * 1024);
-            const float* src = p + j * dstep;
+            const float* src = d[j] + step;
             asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off" : : "s"(dst), "v"(src) : "memory");
         }
     }
@@ -243,18 +242,6 @@ __device__ __forceinline__ void load_fragments(const float* __restrict lds, int 
 template <int MODE, int NBLK>
 __device__ __forceinline__ int tile_pos(int b, int x) { return MODE == MNMAJOR_VEC ? NBLK * x + b : 32 * b + x; }
 
-// XCD-aware, L2-friendly block order.  Hardware deals consecutive workgroup ids round-robin to
-// the 8 XCDs (each with its own L2); give every XCD a contiguous run of tiles, and walk the
-// tiles of a run in groups of GROUP_M tile-rows so that concurrently resident tiles share
-// A rows and B columns.
-__device__ __forceinline__ int64_t xcd_remap(int64_t pid, int64_t n) {
-    constexpr int XCDS = 8;
-    const int64_t q = n / XCDS, rem = n % XCDS;
-    const int64_t xcd = pid % XCDS, local = pid / XCDS;
-    const int64_t base = xcd < rem ? xcd * (q + 1) : rem * (q + 1) + (xcd - rem) * q;
-    return base + local;
-}
-
 // s_waitcnt vmcnt(n) only (expcnt / lgkmcnt left unconstrained), gfx9 encoding
 __device__ __forceinline__ constexpr int vmcnt_imm(int n) { return (n & 0xF) | (0x7 << 4) | (0xF << 8) | ((n >> 4) << 14); }
 
@@ -284,10 +271,13 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
 
     // ---- which tile ----
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-    int64_t pid = TENMO_EXP_XCD ? xcd_remap(blockIdx.x, gridDim.x) : (int64_t)blockIdx.x;
+    // Workgroup ids are dealt round-robin to the 8 XCDs, so with groups of 8 tile-rows each XCD
+    // keeps one 'tile-row' of A hot in its L2 and streams B past it.  (A blocked 8x8-tiles-per-XCD
+    // order was measured: more L2-miss traffic and 1.4 % slower.)
+    const int64_t pid = blockIdx.x;
     const int64_t batch = pid / tiles;
     const int64_t tid = pid % tiles;
-    constexpr int GROUP_M = TENMO_EXP_GROUP_M;
+    constexpr int GROUP_M = 8;
     const int64_t per_group = (int64_t)GROUP_M * g.tiles_n;
     const int64_t first_m = (tid / per_group) * GROUP_M;
     const int64_t gsz = min((int64_t)g.tiles_m - first_m, (int64_t)GROUP_M);
@@ -310,7 +300,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
         k_end = min(g.K, k_begin + g.k_per_split);
     }
     const int64_t nk = (k_end > k_begin) ? (k_end - k_begin + GEMM_BK - 1) / GEMM_BK : 0;
-    const bool rows_interior = (m0 + BM <= g.M) && (n0 + BN <= g.N);
 
     f32x16 acc[MB][NB];
 #pragma unroll
@@ -324,7 +313,9 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     TileLoader<BN, BMODE> lb;
 
     auto mfma_chunk = [&](const float (&fa)[MB][4], const float (&fb)[NB][4]) {
-        if (TENMO_EXP_SETPRIO == 1) __builtin_amdgcn_s_setprio(1);
+        // the co-resident wavefront of the other workgroup gets the LDS / memory issue slots while
+        // this one feeds the matrix pipe (+4 % at 8192^3)
+        __builtin_amdgcn_s_setprio(1);
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
@@ -332,7 +323,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
 #pragma unroll
                 for (int j = 0; j < NB; ++j)
                     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
-        if (TENMO_EXP_SETPRIO == 1) __builtin_amdgcn_s_setprio(0);
+        __builtin_amdgcn_s_setprio(0);
     };
     auto compute = [&](const float* __restrict st) {
 #pragma unroll
@@ -347,11 +338,14 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     int64_t done = 0; // K steps finished by the direct pipeline
     if constexpr (DIRECT) {
         // ---- interior tiles: three-stage direct-to-LDS ring ----
-        const int64_t nfast = rows_interior ? (k_end - k_begin) / GEMM_BK : 0;
+        // ragged tiles stay on the direct path as long as clamping rows is enough
+        const bool a_ok = (m0 + BM <= g.M) || AMODE == KMAJOR_VEC || (g.M % 4 == 0 && g.M >= 4);
+        const bool b_ok = (n0 + BN <= g.N) || BMODE == KMAJOR_VEC || (g.N % 4 == 0 && g.N >= 4);
+        const int64_t nfast = (a_ok && b_ok) ? (k_end - k_begin) / GEMM_BK : 0;
         if (nfast > 0) {
             constexpr int NL = TileLoader<BM, AMODE>::NCH + TileLoader<BN, BMODE>::NCH; // direct loads per wave per K step
-            la.init_direct(Ab, a_row_s, a_k_s, m0, k_begin, t);
-            lb.init_direct(Bb, b_row_s, b_k_s, n0, k_begin, t);
+            la.init_direct(Ab, a_row_s, a_k_s, m0, k_begin, g.M, t);
+            lb.init_direct(Bb, b_row_s, b_k_s, n0, k_begin, g.N, t);
             auto issue = [&](float* st, int64_t it) {
                 la.load_direct(st, it * GEMM_BK, t);
                 lb.load_direct(st + A_FLOATS, it * GEMM_BK, t);

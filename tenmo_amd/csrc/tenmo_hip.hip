@@ -12,6 +12,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <cmath>
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
@@ -67,6 +68,7 @@ struct State {
     // tuning overrides (environment, read once): -1 = automatic
     int force_tile = -1;
     int force_splitk = -1;
+    int verbose = 0;
     int cols_waves_per_cu = 2; // target workgroups per CU of the column-streaming kernels (long K slices stream best)
 };
 State S;
@@ -175,7 +177,8 @@ int launch_gemm_tile(const GemmArgs& g, dim3 grid, int am, int bm) {
 }
 
 struct TileShape { int bm, bn; };
-const TileShape kTiles[3] = {{256, 128}, {128, 128}, {64, 64}};
+constexpr int kNumTiles = 5;
+const TileShape kTiles[kNumTiles] = {{256, 128}, {128, 128}, {64, 64}, {128, 64}, {64, 128}};
 
 int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, int64_t b_rs, int64_t b_cs, float* C,
                   int64_t M, int64_t N, int64_t K, const BatchDesc& bd, int64_t batch_count, int accumulate) {
@@ -197,21 +200,43 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     const int am = operand_mode(a_rs, a_cs, M, K);
     const int bm = operand_mode(b_cs, b_rs, N, K);
 
-    // tile: the largest whose grid still fills the chip
-    auto blocks = [&](int t) { return ((M + kTiles[t].bm - 1) / kTiles[t].bm) * ((N + kTiles[t].bn - 1) / kTiles[t].bn) * batch_count; };
-    int tile = 2;
-    if (blocks(0) >= (int64_t)S.cus * 3 / 2) tile = 0;
-    else if (blocks(1) >= (int64_t)S.cus) tile = 1;
-    if (S.force_tile >= 0 && S.force_tile < 3) tile = S.force_tile;
-
-    // split K when even the chosen tile leaves most of the chip idle and K is long
-    int splits = 1;
-    const int64_t nb = blocks(tile);
-    if (nb < S.cus && K >= 1024) {
-        splits = (int)std::min<int64_t>({(2 * (int64_t)S.cus + nb - 1) / nb, K / 256, (int64_t)32});
-        if (splits < 1) splits = 1;
+    // Pick the workgroup tile and the number of K slices with a small cost model of this chip
+    // (constants fitted to measured launches on MI355X): per CU the matrix-pipe time is the sum over
+    // its workgroups, a lone wavefront per SIMD cannot hide its own barrier/LDS latency, every
+    // workgroup pays a fixed prologue/epilogue, and the launch can never beat its HBM and L2 traffic.
+    int tile = 0, splits = 1;
+    {
+        static const double kOcc[kNumTiles] = {2, 3, 6, 4, 4};             // resident workgroups per CU (LDS / VGPR limits)
+        static const double kEff[kNumTiles] = {0.93, 0.92, 0.86, 0.90, 0.90}; // matrix-pipe efficiency at full occupancy
+        static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
+        const double cus = (double)S.cus;
+        double best = 1e300;
+        for (int t = 0; t < kNumTiles; ++t) {
+            const double tm = (double)((M + kTiles[t].bm - 1) / kTiles[t].bm), tn = (double)((N + kTiles[t].bn - 1) / kTiles[t].bn);
+            const double tiles = tm * tn * (double)batch_count;
+            const double m_us = (kTiles[t].bm / 64) * (kTiles[t].bn / 64) * 8 * 64 / 2400.0; // MFMA time of one K step of one wavefront
+            for (int sp : kSplits) {
+                if (sp > 1 && (K / sp < 64 || (double)sp * batch_count * M * N * 4.0 > 1.0e9)) break;
+                const double wgs = tiles * sp, slots = cus * kOcc[t];
+                // one round = every CU runs `conc` workgroups side by side; the dispatcher refills a CU
+                // only as slots free, so a partial extra round costs a whole one
+                const double rounds = wgs <= slots ? 1.0 : std::ceil(wgs / slots);
+                const double conc = wgs <= slots ? std::ceil(wgs / cus) : kOcc[t];
+                const double iters = std::ceil((double)K / sp / GEMM_BK);
+                const double t_round = iters * std::max(conc * m_us, 0.23 + m_us) / kEff[t] + 2.5;
+                const double bytes = 4.0 * batch_count * ((double)M * K + (double)K * N + (double)M * N * (sp > 1 ? sp + 1.0 : 1.0));
+                const double l2_bytes = 4.0 * batch_count * (double)K * ((double)M * tn + (double)N * tm);
+                double est = std::max({rounds * t_round, bytes / 5.0e6, l2_bytes / 14.0e6}) + 3.0;
+                if (sp > 1) est += 5.0 + 4.0 * batch_count * (double)M * N * (sp + 1.0) / 4.0e6;
+                if (est < best) { best = est; tile = t; splits = sp; }
+            }
+        }
+        if (S.verbose) fprintf(stderr, "tenmo_hip gemm M=%lld N=%lld K=%lld batch=%lld -> tile %dx%d, %d K slice(s), est %.1f us\n",
+                               (long long)M, (long long)N, (long long)K, (long long)batch_count, kTiles[tile].bm, kTiles[tile].bn, splits, best);
     }
+    if (S.force_tile >= 0 && S.force_tile < kNumTiles) tile = S.force_tile;
     if (S.force_splitk > 0) splits = S.force_splitk;
+    const int64_t nb = ((M + kTiles[tile].bm - 1) / kTiles[tile].bm) * ((N + kTiles[tile].bn - 1) / kTiles[tile].bn) * batch_count;
     g.k_splits = splits;
     g.k_per_split = K;
     if (splits > 1) {
@@ -234,6 +259,8 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     switch (tile) {
         case 0: rc = launch_gemm_tile<256, 128>(g, grid, am, bm); break;
         case 1: rc = launch_gemm_tile<128, 128>(g, grid, am, bm); break;
+        case 3: rc = launch_gemm_tile<128, 64>(g, grid, am, bm); break;
+        case 4: rc = launch_gemm_tile<64, 128>(g, grid, am, bm); break;
         default: rc = launch_gemm_tile<64, 64>(g, grid, am, bm); break;
     }
     if (rc) return rc;
@@ -557,6 +584,7 @@ int tenmo_hip_init(int device_id) {
     HIP_TRY(hipEventCreate(&S.ev1));
     S.force_tile = env_int("TENMO_HIP_GEMM_TILE", -1);
     S.force_splitk = env_int("TENMO_HIP_GEMM_SPLITK", -1);
+    S.verbose = env_int("TENMO_HIP_VERBOSE", 0);
     S.ready = true;
     return 0;
 }
