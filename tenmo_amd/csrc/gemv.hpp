@@ -96,7 +96,8 @@ __global__ __launch_bounds__(64 * MV_WAVES) void mv_rows_kernel(const GemvArgs g
 
 // ---- columns kernel: unit stride across the outputs ((R x k) . (k x n), R <= 8) ---------------
 // out[r][j] = sum_k X[r][k] * Mx[k][j].  A workgroup owns 1024 consecutive columns (one 16-byte
-// load per lane per k row: 1 KiB bursts per wavefront) and one slice of k; the R x slice block of
+// load per lane per k row: 1 KiB bursts per wavefront; dword loads when rows are not 16-byte
+// aligned) and one slice of k; the R x slice block of
 // X is staged in LDS and broadcast.  Partial sums of the k slices go to `partial` and are added by
 // colsplit_reduce_kernel, so the result does not depend on scheduling.
 struct ColsArgs {
@@ -114,12 +115,18 @@ struct ColsArgs {
 
 constexpr int COLS_THREADS = 256;
 constexpr int COLS_KCHUNK = 128; // k rows staged per LDS refill
+constexpr int COLS_KSLICE_MIN = 32; // granularity of the K slices handed to workgroups
 
-template <int R>
+// ALIGNED: every row of the matrix starts on a 16-byte boundary -> a lane owns 4 consecutive columns
+// and moves them with one 16-byte load.  Otherwise (row pitch not a multiple of 4 floats, e.g.
+// N = 50257) 16-byte loads would straddle and run at half rate, so a lane owns 4 columns 256 apart
+// and uses dword loads, each still one contiguous 256-byte burst per wavefront.
+template <int R, bool ALIGNED>
 __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
     __shared__ float xs[R][COLS_KCHUNK];
     const int t = threadIdx.x;
-    const int64_t col = ((int64_t)blockIdx.x * COLS_THREADS + t) * 4;
+    const int64_t col0 = (int64_t)blockIdx.x * COLS_THREADS * 4 + (ALIGNED ? 4 * t : t);
+    constexpr int CSTEP = ALIGNED ? 1 : COLS_THREADS; // distance between a lane's 4 columns
     const int64_t batch = blockIdx.z;
     int64_t x_off, m_off;
     batch_offsets(g.batch, batch, x_off, m_off);
@@ -128,12 +135,18 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
 
     const int64_t k_begin = (int64_t)blockIdx.y * g.k_per_split;
     const int64_t k_end = min(g.k, k_begin + g.k_per_split);
-    const bool full = (col + 3 < g.n);
-    const bool any = (col < g.n);
+    const bool full = (col0 + 3 * CSTEP < g.n);
+    const bool any = (col0 < g.n);
 
     f32x4 acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+    auto load4 = [&](const float* __restrict p) -> f32x4 {
+        if constexpr (ALIGNED) return __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
+        else return f32x4{__builtin_nontemporal_load(p), __builtin_nontemporal_load(p + CSTEP),
+                          __builtin_nontemporal_load(p + 2 * CSTEP), __builtin_nontemporal_load(p + 3 * CSTEP)};
+    };
 
     for (int64_t kc = k_begin; kc < k_end; kc += COLS_KCHUNK) {
         const int len = (int)min((int64_t)COLS_KCHUNK, k_end - kc);
@@ -144,31 +157,31 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
         }
         __syncthreads();
         if (full) {
-            const float* __restrict p = Mb + kc * g.m_rs + col;
+            const float* __restrict p = Mb + kc * g.m_rs + col0;
             int kk = 0;
-            constexpr int U = 8; // independent 16-byte loads in flight per lane
+            constexpr int U = 8; // independent row loads in flight per lane
             for (; kk + U <= len; kk += U) {
                 f32x4 m[U];
 #pragma unroll
-                for (int u = 0; u < U; ++u)
-                    m[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(p + (int64_t)(kk + u) * g.m_rs));
+                for (int u = 0; u < U; ++u) m[u] = load4(p + (int64_t)(kk + u) * g.m_rs);
 #pragma unroll
                 for (int u = 0; u < U; ++u)
 #pragma unroll
                     for (int r = 0; r < R; ++r) acc[r] += m[u] * xs[r][kk + u];
             }
             for (; kk < len; ++kk) {
-                f32x4 m0 = *reinterpret_cast<const f32x4_u*>(p + (int64_t)kk * g.m_rs);
+                const f32x4 m0 = load4(p + (int64_t)kk * g.m_rs);
 #pragma unroll
                 for (int r = 0; r < R; ++r) acc[r] += m0 * xs[r][kk];
             }
         } else if (any) {
             for (int kk = 0; kk < len; ++kk) {
-                const float* p = Mb + (kc + kk) * g.m_rs + col;
+                const float* p = Mb + (kc + kk) * g.m_rs + col0;
                 f32x4 m0 = {0.f, 0.f, 0.f, 0.f};
                 m0.x = p[0];
-                if (col + 1 < g.n) m0.y = p[1];
-                if (col + 2 < g.n) m0.z = p[2];
+                if (col0 + CSTEP < g.n) m0.y = p[CSTEP];
+                if (col0 + 2 * CSTEP < g.n) m0.z = p[2 * CSTEP];
+                if (col0 + 3 * CSTEP < g.n) m0.w = p[3 * CSTEP];
 #pragma unroll
                 for (int r = 0; r < R; ++r) acc[r] += m0 * xs[r][kk];
             }
@@ -181,15 +194,16 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
 #pragma unroll
     for (int r = 0; r < R; ++r) {
         if (r >= g.rows) break;
-        float* o = ob + (int64_t)r * g.n + col;
-        if (full) {
+        float* o = ob + (int64_t)r * g.n + col0;
+        if (ALIGNED && full) {
             f32x4 v = acc[r];
             if (accumulate) v += *reinterpret_cast<const f32x4_u*>(o);
             *reinterpret_cast<f32x4_u*>(o) = v;
         } else {
             const float a[4] = {acc[r].x, acc[r].y, acc[r].z, acc[r].w};
+#pragma unroll
             for (int e = 0; e < 4; ++e)
-                if (col + e < g.n) o[e] = accumulate ? o[e] + a[e] : a[e];
+                if (col0 + e * CSTEP < g.n) o[e * CSTEP] = accumulate ? o[e * CSTEP] + a[e] : a[e];
         }
     }
 }

@@ -278,6 +278,13 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
 //   cols kernel : unit stride along the outputs    -> one lane per four outputs, k split over blocks
 // ------------------------------------------------------------------------------------------------
 
+// every row of every batch of the streamed matrix starts on a 16-byte boundary
+bool cols_aligned(const ColsArgs& c) {
+    if ((uintptr_t)c.Mx % 16 != 0 || c.m_rs % 4 != 0) return false;
+    for (int d = 0; d < c.batch.rank; ++d) if (c.batch.b_str[d] % 4 != 0) return false;
+    return true;
+}
+
 // out[b][i] = sum_j Mat[b](i, j) * vec[b](j), i < n_out, j < n_red;  Mat(i,j) = Mx[i*out_s + j*red_s]
 int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* vec, int64_t v_s, float* out,
                     int64_t n_out, int64_t n_red, const BatchDesc& bd_mat_vec, int64_t batch_count, int accumulate) {
@@ -327,10 +334,10 @@ int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* 
         const int64_t col_blocks = (n_out + COLS_THREADS * 4 - 1) / (COLS_THREADS * 4);
         int64_t splits = 1;
         const int64_t want = (int64_t)S.cus * S.cols_waves_per_cu;
-        if (col_blocks * batch_count < want) splits = std::min<int64_t>((want + col_blocks * batch_count - 1) / (col_blocks * batch_count), (n_red + COLS_KCHUNK - 1) / COLS_KCHUNK);
+        if (col_blocks * batch_count < want) splits = std::min<int64_t>((want + col_blocks * batch_count - 1) / (col_blocks * batch_count), (n_red + COLS_KSLICE_MIN - 1) / COLS_KSLICE_MIN);
         splits = std::max<int64_t>(1, std::min<int64_t>(splits, 65535));
         int64_t per = (n_red + splits - 1) / splits;
-        per = (per + COLS_KCHUNK - 1) / COLS_KCHUNK * COLS_KCHUNK;
+        per = (per + COLS_KSLICE_MIN - 1) / COLS_KSLICE_MIN * COLS_KSLICE_MIN;
         splits = (n_red + per - 1) / per;
         c.k_splits = (int32_t)splits; c.k_per_split = per;
         float* target = out;
@@ -340,7 +347,8 @@ int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* 
             target = ws;
         }
         c.out = target;
-        hipLaunchKernelGGL((cols_kernel<1>), dim3((unsigned)col_blocks, (unsigned)splits, (unsigned)batch_count), dim3(COLS_THREADS), 0, S.stream, c);
+        if (cols_aligned(c)) hipLaunchKernelGGL((cols_kernel<1, true>), dim3((unsigned)col_blocks, (unsigned)splits, (unsigned)batch_count), dim3(COLS_THREADS), 0, S.stream, c);
+        else hipLaunchKernelGGL((cols_kernel<1, false>), dim3((unsigned)col_blocks, (unsigned)splits, (unsigned)batch_count), dim3(COLS_THREADS), 0, S.stream, c);
         if (splits > 1) {
             const int64_t n = batch_count * n_out;
             hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
@@ -357,7 +365,10 @@ int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* 
 
 // skinny GEMM: M <= 8 rows against a row-major B — the matrix is streamed once, like vm
 template <int R>
-void launch_cols(const ColsArgs& c, dim3 grid) { hipLaunchKernelGGL((cols_kernel<R>), grid, dim3(COLS_THREADS), 0, S.stream, c); }
+void launch_cols(const ColsArgs& c, dim3 grid) {
+    if (cols_aligned(c)) hipLaunchKernelGGL((cols_kernel<R, true>), grid, dim3(COLS_THREADS), 0, S.stream, c);
+    else hipLaunchKernelGGL((cols_kernel<R, false>), grid, dim3(COLS_THREADS), 0, S.stream, c);
+}
 
 int skinny_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, int64_t b_rs, float* C,
                     int64_t M, int64_t N, int64_t K, const BatchDesc& bd, int64_t batch_count, int accumulate) {
@@ -367,10 +378,10 @@ int skinny_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, 
     const int64_t col_blocks = (N + COLS_THREADS * 4 - 1) / (COLS_THREADS * 4);
     int64_t splits = 1;
     const int64_t want = (int64_t)S.cus * S.cols_waves_per_cu;
-    if (col_blocks * batch_count < want) splits = std::min<int64_t>((want + col_blocks * batch_count - 1) / (col_blocks * batch_count), (K + COLS_KCHUNK - 1) / COLS_KCHUNK);
+    if (col_blocks * batch_count < want) splits = std::min<int64_t>((want + col_blocks * batch_count - 1) / (col_blocks * batch_count), (K + COLS_KSLICE_MIN - 1) / COLS_KSLICE_MIN);
     splits = std::max<int64_t>(1, std::min<int64_t>(splits, 65535));
     int64_t per = (K + splits - 1) / splits;
-    per = (per + COLS_KCHUNK - 1) / COLS_KCHUNK * COLS_KCHUNK;
+    per = (per + COLS_KSLICE_MIN - 1) / COLS_KSLICE_MIN * COLS_KSLICE_MIN;
     splits = (K + per - 1) / per;
     c.k_splits = (int32_t)splits; c.k_per_split = per;
     float* target = C;
@@ -539,6 +550,26 @@ int reduce_to_parent(const float* full, const Geometry& g, const tenmo_view* par
     if (total == 0) return 0;
     hipLaunchKernelGGL(broadcast_reduce_add_kernel, dim3((unsigned)std::min<int64_t>((total + 255) / 256, 65535)), dim3(256), 0, S.stream, r);
     return 0;
+}
+
+// every batch dim of the parent has extent 1 (or the parent has none)
+bool all_broadcast(const tenmo_view* parent, int trailing) {
+    for (int d = 0; d < parent->rank - trailing; ++d) if (parent->shape[d] != 1) return false;
+    return true;
+}
+
+// the batch dims of A stack its [M, K] matrices at a constant row pitch, i.e. A is one
+// [batch*M, K] matrix with row stride A.strides[-2]
+bool rows_fold(const tenmo_view* A, const Geometry& g) {
+    const int own = A->rank - 2;
+    if (own != g.batch_rank) return false;
+    int64_t expect = A->shape[A->rank - 2] * A->strides[A->rank - 2];
+    for (int d = own - 1; d >= 0; --d) {
+        if (A->shape[d] != g.oshape[d]) return false;
+        if (A->shape[d] > 1 && A->strides[d] != expect) return false;
+        expect *= A->shape[d];
+    }
+    return true;
 }
 
 bool same_batch(const Geometry& g, const tenmo_view* parent, int trailing) {
@@ -774,7 +805,17 @@ int tenmo_hip_matmul_backward(const tenmo_view* A, const tenmo_view* B, const fl
     }
     if (grad_B) { // dB = A^T(view) . dC   (tenmo/matmul.mojo:46-48, :127-132)
         const tenmo_view At = transposed_last2(A);
-        if (same_batch(g, B, 2)) {
+        if (!same_batch(g, B, 2) && all_broadcast(B, 2) && rows_fold(A, g)) {
+            // B is shared by every batch (a Linear weight under a batched input): the sum over batches
+            // of A_b^T . dC_b is ONE product with the batch folded into the reduction,
+            // [K, batch*M] . [batch*M, N], accumulated straight into the gradbox — no batched
+            // gradient is materialised and no reduction pass runs.
+            const int64_t M = A->shape[A->rank - 2], K = A->shape[A->rank - 1], N = B->shape[B->rank - 1];
+            BatchDesc none{};
+            for (int d = 0; d < MAX_BATCH_RANK; ++d) none.shape[d] = 1;
+            if (int rc = gemm_dispatch(A->data + A->offset, A->strides[A->rank - 1], A->strides[A->rank - 2], dC, N, 1, grad_B,
+                                       K, N, g.batch_count * M, none, 1, 1)) return rc;
+        } else if (same_batch(g, B, 2)) {
             if (int rc = matmul_views(&At, &dCv, grad_B, 1, "tenmo_hip_matmul_backward")) return rc;
         } else {
             Geometry gg;
