@@ -235,11 +235,18 @@ def mlp_step_times(_lib, torch, np):
         gpu.step_device(xd, yd, lr, sync=False)
     _lib.check(L.tenmo_hip_sync())
     gpu_ms = (time.perf_counter() - t0) * 1e3 / 20
+    # the same 20 steps replayed from the captured graph (parameters keep training; timing only)
+    gpu.step_device(*dev[0], lr, sync=True, graph=True)
+    t0 = time.perf_counter()
+    for xd, yd in dev[10:]:
+        gpu.step_device(xd, yd, lr, sync=False, graph=True)
+    _lib.check(L.tenmo_hip_sync())
+    graph_ms = (time.perf_counter() - t0) * 1e3 / 20
     t0 = time.perf_counter()
     for x, y in batches[10:]:
         cpu.step(x, y, lr)
     cpu_ms = (time.perf_counter() - t0) * 1e3 / 20
-    return {"mlp_step_ms_gpu": round(gpu_ms, 4), "mlp_step_ms_cpu": round(cpu_ms, 4), "mlp_cpu_cores": O.num_physical_cores(),
+    return {"mlp_step_ms_gpu": round(gpu_ms, 4), "mlp_step_ms_gpu_graph": round(graph_ms, 4), "mlp_step_ms_cpu": round(cpu_ms, 4), "mlp_cpu_cores": O.num_physical_cores(),
             "mlp_max_abs_loss_diff_first10": worst}
 
 

@@ -181,6 +181,13 @@ void tenmo_hip_mlp_destroy(tenmo_mlp*);
  * written to loss_out[0] (device).  No host synchronisation unless sync != 0. */
 int tenmo_hip_mlp_step(tenmo_mlp*, const float* x, const int32_t* y, int64_t batch, float lr,
                        float* loss_out, int32_t sync);
+/* Same step, replayed from a HIP graph captured on first use (and re-captured when batch, lr or
+ * loss_out change): one graph launch instead of ~25 kernel launches.  The reference explains its GPU
+ * MNIST time by exactly this launch overhead ("13 kernels per step ... launch latency exceeds
+ * compute", docs/from-bytes-to-gradients.md:454).  Inputs are copied into fixed staging buffers
+ * first, so x and y may differ from call to call.  Needs the library's own stream. */
+int tenmo_hip_mlp_step_graph(tenmo_mlp*, const float* x, const int32_t* y, int64_t batch, float lr,
+                             float* loss_out, int32_t sync);
 int tenmo_hip_mlp_forward(tenmo_mlp*, const float* x, int64_t batch, float* logits_out, int32_t sync);
 /* copy a layer's parameters / last gradients to HOST arrays (synchronises) */
 int tenmo_hip_mlp_get_params(tenmo_mlp*, int32_t layer, float* W_host, float* b_host);

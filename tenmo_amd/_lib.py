@@ -76,6 +76,7 @@ SIGNATURES = {
     "tenmo_hip_mlp_create": (C.c_void_p, [C.c_int32, _i64p, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int64]),
     "tenmo_hip_mlp_destroy": (None, [C.c_void_p]),
     "tenmo_hip_mlp_step": (C.c_int, [C.c_void_p, _ptr, _ptr, C.c_int64, C.c_float, _ptr, C.c_int32]),
+    "tenmo_hip_mlp_step_graph": (C.c_int, [C.c_void_p, _ptr, _ptr, C.c_int64, C.c_float, _ptr, C.c_int32]),
     "tenmo_hip_mlp_forward": (C.c_int, [C.c_void_p, _ptr, C.c_int64, _ptr, C.c_int32]),
     "tenmo_hip_mlp_get_params": (C.c_int, [C.c_void_p, C.c_int32, _ptr, _ptr]),
     "tenmo_hip_mlp_get_grads": (C.c_int, [C.c_void_p, C.c_int32, _ptr, _ptr]),

@@ -1005,6 +1005,13 @@ struct tenmo_mlp {
     int64_t max_batch = 0;
     std::vector<float*> W, b, dW, db, act, grad; // act[l]: output of layer l ([B, dims[l+1]]); grad[l]: its gradient
     float* row_loss = nullptr;
+    // captured training step (tenmo_hip_mlp_step_graph): fixed input staging + the executable graph
+    float* x_stage = nullptr;
+    int32_t* y_stage = nullptr;
+    hipGraphExec_t exec = nullptr;
+    int64_t g_batch = -1;
+    float g_lr = 0.f;
+    float* g_loss = nullptr;
 };
 
 static unsigned grid_for(int64_t n) { return (unsigned)std::max<int64_t>(1, std::min<int64_t>((n + 255) / 256, 4096)); }
@@ -1026,6 +1033,8 @@ tenmo_mlp* tenmo_hip_mlp_create(int32_t L, const int64_t* dims, const float* con
         ok = ok && hipMemcpy(m->b[l], bh[l], bn * 4, hipMemcpyHostToDevice) == hipSuccess;
     }
     ok = ok && hipMalloc(&m->row_loss, (size_t)max_batch * 4) == hipSuccess;
+    ok = ok && hipMalloc(&m->x_stage, (size_t)max_batch * dims[0] * 4) == hipSuccess;
+    ok = ok && hipMalloc(&m->y_stage, (size_t)max_batch * 4) == hipSuccess;
     if (!ok) { fail(TENMO_ERR_HIP, "tenmo_hip_mlp_create: device allocation or upload failed"); tenmo_hip_mlp_destroy(m); return nullptr; }
     return m;
 }
@@ -1036,6 +1045,9 @@ void tenmo_hip_mlp_destroy(tenmo_mlp* m) {
     for (auto* v : {&m->W, &m->b, &m->dW, &m->db, &m->act, &m->grad})
         for (float* p : *v) if (p) hipFree(p);
     if (m->row_loss) hipFree(m->row_loss);
+    if (m->x_stage) hipFree(m->x_stage);
+    if (m->y_stage) hipFree(m->y_stage);
+    if (m->exec) hipGraphExecDestroy(m->exec);
     delete m;
 }
 
@@ -1060,9 +1072,8 @@ int tenmo_hip_mlp_forward(tenmo_mlp* m, const float* x, int64_t B, float* logits
     return finish(sync);
 }
 
-int tenmo_hip_mlp_step(tenmo_mlp* m, const float* x, const int32_t* y, int64_t B, float lr, float* loss_out, int32_t sync) {
-    if (int rc = ensure_ready()) return rc;
-    if (!m || B < 1 || B > m->max_batch) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_mlp_step: batch outside 1..max_batch");
+// enqueues every kernel of one training step on the library stream
+static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int64_t B, float lr, float* loss_out) {
     if (int rc = mlp_forward(m, x, B)) return rc;
     const int L = m->L;
     const int64_t C = m->dims[L];
@@ -1087,6 +1098,39 @@ int tenmo_hip_mlp_step(tenmo_mlp* m, const float* x, const int32_t* y, int64_t B
         hipLaunchKernelGGL(sgd_kernel, dim3(grid_for(wn)), dim3(256), 0, S.stream, m->W[l], m->dW[l], wn, lr);
         hipLaunchKernelGGL(sgd_kernel, dim3(grid_for(bn)), dim3(256), 0, S.stream, m->b[l], m->db[l], bn, lr);
     }
+    return 0;
+}
+
+int tenmo_hip_mlp_step(tenmo_mlp* m, const float* x, const int32_t* y, int64_t B, float lr, float* loss_out, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    if (!m || B < 1 || B > m->max_batch) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_mlp_step: batch outside 1..max_batch");
+    if (int rc = mlp_step_enqueue(m, x, y, B, lr, loss_out)) return rc;
+    return finish(sync);
+}
+
+int tenmo_hip_mlp_step_graph(tenmo_mlp* m, const float* x, const int32_t* y, int64_t B, float lr, float* loss_out, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    if (!m || B < 1 || B > m->max_batch) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_mlp_step_graph: batch outside 1..max_batch");
+    if (S.stream == nullptr) return fail(TENMO_ERR_UNSUPPORTED, "tenmo_hip_mlp_step_graph: cannot capture on the null stream");
+    // the captured kernels read fixed staging buffers; this step's inputs are copied in eagerly
+    HIP_TRY(hipMemcpyAsync(m->x_stage, x, (size_t)B * m->dims[0] * 4, hipMemcpyDeviceToDevice, S.stream));
+    HIP_TRY(hipMemcpyAsync(m->y_stage, y, (size_t)B * 4, hipMemcpyDeviceToDevice, S.stream));
+    if (!m->exec || m->g_batch != B || m->g_lr != lr || m->g_loss != loss_out) {
+        if (m->exec) { HIP_TRY(hipStreamSynchronize(S.stream)); HIP_TRY(hipGraphExecDestroy(m->exec)); m->exec = nullptr; }
+        float* ws;
+        if (int rc = workspace(1, &ws)) return rc; // scratch must exist before capture: no allocation may happen inside it
+        HIP_TRY(hipStreamBeginCapture(S.stream, hipStreamCaptureModeThreadLocal));
+        const int rc = mlp_step_enqueue(m, m->x_stage, m->y_stage, B, lr, loss_out);
+        hipGraph_t graph = nullptr;
+        const hipError_t e = hipStreamEndCapture(S.stream, &graph);
+        if (rc) { if (graph) hipGraphDestroy(graph); return rc; }
+        if (e != hipSuccess) return fail(TENMO_ERR_HIP, "hipStreamEndCapture failed: %s", hipGetErrorString(e));
+        const hipError_t ei = hipGraphInstantiate(&m->exec, graph, nullptr, nullptr, 0);
+        hipGraphDestroy(graph);
+        if (ei != hipSuccess) { m->exec = nullptr; return fail(TENMO_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(ei)); }
+        m->g_batch = B; m->g_lr = lr; m->g_loss = loss_out;
+    }
+    HIP_TRY(hipGraphLaunch(m->exec, S.stream));
     return finish(sync);
 }
 

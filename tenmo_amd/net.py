@@ -135,15 +135,18 @@ class MLP:
                 pass
             self._h = None
 
-    def step_device(self, x: torch.Tensor, y: torch.Tensor, lr: float, sync: bool = False) -> torch.Tensor:
-        """x: fp32 [batch, dims[0]] on the device, y: int32 [batch] on the device. Returns the device scalar loss."""
-        check(_lib.load().tenmo_hip_mlp_step(self._h, x.data_ptr(), y.data_ptr(), x.shape[0], float(lr), self._loss.data_ptr(), 1 if sync else 0))
+    def step_device(self, x: torch.Tensor, y: torch.Tensor, lr: float, sync: bool = False, graph: bool = False) -> torch.Tensor:
+        """x: fp32 [batch, dims[0]] on the device, y: int32 [batch] on the device. Returns the device scalar loss.
+        graph=True replays the step from a captured HIP graph (tenmo_hip_mlp_step_graph)."""
+        L = _lib.load()
+        fn = L.tenmo_hip_mlp_step_graph if graph else L.tenmo_hip_mlp_step
+        check(fn(self._h, x.data_ptr(), y.data_ptr(), x.shape[0], float(lr), self._loss.data_ptr(), 1 if sync else 0))
         return self._loss
 
-    def step(self, x: np.ndarray, y: np.ndarray, lr: float) -> float:
+    def step(self, x: np.ndarray, y: np.ndarray, lr: float, graph: bool = False) -> float:
         xd = torch.from_numpy(np.ascontiguousarray(x, np.float32)).cuda()
         yd = torch.from_numpy(np.ascontiguousarray(y, np.int32)).cuda()
-        self.step_device(xd, yd, lr, sync=True)
+        self.step_device(xd, yd, lr, sync=True, graph=graph)
         return float(self._loss.item())
 
     def forward(self, x: np.ndarray) -> np.ndarray:

@@ -415,3 +415,33 @@ def test_mlp_loss_curve_tracks_cpu(T, oracle):
     # cross-entropy vector of the reference: uniform logits -> -log(1/3)
     m = MLP([2, 3], [np.zeros((2, 3), np.float32)], [np.ones(3, np.float32)], 2)
     assert abs(m.step(np.ones((2, 2), np.float32), np.asarray([0, 1], np.int32), 0.0) - 1.0986122886681098) < 1e-6
+
+
+def test_mlp_graph_replay_matches_eager(T, oracle):
+    """The captured step replayed many times, with eager library work and synchronisations between
+    replays, gives the same losses and parameters as the eager step (and so as the CPU run)."""
+    from tenmo_amd import rng as R
+    from tenmo_amd.net import MLP
+
+    dims, seed, lr = [784, 128, 32, 10], 77, 0.01
+    Ws, bs = R.xavier_mlp(dims, seed)
+    eager, graph, cpu = MLP(dims, Ws, bs, 64), MLP(dims, Ws, bs, 64), oracle.MLP(dims, Ws, bs, 64)
+    side_a = T.Tensor.from_numpy(np.ones((70, 33), np.float32))
+    side_b = T.Tensor.from_numpy(np.ones((33, 20), np.float32))
+    for step in range(12):
+        x, y = R.mnist_like_batch(64, seed, step)
+        le = eager.step(x, y, lr)
+        lg = graph.step(x, y, lr, graph=True)
+        lc = cpu.step(x, y, lr)
+        assert le == lg, (step, le, lg)          # same kernels, same order: bit-identical
+        assert abs(lg - lc) <= 1e-4
+        # unrelated eager work on the same stream between replays
+        assert np.all(side_a.matmul(side_b, track_grad=False).to_numpy() == 33.0)
+    for l in range(3):
+        (We, be), (Wg, bg) = eager.params(l), graph.params(l)
+        np.testing.assert_array_equal(We, Wg)
+        np.testing.assert_array_equal(be, bg)
+    # a different learning rate re-captures
+    x, y = R.mnist_like_batch(64, seed, 99)
+    assert eager.step(x, y, 0.05) == graph.step(x, y, 0.05, graph=True)
+    np.testing.assert_array_equal(eager.params(0)[0], graph.params(0)[0])
