@@ -84,7 +84,7 @@ def test_closed_forms(T, golden):
 
 # ---- 2-D GEMM against oracle and fp64 --------------------------------------------------------------
 
-@pytest.mark.parametrize("tile", [-1, 0, 1, 2])
+@pytest.mark.parametrize("tile", [-1, 0, 1, 2, 3, 4])
 def test_verify_shapes(T, golden, oracle, tile):
     """Shape list of tests/test_matmul_2d_verify.mojo, each with A / B as row-major, transposed view
     and padded view, on every workgroup-tile configuration."""
@@ -107,6 +107,54 @@ def test_verify_shapes(T, golden, oracle, tile):
                     assert rel_fro(got, oracle.mm2d(av, bv)) <= 2 * RTOL_FRO
     finally:
         L.tenmo_hip_set_tuning(b"gemm_tile", -1)
+
+
+@pytest.mark.parametrize("tile", [-1, 0, 1, 3, 4])
+def test_ragged_tiles_and_k_slices(T, oracle, tile):
+    """Extents that leave partial tiles in M, N and K at once, in every operand layout: exercises the
+    direct-to-LDS path with clamped rows (extent divisible by 4 or not), the checked tail, and
+    explicit K slicing with its reduction."""
+    L = T.lib.load()
+    rng = np.random.default_rng(19)
+    try:
+        L.tenmo_hip_set_tuning(b"gemm_tile", tile)
+        for (m, k, n) in [(100, 256, 500), (260, 100, 132), (257, 48, 129), (300, 1000, 68), (1, 64, 4), (4, 4096, 8), (131, 37, 259)]:
+            a = rng.standard_normal((m, k), dtype=np.float32)
+            b = rng.standard_normal((k, n), dtype=np.float32)
+            ref = ref_matmul64(a, b)
+            for av in (a, np.ascontiguousarray(a.T).T):
+                for bv in (b, np.ascontiguousarray(b.T).T):
+                    for sk in (-1, 3):
+                        L.tenmo_hip_set_tuning(b"gemm_splitk", sk)
+                        got = as_strided_tensor(T, av).matmul(as_strided_tensor(T, bv), track_grad=False).to_numpy()
+                        assert rel_fro(got, ref) <= RTOL_FRO, (tile, m, k, n, av.strides, bv.strides, sk)
+    finally:
+        L.tenmo_hip_set_tuning(b"gemm_tile", -1)
+        L.tenmo_hip_set_tuning(b"gemm_splitk", -1)
+
+
+def test_raw_abi_arguments(T):
+    """Argument checking of the kernel-level entry points (status codes + messages, nothing launched)."""
+    L, lib = T.lib.load(), T.lib
+    x = T.Tensor.zeros(4, 4)
+    p = x.buffer.data_ptr()
+    assert L.tenmo_hip_gemm_f32(p, 0, 4, 1, p, 0, 4, 1, p, -1, 4, 4, 0, None, None, None, 0, 0) == -2
+    assert b"negative" in L.tenmo_hip_last_error()
+    assert L.tenmo_hip_gemm_f32(None, 0, 4, 1, p, 0, 4, 1, p, 4, 4, 4, 0, None, None, None, 0, 0) == -3
+    assert L.tenmo_hip_gemm_f32(p, 0, 4, 1, p, 0, 4, 1, p, 4, 4, 4, 7, None, None, None, 0, 0) == -3   # batch rank > 6
+    assert L.tenmo_hip_gemm_f32(p, 0, 4, 1, p, 0, 4, 1, p, 4, 4, 4, 1, None, None, None, 0, 0) == -3   # rank 1 without arrays
+    assert L.tenmo_hip_set_tuning(b"no_such_knob", 1) == -3
+    assert L.tenmo_hip_mv_f32(p, 0, 4, 1, p, 0, 1, p, -2, 4, 0, None, None, None, 0, 0) == -2
+    # a zero-sized problem is a no-op that succeeds
+    assert L.tenmo_hip_gemm_f32(p, 0, 4, 1, p, 0, 4, 1, p, 0, 4, 4, 0, None, None, None, 0, 1) == 0
+    # explicit batch arrays: C[b] = A[b] . B (B broadcast with stride 0), accumulate twice doubles
+    a = np.arange(2 * 3 * 4, dtype=np.float32).reshape(2, 3, 4)
+    b = np.arange(4 * 5, dtype=np.float32).reshape(4, 5)
+    A, B, out = T.Tensor.from_numpy(a), T.Tensor.from_numpy(b), T.Tensor.zeros(2, 3, 5)
+    for _ in range(2):
+        lib.check(L.tenmo_hip_gemm_f32(A.buffer.data_ptr(), 0, 4, 1, B.buffer.data_ptr(), 0, 5, 1, out.buffer.data_ptr(), 3, 5, 4,
+                                       1, lib.i64([2]), lib.i64([12]), lib.i64([0]), 1, 1))
+    np.testing.assert_array_equal(out.to_numpy(), 2 * np.matmul(a, b))
 
 
 def test_odd_strides_and_overlap(T, oracle):
