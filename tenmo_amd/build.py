@@ -1,7 +1,6 @@
 """Builds ``libtenmo_hip.so`` (hipcc, gfx950 only) next to this file.
 
     python -m tenmo_amd.build            # compile
-    python -m tenmo_amd.build --asm      # also keep the gfx950 assembly under _work/ for inspection
 
 The library is built in-tree so that the copy of the tree that runs on the GPU machine carries it.
 """
@@ -31,12 +30,8 @@ FLAGS = [
 ]
 
 
-def build(verbose: bool = False, keep_asm: bool = False) -> str:
+def build(verbose: bool = False) -> str:
     cmd = [HIPCC] + FLAGS + [SRC, "-o", LIB]
-    if keep_asm:
-        work = os.path.join(ROOT, "_work", "asm")
-        os.makedirs(work, exist_ok=True)
-        cmd += ["-save-temps=obj"]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, cwd=os.path.join(HERE, "csrc"), capture_output=True, text=True)
@@ -50,4 +45,4 @@ def build(verbose: bool = False, keep_asm: bool = False) -> str:
 
 
 if __name__ == "__main__":
-    print(build(verbose=True, keep_asm="--asm" in sys.argv))
+    print(build(verbose=True))
