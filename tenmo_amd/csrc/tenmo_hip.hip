@@ -202,12 +202,12 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
 
     // Pick the workgroup tile and the number of K slices with a small cost model of this chip
     // (constants fitted to measured launches on MI355X): per CU the matrix-pipe time is the sum over
-    // its workgroups, a lone wavefront per SIMD cannot hide its own barrier/LDS latency, every
-    // workgroup pays a fixed prologue/epilogue, and the launch can never beat its HBM and L2 traffic.
+    // its workgroups (the K loop runs at full rate from one wavefront per SIMD up), every workgroup
+    // pays a fixed prologue/epilogue, and the launch can never beat its HBM and L2 traffic.
     int tile = 0, splits = 1;
     {
         static const double kOcc[kNumTiles] = {2, 3, 6, 4, 4};             // resident workgroups per CU (LDS / VGPR limits)
-        static const double kEff[kNumTiles] = {0.93, 0.92, 0.86, 0.90, 0.90}; // matrix-pipe efficiency at full occupancy
+        static const double kEff[kNumTiles] = {0.96, 0.95, 0.94, 0.92, 0.92}; // matrix-pipe efficiency of the K loop
         static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
         const double cus = (double)S.cus;
         double best = 1e300;
@@ -223,11 +223,11 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
                 const double rounds = wgs <= slots ? 1.0 : std::ceil(wgs / slots);
                 const double conc = wgs <= slots ? std::ceil(wgs / cus) : kOcc[t];
                 const double iters = std::ceil((double)K / sp / GEMM_BK);
-                const double t_round = iters * std::max(conc * m_us, 0.23 + m_us) / kEff[t] + 2.5;
+                const double t_round = iters * conc * m_us / kEff[t] + 1.5;
                 const double bytes = 4.0 * batch_count * ((double)M * K + (double)K * N + (double)M * N * (sp > 1 ? sp + 1.0 : 1.0));
                 const double l2_bytes = 4.0 * batch_count * (double)K * ((double)M * tn + (double)N * tm);
                 double est = std::max({rounds * t_round, bytes / 5.0e6, l2_bytes / 14.0e6}) + 3.0;
-                if (sp > 1) est += 5.0 + 4.0 * batch_count * (double)M * N * (sp + 1.0) / 4.0e6;
+                if (sp > 1) est += 5.0 + 4.0 * batch_count * (double)M * N * (sp + 1.0) / 6.0e6;
                 if (est < best) { best = est; tile = t; splits = sp; }
             }
         }
