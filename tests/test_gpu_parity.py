@@ -157,6 +157,36 @@ def test_raw_abi_arguments(T):
     np.testing.assert_array_equal(out.to_numpy(), 2 * np.matmul(a, b))
 
 
+def test_direct_path_pitch_limits(T):
+    """Row pitches the direct global->LDS path cannot address with 32-bit lane offsets (huge, negative)
+    fall back to the checked loader and still give the right product; aligned 16-byte rows with a
+    large but admissible pitch stay on the direct path."""
+    rng = np.random.default_rng(29)
+    m, k, n = 6, 64, 40
+    b = rng.standard_normal((k, n), dtype=np.float32)
+    B = T.Tensor.from_numpy(b)
+    for pitch in (3_000_000, 1_000_000):     # above / below the direct path's limit of 2^21 elements
+        store = np.zeros(m * pitch, np.float32)
+        a = rng.standard_normal((m, k), dtype=np.float32)
+        for i in range(m):
+            store[i * pitch:i * pitch + k] = a[i]
+        dev = T.Tensor.from_numpy(store)
+        got = dev.view((m, k), (pitch, 1), 0).matmul(B, track_grad=False).to_numpy()
+        assert rel_fro(got, ref_matmul64(a, b)) <= RTOL_FRO, pitch
+        # the same rows as the K-major right operand: B2 = a^T through a transposed view
+        x = rng.standard_normal((5, m), dtype=np.float32)
+        got = T.Tensor.from_numpy(x).matmul(dev.view((m, k), (pitch, 1), 0), track_grad=False).to_numpy()
+        assert rel_fro(got, ref_matmul64(x, a)) <= RTOL_FRO, pitch
+        del dev
+    # rows walked backwards (negative row stride) and columns walked backwards (negative k stride)
+    a = rng.standard_normal((70, 64), dtype=np.float32)
+    dev = T.Tensor.from_numpy(a.ravel())
+    flipped_rows = dev.view((70, 64), (-64, 1), 69 * 64)
+    assert rel_fro(flipped_rows.matmul(B, track_grad=False).to_numpy(), ref_matmul64(a[::-1], b)) <= RTOL_FRO
+    flipped_cols = dev.view((70, 64), (64, -1), 63)
+    assert rel_fro(flipped_cols.matmul(B, track_grad=False).to_numpy(), ref_matmul64(a[:, ::-1], b)) <= RTOL_FRO
+
+
 def test_odd_strides_and_overlap(T, oracle):
     """Column stride 2, row stride 0 (broadcast rows), overlapping windows (tests/test_mmnd.mojo:143-175)."""
     rng = np.random.default_rng(23)
