@@ -65,7 +65,8 @@ int tenmo_hip_set_stream(void* hip_stream);
 /* Device facts the caller may want for reporting: number of compute units, name. */
 int tenmo_hip_device_info(int* compute_units, char* name, int name_len);
 /* Overrides of the automatic kernel selection, for measurement: "gemm_tile" (0: 256x128, 1: 128x128,
- * 2: 64x64 workgroup tile; -1 automatic) and "gemm_splitk" (number of K slices; -1 automatic).  The
+ * 2: 64x64, 3: 128x64, 4: 64x128 workgroup tile; -1 automatic), "gemm_splitk" (number of K slices;
+ * -1 automatic) and "cols_wg_per_cu" (workgroups per CU the column-streaming kernel aims for).  The
  * environment variables TENMO_HIP_GEMM_TILE / TENMO_HIP_GEMM_SPLITK set the same at init.
  * No counterpart in the reference, whose tile size is the compile-time TILE_SIZE=32
  * (tenmo/ndbuffer.mojo:63). */
@@ -92,6 +93,19 @@ int tenmo_hip_gemm_f32(const float* A, int64_t a_off, int64_t a_rs, int64_t a_cs
                        int32_t batch_rank, const int64_t* batch_shape,
                        const int64_t* a_batch_strides, const int64_t* b_batch_strides,
                        int32_t accumulate, int32_t sync);
+
+/* The same product with the element-wise stages that follow it in a Linear layer done in the
+ * GEMM store: C = A.B, then + bias[col] (N floats, or NULL), then max(., 0) if relu, then zeroed
+ * where mask <= 0 (mask: dense like C, or NULL; with mask = the forward activation of the layer
+ * below, dX = dY.W^T comes out already multiplied by the ReLU gradient).
+ * Replaces: Matmul.forward followed by Adder.forward in Linear.forward (tenmo/net.mojo:193-201),
+ * ReLU.forward and ReLUBackward (tenmo/relu.mojo:99-141, mask = x > 0 at :120-123). */
+int tenmo_hip_gemm_epilogue_f32(const float* A, int64_t a_off, int64_t a_rs, int64_t a_cs,
+                                const float* B, int64_t b_off, int64_t b_rs, int64_t b_cs,
+                                float* C, int64_t M, int64_t N, int64_t K,
+                                int32_t batch_rank, const int64_t* batch_shape,
+                                const int64_t* a_batch_strides, const int64_t* b_batch_strides,
+                                const float* bias, int32_t relu, const float* mask, int32_t sync);
 
 /* out[batch..., m] = Mx[.., m, k] . v[.., k]
  * Replaces: matrix_vector_nd + MatrixVectorNdGpu.launch, tenmo/kernels/matrixvector_kernel.mojo:13-171
@@ -133,6 +147,11 @@ int64_t tenmo_hip_result_shape(int32_t op, const tenmo_view* A, const tenmo_view
 /* MatmulNdGpu.launch(A, B, sync) — tenmo/kernels/matmul_kernel.mojo:128-283 — with the result
  * buffer supplied by the caller (dense, tenmo_hip_result_shape elements). */
 int tenmo_hip_matmul_nd(const tenmo_view* A, const tenmo_view* B, float* C, int32_t sync);
+/* Linear.forward on views: out = X.W + bias (bias: W.shape[-1] floats or NULL), then ReLU if
+ * relu != 0, in one launch — tenmo/net.mojo:179-216 (+ tenmo/relu.mojo:99-141).  Shapes and
+ * broadcasting as tenmo_hip_matmul_nd. */
+int tenmo_hip_linear_nd(const tenmo_view* X, const tenmo_view* W, const float* bias, int32_t relu,
+                        float* out, int32_t sync);
 /* MatrixVectorNdGpu.launch — tenmo/kernels/matrixvector_kernel.mojo:80-171 */
 int tenmo_hip_matrix_vector_nd(const tenmo_view* Mx, const tenmo_view* v, float* out, int32_t sync);
 /* VectorMatmulNdGpu.launch — tenmo/kernels/vectormatrix_kernel.mojo:80-170 */
@@ -170,7 +189,8 @@ void cblas_sgemm(int order, int trans_a, int trans_b, int M, int N, int K, float
 /* Linear(x.W + b) -> ReLU -> ... -> Linear -> CrossEntropy(mean) -> backward -> SGD(lr), the step
  * of examples/mnist.mojo:150-162 over tenmo/net.mojo:179-216, relu.mojo:99-141,
  * crossentropy.mojo:285-432,:775-793, optim.mojo:93-120.  All GEMMs go through
- * tenmo_hip_gemm_f32; the element-wise stages are small fused kernels on the same stream.
+ * the GEMM kernel with bias, ReLU and the ReLU gradient applied in its store; the remaining
+ * element-wise stages are small kernels on the same stream.
  * dims[0..n_layers] are the layer widths; W[l] is [dims[l], dims[l+1]] row-major (the reference
  * stores weights [in, out], net.mojo:91-97), b[l] is [dims[l+1]]; both HOST arrays, copied in. */
 typedef struct tenmo_mlp tenmo_mlp;

@@ -58,6 +58,9 @@ SIGNATURES = {
     "tenmo_hip_gemm_f32": (C.c_int, [_ptr, C.c_int64, C.c_int64, C.c_int64, _ptr, C.c_int64, C.c_int64, C.c_int64,
                                      _ptr, C.c_int64, C.c_int64, C.c_int64, C.c_int32, _i64p, _i64p, _i64p,
                                      C.c_int32, C.c_int32]),
+    "tenmo_hip_gemm_epilogue_f32": (C.c_int, [_ptr, C.c_int64, C.c_int64, C.c_int64, _ptr, C.c_int64, C.c_int64, C.c_int64,
+                                              _ptr, C.c_int64, C.c_int64, C.c_int64, C.c_int32, _i64p, _i64p, _i64p,
+                                              _ptr, C.c_int32, _ptr, C.c_int32]),
     "tenmo_hip_mv_f32": (C.c_int, [_ptr, C.c_int64, C.c_int64, C.c_int64, _ptr, C.c_int64, C.c_int64, _ptr,
                                    C.c_int64, C.c_int64, C.c_int32, _i64p, _i64p, _i64p, C.c_int32, C.c_int32]),
     "tenmo_hip_vm_f32": (C.c_int, [_ptr, C.c_int64, C.c_int64, _ptr, C.c_int64, C.c_int64, C.c_int64, _ptr,
@@ -66,6 +69,7 @@ SIGNATURES = {
     "tenmo_hip_classify_matmul": (C.c_int, [C.c_int32, _i64p, C.c_int32, _i64p]),
     "tenmo_hip_result_shape": (C.c_int64, [C.c_int32, _vp, _vp, _i64p, _i32p]),
     "tenmo_hip_matmul_nd": (C.c_int, [_vp, _vp, _ptr, C.c_int32]),
+    "tenmo_hip_linear_nd": (C.c_int, [_vp, _vp, _ptr, C.c_int32, _ptr, C.c_int32]),
     "tenmo_hip_matrix_vector_nd": (C.c_int, [_vp, _vp, _ptr, C.c_int32]),
     "tenmo_hip_vector_matmul_nd": (C.c_int, [_vp, _vp, _ptr, C.c_int32]),
     "tenmo_hip_matmul_backward": (C.c_int, [_vp, _vp, _ptr, _ptr, _ptr, C.c_int32]),

@@ -89,22 +89,6 @@ __global__ void fill_kernel(float* p, int64_t n, float value) {
 }
 
 // ---- MLP harness stages -----------------------------------------------------------------------
-// z[r][c] += b[c]; if relu: z = max(z, 0)   (tenmo/net.mojo:198-201, tenmo/relu.mojo:99-141)
-__global__ void bias_act_kernel(float* __restrict z, const float* __restrict b, int64_t rows, int64_t cols, int relu) {
-    const int64_t total = rows * cols;
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
-        float x = z[i] + b[i % cols];
-        z[i] = (relu && !(x > 0.f)) ? 0.f : x;
-    }
-}
-
-// g[i] = (h[i] > 0) ? g[i] : 0     ReLU backward with the mask recomputed from the activation
-// (mask = x > 0 in tenmo/relu.mojo:120-123; h > 0 exactly when x > 0)
-__global__ void relu_backward_kernel(float* __restrict g, const float* __restrict h, int64_t n) {
-    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x)
-        if (!(h[i] > 0.f)) g[i] = 0.f;
-}
-
 // Fused class-index cross-entropy, mean reduction (tenmo/crossentropy.mojo:285-432) and its
 // gradient (softmax - onehot) / valid_count (:775-793, :451-481).  One thread per row (C is tiny in
 // the harness); per-row losses go to row_loss for the ordered sum below.
@@ -142,8 +126,20 @@ __global__ void column_sum_kernel(const float* __restrict g, int64_t rows, int64
     db[c] = s;
 }
 
-// p -= lr * g   (tenmo/optim.mojo:93-120, no momentum, no weight decay)
-__global__ void sgd_kernel(float* __restrict p, const float* __restrict g, int64_t n, float lr) {
+// p -= lr * g   (tenmo/optim.mojo:93-120, no momentum, no weight decay) for up to SGD_MAX_TENSORS
+// parameter tensors in one launch (blockIdx.y = tensor)
+constexpr int SGD_MAX_TENSORS = 16;
+struct SgdArgs {
+    float* p[SGD_MAX_TENSORS];
+    const float* g[SGD_MAX_TENSORS];
+    int64_t n[SGD_MAX_TENSORS];
+    int32_t count;
+};
+__global__ void sgd_multi_kernel(const SgdArgs a, float lr) {
+    const int k = blockIdx.y;
+    float* __restrict p = a.p[k];
+    const float* __restrict g = a.g[k];
+    const int64_t n = a.n[k];
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = p[i] - lr * g[i];
 }
 

@@ -72,8 +72,20 @@ struct GemmArgs {
     int64_t batch_count;
     int64_t k_per_split;  // multiple of GEMM_BK
     float* partial;       // [k_splits][batch*M*N] when k_splits > 1
+    // fused epilogue, applied to the finished sums (by the slice reduction when k_splits > 1):
+    const float* bias;    // + bias[col], or null                         (Linear: x.W + b)
+    const float* mask;    // dense like C: result zeroed where mask <= 0, or null   (ReLU backward on dX)
+    int32_t relu;         // max(.,0) after the bias                      (ReLU forward)
     BatchDesc batch;
 };
+
+// bias, ReLU and ReLU-backward mask on one finished element (i = flat index into the dense C)
+__device__ __forceinline__ float epilogue_value(float v, const float* __restrict bias, const float* __restrict mask, int relu, int64_t i, int64_t col) {
+    if (bias) v += bias[col];
+    if (relu && !(v > 0.f)) v = 0.f;
+    if (mask && !(mask[i] > 0.f)) v = 0.f;
+    return v;
+}
 
 __device__ __forceinline__ void batch_offsets(const BatchDesc& bd, int64_t b, int64_t& a_off, int64_t& b_off) {
     a_off = 0; b_off = 0;
@@ -495,6 +507,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     } else {
         Cb = g.C + batch * g.M * g.N;
     }
+    const bool fused = g.k_splits == 1 && (g.bias != nullptr || g.mask != nullptr || g.relu != 0);
+    const float* __restrict mask = g.mask ? g.mask + batch * g.M * g.N : nullptr;
     const int h = lane >> 5, x = lane & 31;
 #pragma unroll
     for (int i = 0; i < MB; ++i) {
@@ -504,6 +518,14 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
             const int64_t row = m0 + wm * TM + tile_pos<AMODE, MB>(i, ip);
             if (row >= g.M) continue;
             float* crow = Cb + row * g.N;
+            if (fused) { // rare enough to stay scalar
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
+                    const int64_t col = n0 + wn * TN + tile_pos<BMODE, NB>(j, x);
+                    if (col < g.N) crow[col] = epilogue_value(acc[i][j][e], g.bias, mask, g.relu, row * g.N + col, col);
+                }
+                continue;
+            }
             if constexpr (BMODE == MNMAJOR_VEC && NB > 1) {
                 const int64_t col = n0 + wn * TN + NB * x;
                 if (col + NB <= g.N) {
@@ -532,9 +554,10 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     }
 }
 
-// Sums the k_splits partial results into C (plain or accumulating), slices in a fixed order.
-// One thread per output; eight slice loads in flight per thread.
-__global__ void splitk_reduce_kernel(const float* __restrict partial, float* __restrict C, int64_t n, int splits, int accumulate) {
+// Sums the k_splits partial results into C (plain or accumulating), slices in a fixed order, then
+// applies the fused epilogue.  One thread per output; eight slice loads in flight per thread.
+__global__ void splitk_reduce_kernel(const float* __restrict partial, float* __restrict C, int64_t n, int splits, int accumulate,
+                                     const float* __restrict bias, const float* __restrict mask, int relu, int64_t N) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
     for (; i < n; i += stride) {
@@ -548,6 +571,7 @@ __global__ void splitk_reduce_kernel(const float* __restrict partial, float* __r
             for (int u = 0; u < 8; ++u) s += v[u];
         }
         for (; p < splits; ++p) s += partial[(int64_t)p * n + i];
+        if (bias || mask || relu) s = epilogue_value(s, bias, mask, relu, i, i % N);
         C[i] = s;
     }
 }

@@ -180,10 +180,20 @@ struct TileShape { int bm, bn; };
 constexpr int kNumTiles = 5;
 const TileShape kTiles[kNumTiles] = {{256, 128}, {128, 128}, {64, 64}, {128, 64}, {64, 128}};
 
+// what the GEMM store does besides writing the sums (all optional)
+struct Epilogue {
+    const float* bias = nullptr; // + bias[col]
+    const float* mask = nullptr; // dense like C: zero the result where mask <= 0
+    int relu = 0;                // max(., 0) after the bias
+    bool any() const { return bias || mask || relu; }
+};
+
 int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, int64_t b_rs, int64_t b_cs, float* C,
-                  int64_t M, int64_t N, int64_t K, const BatchDesc& bd, int64_t batch_count, int accumulate) {
+                  int64_t M, int64_t N, int64_t K, const BatchDesc& bd, int64_t batch_count, int accumulate, const Epilogue& ep = Epilogue()) {
     if (M == 0 || N == 0 || batch_count == 0) return 0;
+    if (ep.any() && accumulate) return fail(TENMO_ERR_INVALID_ARGUMENT, "a fused epilogue cannot be combined with accumulate");
     if (K == 0) { // empty reduction: the reference's zero-initialised result
+        if (ep.any()) return fail(TENMO_ERR_UNSUPPORTED, "fused epilogue with K = 0");
         if (!accumulate) {
             const int64_t n = batch_count * M * N;
             hipLaunchKernelGGL(fill_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 65535)), dim3(256), 0, S.stream, C, n, 0.f);
@@ -195,6 +205,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     g.a_rs = a_rs; g.a_cs = a_cs; g.b_rs = b_rs; g.b_cs = b_cs;
     g.M = M; g.N = N; g.K = K;
     g.accumulate = accumulate;
+    g.bias = ep.bias; g.mask = ep.mask; g.relu = ep.relu;
     g.batch = bd;
     g.batch_count = batch_count;
     const int am = operand_mode(a_rs, a_cs, M, K);
@@ -267,7 +278,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     if (splits > 1) {
         const int64_t n = batch_count * M * N;
         hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
-                           g.partial, C, n, splits, accumulate);
+                           g.partial, C, n, splits, accumulate, ep.bias, ep.mask, ep.relu, N);
     }
     return 0;
 }
@@ -352,7 +363,7 @@ int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* 
         if (splits > 1) {
             const int64_t n = batch_count * n_out;
             hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
-                               target, out, n, (int)splits, accumulate);
+                               target, out, n, (int)splits, accumulate, (const float*)nullptr, (const float*)nullptr, 0, (int64_t)1);
         }
         return 0;
     }
@@ -399,7 +410,7 @@ int skinny_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, 
     if (splits > 1) {
         const int64_t n = batch_count * M * N;
         hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
-                           target, C, n, (int)splits, accumulate);
+                           target, C, n, (int)splits, accumulate, (const float*)nullptr, (const float*)nullptr, 0, (int64_t)1);
     }
     return 0;
 }
@@ -511,7 +522,7 @@ tenmo_view dense_view(const float* p, const int64_t* shape, int rank) {
     return v;
 }
 
-int matmul_views(const tenmo_view* A, const tenmo_view* B, float* C, int accumulate, const char* who) {
+int matmul_views(const tenmo_view* A, const tenmo_view* B, float* C, int accumulate, const char* who, const Epilogue& ep = Epilogue()) {
     Geometry g;
     if (int rc = resolve(TENMO_OP_MM, A, B, &g, who)) return rc;
     int64_t batch_count = g.batch_count;
@@ -522,9 +533,9 @@ int matmul_views(const tenmo_view* A, const tenmo_view* B, float* C, int accumul
     const float* Bp = B->data + B->offset;
     const int64_t a_rs = A->strides[A->rank - 2], a_cs = A->strides[A->rank - 1];
     const int64_t b_rs = B->strides[B->rank - 2], b_cs = B->strides[B->rank - 1];
-    if (M <= 8 && (b_cs == 1 || N == 1) && N >= 2048 && K > 0)
+    if (M <= 8 && (b_cs == 1 || N == 1) && N >= 2048 && K > 0 && !ep.any())
         return skinny_dispatch(Ap, a_rs, a_cs, Bp, b_rs, C, M, N, K, bd, batch_count, accumulate);
-    return gemm_dispatch(Ap, a_rs, a_cs, Bp, b_rs, b_cs, C, M, N, K, bd, batch_count, accumulate);
+    return gemm_dispatch(Ap, a_rs, a_cs, Bp, b_rs, b_cs, C, M, N, K, bd, batch_count, accumulate, ep);
 }
 
 // dst (dense, parent's shape) += sum over the batch dims of `full` that the parent broadcast
@@ -694,6 +705,25 @@ int tenmo_hip_gemm_f32(const float* A, int64_t a_off, int64_t a_rs, int64_t a_cs
     return finish(sync);
 }
 
+int tenmo_hip_gemm_epilogue_f32(const float* A, int64_t a_off, int64_t a_rs, int64_t a_cs,
+                                const float* B, int64_t b_off, int64_t b_rs, int64_t b_cs,
+                                float* C, int64_t M, int64_t N, int64_t K,
+                                int32_t batch_rank, const int64_t* batch_shape,
+                                const int64_t* a_batch_strides, const int64_t* b_batch_strides,
+                                const float* bias, int32_t relu, const float* mask, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    if (M < 0 || N < 0 || K < 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_gemm_epilogue_f32: negative dimension");
+    if ((!A || !B || !C) && M * N > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_gemm_epilogue_f32: null pointer");
+    if (K == 0 && M * N > 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_gemm_epilogue_f32: K = 0");
+    BatchDesc bd{};
+    int64_t count = 1;
+    if (int rc = fill_batch(bd, batch_rank, batch_shape, a_batch_strides, b_batch_strides, &count)) return rc;
+    Epilogue ep;
+    ep.bias = bias; ep.relu = relu ? 1 : 0; ep.mask = mask;
+    if (int rc = gemm_dispatch(A + a_off, a_rs, a_cs, B + b_off, b_rs, b_cs, C, M, N, K, bd, count, 0, ep)) return rc;
+    return finish(sync);
+}
+
 int tenmo_hip_mv_f32(const float* Mx, int64_t m_off, int64_t m_rs, int64_t m_cs,
                      const float* v, int64_t v_off, int64_t v_s,
                      float* out, int64_t m, int64_t k,
@@ -757,6 +787,14 @@ int64_t tenmo_hip_result_shape(int32_t op, const tenmo_view* A, const tenmo_view
 int tenmo_hip_matmul_nd(const tenmo_view* A, const tenmo_view* B, float* C, int32_t sync) {
     if (int rc = ensure_ready()) return rc;
     if (int rc = matmul_views(A, B, C, 0, "tenmo_hip_matmul_nd")) return rc;
+    return finish(sync);
+}
+
+int tenmo_hip_linear_nd(const tenmo_view* X, const tenmo_view* W, const float* bias, int32_t relu, float* out, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    Epilogue ep;
+    ep.bias = bias; ep.relu = relu ? 1 : 0;
+    if (int rc = matmul_views(X, W, out, 0, "tenmo_hip_linear_nd", ep)) return rc;
     return finish(sync);
 }
 
@@ -1057,8 +1095,9 @@ static int mlp_forward(tenmo_mlp* m, const float* x, int64_t B) {
     const float* in = x;
     for (int l = 0; l < m->L; ++l) {
         const int64_t I = m->dims[l], O = m->dims[l + 1];
-        if (int rc = gemm_dispatch(in, I, 1, m->W[l], O, 1, m->act[l], B, O, I, bd, 1, 0)) return rc;
-        hipLaunchKernelGGL(bias_act_kernel, dim3(grid_for(B * O)), dim3(256), 0, S.stream, m->act[l], m->b[l], B, O, l + 1 < m->L ? 1 : 0);
+        Epilogue ep; // bias add and ReLU happen in the GEMM store
+        ep.bias = m->b[l]; ep.relu = l + 1 < m->L ? 1 : 0;
+        if (int rc = gemm_dispatch(in, I, 1, m->W[l], O, 1, m->act[l], B, O, I, bd, 1, 0, ep)) return rc;
         in = m->act[l];
     }
     return 0;
@@ -1089,14 +1128,22 @@ static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int6
         // dW = in^T(view) . g        (tenmo/matmul.mojo:46-48)
         if (int rc = gemm_dispatch(in, 1, I, gl, O, 1, m->dW[l], I, O, B, bd, 1, 0)) return rc;
         if (l > 0) { // dX = g . W^T(view)  (tenmo/matmul.mojo:36-38); the network input needs no gradient (:34)
-            if (int rc = gemm_dispatch(gl, O, 1, m->W[l], 1, O, m->grad[l - 1], B, I, O, bd, 1, 0)) return rc;
-            hipLaunchKernelGGL(relu_backward_kernel, dim3(grid_for(B * I)), dim3(256), 0, S.stream, m->grad[l - 1], m->act[l - 1], B * I);
+            Epilogue ep; // ReLU backward in the GEMM store: zero where the forward activation was not positive
+            ep.mask = m->act[l - 1];
+            if (int rc = gemm_dispatch(gl, O, 1, m->W[l], 1, O, m->grad[l - 1], B, I, O, bd, 1, 0, ep)) return rc;
         }
     }
-    for (int l = 0; l < L; ++l) {
-        const int64_t wn = m->dims[l] * m->dims[l + 1], bn = m->dims[l + 1];
-        hipLaunchKernelGGL(sgd_kernel, dim3(grid_for(wn)), dim3(256), 0, S.stream, m->W[l], m->dW[l], wn, lr);
-        hipLaunchKernelGGL(sgd_kernel, dim3(grid_for(bn)), dim3(256), 0, S.stream, m->b[l], m->db[l], bn, lr);
+    // every parameter tensor in one launch
+    for (int l0 = 0; l0 < L; l0 += SGD_MAX_TENSORS / 2) {
+        SgdArgs sa{};
+        int64_t largest = 0;
+        for (int l = l0; l < L && sa.count + 2 <= SGD_MAX_TENSORS; ++l) {
+            const int64_t wn = m->dims[l] * m->dims[l + 1], bn = m->dims[l + 1];
+            sa.p[sa.count] = m->W[l]; sa.g[sa.count] = m->dW[l]; sa.n[sa.count] = wn; ++sa.count;
+            sa.p[sa.count] = m->b[l]; sa.g[sa.count] = m->db[l]; sa.n[sa.count] = bn; ++sa.count;
+            largest = std::max(largest, wn);
+        }
+        hipLaunchKernelGGL(sgd_multi_kernel, dim3(grid_for(largest), (unsigned)sa.count), dim3(256), 0, S.stream, sa, lr);
     }
     return 0;
 }

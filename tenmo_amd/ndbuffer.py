@@ -127,6 +127,21 @@ class NDBuffer:
         """NDBuffer.matmul_nd (tenmo/ndbuffer.mojo:2445-2501)."""
         return self._product(OP_MM, other, "tenmo_hip_matmul_nd", sync)
 
+    def linear(self, weight: "NDBuffer", bias: "NDBuffer", relu: bool = False, sync: bool = False) -> "NDBuffer":
+        """self . weight + bias (then ReLU) in one launch: Linear.forward, tenmo/net.mojo:193-201."""
+        if bias.rank() != 1 or bias.strides[0] != 1 or bias.shape[0] != weight.shape[-1]:
+            raise TenmoHipError(-2, f"linear: bias of shape {bias.shape} does not match weight {weight.shape}")
+        L = _lib.load()
+        a, b = self.c_view(), weight.c_view()
+        _lib.init()
+        oshape = (C.c_int64 * (_lib.MAX_RANK + 2))()
+        orank = C.c_int32()
+        check(L.tenmo_hip_result_shape(OP_MM, C.byref(a), C.byref(b), oshape, C.byref(orank)))
+        out = NDBuffer.empty(tuple(oshape[i] for i in range(orank.value)))
+        check(L.tenmo_hip_linear_nd(C.byref(a), C.byref(b), bias.data_ptr() + 4 * bias.offset, 1 if relu else 0,
+                                    out.data_ptr(), 1 if sync else 0))
+        return out
+
     def matrix_vector(self, v: "NDBuffer", sync: bool = False) -> "NDBuffer":
         return self._product(OP_MV, v, "tenmo_hip_matrix_vector_nd", sync)
 

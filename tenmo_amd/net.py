@@ -1,9 +1,10 @@
 """Callers of the matrix-product path: ``Linear`` and the MNIST-shaped MLP training step.
 
-``Linear``        y = x.W + b with W stored [in, out] (tenmo/net.mojo:49-216, :91-97).  The bias add
-                  and the bias gradient are expressed as rank-1 products on the same GEMM entry
-                  (ones[rows,1] . b[1,out], then += x.W;  db = ones[1,rows] . dY), so the layer never
-                  leaves ``libtenmo_hip.so``.
+``Linear``        y = x.W + b with W stored [in, out] (tenmo/net.mojo:49-216, :91-97).  For matrix
+                  inputs the bias is added in the GEMM store (one launch); for a vector input it
+                  is a rank-1 product on the GEMM entry (ones[rows,1] . b[1,out], accumulated),
+                  as is the bias gradient (db = ones[1,rows] . dY), so the layer never leaves
+                  ``libtenmo_hip.so``.
 ``MLP``           the whole training step of examples/mnist.mojo:150-162 on the device:
                   Linear -> ReLU -> ... -> Linear -> CrossEntropyLoss(mean) -> backward -> SGD(lr).
 ``xavier_uniform``  U(+-sqrt(6/(in+out))) weights, zero bias (tenmo/net.mojo:87-114).
@@ -19,7 +20,7 @@ import torch
 
 from . import _lib
 from ._lib import TenmoHipError, check
-from .matmul import Matmul
+from .matmul import Matmul, Matmul2dBackward, MatmulNdBackward
 from .ndbuffer import NDBuffer
 from .tensor import Tensor, mm
 
@@ -52,15 +53,24 @@ class Linear:
     def __call__(self, xs: Tensor, sync: bool = True) -> Tensor:
         if xs.shape()[-1] != self.weight.shape()[0]:
             raise TenmoHipError(-2, f"LinearBLAS forward: input dim mismatch: input shape -> {xs.shape()} and weights shape -> {self.weight.shape()}")
-        out = Matmul.forward(xs, self.weight, track_grad=self.training, mode=mm, sync=False)
         if self.bias is None:
-            return out
-        # out += ones[rows,1] . b[1,out]  — Adder.forward with broadcasting (tenmo/addition.mojo:73-112)
+            return Matmul.forward(xs, self.weight, track_grad=self.training, mode=mm, sync=sync)
         L = _lib.load()
-        rows = out.numels() // self.out_features
-        ones = torch.ones(rows, dtype=torch.float32, device="cuda")
-        check(L.tenmo_hip_gemm_f32(ones.data_ptr(), 0, 1, 1, self.bias.buffer.data_ptr(), self.bias.buffer.offset, self.out_features, 1,
-                                   out.buffer.data_ptr(), rows, self.out_features, 1, 0, None, None, None, 1, 1 if sync else 0))
+        if xs.rank() >= 2:
+            # x.W + b in one launch: the bias is added in the GEMM store
+            out = Tensor(xs.buffer.linear(self.weight.buffer, self.bias.buffer, relu=False, sync=sync), requires_grad=False)
+            if self.training and (xs.requires_grad or self.weight.requires_grad):
+                out.requires_grad = True
+                out.add_ancestry((Matmul2dBackward if xs.rank() == 2 else MatmulNdBackward).backward, xs, self.weight)
+            rows = out.numels() // self.out_features
+            ones = torch.ones(rows, dtype=torch.float32, device="cuda") if self.training and self.bias.requires_grad else None
+        else:
+            out = Matmul.forward(xs, self.weight, track_grad=self.training, mode=mm, sync=False)
+            # out += ones[rows,1] . b[1,out]  — Adder.forward with broadcasting (tenmo/addition.mojo:73-112)
+            rows = out.numels() // self.out_features
+            ones = torch.ones(rows, dtype=torch.float32, device="cuda")
+            check(L.tenmo_hip_gemm_f32(ones.data_ptr(), 0, 1, 1, self.bias.buffer.data_ptr(), self.bias.buffer.offset, self.out_features, 1,
+                                       out.buffer.data_ptr(), rows, self.out_features, 1, 0, None, None, None, 1, 1 if sync else 0))
         if self.training and (out.backward_fn is not None or self.bias.requires_grad):
             inner, bias, parents = out.backward_fn, self.bias, list(out.ancestors)
 

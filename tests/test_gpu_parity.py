@@ -187,6 +187,55 @@ def test_direct_path_pitch_limits(T):
     assert rel_fro(flipped_cols.matmul(B, track_grad=False).to_numpy(), ref_matmul64(a[:, ::-1], b)) <= RTOL_FRO
 
 
+@pytest.mark.parametrize("tile", [-1, 0, 2, 3])
+def test_fused_epilogue(T, tile):
+    """bias + ReLU + ReLU-gradient mask applied in the GEMM store equal the separate steps, on every
+    path that can finish a tile: plain store, K slices + reduction, batched, ragged extents."""
+    L, lib = T.lib.load(), T.lib
+    rng = np.random.default_rng(31)
+    try:
+        L.tenmo_hip_set_tuning(b"gemm_tile", tile)
+        for (bsz, m, k, n, sk) in [(1, 64, 784, 128, -1), (1, 64, 784, 128, 3), (1, 300, 100, 77, -1), (3, 70, 48, 130, -1), (1, 5, 1000, 9, 4)]:
+            L.tenmo_hip_set_tuning(b"gemm_splitk", sk)
+            a = rng.standard_normal((bsz, m, k), dtype=np.float32)
+            b = rng.standard_normal((k, n), dtype=np.float32)
+            bias = rng.standard_normal(n).astype(np.float32)
+            mask = rng.standard_normal((bsz, m, n)).astype(np.float32)
+            A, B, Bi, Mk = (T.Tensor.from_numpy(x) for x in (a, b, bias, mask))
+            out = T.Tensor.zeros(bsz, m, n)
+            z = ref_matmul64(a, b)
+            for relu, use_bias, use_mask in [(0, 1, 0), (1, 1, 0), (1, 0, 0), (0, 0, 1), (1, 1, 1)]:
+                lib.check(L.tenmo_hip_gemm_epilogue_f32(
+                    A.buffer.data_ptr(), 0, k, 1, B.buffer.data_ptr(), 0, n, 1, out.buffer.data_ptr(), m, n, k,
+                    1, lib.i64([bsz]), lib.i64([m * k]), lib.i64([0]),
+                    Bi.buffer.data_ptr() if use_bias else None, relu, Mk.buffer.data_ptr() if use_mask else None, 1))
+                ref = z + (bias if use_bias else 0.0)
+                if relu:
+                    ref = np.where(ref > 0, ref, 0.0)
+                if use_mask:
+                    ref = np.where(mask > 0, ref, 0.0)
+                got = out.to_numpy()
+                # elements within rounding of the ReLU threshold may legitimately land on either side
+                near = np.abs(z + (bias if use_bias else 0.0)) < 1e-4
+                assert rel_fro(np.where(near, 0, got), np.where(near, 0, ref)) <= RTOL_FRO, (tile, bsz, m, k, n, sk, relu, use_bias, use_mask)
+                if use_mask:
+                    assert np.all(got[mask <= 0] == 0)
+        # view-level Linear entry against the unfused sequence
+        x = rng.standard_normal((4, 33, 50), dtype=np.float32)
+        w = rng.standard_normal((50, 20), dtype=np.float32)
+        bias = rng.standard_normal(20).astype(np.float32)
+        X, W, Bi = T.Tensor.from_numpy(x), T.Tensor.from_numpy(w), T.Tensor.from_numpy(bias)
+        got = X.buffer.linear(W.buffer, Bi.buffer, relu=True, sync=True).to_numpy()
+        ref = np.maximum(ref_matmul64(x, w) + bias, 0)
+        assert got.shape == (4, 33, 20) and rel_fro(got, ref) <= RTOL_FRO
+        # accumulate and a fused epilogue exclude each other; K = 0 has no sums to finish
+        assert L.tenmo_hip_gemm_epilogue_f32(A.buffer.data_ptr(), 0, 4, 1, B.buffer.data_ptr(), 0, 4, 1, out.buffer.data_ptr(), 2, 2, 0,
+                                             0, None, None, None, Bi.buffer.data_ptr(), 0, None, 1) == -2
+    finally:
+        L.tenmo_hip_set_tuning(b"gemm_tile", -1)
+        L.tenmo_hip_set_tuning(b"gemm_splitk", -1)
+
+
 def test_odd_strides_and_overlap(T, oracle):
     """Column stride 2, row stride 0 (broadcast rows), overlapping windows (tests/test_mmnd.mojo:143-175)."""
     rng = np.random.default_rng(23)
