@@ -91,21 +91,39 @@ __global__ void fill_kernel(float* p, int64_t n, float value) {
 // ---- MLP harness stages -----------------------------------------------------------------------
 // Fused class-index cross-entropy, mean reduction (tenmo/crossentropy.mojo:285-432) and its
 // gradient (softmax - onehot) / valid_count (:775-793, :451-481).  One thread per row (C is tiny in
-// the harness); per-row losses go to row_loss for the ordered sum below.
+// the harness); per-row losses go to row_loss for the ordered sum.  When the whole batch fits one
+// workgroup (gridDim.x == 1) and loss_out / db_out are given, the same launch also finishes the
+// ordered mean and the bias gradient of the last layer (column sums of dz, rows ascending).
 __global__ void cross_entropy_kernel(const float* __restrict logits, const int32_t* __restrict y, int64_t rows, int64_t C,
-                                     float* __restrict dz, float* __restrict row_loss) {
+                                     float* __restrict dz, float* __restrict row_loss, float* __restrict loss_out, float* __restrict db_out) {
     const int64_t r = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (r >= rows) return;
-    const float* x = logits + r * C;
-    float mx = -3.402823466e+38f;
-    for (int64_t c = 0; c < C; ++c) mx = fmaxf(mx, x[c]);
-    float sum_exp = 0.f;
-    for (int64_t c = 0; c < C; ++c) sum_exp += expf(x[c] - mx);
-    const float lse = logf(fmaxf(sum_exp, 1e-7f));
-    const int32_t t = y[r];
-    row_loss[r] = -(x[t] - mx - lse);
-    const float inv = 1.f / sum_exp, scale = 1.f / (float)rows;
-    for (int64_t c = 0; c < C; ++c) dz[r * C + c] = (expf(x[c] - mx) * inv - (c == t ? 1.f : 0.f)) * scale;
+    if (r < rows) {
+        const float* x = logits + r * C;
+        float mx = -3.402823466e+38f;
+        for (int64_t c = 0; c < C; ++c) mx = fmaxf(mx, x[c]);
+        float sum_exp = 0.f;
+        for (int64_t c = 0; c < C; ++c) sum_exp += expf(x[c] - mx);
+        const float lse = logf(fmaxf(sum_exp, 1e-7f));
+        const int32_t t = y[r];
+        row_loss[r] = -(x[t] - mx - lse);
+        const float inv = 1.f / sum_exp, scale = 1.f / (float)rows;
+        for (int64_t c = 0; c < C; ++c) dz[r * C + c] = (expf(x[c] - mx) * inv - (c == t ? 1.f : 0.f)) * scale;
+    }
+    if (gridDim.x == 1 && (loss_out || db_out)) {
+        __syncthreads(); // this workgroup wrote every row
+        if (loss_out && threadIdx.x == 0) {
+            float s = 0.f;
+            for (int64_t q = 0; q < rows; ++q) s += row_loss[q];
+            *loss_out = s / (float)rows;
+        }
+        if (db_out) {
+            for (int64_t c = threadIdx.x; c < C; c += blockDim.x) {
+                float s = 0.f;
+                for (int64_t q = 0; q < rows; ++q) s += dz[q * C + c];
+                db_out[c] = s;
+            }
+        }
+    }
 }
 
 // loss = (sum of row losses in row order) / rows — the order of the reference's scalar loop

@@ -1116,15 +1116,20 @@ static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int6
     if (int rc = mlp_forward(m, x, B)) return rc;
     const int L = m->L;
     const int64_t C = m->dims[L];
-    hipLaunchKernelGGL(cross_entropy_kernel, dim3((unsigned)((B + 63) / 64)), dim3(64), 0, S.stream, m->act[L - 1], y, B, C, m->grad[L - 1], m->row_loss);
-    hipLaunchKernelGGL(ordered_mean_kernel, dim3(1), dim3(64), 0, S.stream, m->row_loss, B, loss_out);
+    const bool one_block = B <= 256; // loss, its gradient, the mean and the last bias gradient in one launch
+    if (one_block) {
+        hipLaunchKernelGGL(cross_entropy_kernel, dim3(1), dim3((unsigned)((B + 63) / 64 * 64)), 0, S.stream, m->act[L - 1], y, B, C, m->grad[L - 1], m->row_loss, loss_out, m->db[L - 1]);
+    } else {
+        hipLaunchKernelGGL(cross_entropy_kernel, dim3((unsigned)((B + 63) / 64)), dim3(64), 0, S.stream, m->act[L - 1], y, B, C, m->grad[L - 1], m->row_loss, (float*)nullptr, (float*)nullptr);
+        hipLaunchKernelGGL(ordered_mean_kernel, dim3(1), dim3(64), 0, S.stream, m->row_loss, B, loss_out);
+    }
     BatchDesc bd{};
     for (int d = 0; d < MAX_BATCH_RANK; ++d) bd.shape[d] = 1;
     for (int l = L - 1; l >= 0; --l) {
         const int64_t I = m->dims[l], O = m->dims[l + 1];
         const float* in = l == 0 ? x : m->act[l - 1];
         const float* gl = m->grad[l];
-        hipLaunchKernelGGL(column_sum_kernel, dim3((unsigned)((O + 63) / 64)), dim3(64), 0, S.stream, gl, B, O, m->db[l]);
+        if (!(one_block && l == L - 1)) hipLaunchKernelGGL(column_sum_kernel, dim3((unsigned)((O + 63) / 64)), dim3(64), 0, S.stream, gl, B, O, m->db[l]);
         // dW = in^T(view) . g        (tenmo/matmul.mojo:46-48)
         if (int rc = gemm_dispatch(in, 1, I, gl, O, 1, m->dW[l], I, O, B, bd, 1, 0)) return rc;
         if (l > 0) { // dX = g . W^T(view)  (tenmo/matmul.mojo:36-38); the network input needs no gradient (:34)

@@ -536,9 +536,21 @@ def test_mlp_loss_curve_tracks_cpu(T, oracle):
         (Wg, bg), (Wc, bc) = gpu.params(l), cpu.params(l)
         assert rel_fro(Wg, Wc) <= 1e-5 and np.abs(bg - bc).max() <= 1e-5
         (dWg, dbg), (dWc, dbc) = gpu.grads(l), cpu.grads(l)
-        assert rel_fro(dWg, dWc) <= 1e-4
+        assert rel_fro(dWg, dWc) <= 1e-4 and rel_fro(dbg, dbc) <= 1e-4
     x, _ = R.mnist_like_batch(64, seed, 99)
     assert rel_fro(gpu.forward(x), cpu.forward(x)) <= 1e-5
+    # a batch larger than one workgroup takes the separate loss-mean / bias-gradient launches
+    dims = [40, 24, 5]
+    Ws, bs = R.xavier_mlp(dims, seed + 1)
+    gpu, cpu = MLP(dims, Ws, bs, 300), oracle.MLP(dims, Ws, bs, 300)
+    rs = np.random.default_rng(5)
+    for step in range(5):
+        x = rs.standard_normal((300, 40)).astype(np.float32)
+        y = rs.integers(0, 5, 300).astype(np.int32)
+        assert abs(gpu.step(x, y, 0.05) - cpu.step(x, y, 0.05)) <= 1e-4, step
+    for l in range(2):
+        (dWg, dbg), (dWc, dbc) = gpu.grads(l), cpu.grads(l)
+        assert rel_fro(dWg, dWc) <= 1e-4 and rel_fro(dbg, dbc) <= 1e-4
     # cross-entropy vector of the reference: uniform logits -> -log(1/3)
     m = MLP([2, 3], [np.zeros((2, 3), np.float32)], [np.ones(3, np.float32)], 2)
     assert abs(m.step(np.ones((2, 2), np.float32), np.asarray([0, 1], np.int32), 0.0) - 1.0986122886681098) < 1e-6
