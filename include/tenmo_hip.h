@@ -126,6 +126,13 @@ int tenmo_hip_vm_f32(const float* v, int64_t v_off, int64_t v_s,
                      const int64_t* v_batch_strides, const int64_t* m_batch_strides,
                      int32_t accumulate, int32_t sync);
 
+/* out[c] (+)= sum over r < rows of G[g_off + r*g_rs + c], c < cols: the bias gradient of a Linear
+ * layer, i.e. the upstream gradient summed over its broadcast (row) axis — what
+ * sum_over_broadcasted_axes does for the bias operand of Adder (tenmo/broadcast.mojo:66-88,
+ * tenmo/addition.mojo:73-112).  G is streamed once at HBM rate. */
+int tenmo_hip_column_sum_f32(const float* G, int64_t g_off, int64_t g_rs, int64_t rows, int64_t cols,
+                             float* out, int32_t accumulate, int32_t sync);
+
 /* out[0] = sum_i a[i]*b[i]   (a stride of 0 broadcasts a one-element operand,
  * tenmo/dotproduct.mojo:67-74).  Replaces: DotproductKernel.launch,
  * tenmo/kernels/dotproduct_kernel.mojo:19-110. */

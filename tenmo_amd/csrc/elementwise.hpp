@@ -105,7 +105,9 @@ __global__ void cross_entropy_kernel(const float* __restrict logits, const int32
         for (int64_t c = 0; c < C; ++c) sum_exp += expf(x[c] - mx);
         const float lse = logf(fmaxf(sum_exp, 1e-7f));
         const int32_t t = y[r];
-        row_loss[r] = -(x[t] - mx - lse);
+        // a label outside [0, C) (the reference rejects it on the host, crossentropy.mojo:116-123) must
+        // not turn into an out-of-bounds read: its loss is NaN, its row gets no one-hot term
+        row_loss[r] = (t >= 0 && t < C) ? -(x[t] - mx - lse) : __builtin_nanf("");
         const float inv = 1.f / sum_exp, scale = 1.f / (float)rows;
         for (int64_t c = 0; c < C; ++c) dz[r * C + c] = (expf(x[c] - mx) * inv - (c == t ? 1.f : 0.f)) * scale;
     }

@@ -65,6 +65,7 @@ struct State {
     float* stage[3] = {nullptr, nullptr, nullptr};
     size_t stage_bytes[3] = {0, 0, 0};
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    float* one = nullptr; // device constant 1.0f: a stride-0 vector of ones for column sums
     // tuning overrides (environment, read once): -1 = automatic
     int force_tile = -1;
     int force_splitk = -1;
@@ -419,11 +420,18 @@ int skinny_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, 
 // view helpers
 // ------------------------------------------------------------------------------------------------
 
-int check_view(const tenmo_view* v, const char* who) {
+int check_view(const tenmo_view* v, const char* who, bool need_data) {
     if (!v) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: null view", who);
     if (v->rank < 0 || v->rank > TENMO_MAX_RANK) return fail(TENMO_ERR_INVALID_SHAPE, "%s: rank %d exceeds max_rank %d", who, v->rank, TENMO_MAX_RANK);
     for (int d = 0; d < v->rank; ++d)
         if (v->shape[d] < 0) return fail(TENMO_ERR_INVALID_SHAPE, "%s: negative dimension", who);
+    if (need_data && !v->data && product(v->shape, v->rank) > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: view without data", who);
+    return 0;
+}
+
+// a result / gradient pointer that will be written must not be null
+int need(const void* p, bool written, const char* who, const char* what) {
+    if (!p && written) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: null %s", who, what);
     return 0;
 }
 
@@ -458,9 +466,10 @@ struct Geometry {
 };
 
 // trailing dims: MM (2,2), MV (2,1), VM (1,2)
-int resolve(int op, const tenmo_view* A, const tenmo_view* B, Geometry* g, const char* who) {
-    if (int rc = check_view(A, who)) return rc;
-    if (int rc = check_view(B, who)) return rc;
+// need_data = false for pure shape queries, which never touch the operands
+int resolve(int op, const tenmo_view* A, const tenmo_view* B, Geometry* g, const char* who, bool need_data = true) {
+    if (int rc = check_view(A, who, need_data)) return rc;
+    if (int rc = check_view(B, who, need_data)) return rc;
     const int ta = op == TENMO_OP_VM ? 1 : 2, tb = op == TENMO_OP_MV ? 1 : 2;
     if (op == TENMO_OP_MM) {
         if (A->rank < 2) return fail(TENMO_ERR_INVALID_SHAPE, "MatmulNdGpu: A must have rank >= 2");
@@ -527,6 +536,7 @@ int matmul_views(const tenmo_view* A, const tenmo_view* B, float* C, int accumul
     if (int rc = resolve(TENMO_OP_MM, A, B, &g, who)) return rc;
     int64_t batch_count = g.batch_count;
     if (batch_count == 0) return 0; // no output elements (the reference only widens the loop count, matmul_cpu.mojo:666-667)
+    if (int rc = need(C, product(g.oshape, g.orank) > 0, who, "result pointer")) return rc;
     const BatchDesc bd = make_batch(g, A, 2, B, 2);
     const int64_t M = A->shape[A->rank - 2], K = A->shape[A->rank - 1], N = B->shape[B->rank - 1];
     const float* Ap = A->data + A->offset;
@@ -624,6 +634,9 @@ int tenmo_hip_init(int device_id) {
     S.stream = S.own_stream;
     HIP_TRY(hipEventCreate(&S.ev0));
     HIP_TRY(hipEventCreate(&S.ev1));
+    HIP_TRY(hipMalloc(&S.one, sizeof(float)));
+    const float one = 1.0f;
+    HIP_TRY(hipMemcpy(S.one, &one, sizeof one, hipMemcpyHostToDevice));
     S.force_tile = env_int("TENMO_HIP_GEMM_TILE", -1);
     S.force_splitk = env_int("TENMO_HIP_GEMM_SPLITK", -1);
     S.verbose = env_int("TENMO_HIP_VERBOSE", 0);
@@ -634,13 +647,15 @@ int tenmo_hip_init(int device_id) {
 int tenmo_hip_shutdown(void) {
     std::lock_guard<std::mutex> lock(S_mu);
     if (!S.ready) return 0;
-    hipStreamSynchronize(S.stream);
-    if (S.ws) hipFree(S.ws);
-    if (S.ws2) hipFree(S.ws2);
-    for (int i = 0; i < 3; ++i) if (S.stage[i]) hipFree(S.stage[i]);
-    hipEventDestroy(S.ev0);
-    hipEventDestroy(S.ev1);
-    hipStreamDestroy(S.own_stream);
+    // teardown: nothing useful can be done with a failure here
+    (void)hipStreamSynchronize(S.stream);
+    if (S.ws) (void)hipFree(S.ws);
+    if (S.ws2) (void)hipFree(S.ws2);
+    if (S.one) (void)hipFree(S.one);
+    for (int i = 0; i < 3; ++i) if (S.stage[i]) (void)hipFree(S.stage[i]);
+    (void)hipEventDestroy(S.ev0);
+    (void)hipEventDestroy(S.ev1);
+    (void)hipStreamDestroy(S.own_stream);
     S = State();
     return 0;
 }
@@ -697,7 +712,8 @@ int tenmo_hip_gemm_f32(const float* A, int64_t a_off, int64_t a_rs, int64_t a_cs
                        int32_t accumulate, int32_t sync) {
     if (int rc = ensure_ready()) return rc;
     if (M < 0 || N < 0 || K < 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_gemm_f32: negative dimension");
-    if ((!A || !B || !C) && M * N > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_gemm_f32: null pointer");
+    if (int rc = need(C, M * N > 0, "tenmo_hip_gemm_f32", "result pointer")) return rc;
+    if ((!A || !B) && M * N * K > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_gemm_f32: null pointer");
     BatchDesc bd{};
     int64_t count = 1;
     if (int rc = fill_batch(bd, batch_rank, batch_shape, a_batch_strides, b_batch_strides, &count)) return rc;
@@ -713,7 +729,8 @@ int tenmo_hip_gemm_epilogue_f32(const float* A, int64_t a_off, int64_t a_rs, int
                                 const float* bias, int32_t relu, const float* mask, int32_t sync) {
     if (int rc = ensure_ready()) return rc;
     if (M < 0 || N < 0 || K < 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_gemm_epilogue_f32: negative dimension");
-    if ((!A || !B || !C) && M * N > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_gemm_epilogue_f32: null pointer");
+    if (int rc = need(C, M * N > 0, "tenmo_hip_gemm_epilogue_f32", "result pointer")) return rc;
+    if ((!A || !B) && M * N * K > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_gemm_epilogue_f32: null pointer");
     if (K == 0 && M * N > 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_gemm_epilogue_f32: K = 0");
     BatchDesc bd{};
     int64_t count = 1;
@@ -735,6 +752,8 @@ int tenmo_hip_mv_f32(const float* Mx, int64_t m_off, int64_t m_rs, int64_t m_cs,
     BatchDesc bd{};
     int64_t count = 1;
     if (int rc = fill_batch(bd, batch_rank, batch_shape, m_batch_strides, v_batch_strides, &count)) return rc;
+    if (int rc = need(out, m * count > 0, "tenmo_hip_mv_f32", "result pointer")) return rc;
+    if ((!Mx || !v) && m * k * count > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_mv_f32: null operand");
     if (int rc = matvec_dispatch(Mx + m_off, m_rs, m_cs, v + v_off, v_s, out, m, k, bd, count, accumulate)) return rc;
     return finish(sync);
 }
@@ -751,8 +770,23 @@ int tenmo_hip_vm_f32(const float* v, int64_t v_off, int64_t v_s,
     int64_t count = 1;
     // matvec_dispatch wants (matrix, vector) order in the batch descriptor
     if (int rc = fill_batch(bd, batch_rank, batch_shape, m_batch_strides, v_batch_strides, &count)) return rc;
+    if (int rc = need(out, n * count > 0, "tenmo_hip_vm_f32", "result pointer")) return rc;
+    if ((!Mx || !v) && n * k * count > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_vm_f32: null operand");
     // out[j] = sum_i Mx(i, j) v(i): outputs walk the matrix columns, the reduction walks its rows
     if (int rc = matvec_dispatch(Mx + m_off, m_cs, m_rs, v + v_off, v_s, out, n, k, bd, count, accumulate)) return rc;
+    return finish(sync);
+}
+
+int tenmo_hip_column_sum_f32(const float* G, int64_t g_off, int64_t g_rs, int64_t rows, int64_t cols,
+                             float* out, int32_t accumulate, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    if (rows < 0 || cols < 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_column_sum_f32: negative dimension");
+    if (int rc = need(out, cols > 0, "tenmo_hip_column_sum_f32", "result pointer")) return rc;
+    if (!G && rows * cols > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_column_sum_f32: null operand");
+    // ones[rows] . G[rows, cols] with the ones read through stride 0: the matrix is streamed once
+    BatchDesc bd{};
+    for (int d = 0; d < MAX_BATCH_RANK; ++d) bd.shape[d] = 1;
+    if (int rc = matvec_dispatch(G + g_off, 1, g_rs, S.one, 0, out, cols, rows, bd, 1, accumulate)) return rc;
     return finish(sync);
 }
 
@@ -760,6 +794,8 @@ int tenmo_hip_dot_f32(const float* a, int64_t a_off, int64_t a_s, const float* b
                       int64_t n, float* out, int32_t sync) {
     if (int rc = ensure_ready()) return rc;
     if (n < 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_dot_f32: negative length");
+    if (int rc = need(out, true, "tenmo_hip_dot_f32", "result pointer")) return rc;
+    if ((!a || !b) && n > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_dot_f32: null operand");
     const int parts = (int)std::max<int64_t>(1, std::min<int64_t>((n + DOT_THREADS * 8 - 1) / (DOT_THREADS * 8), 1024));
     float* ws;
     if (int rc = workspace(parts * sizeof(float), &ws)) return rc;
@@ -778,7 +814,7 @@ int tenmo_hip_classify_matmul(int32_t ra, const int64_t* a, int32_t rb, const in
 
 int64_t tenmo_hip_result_shape(int32_t op, const tenmo_view* A, const tenmo_view* B, int64_t* out_shape, int32_t* out_rank) {
     Geometry g;
-    if (int rc = resolve(op, A, B, &g, "tenmo_hip_result_shape")) return rc;
+    if (int rc = resolve(op, A, B, &g, "tenmo_hip_result_shape", false)) return rc;
     if (out_shape) std::copy(g.oshape, g.oshape + g.orank, out_shape);
     if (out_rank) *out_rank = g.orank;
     return product(g.oshape, g.orank);
@@ -802,6 +838,7 @@ int tenmo_hip_matrix_vector_nd(const tenmo_view* Mx, const tenmo_view* v, float*
     if (int rc = ensure_ready()) return rc;
     Geometry g;
     if (int rc = resolve(TENMO_OP_MV, Mx, v, &g, "tenmo_hip_matrix_vector_nd")) return rc;
+    if (int rc = need(out, product(g.oshape, g.orank) > 0, "tenmo_hip_matrix_vector_nd", "result pointer")) return rc;
     const BatchDesc bd = make_batch(g, Mx, 2, v, 1);
     const int64_t m = Mx->shape[Mx->rank - 2], k = Mx->shape[Mx->rank - 1];
     if (int rc = matvec_dispatch(Mx->data + Mx->offset, Mx->strides[Mx->rank - 2], Mx->strides[Mx->rank - 1],
@@ -813,6 +850,7 @@ int tenmo_hip_vector_matmul_nd(const tenmo_view* v, const tenmo_view* Mx, float*
     if (int rc = ensure_ready()) return rc;
     Geometry g;
     if (int rc = resolve(TENMO_OP_VM, v, Mx, &g, "tenmo_hip_vector_matmul_nd")) return rc;
+    if (int rc = need(out, product(g.oshape, g.orank) > 0, "tenmo_hip_vector_matmul_nd", "result pointer")) return rc;
     const BatchDesc bd = make_batch(g, Mx, 2, v, 1); // (matrix, vector) order
     const int64_t k = Mx->shape[Mx->rank - 2], n = Mx->shape[Mx->rank - 1];
     if (int rc = matvec_dispatch(Mx->data + Mx->offset, Mx->strides[Mx->rank - 1], Mx->strides[Mx->rank - 2],
@@ -826,6 +864,7 @@ int tenmo_hip_matmul_backward(const tenmo_view* A, const tenmo_view* B, const fl
     Geometry g;
     if (int rc = resolve(TENMO_OP_MM, A, B, &g, "tenmo_hip_matmul_backward")) return rc;
     if (g.batch_count == 0) return 0;
+    if (int rc = need(dC, product(g.oshape, g.orank) > 0 && (grad_A || grad_B), "tenmo_hip_matmul_backward", "upstream gradient")) return rc;
     const tenmo_view dCv = dense_view(dC, g.oshape, g.orank);
     if (grad_A) { // dA = dC . B^T(view)   (tenmo/matmul.mojo:36-38, :116-121)
         const tenmo_view Bt = transposed_last2(B);
@@ -896,6 +935,7 @@ int tenmo_hip_mv_backward(const tenmo_view* Mx, const tenmo_view* v, const float
     Geometry g;
     if (int rc = resolve(TENMO_OP_MV, Mx, v, &g, "tenmo_hip_mv_backward")) return rc;
     if (g.batch_count == 0) return 0;
+    if (int rc = need(dy, product(g.oshape, g.orank) > 0 && (grad_M || grad_v), "tenmo_hip_mv_backward", "upstream gradient")) return rc;
     const int64_t m = Mx->shape[Mx->rank - 2], k = Mx->shape[Mx->rank - 1];
     int64_t dy_bstr[MAX_BATCH_RANK] = {0}, v_bstr[MAX_BATCH_RANK] = {0}, m_bstr[MAX_BATCH_RANK] = {0};
     { int64_t acc = m; for (int d = g.batch_rank - 1; d >= 0; --d) { dy_bstr[d] = acc; acc *= g.oshape[d]; } }
@@ -933,6 +973,7 @@ int tenmo_hip_vm_backward(const tenmo_view* v, const tenmo_view* Mx, const float
     Geometry g;
     if (int rc = resolve(TENMO_OP_VM, v, Mx, &g, "tenmo_hip_vm_backward")) return rc;
     if (g.batch_count == 0) return 0;
+    if (int rc = need(dy, product(g.oshape, g.orank) > 0 && (grad_v || grad_M), "tenmo_hip_vm_backward", "upstream gradient")) return rc;
     const int64_t k = Mx->shape[Mx->rank - 2], n = Mx->shape[Mx->rank - 1];
     int64_t dy_bstr[MAX_BATCH_RANK] = {0}, v_bstr[MAX_BATCH_RANK] = {0}, m_bstr[MAX_BATCH_RANK] = {0};
     { int64_t acc = n; for (int d = g.batch_rank - 1; d >= 0; --d) { dy_bstr[d] = acc; acc *= g.oshape[d]; } }
@@ -1050,6 +1091,7 @@ struct tenmo_mlp {
     int64_t g_batch = -1;
     float g_lr = 0.f;
     float* g_loss = nullptr;
+    float* g_ws = nullptr;      // library scratch pointer the captured kernels hold
 };
 
 static unsigned grid_for(int64_t n) { return (unsigned)std::max<int64_t>(1, std::min<int64_t>((n + 255) / 256, 4096)); }
@@ -1079,13 +1121,13 @@ tenmo_mlp* tenmo_hip_mlp_create(int32_t L, const int64_t* dims, const float* con
 
 void tenmo_hip_mlp_destroy(tenmo_mlp* m) {
     if (!m) return;
-    if (S.ready) hipStreamSynchronize(S.stream);
+    if (S.ready) (void)hipStreamSynchronize(S.stream);
     for (auto* v : {&m->W, &m->b, &m->dW, &m->db, &m->act, &m->grad})
-        for (float* p : *v) if (p) hipFree(p);
-    if (m->row_loss) hipFree(m->row_loss);
-    if (m->x_stage) hipFree(m->x_stage);
-    if (m->y_stage) hipFree(m->y_stage);
-    if (m->exec) hipGraphExecDestroy(m->exec);
+        for (float* p : *v) if (p) (void)hipFree(p);
+    if (m->row_loss) (void)hipFree(m->row_loss);
+    if (m->x_stage) (void)hipFree(m->x_stage);
+    if (m->y_stage) (void)hipFree(m->y_stage);
+    if (m->exec) (void)hipGraphExecDestroy(m->exec);
     delete m;
 }
 
@@ -1106,6 +1148,7 @@ static int mlp_forward(tenmo_mlp* m, const float* x, int64_t B) {
 int tenmo_hip_mlp_forward(tenmo_mlp* m, const float* x, int64_t B, float* logits_out, int32_t sync) {
     if (int rc = ensure_ready()) return rc;
     if (!m || B < 1 || B > m->max_batch) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_mlp_forward: batch outside 1..max_batch");
+    if (!x || !logits_out) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_mlp_forward: null pointer");
     if (int rc = mlp_forward(m, x, B)) return rc;
     HIP_TRY(hipMemcpyAsync(logits_out, m->act[m->L - 1], (size_t)B * m->dims[m->L] * 4, hipMemcpyDeviceToDevice, S.stream));
     return finish(sync);
@@ -1129,7 +1172,13 @@ static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int6
         const int64_t I = m->dims[l], O = m->dims[l + 1];
         const float* in = l == 0 ? x : m->act[l - 1];
         const float* gl = m->grad[l];
-        if (!(one_block && l == L - 1)) hipLaunchKernelGGL(column_sum_kernel, dim3((unsigned)((O + 63) / 64)), dim3(64), 0, S.stream, gl, B, O, m->db[l]);
+        if (one_block && l == L - 1) {
+            // done by the cross-entropy launch
+        } else if (B * O >= (int64_t)1 << 18) { // large: stream the gradient once at HBM rate
+            if (int rc = matvec_dispatch(gl, 1, O, S.one, 0, m->db[l], O, B, bd, 1, 0)) return rc;
+        } else {
+            hipLaunchKernelGGL(column_sum_kernel, dim3((unsigned)((O + 63) / 64)), dim3(64), 0, S.stream, gl, B, O, m->db[l]);
+        }
         // dW = in^T(view) . g        (tenmo/matmul.mojo:46-48)
         if (int rc = gemm_dispatch(in, 1, I, gl, O, 1, m->dW[l], I, O, B, bd, 1, 0)) return rc;
         if (l > 0) { // dX = g . W^T(view)  (tenmo/matmul.mojo:36-38); the network input needs no gradient (:34)
@@ -1156,6 +1205,7 @@ static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int6
 int tenmo_hip_mlp_step(tenmo_mlp* m, const float* x, const int32_t* y, int64_t B, float lr, float* loss_out, int32_t sync) {
     if (int rc = ensure_ready()) return rc;
     if (!m || B < 1 || B > m->max_batch) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_mlp_step: batch outside 1..max_batch");
+    if (!x || !y || !loss_out) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_mlp_step: null pointer");
     if (int rc = mlp_step_enqueue(m, x, y, B, lr, loss_out)) return rc;
     return finish(sync);
 }
@@ -1163,24 +1213,26 @@ int tenmo_hip_mlp_step(tenmo_mlp* m, const float* x, const int32_t* y, int64_t B
 int tenmo_hip_mlp_step_graph(tenmo_mlp* m, const float* x, const int32_t* y, int64_t B, float lr, float* loss_out, int32_t sync) {
     if (int rc = ensure_ready()) return rc;
     if (!m || B < 1 || B > m->max_batch) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_mlp_step_graph: batch outside 1..max_batch");
+    if (!x || !y || !loss_out) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_mlp_step_graph: null pointer");
     if (S.stream == nullptr) return fail(TENMO_ERR_UNSUPPORTED, "tenmo_hip_mlp_step_graph: cannot capture on the null stream");
     // the captured kernels read fixed staging buffers; this step's inputs are copied in eagerly
     HIP_TRY(hipMemcpyAsync(m->x_stage, x, (size_t)B * m->dims[0] * 4, hipMemcpyDeviceToDevice, S.stream));
     HIP_TRY(hipMemcpyAsync(m->y_stage, y, (size_t)B * 4, hipMemcpyDeviceToDevice, S.stream));
-    if (!m->exec || m->g_batch != B || m->g_lr != lr || m->g_loss != loss_out) {
+    float* ws;
+    if (int rc = workspace(1, &ws)) return rc; // scratch must exist before capture: no allocation may happen inside it
+    // the captured kernels hold the scratch pointer: a capture made before the scratch buffer grew is stale
+    if (!m->exec || m->g_batch != B || m->g_lr != lr || m->g_loss != loss_out || m->g_ws != ws) {
         if (m->exec) { HIP_TRY(hipStreamSynchronize(S.stream)); HIP_TRY(hipGraphExecDestroy(m->exec)); m->exec = nullptr; }
-        float* ws;
-        if (int rc = workspace(1, &ws)) return rc; // scratch must exist before capture: no allocation may happen inside it
         HIP_TRY(hipStreamBeginCapture(S.stream, hipStreamCaptureModeThreadLocal));
         const int rc = mlp_step_enqueue(m, m->x_stage, m->y_stage, B, lr, loss_out);
         hipGraph_t graph = nullptr;
         const hipError_t e = hipStreamEndCapture(S.stream, &graph);
-        if (rc) { if (graph) hipGraphDestroy(graph); return rc; }
+        if (rc) { if (graph) (void)hipGraphDestroy(graph); return rc; }
         if (e != hipSuccess) return fail(TENMO_ERR_HIP, "hipStreamEndCapture failed: %s", hipGetErrorString(e));
         const hipError_t ei = hipGraphInstantiate(&m->exec, graph, nullptr, nullptr, 0);
-        hipGraphDestroy(graph);
+        (void)hipGraphDestroy(graph);
         if (ei != hipSuccess) { m->exec = nullptr; return fail(TENMO_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(ei)); }
-        m->g_batch = B; m->g_lr = lr; m->g_loss = loss_out;
+        m->g_batch = B; m->g_lr = lr; m->g_loss = loss_out; m->g_ws = ws;
     }
     HIP_TRY(hipGraphLaunch(m->exec, S.stream));
     return finish(sync);

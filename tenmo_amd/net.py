@@ -2,9 +2,9 @@
 
 ``Linear``        y = x.W + b with W stored [in, out] (tenmo/net.mojo:49-216, :91-97).  For matrix
                   inputs the bias is added in the GEMM store (one launch); for a vector input it
-                  is a rank-1 product on the GEMM entry (ones[rows,1] . b[1,out], accumulated),
-                  as is the bias gradient (db = ones[1,rows] . dY), so the layer never leaves
-                  ``libtenmo_hip.so``.
+                  is a rank-1 product on the GEMM entry (ones[rows,1] . b[1,out], accumulated).
+                  The bias gradient is the column sum of dY (one streaming pass), so the layer
+                  never leaves ``libtenmo_hip.so``.
 ``MLP``           the whole training step of examples/mnist.mojo:150-162 on the device:
                   Linear -> ReLU -> ... -> Linear -> CrossEntropyLoss(mean) -> backward -> SGD(lr).
 ``xavier_uniform``  U(+-sqrt(6/(in+out))) weights, zero bias (tenmo/net.mojo:87-114).
@@ -63,7 +63,6 @@ class Linear:
                 out.requires_grad = True
                 out.add_ancestry((Matmul2dBackward if xs.rank() == 2 else MatmulNdBackward).backward, xs, self.weight)
             rows = out.numels() // self.out_features
-            ones = torch.ones(rows, dtype=torch.float32, device="cuda") if self.training and self.bias.requires_grad else None
         else:
             out = Matmul.forward(xs, self.weight, track_grad=self.training, mode=mm, sync=False)
             # out += ones[rows,1] . b[1,out]  — Adder.forward with broadcasting (tenmo/addition.mojo:73-112)
@@ -79,8 +78,8 @@ class Linear:
                 updated = []
                 if bias.requires_grad:
                     g = bias.ensure_gradbox()
-                    check(L.tenmo_hip_gemm_f32(ones.data_ptr(), 0, rows, 1, output.gradbox.data_ptr(), 0, self.out_features, 1,
-                                               g.data_ptr(), 1, self.out_features, rows, 0, None, None, None, 1, 0))
+                    check(L.tenmo_hip_column_sum_f32(output.gradbox.data_ptr(), 0, self.out_features, rows, self.out_features,
+                                                     g.data_ptr(), 1, 0))
                     updated.append(bias)
                 if inner is not None:
                     updated += inner(output, retain_graph)

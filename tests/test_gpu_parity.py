@@ -145,6 +145,20 @@ def test_raw_abi_arguments(T):
     assert L.tenmo_hip_gemm_f32(p, 0, 4, 1, p, 0, 4, 1, p, 4, 4, 4, 1, None, None, None, 0, 0) == -3   # rank 1 without arrays
     assert L.tenmo_hip_set_tuning(b"no_such_knob", 1) == -3
     assert L.tenmo_hip_mv_f32(p, 0, 4, 1, p, 0, 1, p, -2, 4, 0, None, None, None, 0, 0) == -2
+    # null pointers are refused before anything is launched
+    assert L.tenmo_hip_mv_f32(p, 0, 4, 1, p, 0, 1, None, 4, 4, 0, None, None, None, 0, 0) == -3
+    assert L.tenmo_hip_mv_f32(None, 0, 4, 1, p, 0, 1, p, 4, 4, 0, None, None, None, 0, 0) == -3
+    assert L.tenmo_hip_vm_f32(p, 0, 1, p, 0, 4, 1, None, 4, 4, 0, None, None, None, 0, 0) == -3
+    assert L.tenmo_hip_dot_f32(p, 0, 1, p, 0, 1, 4, None, 0) == -3
+    assert L.tenmo_hip_dot_f32(None, 0, 1, p, 0, 1, 4, p, 0) == -3
+    assert L.tenmo_hip_gemm_f32(p, 0, 4, 1, p, 0, 4, 1, None, 4, 4, 0, 0, None, None, None, 0, 0) == -3  # K = 0 still writes C
+    v = lib.make_view(p, 0, (4, 4), (4, 1))
+    nv = lib.make_view(None, 0, (4, 4), (4, 1))
+    import ctypes as C
+    assert L.tenmo_hip_matmul_nd(C.byref(v), C.byref(v), None, 0) == -3
+    assert L.tenmo_hip_matmul_nd(C.byref(nv), C.byref(v), p, 0) == -3
+    assert L.tenmo_hip_matrix_vector_nd(C.byref(v), C.byref(lib.make_view(p, 0, (4,), (1,))), None, 0) == -3
+    assert L.tenmo_hip_matmul_backward(C.byref(v), C.byref(v), None, p, p, 0) == -3
     # a zero-sized problem is a no-op that succeeds
     assert L.tenmo_hip_gemm_f32(p, 0, 4, 1, p, 0, 4, 1, p, 0, 4, 4, 0, None, None, None, 0, 1) == 0
     # explicit batch arrays: C[b] = A[b] . B (B broadcast with stride 0), accumulate twice doubles
@@ -234,6 +248,27 @@ def test_fused_epilogue(T, tile):
     finally:
         L.tenmo_hip_set_tuning(b"gemm_tile", -1)
         L.tenmo_hip_set_tuning(b"gemm_splitk", -1)
+
+
+def test_column_sum(T):
+    """Bias gradient = column sums of the upstream gradient (tenmo/broadcast.mojo:81-87): small, ragged,
+    padded rows, accumulate, and a size that takes the K-sliced streaming path."""
+    L, lib = T.lib.load(), T.lib
+    rng = np.random.default_rng(37)
+    for rows, cols, pitch in [(1, 1, 1), (3, 5, 5), (64, 10, 10), (300, 77, 80), (8192, 2304, 2304), (4096, 1000, 1003)]:
+        g = rng.standard_normal((rows, pitch), dtype=np.float32)
+        G = T.Tensor.from_numpy(g)
+        out = T.Tensor.from_numpy(np.ones(cols, np.float32))
+        lib.check(L.tenmo_hip_column_sum_f32(G.buffer.data_ptr(), 0, pitch, rows, cols, out.buffer.data_ptr(), 0, 1))
+        ref = g[:, :cols].astype(np.float64).sum(axis=0)
+        assert rel_fro(out.to_numpy(), ref) <= RTOL_FRO, (rows, cols, pitch)
+        lib.check(L.tenmo_hip_column_sum_f32(G.buffer.data_ptr(), 0, pitch, rows, cols, out.buffer.data_ptr(), 1, 1))
+        assert rel_fro(out.to_numpy(), 2 * ref) <= RTOL_FRO, (rows, cols, pitch, "accumulate")
+    assert L.tenmo_hip_column_sum_f32(None, 0, 4, 4, 4, None, 0, 1) == -3
+    assert L.tenmo_hip_column_sum_f32(None, 0, 4, 0, 4, None, 0, 1) == -3     # an empty sum still writes zeros
+    out = T.Tensor.from_numpy(np.ones(4, np.float32))
+    assert L.tenmo_hip_column_sum_f32(None, 0, 4, 0, 4, out.buffer.data_ptr(), 0, 1) == 0
+    assert np.all(out.to_numpy() == 0)
 
 
 def test_odd_strides_and_overlap(T, oracle):
