@@ -180,6 +180,34 @@ int tenmo_hip_mv_backward(const tenmo_view* Mx, const tenmo_view* v, const float
 int tenmo_hip_vm_backward(const tenmo_view* v, const tenmo_view* Mx, const float* dy,
                           float* grad_v, float* grad_M, int32_t sync);
 
+/* ---- adjacent operators of the training step ------------------------------------------------ */
+
+/* CrossEntropyFusedKernel.launch — tenmo/kernels/crossentropy_fused_kernel.mojo:285-391 (CPU form:
+ * tenmo/crossentropy.mojo:285-432): class-index cross-entropy of logits [M, C] (dense) against
+ * target [M] (int64 when target_is_int64, else int32), with ignore_index and label smoothing.
+ * Writes softmax_out [M, C] (may be NULL when no gradient is needed), per_sample_loss [M]
+ * (0 for ignored rows), loss_sum [1] = their sum and valid_count [1] = rows not ignored — all
+ * DEVICE pointers; the mean is loss_sum / valid_count as in crossentropy.mojo:1022-1024.
+ * The sum is formed in a fixed order (the reference's kernel uses atomics). */
+int tenmo_hip_cross_entropy_forward_f32(const float* logits, const void* target, int32_t target_is_int64,
+                                        int64_t M, int64_t C, int64_t ignore_index, float label_smoothing,
+                                        float* softmax_out, float* per_sample_loss, float* loss_sum,
+                                        int32_t* valid_count, int32_t sync);
+/* CrossEntropyFusedKernel.launch_backward — crossentropy_fused_kernel.mojo:192-275, :439-540:
+ * grad[m,c] = (softmax[m,c] - (1-ls)*onehot[m,c] - ls/C) * [target[m] != ignore_index] * scale[m];
+ * reduction 0 (none): scale = upstream[m]; 1 (sum): upstream[0]; 2 (mean): upstream[0] /
+ * max(valid_count, 1).  upstream is a DEVICE pointer.  accumulate != 0 adds into grad_logits (the
+ * Gradbox +=) instead of overwriting it. */
+int tenmo_hip_cross_entropy_backward_f32(const float* softmax, const void* target, int32_t target_is_int64,
+                                         const float* upstream, int64_t M, int64_t C, int64_t ignore_index,
+                                         float label_smoothing, int32_t reduction, int32_t valid_count,
+                                         float* grad_logits, int32_t accumulate, int32_t sync);
+/* SGDStep.launch_no_momentum / launch_momentum — tenmo/kernels/sgd_kernel.mojo:56-143 (CPU form:
+ * tenmo/optim.mojo:93-160): g += weight_decay * p when weight_decay > 0; with velocity != NULL
+ * v = momentum * v + g, p -= lr * v; else p -= lr * g. */
+int tenmo_hip_sgd_step_f32(float* param, const float* grad, float* velocity, int64_t n,
+                           float lr, float momentum, float weight_decay, int32_t sync);
+
 /* ---- the reference's existing plugin ABI --------------------------------------------------- */
 
 /* Exact CBLAS prototype the reference binds with

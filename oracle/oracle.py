@@ -84,6 +84,9 @@ def lib():
         L.oracle_mlp_forward.argtypes = [C.c_void_p, fp, C.c_int64, fp, C.c_int]
         L.oracle_mlp_get_params.argtypes = [C.c_void_p, C.c_int, fp, fp]
         L.oracle_mlp_get_grads.argtypes = [C.c_void_p, C.c_int, fp, fp]
+        L.oracle_cross_entropy_forward_f32.argtypes = [fp, i64p, C.c_int64, C.c_int64, C.c_int64, C.c_float, fp, fp, fp, i32p]
+        L.oracle_cross_entropy_backward_f32.argtypes = [fp, i64p, fp, C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_int, C.c_int32, fp]
+        L.oracle_sgd_step_f32.argtypes = [fp, fp, fp, C.c_int64, C.c_float, C.c_float, C.c_float]
         _lib = L
     return _lib
 
@@ -344,3 +347,45 @@ class MLP:
         b = np.empty((self.dims[layer + 1],), np.float32)
         _check(lib().oracle_mlp_get_grads(self._h, layer, W.ctypes.data, b.ctypes.data))
         return W, b
+
+
+REDUCTION_NONE, REDUCTION_SUM, REDUCTION_MEAN = 0, 1, 2
+
+
+def cross_entropy_forward(logits: np.ndarray, target: np.ndarray, ignore_index: int = -100, label_smoothing: float = 0.0):
+    """(softmax [M,C], per-sample loss [M], loss sum, valid count) — tenmo/crossentropy.mojo:285-432."""
+    logits = np.ascontiguousarray(logits, np.float32)
+    target = np.ascontiguousarray(target, np.int64)
+    M, Cn = logits.shape
+    sm = np.empty((M, Cn), np.float32)
+    rows = np.empty(M, np.float32)
+    total = np.zeros(1, np.float32)
+    valid = np.zeros(1, np.int32)
+    _check(lib().oracle_cross_entropy_forward_f32(logits.ctypes.data_as(C.POINTER(C.c_float)), target.ctypes.data_as(C.POINTER(C.c_int64)),
+                                                  M, Cn, ignore_index, label_smoothing,
+                                                  sm.ctypes.data_as(C.POINTER(C.c_float)), rows.ctypes.data_as(C.POINTER(C.c_float)),
+                                                  total.ctypes.data_as(C.POINTER(C.c_float)), valid.ctypes.data_as(C.POINTER(C.c_int32))))
+    return sm, rows, float(total[0]), int(valid[0])
+
+
+def cross_entropy_backward(softmax: np.ndarray, target: np.ndarray, upstream: np.ndarray, reduction: int, valid_count: int,
+                           ignore_index: int = -100, label_smoothing: float = 0.0) -> np.ndarray:
+    """Gradient with respect to the logits — tenmo/crossentropy.mojo:744-770, :451-481."""
+    softmax = np.ascontiguousarray(softmax, np.float32)
+    target = np.ascontiguousarray(target, np.int64)
+    upstream = np.ascontiguousarray(np.atleast_1d(upstream), np.float32)
+    M, Cn = softmax.shape
+    grad = np.empty((M, Cn), np.float32)
+    _check(lib().oracle_cross_entropy_backward_f32(softmax.ctypes.data_as(C.POINTER(C.c_float)), target.ctypes.data_as(C.POINTER(C.c_int64)),
+                                                   upstream.ctypes.data_as(C.POINTER(C.c_float)), M, Cn, ignore_index, label_smoothing,
+                                                   reduction, valid_count, grad.ctypes.data_as(C.POINTER(C.c_float))))
+    return grad
+
+
+def sgd_step(param: np.ndarray, grad: np.ndarray, velocity: Optional[np.ndarray], lr: float, momentum: float = 0.0,
+             weight_decay: float = 0.0) -> None:
+    """In-place optimiser step on contiguous fp32 arrays — tenmo/optim.mojo:93-160."""
+    assert param.dtype == np.float32 and param.flags.c_contiguous and grad.dtype == np.float32
+    fpp = C.POINTER(C.c_float)
+    _check(lib().oracle_sgd_step_f32(param.ctypes.data_as(fpp), np.ascontiguousarray(grad).ctypes.data_as(fpp),
+                                     velocity.ctypes.data_as(fpp) if velocity is not None else None, param.size, lr, momentum, weight_decay))

@@ -575,4 +575,96 @@ int oracle_mlp_get_grads(oracle_mlp* m, int l, float* dW, float* db) {
     return 0;
 }
 
+// ---- class-index cross-entropy (tenmo/crossentropy.mojo:285-432) --------------------------------
+// Row loop with the reference's three passes: max, exp + sum_exp (+ sum of logits under label
+// smoothing), loss from the target's logit, then the softmax normalisation.  The row losses are
+// added in row order (scalar_loss += loss, :394); valid rows are those whose target differs from
+// ignore_index (:369-389).
+int oracle_cross_entropy_forward_f32(const float* logits, const int64_t* target, int64_t M, int64_t C, int64_t ignore_index,
+                                     float label_smoothing, float* softmax, float* per_sample_loss, float* loss_sum, int32_t* valid_count) {
+    if (M < 0 || C < 1) return fail("cross entropy needs M >= 0 and C >= 1");
+    if (!(label_smoothing >= 0.f && label_smoothing <= 1.f)) return fail("CrossEntropyLoss: label_smoothing must be in [0, 1]");
+    const bool has_ls = label_smoothing > 0.f;
+    float scalar_loss = 0.f;
+    int32_t valid = 0;
+    for (int64_t row = 0; row < M; ++row) {
+        const float* x = logits + row * C;
+        float max_val = -std::numeric_limits<float>::max();          // min_finite, :332
+        for (int64_t c = 0; c < C; ++c) max_val = std::max(max_val, x[c]);
+        float sum_exp = 0.f, sum_logits = 0.f;
+        for (int64_t c = 0; c < C; ++c) {
+            const float e = std::exp(x[c] - max_val);
+            sum_exp += e;
+            if (has_ls) sum_logits += x[c];
+            if (softmax) softmax[row * C + c] = e;
+        }
+        const float log_sum_exp = std::log(std::max(sum_exp, 1e-7f)); // Epsilon[float32], :366-367
+        float loss = 0.f;
+        if (target[row] != ignore_index) {
+            const int64_t t = target[row];
+            if (t < 0 || t >= C) return fail("cross entropy: target index outside [0, C)"); // validated at :116-123
+            const float log_softmax_tgt = x[t] - max_val - log_sum_exp;
+            loss = -log_softmax_tgt;
+            if (has_ls) {
+                const float inv_C = 1.f / (float)C;
+                const float mean_log_softmax = sum_logits * inv_C - max_val - log_sum_exp;
+                loss = (1.f - label_smoothing) * loss - label_smoothing * mean_log_softmax;
+            }
+            ++valid;
+        }
+        if (per_sample_loss) per_sample_loss[row] = loss;
+        scalar_loss += loss;
+        if (softmax) {
+            const float inv = 1.f / sum_exp;
+            for (int64_t c = 0; c < C; ++c) softmax[row * C + c] *= inv;
+        }
+    }
+    if (loss_sum) *loss_sum = scalar_loss;
+    if (valid_count) *valid_count = valid;
+    return 0;
+}
+
+// Gradient with respect to the logits (tenmo/crossentropy.mojo:744-770 with scale_grad_by_upstream
+// :451-481): (softmax - (1-ls)*onehot - ls/C) * ignore_mask * upstream / (valid_count for mean).
+// reduction: 0 none (upstream has M entries), 1 sum, 2 mean.
+int oracle_cross_entropy_backward_f32(const float* softmax, const int64_t* target, const float* upstream, int64_t M, int64_t C,
+                                      int64_t ignore_index, float label_smoothing, int reduction, int32_t valid_count, float* grad) {
+    if (reduction < 0 || reduction > 2) return fail("reduction must be 0, 1 or 2");
+    const float ls = label_smoothing;
+    const float ls_uniform = ls / (float)C;
+    for (int64_t row = 0; row < M; ++row) {
+        const bool valid = target[row] != ignore_index;
+        float scale;
+        if (reduction == 0) scale = upstream[row];
+        else scale = upstream[0] / (float)((reduction == 2 && valid_count > 0) ? valid_count : 1);
+        for (int64_t c = 0; c < C; ++c) {
+            const float onehot = (valid && c == target[row]) ? 1.f : 0.f;
+            float g = softmax[row * C + c];
+            if (ls > 0.f) g = (g - onehot * (1.f - ls)) - ls_uniform;
+            else g = g - onehot;
+            g = g * (valid ? 1.f : 0.f);
+            grad[row * C + c] = g * scale;
+        }
+    }
+    return 0;
+}
+
+// One SGD step on one tensor (tenmo/optim.mojo:93-160): g += weight_decay * p when weight_decay > 0;
+// with a velocity buffer v = momentum * v + g and p -= lr * v, otherwise p -= lr * g.
+int oracle_sgd_step_f32(float* param, const float* grad, float* velocity, int64_t n, float lr, float momentum, float weight_decay) {
+    for (int64_t i = 0; i < n; ++i) {
+        const float p = param[i];
+        float g = grad[i];
+        if (weight_decay > 0.f) g += p * weight_decay;
+        if (velocity) {
+            const float v = momentum * velocity[i] + g;
+            velocity[i] = v;
+            param[i] = p - lr * v;
+        } else {
+            param[i] = p - lr * g;
+        }
+    }
+    return 0;
+}
+
 } // extern "C"

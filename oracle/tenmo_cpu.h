@@ -91,6 +91,15 @@ int oracle_mlp_get_params(oracle_mlp*, int layer, float* W, float* b);
 /* last step's parameter gradients */
 int oracle_mlp_get_grads(oracle_mlp*, int layer, float* dW, float* db);
 
+/* class-index cross-entropy, tenmo/crossentropy.mojo:285-432 (forward) and :744-770, :451-481
+ * (gradient); reduction 0 none, 1 sum, 2 mean */
+int oracle_cross_entropy_forward_f32(const float* logits, const int64_t* target, int64_t M, int64_t C, int64_t ignore_index,
+                                     float label_smoothing, float* softmax, float* per_sample_loss, float* loss_sum, int32_t* valid_count);
+int oracle_cross_entropy_backward_f32(const float* softmax, const int64_t* target, const float* upstream, int64_t M, int64_t C,
+                                      int64_t ignore_index, float label_smoothing, int reduction, int32_t valid_count, float* grad);
+/* SGD step, tenmo/optim.mojo:93-160 */
+int oracle_sgd_step_f32(float* param, const float* grad, float* velocity, int64_t n, float lr, float momentum, float weight_decay);
+
 #ifdef __cplusplus
 }
 #endif

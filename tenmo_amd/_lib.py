@@ -76,6 +76,11 @@ SIGNATURES = {
     "tenmo_hip_matmul_backward": (C.c_int, [_vp, _vp, _ptr, _ptr, _ptr, C.c_int32]),
     "tenmo_hip_mv_backward": (C.c_int, [_vp, _vp, _ptr, _ptr, _ptr, C.c_int32]),
     "tenmo_hip_vm_backward": (C.c_int, [_vp, _vp, _ptr, _ptr, _ptr, C.c_int32]),
+    "tenmo_hip_cross_entropy_forward_f32": (C.c_int, [_ptr, _ptr, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_float,
+                                                      _ptr, _ptr, _ptr, _ptr, C.c_int32]),
+    "tenmo_hip_cross_entropy_backward_f32": (C.c_int, [_ptr, _ptr, C.c_int32, _ptr, C.c_int64, C.c_int64, C.c_int64, C.c_float,
+                                                       C.c_int32, C.c_int32, _ptr, C.c_int32, C.c_int32]),
+    "tenmo_hip_sgd_step_f32": (C.c_int, [_ptr, _ptr, _ptr, C.c_int64, C.c_float, C.c_float, C.c_float, C.c_int32]),
     "cblas_sgemm": (None, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, _ptr, C.c_int,
                            _ptr, C.c_int, C.c_float, _ptr, C.c_int]),
     "tenmo_hip_mlp_create": (C.c_void_p, [C.c_int32, _i64p, C.POINTER(C.c_void_p), C.POINTER(C.c_void_p), C.c_int64]),

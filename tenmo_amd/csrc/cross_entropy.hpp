@@ -1,0 +1,340 @@
+// Fused class-index cross-entropy for gfx950: softmax, per-row loss (label smoothing, ignore_index),
+// loss sum / valid count, and the gradient with respect to the logits.
+//
+// Replaces the two launches of CrossEntropyFusedKernel
+// (tenmo/kernels/crossentropy_fused_kernel.mojo:39-160 forward, :192-275 backward; the CPU form of the
+// same arithmetic is tenmo/crossentropy.mojo:285-432 and :744-770).  Both are HBM-bound: the forward
+// keeps a row of up to 65533 classes in registers, so it reads the logits once and writes the softmax
+// once (longer rows take three passes); the backward reads the softmax and writes the gradient.
+//
+//   forward, per row m:  mx = max_c x[c];  S = sum_c exp(x[c]-mx);  lse = log(S)
+//                        loss = -(x[t]-mx-lse)                                    t = target[m] != ignore_index
+//                        loss = (1-ls)*loss - ls*(sum_c x[c]/C - mx - lse)        with label smoothing ls > 0
+//                        loss = 0                                                 t == ignore_index
+//                        softmax[c] = exp(x[c]-mx)/S
+//   backward:            g[c] = softmax[c] - (1-ls)*[c==t] - ls/C   (0 for an ignored row), times
+//                        upstream[m] (reduction none), upstream[0] (sum), upstream[0]/max(valid,1) (mean)
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+namespace tenmo {
+
+constexpr int CE_THREADS = 256;
+constexpr float CE_MAX_INIT = -3.402823466e+38f; // the reference's MAX_INIT
+
+struct CeForwardArgs {
+    const float* logits;  // [M, C] dense
+    const void* target;   // [M] int64 or int32 class indices
+    float* softmax_out;   // [M, C] or null (no gradient tracked)
+    float* row_loss;      // [M]
+    int64_t M, C;
+    int64_t ignore_index;
+    float label_smoothing;
+};
+
+template <typename IdxT>
+__device__ __forceinline__ float ce_row_loss(const float* __restrict x, const IdxT* __restrict target, int64_t row, int64_t C,
+                                             int64_t ignore_index, float ls, float mx, float lse, float sum_logits) {
+    const int64_t t = (int64_t)target[row];
+    if (t == ignore_index) return 0.f;
+    // the reference validates the indices on the host (crossentropy.mojo:116-123); an index that
+    // slipped through must not become an out-of-bounds read
+    if (t < 0 || t >= C) return __builtin_nanf("");
+    float loss = -((x[t] - mx) - lse);
+    if (ls > 0.f) {
+        const float mean_log_softmax = sum_logits * (1.f / (float)C) - mx - lse;
+        loss = (1.f - ls) * loss - ls * mean_log_softmax;
+    }
+    return loss;
+}
+
+// Few classes: one thread per row (the rows are too short to share).
+template <typename IdxT>
+__global__ void ce_forward_rows_kernel(const CeForwardArgs a) {
+    const int64_t row = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (row >= a.M) return;
+    const float* __restrict x = a.logits + row * a.C;
+    float mx = CE_MAX_INIT;
+    for (int64_t c = 0; c < a.C; ++c) mx = fmaxf(mx, x[c]);
+    float s = 0.f, sl = 0.f;
+    for (int64_t c = 0; c < a.C; ++c) { s += expf(x[c] - mx); sl += x[c]; }
+    const float lse = logf(s);
+    a.row_loss[row] = ce_row_loss(x, (const IdxT*)a.target, row, a.C, a.ignore_index, a.label_smoothing, mx, lse, sl);
+    if (a.softmax_out) {
+        float* __restrict p = a.softmax_out + row * a.C;
+        const float inv = 1.f / s;
+        for (int64_t c = 0; c < a.C; ++c) p[c] = expf(x[c] - mx) * inv;
+    }
+}
+
+__device__ __forceinline__ float ce_wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+__device__ __forceinline__ float ce_wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// One workgroup per row.  VEC: the row starts on a 16-byte boundary and C % 4 == 0.
+template <typename IdxT, bool VEC>
+__global__ __launch_bounds__(CE_THREADS) void ce_forward_block_kernel(const CeForwardArgs a) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    __shared__ float red[CE_THREADS / 64];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    for (int64_t row = blockIdx.x; row < a.M; row += gridDim.x) {
+        const float* __restrict x = a.logits + row * a.C;
+        const int64_t C = a.C;
+        // ---- max ----
+        float mx = CE_MAX_INIT;
+        if constexpr (VEC) {
+            const f4* __restrict x4 = reinterpret_cast<const f4*>(x);
+            for (int64_t i = tid; i < C / 4; i += CE_THREADS) {
+                const f4 v = x4[i];
+                mx = fmaxf(fmaxf(mx, fmaxf(v.x, v.y)), fmaxf(v.z, v.w));
+            }
+        } else {
+            for (int64_t c = tid; c < C; c += CE_THREADS) mx = fmaxf(mx, x[c]);
+        }
+        mx = ce_wave_max(mx);
+        if (lane == 0) red[wave] = mx;
+        __syncthreads();
+        mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+        __syncthreads();
+        // ---- sum of exp (and of the logits, for label smoothing) ----
+        float s = 0.f, sl = 0.f;
+        if constexpr (VEC) {
+            const f4* __restrict x4 = reinterpret_cast<const f4*>(x);
+            for (int64_t i = tid; i < C / 4; i += CE_THREADS) {
+                const f4 v = x4[i];
+                s += (expf(v.x - mx) + expf(v.y - mx)) + (expf(v.z - mx) + expf(v.w - mx));
+                sl += (v.x + v.y) + (v.z + v.w);
+            }
+        } else {
+            for (int64_t c = tid; c < C; c += CE_THREADS) { const float v = x[c]; s += expf(v - mx); sl += v; }
+        }
+        s = ce_wave_sum(s);
+        if (lane == 0) red[wave] = s;
+        __syncthreads();
+        s = (red[0] + red[1]) + (red[2] + red[3]);
+        __syncthreads();
+        sl = ce_wave_sum(sl);
+        if (lane == 0) red[wave] = sl;
+        __syncthreads();
+        sl = (red[0] + red[1]) + (red[2] + red[3]);
+        __syncthreads();
+        const float lse = logf(s);
+        if (tid == 0)
+            a.row_loss[row] = ce_row_loss(x, (const IdxT*)a.target, row, C, a.ignore_index, a.label_smoothing, mx, lse, sl);
+        // ---- softmax ----
+        if (a.softmax_out) {
+            float* __restrict p = a.softmax_out + row * C;
+            const float inv = 1.f / s;
+            if constexpr (VEC) {
+                const f4* __restrict x4 = reinterpret_cast<const f4*>(x);
+                f4* __restrict p4 = reinterpret_cast<f4*>(p);
+                for (int64_t i = tid; i < C / 4; i += CE_THREADS) {
+                    const f4 v = x4[i];
+                    f4 o = {expf(v.x - mx) * inv, expf(v.y - mx) * inv, expf(v.z - mx) * inv, expf(v.w - mx) * inv};
+                    p4[i] = o;
+                }
+            } else {
+                for (int64_t c = tid; c < C; c += CE_THREADS) p[c] = expf(x[c] - mx) * inv;
+            }
+        }
+    }
+}
+
+// One workgroup per row with the whole row held in registers: the logits are read once and the
+// softmax written once (the algorithmic minimum).  THREADS * EPT >= C + 3.
+// VEC: logits and softmax_out are congruent modulo 16 bytes, so a row of either starts the same
+// number m of elements past a 16-byte boundary.  The row is then walked in aligned groups of four
+// counted from that boundary: groups that lie wholly inside the row move as one 16-byte access, the
+// (at most two) groups that straddle its ends element by element — nothing outside the row is touched.
+template <typename IdxT, int THREADS, int EPT, bool VEC>
+__global__ __launch_bounds__(THREADS) void ce_forward_regs_kernel(const CeForwardArgs a) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    constexpr int WAVES = THREADS / 64;
+    __shared__ float red[3][WAVES];
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int C = (int)a.C; // <= THREADS * EPT - 3
+    for (int64_t row = blockIdx.x; row < a.M; row += gridDim.x) {
+        const float* __restrict x = a.logits + row * C;
+        const int m = VEC ? (int)(((uintptr_t)x >> 2) & 3) : 0;
+        const int span = C + m;            // elements from the aligned origin to the end of the row
+        // the row elements outside whole aligned groups: `head` at the front, `tail` at the back
+        const int head = m ? 4 - m : 0, tail = span & 3;
+        const int extra_n = VEC ? (tid == 0 ? head : tid == 1 ? tail : 0) : 0;
+        const int extra_at = tid == 0 ? 0 : C - tail;
+        float v[EPT], ex[3];
+        float mx = CE_MAX_INIT, sl = 0.f;
+        if constexpr (VEC) {
+            const f4* __restrict x4 = reinterpret_cast<const f4*>(x - m);
+#pragma unroll
+            for (int j = 0; j < EPT / 4; ++j) {
+                const int g = tid + THREADS * j; // aligned group number
+                f4 t = {CE_MAX_INIT, CE_MAX_INIT, CE_MAX_INIT, CE_MAX_INIT};
+                if (4 * g >= m && 4 * g + 4 <= span) { t = x4[g]; sl += (t.x + t.y) + (t.z + t.w); }
+                v[4 * j] = t.x; v[4 * j + 1] = t.y; v[4 * j + 2] = t.z; v[4 * j + 3] = t.w;
+                mx = fmaxf(fmaxf(mx, fmaxf(t.x, t.y)), fmaxf(t.z, t.w));
+            }
+#pragma unroll
+            for (int e = 0; e < 3; ++e) {
+                ex[e] = CE_MAX_INIT;
+                if (e < extra_n) { ex[e] = x[extra_at + e]; sl += ex[e]; }
+                mx = fmaxf(mx, ex[e]);
+            }
+        } else {
+#pragma unroll
+            for (int j = 0; j < EPT; ++j) {
+                const int c = tid + THREADS * j;
+                float q = CE_MAX_INIT;
+                if (c < C) { q = x[c]; sl += q; }
+                v[j] = q;
+                mx = fmaxf(mx, q);
+            }
+#pragma unroll
+            for (int e = 0; e < 3; ++e) ex[e] = CE_MAX_INIT;
+        }
+        mx = ce_wave_max(mx);
+        sl = ce_wave_sum(sl);
+        if (lane == 0) { red[0][wave] = mx; red[1][wave] = sl; }
+        __syncthreads();
+        mx = red[0][0]; sl = red[1][0];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) { mx = fmaxf(mx, red[0][w]); sl += red[1][w]; }
+        // empty slots hold -FLT_MAX: their exponential is exactly 0
+        float s = 0.f;
+#pragma unroll
+        for (int j = 0; j < EPT; ++j) { v[j] = expf(v[j] - mx); s += v[j]; }
+#pragma unroll
+        for (int e = 0; e < 3; ++e) { ex[e] = expf(ex[e] - mx); s += ex[e]; }
+        s = ce_wave_sum(s);
+        if (lane == 0) red[2][wave] = s;
+        __syncthreads();
+        s = red[2][0];
+#pragma unroll
+        for (int w = 1; w < WAVES; ++w) s += red[2][w];
+        __syncthreads(); // red is reused by the next row
+        if (tid == 0)
+            a.row_loss[row] = ce_row_loss(x, (const IdxT*)a.target, row, (int64_t)C, a.ignore_index, a.label_smoothing, mx, logf(s), sl);
+        if (a.softmax_out) {
+            float* __restrict p = a.softmax_out + row * C;
+            const float inv = 1.f / s;
+            if constexpr (VEC) {
+                f4* __restrict p4 = reinterpret_cast<f4*>(p - m);
+#pragma unroll
+                for (int j = 0; j < EPT / 4; ++j) {
+                    const int g = tid + THREADS * j;
+                    if (4 * g >= m && 4 * g + 4 <= span) {
+                        const f4 o = {v[4 * j] * inv, v[4 * j + 1] * inv, v[4 * j + 2] * inv, v[4 * j + 3] * inv};
+                        p4[g] = o;
+                    }
+                }
+#pragma unroll
+                for (int e = 0; e < 3; ++e)
+                    if (e < extra_n) p[extra_at + e] = ex[e] * inv;
+            } else {
+#pragma unroll
+                for (int j = 0; j < EPT; ++j) {
+                    const int c = tid + THREADS * j;
+                    if (c < C) p[c] = v[j] * inv;
+                }
+            }
+        }
+    }
+}
+
+// loss_sum = sum of the row losses, valid = number of rows whose target is not ignore_index.
+// One workgroup; every thread adds a contiguous run of rows in order and the partial sums are
+// combined in a fixed tree, so the result does not depend on scheduling (the reference's kernel
+// adds with atomics, crossentropy_fused_kernel.mojo:157-159; its CPU loop adds in row order).
+template <typename IdxT>
+__global__ __launch_bounds__(1024) void ce_finish_kernel(const float* __restrict row_loss, const IdxT* __restrict target, int64_t M,
+                                                         int64_t ignore_index, float* __restrict loss_sum, int32_t* __restrict valid) {
+    __shared__ float ps[1024];
+    __shared__ int pv[1024];
+    const int tid = threadIdx.x;
+    const int64_t per = (M + 1023) / 1024;
+    const int64_t lo = (int64_t)tid * per, hi = lo + per < M ? lo + per : M;
+    float s = 0.f;
+    int v = 0;
+    for (int64_t r = lo; r < hi; ++r) { s += row_loss[r]; v += ((int64_t)target[r] != ignore_index) ? 1 : 0; }
+    ps[tid] = s; pv[tid] = v;
+    __syncthreads();
+    for (int stride = 512; stride > 0; stride >>= 1) {
+        if (tid < stride) { ps[tid] += ps[tid + stride]; pv[tid] += pv[tid + stride]; }
+        __syncthreads();
+    }
+    if (tid == 0) { *loss_sum = ps[0]; *valid = pv[0]; }
+}
+
+struct CeBackwardArgs {
+    const float* softmax;  // [M, C]
+    const void* target;    // [M]
+    const float* upstream; // [M] for reduction none, [1] otherwise
+    float* grad;           // [M, C]
+    int64_t M, C;
+    int64_t ignore_index;
+    float label_smoothing;
+    int32_t reduction;     // 0 none, 1 sum, 2 mean (the reference kernel's encoding)
+    int32_t valid_count;
+    int32_t accumulate;    // grad += instead of grad =
+    int32_t chunks;        // workgroups per row
+};
+
+template <typename IdxT, bool VEC>
+__global__ __launch_bounds__(CE_THREADS) void ce_backward_kernel(const CeBackwardArgs a) {
+    const int64_t row = blockIdx.x / a.chunks;
+    const int chunk = blockIdx.x % a.chunks;
+    if (row >= a.M) return;
+    const int64_t t = (int64_t)((const IdxT*)a.target)[row];
+    const bool valid = t != a.ignore_index;
+    float scale = a.reduction == 0 ? a.upstream[row] : a.upstream[0];
+    if (a.reduction == 2) scale = scale / (float)(a.valid_count > 0 ? a.valid_count : 1);
+    const float ls = a.label_smoothing;
+    const bool has_ls = ls > 0.f;
+    const float ls_uniform = ls * (1.f / (float)a.C);
+    const float* __restrict sm = a.softmax + row * a.C;
+    float* __restrict g = a.grad + row * a.C;
+    auto value = [&](float p, int64_t c) {
+        float v = 0.f;
+        if (valid) {
+            v = p;
+            if (c == t) { v = v - 1.f; if (has_ls) v = v + ls; }
+            if (has_ls) v = v - ls_uniform;
+        }
+        return v * scale;
+    };
+    if constexpr (VEC) { // softmax and grad congruent modulo 16 bytes: aligned groups of four, as in the forward
+        typedef float f4 __attribute__((ext_vector_type(4)));
+        const int m = (int)(((uintptr_t)sm >> 2) & 3);
+        const int64_t span = a.C + m;
+        const f4* __restrict sm4 = reinterpret_cast<const f4*>(sm - m);
+        f4* __restrict g4 = reinterpret_cast<f4*>(g - m);
+        for (int64_t i = (int64_t)chunk * CE_THREADS + threadIdx.x; 4 * i < span; i += (int64_t)a.chunks * CE_THREADS) {
+            const int64_t e0 = 4 * i;
+            if (e0 >= m && e0 + 4 <= span) {
+                const f4 p = sm4[i];
+                f4 o = {value(p.x, e0 - m), value(p.y, e0 - m + 1), value(p.z, e0 - m + 2), value(p.w, e0 - m + 3)};
+                if (a.accumulate) o += g4[i];
+                g4[i] = o;
+            } else {
+                for (int e = 0; e < 4; ++e) {
+                    const int64_t c = e0 + e - m;
+                    if (c >= 0 && c < a.C) { const float v = value(sm[c], c); g[c] = a.accumulate ? g[c] + v : v; }
+                }
+            }
+        }
+    } else {
+        for (int64_t c = (int64_t)chunk * CE_THREADS + threadIdx.x; c < a.C; c += (int64_t)a.chunks * CE_THREADS) {
+            const float v = value(sm[c], c);
+            g[c] = a.accumulate ? g[c] + v : v;
+        }
+    }
+}
+
+} // namespace tenmo

@@ -163,4 +163,50 @@ __global__ void sgd_multi_kernel(const SgdArgs a, float lr) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = p[i] - lr * g[i];
 }
 
+// One optimiser step on one tensor, with the options of the reference's two SGD kernels
+// (tenmo/kernels/sgd_kernel.mojo:8-26 without, :29-53 with momentum): g += wd * p when wd > 0;
+// with a velocity buffer v = momentum * v + g and p -= lr * v, else p -= lr * g.
+__device__ __forceinline__ void sgd_update(float& p, float g, float* v, float lr, float momentum, float weight_decay) {
+    if (weight_decay > 0.f) g += p * weight_decay;
+    if (v) {
+        *v = momentum * *v + g;
+        p = p - lr * *v;
+    } else {
+        p = p - lr * g;
+    }
+}
+// VEC: all three arrays start on 16-byte boundaries; the tail of n % 4 elements is done by thread 0
+template <bool VEC>
+__global__ void sgd_step_kernel(float* __restrict p, const float* __restrict g, float* __restrict vel, int64_t n, float lr, float momentum, float weight_decay) {
+    const int64_t tid = (int64_t)blockIdx.x * blockDim.x + threadIdx.x, stride = (int64_t)gridDim.x * blockDim.x;
+    if constexpr (VEC) {
+        typedef float f4 __attribute__((ext_vector_type(4)));
+        f4* __restrict p4 = reinterpret_cast<f4*>(p);
+        const f4* __restrict g4 = reinterpret_cast<const f4*>(g);
+        f4* __restrict v4 = reinterpret_cast<f4*>(vel);
+        for (int64_t i = tid; i < n / 4; i += stride) {
+            const f4 pp = p4[i], gg = g4[i];
+            float pa[4] = {pp.x, pp.y, pp.z, pp.w};
+            const float ga[4] = {gg.x, gg.y, gg.z, gg.w};
+            if (vel) {
+                const f4 vv = v4[i];
+                float va[4] = {vv.x, vv.y, vv.z, vv.w};
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sgd_update(pa[e], ga[e], &va[e], lr, momentum, weight_decay);
+                const f4 vo = {va[0], va[1], va[2], va[3]};
+                v4[i] = vo;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 4; ++e) sgd_update(pa[e], ga[e], nullptr, lr, momentum, weight_decay);
+            }
+            const f4 po = {pa[0], pa[1], pa[2], pa[3]};
+            p4[i] = po;
+        }
+        if (tid == 0)
+            for (int64_t i = n / 4 * 4; i < n; ++i) sgd_update(p[i], g[i], vel ? vel + i : nullptr, lr, momentum, weight_decay);
+    } else {
+        for (int64_t i = tid; i < n; i += stride) sgd_update(p[i], g[i], vel ? vel + i : nullptr, lr, momentum, weight_decay);
+    }
+}
+
 } // namespace tenmo

@@ -22,6 +22,7 @@
 #include <vector>
 
 #include "../../include/tenmo_hip.h"
+#include "cross_entropy.hpp"
 #include "elementwise.hpp"
 #include "gemm_mfma.hpp"
 #include "gemv.hpp"
@@ -604,6 +605,31 @@ bool same_batch(const Geometry& g, const tenmo_view* parent, int trailing) {
     return true;
 }
 
+// ---- cross-entropy forward: pick the kernel that reads a row once --------------------------------
+template <typename IdxT, bool VEC>
+void launch_ce_forward_t(const CeForwardArgs& a) {
+    const int64_t C = a.C, M = a.M;
+    // the row lives in registers: THREADS * EPT >= C, the smallest EPT that fits
+#define TENMO_CE_REGS(THREADS, EPT)                                                                                      \
+    if (C + 3 <= (int64_t)(THREADS) * (EPT)) {                                                                           \
+        const dim3 grid((unsigned)std::min<int64_t>(M, (int64_t)S.cus * (2048 / (THREADS)))), block(THREADS);             \
+        hipLaunchKernelGGL((ce_forward_regs_kernel<IdxT, THREADS, EPT, VEC>), grid, block, 0, S.stream, a);               \
+        return;                                                                                                          \
+    }
+    TENMO_CE_REGS(256, 4) TENMO_CE_REGS(256, 8) TENMO_CE_REGS(256, 16) TENMO_CE_REGS(256, 32)
+    TENMO_CE_REGS(1024, 16) TENMO_CE_REGS(1024, 32) TENMO_CE_REGS(1024, 64)
+#undef TENMO_CE_REGS
+    // longer rows: three passes over the row (16-byte accesses only when every row is aligned)
+    const dim3 grid((unsigned)std::min<int64_t>(M, (int64_t)S.cus * 8)), block(CE_THREADS);
+    if (VEC && C % 4 == 0 && (uintptr_t)a.logits % 16 == 0) hipLaunchKernelGGL((ce_forward_block_kernel<IdxT, true>), grid, block, 0, S.stream, a);
+    else hipLaunchKernelGGL((ce_forward_block_kernel<IdxT, false>), grid, block, 0, S.stream, a);
+}
+
+void launch_ce_forward(const CeForwardArgs& a, bool int64_target, bool vec) {
+    if (int64_target) { if (vec) launch_ce_forward_t<int64_t, true>(a); else launch_ce_forward_t<int64_t, false>(a); }
+    else { if (vec) launch_ce_forward_t<int32_t, true>(a); else launch_ce_forward_t<int32_t, false>(a); }
+}
+
 } // namespace
 
 // ================================================================================================
@@ -787,6 +813,78 @@ int tenmo_hip_column_sum_f32(const float* G, int64_t g_off, int64_t g_rs, int64_
     BatchDesc bd{};
     for (int d = 0; d < MAX_BATCH_RANK; ++d) bd.shape[d] = 1;
     if (int rc = matvec_dispatch(G + g_off, 1, g_rs, S.one, 0, out, cols, rows, bd, 1, accumulate)) return rc;
+    return finish(sync);
+}
+
+int tenmo_hip_cross_entropy_forward_f32(const float* logits, const void* target, int32_t target_is_int64, int64_t M, int64_t C,
+                                        int64_t ignore_index, float label_smoothing,
+                                        float* softmax_out, float* per_sample_loss, float* loss_sum, int32_t* valid_count, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    const char* who = "tenmo_hip_cross_entropy_forward_f32";
+    if (M < 0 || C < 1) return fail(TENMO_ERR_INVALID_SHAPE, "%s: needs M >= 0 rows and C >= 1 classes", who);
+    if (!(label_smoothing >= 0.f && label_smoothing <= 1.f))
+        return fail(TENMO_ERR_INVALID_ARGUMENT, "CrossEntropyLoss: label_smoothing must be in [0, 1], got %g", (double)label_smoothing);
+    if (int rc = need(loss_sum, true, who, "loss_sum")) return rc;
+    if (int rc = need(valid_count, true, who, "valid_count")) return rc;
+    if (M > 0 && (!logits || !target || !per_sample_loss)) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    if (M > 0) {
+        CeForwardArgs a{};
+        a.logits = logits; a.target = target; a.softmax_out = softmax_out; a.row_loss = per_sample_loss;
+        a.M = M; a.C = C; a.ignore_index = ignore_index; a.label_smoothing = label_smoothing;
+        if (C <= 32) { // short rows: a thread each
+            const dim3 grid((unsigned)((M + 127) / 128)), block(128);
+            if (target_is_int64) hipLaunchKernelGGL(ce_forward_rows_kernel<int64_t>, grid, block, 0, S.stream, a);
+            else hipLaunchKernelGGL(ce_forward_rows_kernel<int32_t>, grid, block, 0, S.stream, a);
+        } else {
+            // 16-byte accesses need the two arrays congruent modulo 16 bytes (then their rows are too)
+            const bool vec = (uintptr_t)logits % 4 == 0 && (!softmax_out || (uintptr_t)softmax_out % 16 == (uintptr_t)logits % 16);
+            launch_ce_forward(a, target_is_int64 != 0, vec);
+        }
+    }
+    if (target_is_int64) hipLaunchKernelGGL(ce_finish_kernel<int64_t>, dim3(1), dim3(1024), 0, S.stream, per_sample_loss, (const int64_t*)target, M, ignore_index, loss_sum, valid_count);
+    else hipLaunchKernelGGL(ce_finish_kernel<int32_t>, dim3(1), dim3(1024), 0, S.stream, per_sample_loss, (const int32_t*)target, M, ignore_index, loss_sum, valid_count);
+    return finish(sync);
+}
+
+int tenmo_hip_cross_entropy_backward_f32(const float* softmax, const void* target, int32_t target_is_int64, const float* upstream,
+                                         int64_t M, int64_t C, int64_t ignore_index, float label_smoothing,
+                                         int32_t reduction, int32_t valid_count, float* grad_logits, int32_t accumulate, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    const char* who = "tenmo_hip_cross_entropy_backward_f32";
+    if (M < 0 || C < 1) return fail(TENMO_ERR_INVALID_SHAPE, "%s: needs M >= 0 rows and C >= 1 classes", who);
+    if (reduction < 0 || reduction > 2) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: reduction must be 0 (none), 1 (sum) or 2 (mean)", who);
+    if (M == 0) return 0;
+    if (!softmax || !target || !upstream || !grad_logits) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    CeBackwardArgs a{};
+    a.softmax = softmax; a.target = target; a.upstream = upstream; a.grad = grad_logits;
+    a.M = M; a.C = C; a.ignore_index = ignore_index; a.label_smoothing = label_smoothing;
+    a.reduction = reduction; a.valid_count = valid_count; a.accumulate = accumulate ? 1 : 0;
+    // enough workgroups per row to fill the chip when there are few long rows
+    int64_t chunks = std::max<int64_t>(1, std::min<int64_t>((C + CE_THREADS * 8 - 1) / (CE_THREADS * 8), ((int64_t)S.cus * 8 + M - 1) / M));
+    if (M * chunks > 0x7fffffffLL) return fail(TENMO_ERR_UNSUPPORTED, "%s: grid too large", who);
+    a.chunks = (int32_t)chunks;
+    const dim3 grid((unsigned)(M * chunks)), block(CE_THREADS);
+    const bool vec = (uintptr_t)softmax % 4 == 0 && (uintptr_t)softmax % 16 == (uintptr_t)grad_logits % 16;
+    if (target_is_int64) {
+        if (vec) hipLaunchKernelGGL((ce_backward_kernel<int64_t, true>), grid, block, 0, S.stream, a);
+        else hipLaunchKernelGGL((ce_backward_kernel<int64_t, false>), grid, block, 0, S.stream, a);
+    } else {
+        if (vec) hipLaunchKernelGGL((ce_backward_kernel<int32_t, true>), grid, block, 0, S.stream, a);
+        else hipLaunchKernelGGL((ce_backward_kernel<int32_t, false>), grid, block, 0, S.stream, a);
+    }
+    return finish(sync);
+}
+
+int tenmo_hip_sgd_step_f32(float* param, const float* grad, float* velocity, int64_t n, float lr, float momentum, float weight_decay, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    if (n < 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_sgd_step_f32: negative length");
+    if (n == 0) return 0;
+    if (!param || !grad) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_sgd_step_f32: null pointer");
+    const bool vec = (uintptr_t)param % 16 == 0 && (uintptr_t)grad % 16 == 0 && (uintptr_t)velocity % 16 == 0;
+    const int64_t work = vec ? (n + 3) / 4 : n;
+    const dim3 grid((unsigned)std::max<int64_t>(1, std::min<int64_t>((work + 255) / 256, (int64_t)S.cus * 16))), block(256);
+    if (vec) hipLaunchKernelGGL(sgd_step_kernel<true>, grid, block, 0, S.stream, param, grad, velocity, n, lr, momentum, weight_decay);
+    else hipLaunchKernelGGL(sgd_step_kernel<false>, grid, block, 0, S.stream, param, grad, velocity, n, lr, momentum, weight_decay);
     return finish(sync);
 }
 

@@ -34,3 +34,20 @@ def rel_fro(x, ref):
 
 def ref_matmul64(a, b):
     return np.matmul(np.asarray(a, np.float64), np.asarray(b, np.float64))
+
+
+def ce_reference64(logits, target, ignore_index=-100, ls=0.0):
+    """Independent fp64 statement of class-index cross-entropy: per-row loss and d(sum of losses)/d logits."""
+    x = np.asarray(logits, np.float64)
+    M, C = x.shape
+    lse = np.log(np.exp(x - x.max(1, keepdims=True)).sum(1)) + x.max(1)
+    logp = x - lse[:, None]
+    p = np.exp(logp)
+    valid = np.asarray(target) != ignore_index
+    t = np.where(valid, target, 0)
+    nll = -logp[np.arange(M), t]
+    loss = np.where(valid, (1 - ls) * nll + ls * (-logp.mean(1)), 0.0)
+    onehot = np.zeros((M, C))
+    onehot[np.arange(M), t] = 1.0
+    grad = (p - (1 - ls) * onehot - ls / C) * valid[:, None]
+    return p, loss, grad

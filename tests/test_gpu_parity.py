@@ -9,7 +9,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from helpers import RTOL_FRO, numpy_view, ref_matmul64, rel_fro, storage_of, strides_of
+from helpers import RTOL_FRO, ce_reference64, numpy_view, ref_matmul64, rel_fro, storage_of, strides_of
 
 pytestmark = pytest.mark.gpu
 
@@ -619,3 +619,110 @@ def test_mlp_graph_replay_matches_eager(T, oracle):
     x, y = R.mnist_like_batch(64, seed, 99)
     assert eager.step(x, y, 0.05) == graph.step(x, y, 0.05, graph=True)
     np.testing.assert_array_equal(eager.params(0)[0], graph.params(0)[0])
+
+
+@pytest.mark.gpu
+def test_cross_entropy_entries(T, oracle):
+    """tenmo_hip_cross_entropy_forward_f32 / _backward_f32 against the CPU restatement: thread-per-row
+    and workgroup-per-row kernels, aligned and unaligned rows, int64 and int32 targets, ignore_index,
+    label smoothing, the three reductions, accumulate."""
+    import ctypes as C
+    import torch
+
+    L, lib = T.lib.load(), T.lib
+    rng = np.random.default_rng(43)
+    for M, Cn, ls, is64 in [(2, 3, 0.0, True), (64, 10, 0.0, False), (33, 17, 0.2, True), (5, 1000, 0.05, True),
+                            (7, 1001, 0.1, False), (300, 64, 0.0, True), (3, 50257, 0.1, True)]:
+        x = (3 * rng.standard_normal((M, Cn))).astype(np.float32)
+        t = rng.integers(0, Cn, M)
+        t[rng.random(M) < 0.3] = -100
+        sm_ref, rows_ref, total_ref, valid_ref = oracle.cross_entropy_forward(x, t, label_smoothing=ls)
+        X = torch.from_numpy(x).cuda()
+        Tg = torch.from_numpy(t.astype(np.int64 if is64 else np.int32)).cuda()
+        sm = torch.empty((M, Cn), dtype=torch.float32, device="cuda")
+        rows = torch.empty(M, dtype=torch.float32, device="cuda")
+        total = torch.zeros(1, dtype=torch.float32, device="cuda")
+        valid = torch.zeros(1, dtype=torch.int32, device="cuda")
+        lib.check(L.tenmo_hip_cross_entropy_forward_f32(X.data_ptr(), Tg.data_ptr(), 1 if is64 else 0, M, Cn, -100, ls,
+                                                        sm.data_ptr(), rows.data_ptr(), total.data_ptr(), valid.data_ptr(), 1))
+        case = (M, Cn, ls, is64)
+        assert int(valid.item()) == valid_ref, case
+        # against fp64 at the stated tolerance; against the CPU restatement a little looser for long
+        # rows, whose sum of exponentials the restatement adds serially in fp32 (as the reference does)
+        p64, loss64, _ = ce_reference64(x, t, -100, ls)
+        assert np.allclose(sm.cpu().numpy(), p64, rtol=1e-5, atol=1e-7), case
+        assert np.allclose(rows.cpu().numpy(), loss64, rtol=1e-5, atol=1e-5), case
+        assert np.allclose(sm.cpu().numpy(), sm_ref, rtol=2e-4, atol=1e-7), case
+        assert np.allclose(rows.cpu().numpy(), rows_ref, rtol=1e-5, atol=1e-5), case
+        assert abs(float(total.item()) - total_ref) <= 1e-5 * max(1.0, abs(total_ref)), case
+        # a softmax buffer that is not congruent with the logits modulo 16 bytes takes the element-wise path
+        sm_odd = torch.empty(M * Cn + 1, dtype=torch.float32, device="cuda")
+        lib.check(L.tenmo_hip_cross_entropy_forward_f32(X.data_ptr(), Tg.data_ptr(), 1 if is64 else 0, M, Cn, -100, ls,
+                                                        sm_odd.data_ptr() + 4, rows.data_ptr(), total.data_ptr(), valid.data_ptr(), 1))
+        assert np.allclose(sm_odd[1:].cpu().numpy().reshape(M, Cn), p64, rtol=1e-5, atol=1e-7), case
+        g_odd = torch.empty(M * Cn + 1, dtype=torch.float32, device="cuda")
+        one = torch.ones(1, dtype=torch.float32, device="cuda")
+        lib.check(L.tenmo_hip_cross_entropy_backward_f32(sm.data_ptr(), Tg.data_ptr(), 1 if is64 else 0, one.data_ptr(), M, Cn, -100, ls,
+                                                         1, valid_ref, g_odd.data_ptr() + 4, 0, 1))
+        ref_odd = oracle.cross_entropy_backward(sm.cpu().numpy(), t, np.ones(1, np.float32), 1, valid_ref, label_smoothing=ls)
+        assert np.allclose(g_odd[1:].cpu().numpy().reshape(M, Cn), ref_odd, rtol=1e-5, atol=1e-7), case
+        # without a softmax buffer the losses are the same
+        rows2 = torch.empty_like(rows)
+        lib.check(L.tenmo_hip_cross_entropy_forward_f32(X.data_ptr(), Tg.data_ptr(), 1 if is64 else 0, M, Cn, -100, ls,
+                                                        None, rows2.data_ptr(), total.data_ptr(), valid.data_ptr(), 1))
+        assert torch.allclose(rows, rows2, rtol=1e-6, atol=1e-6), case
+        up = rng.standard_normal(M).astype(np.float32)
+        Up = torch.from_numpy(up).cuda()
+        grad = torch.empty((M, Cn), dtype=torch.float32, device="cuda")
+        for red in (oracle.REDUCTION_NONE, oracle.REDUCTION_SUM, oracle.REDUCTION_MEAN):
+            ref = oracle.cross_entropy_backward(sm.cpu().numpy(), t, up if red == 0 else up[:1], red, valid_ref, label_smoothing=ls)
+            lib.check(L.tenmo_hip_cross_entropy_backward_f32(sm.data_ptr(), Tg.data_ptr(), 1 if is64 else 0, Up.data_ptr(), M, Cn, -100, ls,
+                                                             red, valid_ref, grad.data_ptr(), 0, 1))
+            assert np.allclose(grad.cpu().numpy(), ref, rtol=1e-5, atol=1e-7), (case, red)
+        lib.check(L.tenmo_hip_cross_entropy_backward_f32(sm.data_ptr(), Tg.data_ptr(), 1 if is64 else 0, Up.data_ptr(), M, Cn, -100, ls,
+                                                         2, valid_ref, grad.data_ptr(), 1, 1))
+        assert np.allclose(grad.cpu().numpy(), 2 * ref, rtol=1e-5, atol=1e-7), (case, "accumulate")
+    # argument checks
+    assert L.tenmo_hip_cross_entropy_forward_f32(X.data_ptr(), Tg.data_ptr(), 1, 3, 0, -100, 0.0, None, rows.data_ptr(), total.data_ptr(), valid.data_ptr(), 1) == -2
+    assert L.tenmo_hip_cross_entropy_forward_f32(X.data_ptr(), Tg.data_ptr(), 1, 3, 4, -100, 1.5, None, rows.data_ptr(), total.data_ptr(), valid.data_ptr(), 1) == -3
+    assert b"label_smoothing" in L.tenmo_hip_last_error()
+    assert L.tenmo_hip_cross_entropy_forward_f32(None, Tg.data_ptr(), 1, 3, 4, -100, 0.0, None, rows.data_ptr(), total.data_ptr(), valid.data_ptr(), 1) == -3
+    assert L.tenmo_hip_cross_entropy_backward_f32(sm.data_ptr(), Tg.data_ptr(), 1, Up.data_ptr(), 3, 4, -100, 0.0, 3, 1, grad.data_ptr(), 0, 1) == -3
+    # no rows: sum 0, nothing valid
+    lib.check(L.tenmo_hip_cross_entropy_forward_f32(None, None, 1, 0, 4, -100, 0.0, None, None, total.data_ptr(), valid.data_ptr(), 1))
+    assert float(total.item()) == 0.0 and int(valid.item()) == 0
+
+
+@pytest.mark.gpu
+def test_sgd_entry(T, golden, oracle):
+    import torch
+
+    L, lib = T.lib.load(), T.lib
+    H = golden["harness"]
+    g = H["sgd_momentum_three_steps"]
+    w = torch.tensor(g["w"], dtype=torch.float32, device="cuda")
+    v = torch.zeros(1, dtype=torch.float32, device="cuda")
+    gr = torch.tensor(g["grad"], dtype=torch.float32, device="cuda")
+    for want in g["expect_after_each"]:
+        lib.check(L.tenmo_hip_sgd_step_f32(w.data_ptr(), gr.data_ptr(), v.data_ptr(), 1, g["lr"], g["momentum"], 0.0, 1))
+        assert abs(float(w.item()) - want) < 1e-6
+    g = H["sgd_weight_decay"]
+    w = torch.tensor(g["w"], dtype=torch.float32, device="cuda")
+    gr = torch.tensor(g["grad"], dtype=torch.float32, device="cuda")
+    lib.check(L.tenmo_hip_sgd_step_f32(w.data_ptr(), gr.data_ptr(), None, 3, g["lr"], 0.0, g["weight_decay"], 1))
+    assert np.allclose(w.cpu().numpy(), g["expect"], rtol=1e-6)
+    # a large tensor, both forms, against the CPU restatement
+    rng = np.random.default_rng(47)
+    n = 1_000_003
+    p0, gr0, v0 = (rng.standard_normal(n).astype(np.float32) for _ in range(3))
+    for vel, mom, wd in [(False, 0.0, 0.0), (False, 0.0, 0.01), (True, 0.9, 0.0), (True, 0.9, 0.01)]:
+        p_ref, v_ref = p0.copy(), v0.copy()
+        oracle.sgd_step(p_ref, gr0, v_ref if vel else None, 0.05, mom, wd)
+        P, G, V = torch.from_numpy(p0.copy()).cuda(), torch.from_numpy(gr0).cuda(), torch.from_numpy(v0.copy()).cuda()
+        lib.check(L.tenmo_hip_sgd_step_f32(P.data_ptr(), G.data_ptr(), V.data_ptr() if vel else None, n, 0.05, mom, wd, 1))
+        # one rounding of difference per product (fused multiply-add on the GPU): absolute, since sums cancel
+        assert np.allclose(P.cpu().numpy(), p_ref, rtol=1e-6, atol=1e-6), (vel, mom, wd)
+        if vel:
+            assert np.allclose(V.cpu().numpy(), v_ref, rtol=1e-6, atol=1e-6)
+    assert L.tenmo_hip_sgd_step_f32(None, G.data_ptr(), None, 4, 0.1, 0.0, 0.0, 1) == -3
+    assert L.tenmo_hip_sgd_step_f32(None, None, None, 0, 0.1, 0.0, 0.0, 1) == 0

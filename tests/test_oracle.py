@@ -3,7 +3,7 @@ vectors, fp64 brute force, closed forms and algebraic invariants.  Runs without 
 import numpy as np
 import pytest
 
-from helpers import numpy_view, ref_matmul64, rel_fro, storage_of, strides_of
+from helpers import ce_reference64, numpy_view, ref_matmul64, rel_fro, storage_of, strides_of
 
 
 def _view(O, t):
@@ -281,3 +281,90 @@ def test_mlp_step_matches_numpy_fp64(oracle):
         for l in range(3):
             W, b = m.params(l)
             assert rel_fro(W, W64[l]) < 1e-5 and np.abs(b - b64[l]).max() < 1e-6
+
+
+def test_cross_entropy_oracle_is_pinned(golden, oracle):
+    """Closed forms and vectors of tests/test_cross_entropy.mojo, an independent fp64 statement, the
+    invariants the reference tests (row gradients sum to zero, ignored rows vanish, mean = sum / valid)
+    and finite differences of the loss."""
+    H = golden["harness"]
+    # uniform logits -> log(C)   (tests/test_cross_entropy.mojo:724-743, :1600-1609)
+    sm, rows, total, valid = oracle.cross_entropy_forward(np.ones((2, 3), np.float32), np.array([0, 1]))
+    assert valid == 2 and abs(total / valid - H["ce_uniform_logits"]["loss"]) < 1e-6 and np.allclose(sm, 1 / 3, atol=1e-7)
+    # two rows, mean (:1227-1241)
+    g = H["ce_two_rows_mean"]
+    x = np.array(g["logits"], np.float32)
+    e = np.exp(np.array(g["logits"], np.float64))
+    want = (-np.log(e[0, 0] / e[0].sum()) - np.log(e[1, 1] / e[1].sum())) / 2
+    sm, rows, total, valid = oracle.cross_entropy_forward(x, np.array(g["targets"]))
+    assert abs(total / valid - want) < 1e-6
+    # gradient of the mean: (softmax - onehot) / batch (:1449-1476)
+    grad = oracle.cross_entropy_backward(sm, np.array(g["targets"]), np.ones(1, np.float32), oracle.REDUCTION_MEAN, valid)
+    p64 = e / e.sum(1, keepdims=True)
+    assert np.allclose(grad, (p64 - np.eye(3)[g["targets"]]) / 2, atol=1e-6)
+    # label smoothing (:2425-2443, :2731-2746)
+    g = H["ce_label_smoothing_formula"]
+    x, ls = np.array(g["logits"], np.float32), g["label_smoothing"]
+    p = np.exp(np.array(g["logits"][0], np.float64)); p /= p.sum()
+    sm, rows, total, valid = oracle.cross_entropy_forward(x, np.array(g["targets"]), label_smoothing=ls)
+    assert abs(total - ((1 - ls) * -np.log(p[0]) + ls * np.mean(-np.log(p)))) < 1e-6
+    grad = oracle.cross_entropy_backward(sm, np.array(g["targets"]), np.ones(1, np.float32), oracle.REDUCTION_MEAN, valid, label_smoothing=ls)
+    assert abs(grad[0, 0] - (p[0] - (1 - ls) - ls / 3)) < 1e-6 and abs(grad[0, 1] - (p[1] - ls / 3)) < 1e-6
+    # ignore_index (:247-323)
+    g = H["ce_ignore_index"]
+    x, t = np.array(g["logits"], np.float32), np.array(g["targets"])
+    sm, rows, total, valid = oracle.cross_entropy_forward(x, t, ignore_index=g["ignore_index"])
+    assert valid == 2 and rows[1] == 0 and rows[0] > 0 and rows[2] > 0
+    grad = oracle.cross_entropy_backward(sm, t, np.ones(1, np.float32), oracle.REDUCTION_MEAN, valid, ignore_index=g["ignore_index"])
+    assert np.all(grad[1] == 0) and abs(grad[0, 0]) > 1e-6 and abs(grad[2, 0]) > 1e-6
+    sm, rows, total, valid = oracle.cross_entropy_forward(x[:2], np.array([-100, -100]))
+    assert valid == 0 and total == 0
+    assert np.all(oracle.cross_entropy_backward(sm, np.array([-100, -100]), np.ones(1, np.float32), oracle.REDUCTION_MEAN, valid) == 0)
+    # random cases against the fp64 statement, all reductions, smoothing and ignored rows together
+    rng = np.random.default_rng(41)
+    for M, C, ls in [(7, 5, 0.0), (33, 17, 0.2), (4, 1000, 0.05), (64, 10, 0.0)]:
+        x = (3 * rng.standard_normal((M, C))).astype(np.float32)
+        t = rng.integers(0, C, M)
+        t[rng.random(M) < 0.3] = -100
+        p64, loss64, grad64 = ce_reference64(x, t, -100, ls)
+        sm, rows, total, valid = oracle.cross_entropy_forward(x, t, label_smoothing=ls)
+        assert valid == int((t != -100).sum())
+        assert np.allclose(sm, p64, rtol=1e-5, atol=1e-7) and np.allclose(rows, loss64, rtol=1e-5, atol=1e-6)
+        assert abs(total - loss64.sum()) <= 1e-5 * max(1.0, abs(loss64.sum()))
+        up = rng.standard_normal(M).astype(np.float32)
+        assert np.allclose(oracle.cross_entropy_backward(sm, t, up, oracle.REDUCTION_NONE, valid, label_smoothing=ls), grad64 * up[:, None], rtol=1e-4, atol=1e-6)
+        assert np.allclose(oracle.cross_entropy_backward(sm, t, up[:1], oracle.REDUCTION_SUM, valid, label_smoothing=ls), grad64 * up[0], rtol=1e-4, atol=1e-6)
+        gm = oracle.cross_entropy_backward(sm, t, up[:1], oracle.REDUCTION_MEAN, valid, label_smoothing=ls)
+        assert np.allclose(gm, grad64 * up[0] / max(valid, 1), rtol=1e-4, atol=1e-6)
+        assert np.abs(gm.sum(1)).max() < 1e-6          # every row of the gradient sums to zero (:797-823)
+    # finite differences of the summed loss in fp64 agree with the analytic gradient
+    x = rng.standard_normal((3, 4)).astype(np.float32)
+    t = np.array([1, -100, 3])
+    sm, rows, total, valid = oracle.cross_entropy_forward(x, t, label_smoothing=0.1)
+    grad = oracle.cross_entropy_backward(sm, t, np.ones(1, np.float32), oracle.REDUCTION_SUM, valid, label_smoothing=0.1)
+    for (i, j) in [(0, 0), (0, 1), (2, 3), (1, 2)]:
+        h = 1e-5
+        xp, xm = x.astype(np.float64), x.astype(np.float64)
+        xp[i, j] += h; xm[i, j] -= h
+        fd = (ce_reference64(xp, t, -100, 0.1)[1].sum() - ce_reference64(xm, t, -100, 0.1)[1].sum()) / (2 * h)
+        assert abs(grad[i, j] - fd) < 1e-5
+
+
+def test_sgd_oracle_is_pinned(golden, oracle):
+    """tests/test_sgd.mojo vectors: plain, weight decay, momentum over three steps."""
+    H = golden["harness"]
+    for key in ("sgd_single_step", "sgd_three_steps", "sgd_2d"):
+        g = H[key]
+        w = np.array(g["w"], np.float32)
+        for _ in range(g["steps"]):
+            oracle.sgd_step(w, np.array(g["grad"], np.float32), None, g["lr"])
+        assert np.allclose(w, g["expect"], rtol=1e-6)
+    g = H["sgd_weight_decay"]
+    w = np.array(g["w"], np.float32)
+    oracle.sgd_step(w, np.array(g["grad"], np.float32), None, g["lr"], weight_decay=g["weight_decay"])
+    assert np.allclose(w, g["expect"], rtol=1e-6)
+    g = H["sgd_momentum_three_steps"]
+    w, v = np.array(g["w"], np.float32), np.zeros(1, np.float32)
+    for want in g["expect_after_each"]:
+        oracle.sgd_step(w, np.array(g["grad"], np.float32), v, g["lr"], momentum=g["momentum"])
+        assert abs(w[0] - want) < 1e-6
