@@ -288,37 +288,41 @@ __device__ __forceinline__ void bare_barrier() {
     asm volatile("" ::: "memory");
 }
 
-template <int BM, int BN, int AMODE, int BMODE>
-__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmArgs g) {
-    constexpr int TM = BM / 2, TN = BN / 2;     // wave tile (2x2 waves)
-    constexpr int MB = TM / 32, NB = TN / 32;   // 32x32 MFMA blocks per wave tile
-    constexpr int A_FLOATS = BM * GEMM_BK;
-    constexpr int STAGE_FLOATS = (BM + BN) * GEMM_BK;
-    constexpr bool DIRECT = (AMODE != KMAJOR_GEN) && (BMODE != KMAJOR_GEN);
-    // three separate objects: the compiler can then tell that a direct load into one stage does
-    // not alias the operand fetch from another
-    __shared__ __attribute__((aligned(1024))) float stage0[STAGE_FLOATS];
-    __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
-    __shared__ __attribute__((aligned(1024))) float stage2[DIRECT ? STAGE_FLOATS : 4];
-
-    const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int wm = wave >> 1, wn = wave & 1;
-
-    // ---- which tile ----
-    const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-    // Workgroup ids are dealt round-robin to the 8 XCDs (checked with HW_REG_XCC_ID), so with groups
-    // of 8 tile-rows each XCD keeps one tile-row of A hot in its L2 and streams B past it.  Giving
-    // each XCD a compact 8x8 block of tiles instead was measured: 1.8x the L2-miss traffic (a tall A
-    // panel at a power-of-two row pitch thrashes a few L2 sets) and up to 4 % slower.
-    const int64_t pid = blockIdx.x;
-    const int64_t batch = pid / tiles;
-    const int64_t tid = pid % tiles;
+// position of tile number `tid` (0 .. tiles_m*tiles_n-1) in the tile grid.
+// Workgroup ids are dealt round-robin to the 8 XCDs (checked with HW_REG_XCC_ID), so with groups
+// of 8 tile-rows each XCD keeps one tile-row of A hot in its L2 and streams B past it.  Giving
+// each XCD a compact 8x8 block of tiles instead was measured: 1.8x the L2-miss traffic (a tall A
+// panel at a power-of-two row pitch thrashes a few L2 sets) and up to 4 % slower.
+__device__ __forceinline__ void tile_coords(const GemmArgs& g, int64_t tid, int64_t& tile_m, int64_t& tile_n) {
     constexpr int GROUP_M = 8;
     const int64_t per_group = (int64_t)GROUP_M * g.tiles_n;
     const int64_t first_m = (tid / per_group) * GROUP_M;
     const int64_t gsz = min((int64_t)g.tiles_m - first_m, (int64_t)GROUP_M);
-    const int64_t tile_m = first_m + (tid % per_group) % gsz;
-    const int64_t tile_n = (tid % per_group) / gsz;
+    tile_m = first_m + (tid % per_group) % gsz;
+    tile_n = (tid % per_group) / gsz;
+}
+
+// where a finished tile goes: element (row, col) of the product is written to
+// base[(row - row0) * ld + (col - col0)]
+struct TileDest {
+    float* base;
+    int64_t ld, row0, col0;
+    bool accumulate; // += instead of =
+    bool fused;      // apply g.bias / g.relu / g.mask (never together with accumulate)
+};
+
+// One tile of C over the K range [k_begin, k_end) (k_begin a multiple of GEMM_BK), by the whole
+// workgroup.  The three LDS stages are the caller's; on return every wavefront has left them.
+template <int BM, int BN, int AMODE, int BMODE>
+__device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, float* stage1, float* stage2,
+                                          int64_t batch, int64_t tile_m, int64_t tile_n, int64_t k_begin, int64_t k_end, const TileDest dst) {
+    constexpr int TM = BM / 2, TN = BN / 2;     // wave tile (2x2 waves)
+    constexpr int MB = TM / 32, NB = TN / 32;   // 32x32 MFMA blocks per wave tile
+    constexpr int A_FLOATS = BM * GEMM_BK;
+    constexpr bool DIRECT = (AMODE != KMAJOR_GEN) && (BMODE != KMAJOR_GEN);
+
+    const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int wm = wave >> 1, wn = wave & 1;
     const int64_t m0 = tile_m * BM, n0 = tile_n * BN;
 
     int64_t a_boff, b_boff;
@@ -330,11 +334,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     const int64_t a_row_s = g.a_rs, a_k_s = g.a_cs;   // A(m,k)
     const int64_t b_row_s = g.b_cs, b_k_s = g.b_rs;   // B(n,k) = Bmem[k*b_rs + n*b_cs]
 
-    int64_t k_begin = 0, k_end = g.K;
-    if (g.k_splits > 1) {
-        k_begin = (int64_t)blockIdx.y * g.k_per_split;
-        k_end = min(g.K, k_begin + g.k_per_split);
-    }
     const int64_t nk = (k_end > k_begin) ? (k_end - k_begin + GEMM_BK - 1) / GEMM_BK : 0;
 
     f32x16 acc[MB][NB];
@@ -499,15 +498,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     }
 
     // ---- epilogue ----
-    float* __restrict Cb;
-    bool accumulate = g.accumulate != 0;
-    if (g.k_splits > 1) {
-        Cb = g.partial + ((int64_t)blockIdx.y * g.batch_count + batch) * g.M * g.N;
-        accumulate = false;
-    } else {
-        Cb = g.C + batch * g.M * g.N;
-    }
-    const bool fused = g.k_splits == 1 && (g.bias != nullptr || g.mask != nullptr || g.relu != 0);
+    const bool accumulate = dst.accumulate;
+    const bool fused = dst.fused && (g.bias != nullptr || g.mask != nullptr || g.relu != 0);
     const float* __restrict mask = g.mask ? g.mask + batch * g.M * g.N : nullptr;
     const int h = lane >> 5, x = lane & 31;
 #pragma unroll
@@ -517,7 +509,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
             const int ip = 8 * (e >> 2) + 4 * h + (e & 3); // MFMA row of accumulator element e
             const int64_t row = m0 + wm * TM + tile_pos<AMODE, MB>(i, ip);
             if (row >= g.M) continue;
-            float* crow = Cb + row * g.N;
+            float* crow = dst.base + (row - dst.row0) * dst.ld - dst.col0;
             if (fused) { // rare enough to stay scalar
 #pragma unroll
                 for (int j = 0; j < NB; ++j) {
@@ -550,6 +542,132 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
                     if (col < g.N) crow[col] = accumulate ? crow[col] + acc[i][j][e] : acc[i][j][e];
                 }
             }
+        }
+    }
+}
+
+// One workgroup per tile (and per K slice when g.k_splits > 1).
+template <int BM, int BN, int AMODE, int BMODE>
+__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmArgs g) {
+    constexpr int STAGE_FLOATS = (BM + BN) * GEMM_BK;
+    constexpr bool DIRECT = (AMODE != KMAJOR_GEN) && (BMODE != KMAJOR_GEN);
+    // three separate objects: the compiler can then tell that a direct load into one stage does
+    // not alias the operand fetch from another
+    __shared__ __attribute__((aligned(1024))) float stage0[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage2[DIRECT ? STAGE_FLOATS : 4];
+
+    const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+    const int64_t pid = blockIdx.x;
+    const int64_t batch = pid / tiles;
+    int64_t tile_m, tile_n;
+    tile_coords(g, pid % tiles, tile_m, tile_n);
+
+    int64_t k_begin = 0, k_end = g.K;
+    TileDest dst;
+    dst.ld = g.N; dst.row0 = 0; dst.col0 = 0;
+    if (g.k_splits > 1) { // partial sums of this K slice; the slice reduction finishes them
+        k_begin = (int64_t)blockIdx.y * g.k_per_split;
+        k_end = min(g.K, k_begin + g.k_per_split);
+        dst.base = g.partial + ((int64_t)blockIdx.y * g.batch_count + batch) * g.M * g.N;
+        dst.accumulate = false; dst.fused = false;
+    } else {
+        dst.base = g.C + batch * g.M * g.N;
+        dst.accumulate = g.accumulate != 0; dst.fused = true;
+    }
+    gemm_tile<BM, BN, AMODE, BMODE>(g, stage0, stage1, stage2, batch, tile_m, tile_n, k_begin, k_end, dst);
+}
+
+// ---- stream-K --------------------------------------------------------------------------------
+// The launch's work is cut into K steps ("iterations": tile-major, K-minor, batches outermost) and
+// every workgroup of a persistent grid takes an equal contiguous run of them, so the chip stays
+// full whatever the tile count.  A workgroup whose run covers a whole tile stores it as usual; the
+// pieces of a tile that is shared between workgroups go to compact partial tiles (two slots per
+// workgroup: slot 2w for a piece that starts inside the tile, 2w+1 for one that starts at its
+// beginning) and streamk_fixup_kernel adds them in workgroup order — deterministic, no spinning.
+struct StreamKArgs {
+    int64_t total;   // iterations in the launch = tiles * nks
+    int64_t per_wg;  // iterations per workgroup
+    int64_t nks;     // K steps per tile
+    float* partial;  // [2 * workgroups][BM * BN]
+};
+
+template <int BM, int BN, int AMODE, int BMODE>
+__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_streamk_kernel(const GemmArgs g, const StreamKArgs sk) {
+    constexpr int STAGE_FLOATS = (BM + BN) * GEMM_BK;
+    constexpr bool DIRECT = (AMODE != KMAJOR_GEN) && (BMODE != KMAJOR_GEN);
+    __shared__ __attribute__((aligned(1024))) float stage0[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage2[DIRECT ? STAGE_FLOATS : 4];
+    const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+    const int64_t w = blockIdx.x;
+    int64_t it = w * sk.per_wg;
+    const int64_t end = min(sk.total, it + sk.per_wg);
+    while (it < end) {
+        const int64_t gt = it / sk.nks, k0 = it % sk.nks;
+        const int64_t k1 = min(sk.nks, k0 + (end - it));
+        const int64_t batch = gt / tiles;
+        int64_t tile_m, tile_n;
+        tile_coords(g, gt % tiles, tile_m, tile_n);
+        TileDest dst;
+        if (k0 == 0 && k1 == sk.nks) {
+            dst.base = g.C + batch * g.M * g.N; dst.ld = g.N; dst.row0 = 0; dst.col0 = 0;
+            dst.accumulate = g.accumulate != 0; dst.fused = true;
+        } else {
+            dst.base = sk.partial + (2 * w + (k0 == 0 ? 1 : 0)) * (int64_t)(BM * BN); dst.ld = BN;
+            dst.row0 = tile_m * BM; dst.col0 = tile_n * BN;
+            dst.accumulate = false; dst.fused = false;
+        }
+        gemm_tile<BM, BN, AMODE, BMODE>(g, stage0, stage1, stage2, batch, tile_m, tile_n, k0 * GEMM_BK, min(g.K, k1 * GEMM_BK), dst);
+        it += k1 - k0;
+    }
+}
+
+// A tile that was shared between workgroups is the sum of their partial tiles (ascending workgroup
+// order), finished with accumulate / the fused epilogue.  blockIdx.x = tile, blockIdx.y = one of
+// gridDim.y equal parts of the tile, so that a launch with few tiles still fills the chip.
+template <int BM, int BN>
+__global__ void streamk_fixup_kernel(const GemmArgs g, const StreamKArgs sk) {
+    const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+    const int64_t gt = blockIdx.x;
+    const int64_t it0 = gt * sk.nks, it1 = it0 + sk.nks;
+    const int64_t w_first = it0 / sk.per_wg, w_last = (it1 - 1) / sk.per_wg;
+    if (w_first == w_last) return; // one workgroup had the whole tile and stored it
+    const int64_t batch = gt / tiles;
+    int64_t tile_m, tile_n;
+    tile_coords(g, gt % tiles, tile_m, tile_n);
+    float* __restrict Cb = g.C + batch * g.M * g.N;
+    const float* __restrict mask = g.mask ? g.mask + batch * g.M * g.N : nullptr;
+    const bool fused = g.bias != nullptr || g.mask != nullptr || g.relu != 0;
+    // the first contributor's piece starts at the tile's beginning (slot 2w+1) exactly when its run
+    // began at or before the tile; every later contributor's piece starts inside the tile (slot 2w)
+    const float* __restrict first = sk.partial + (2 * w_first + (w_first * sk.per_wg <= it0 ? 1 : 0)) * (int64_t)(BM * BN);
+    constexpr int PER_TILE = BM * BN / 4; // float4 positions
+    const int part = PER_TILE / gridDim.y;
+    for (int q4 = blockIdx.y * part + threadIdx.x; q4 < (int)(blockIdx.y + 1) * part; q4 += blockDim.x) {
+        const int e = 4 * q4, r = e / BN, c = e % BN;
+        const int64_t row = tile_m * BM + r, col = tile_n * BN + c;
+        if (row >= g.M || col >= g.N) continue;
+        f32x4 s = *reinterpret_cast<const f32x4*>(first + e);
+        int64_t w = w_first + 1;
+        for (; w + 3 <= w_last; w += 4) { // four loads in flight, added in workgroup order
+            const float* __restrict p = sk.partial + (2 * w) * (int64_t)(BM * BN) + e;
+            const f32x4 v0 = *reinterpret_cast<const f32x4*>(p);
+            const f32x4 v1 = *reinterpret_cast<const f32x4*>(p + 2 * (int64_t)(BM * BN));
+            const f32x4 v2 = *reinterpret_cast<const f32x4*>(p + 4 * (int64_t)(BM * BN));
+            const f32x4 v3 = *reinterpret_cast<const f32x4*>(p + 6 * (int64_t)(BM * BN));
+            s += v0; s += v1; s += v2; s += v3;
+        }
+        for (; w <= w_last; ++w) s += *reinterpret_cast<const f32x4*>(sk.partial + (2 * w) * (int64_t)(BM * BN) + e);
+        const float v[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            if (col + q >= g.N) break;
+            const int64_t i = row * g.N + col + q;
+            float o = v[q];
+            if (g.accumulate) o += Cb[i];
+            if (fused) o = epilogue_value(o, g.bias, mask, g.relu, i, col + q);
+            Cb[i] = o;
         }
     }
 }

@@ -70,6 +70,7 @@ struct State {
     // tuning overrides (environment, read once): -1 = automatic
     int force_tile = -1;
     int force_splitk = -1;
+    int force_streamk = -1;    // -1 automatic, 0 never, n > 0: stream-K with n workgroups per CU
     int verbose = 0;
     int cols_waves_per_cu = 2; // target workgroups per CU of the column-streaming kernels (long K slices stream best)
 };
@@ -178,6 +179,22 @@ int launch_gemm_tile(const GemmArgs& g, dim3 grid, int am, int bm) {
     return fail(TENMO_ERR_UNSUPPORTED, "no GEMM variant for operand modes %d/%d", am, bm);
 }
 
+// stream-K: persistent workgroups + fix-up of the shared tiles (vector operand modes only)
+template <int BM, int BN>
+int launch_streamk_tile(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, int64_t tiles_total, bool need_fixup, int am, int bm) {
+#define TENMO_CASE(A_, B_) if (am == A_ && bm == B_) { hipLaunchKernelGGL((gemm_streamk_kernel<BM, BN, A_, B_>), dim3(wgs), dim3(GEMM_THREADS), 0, S.stream, g, sk); }
+    TENMO_CASE(KMAJOR_VEC, KMAJOR_VEC) else TENMO_CASE(KMAJOR_VEC, MNMAJOR_VEC) else TENMO_CASE(MNMAJOR_VEC, KMAJOR_VEC) else TENMO_CASE(MNMAJOR_VEC, MNMAJOR_VEC)
+    else return fail(TENMO_ERR_UNSUPPORTED, "no stream-K variant for operand modes %d/%d", am, bm);
+#undef TENMO_CASE
+    if (need_fixup) {
+        // parts per tile: a power of two that brings the launch to a few workgroups per CU
+        unsigned parts = 1;
+        while (parts < 32 && (int64_t)tiles_total * parts < (int64_t)S.cus * 4) parts *= 2;
+        hipLaunchKernelGGL((streamk_fixup_kernel<BM, BN>), dim3((unsigned)tiles_total, parts), dim3(256), 0, S.stream, g, sk);
+    }
+    return 0;
+}
+
 struct TileShape { int bm, bn; };
 constexpr int kNumTiles = 5;
 const TileShape kTiles[kNumTiles] = {{256, 128}, {128, 128}, {64, 64}, {128, 64}, {64, 128}};
@@ -218,9 +235,11 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     // its workgroups (the K loop runs at full rate from one wavefront per SIMD up), every workgroup
     // pays a fixed prologue/epilogue, and the launch can never beat its HBM and L2 traffic.
     int tile = 0, splits = 1;
+    int sk_tile = 0, sk_wpc = 0;
+    double best_sk = 1e300;
     {
         static const double kOcc[kNumTiles] = {2, 3, 6, 4, 4};             // resident workgroups per CU (LDS / VGPR limits)
-        static const double kEff[kNumTiles] = {0.96, 0.95, 0.94, 0.92, 0.92}; // matrix-pipe efficiency of the K loop
+        static const double kEff[kNumTiles] = {0.96, 0.93, 0.84, 0.90, 0.90}; // matrix-pipe efficiency of the K loop
         static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
         const double cus = (double)S.cus;
         double best = 1e300;
@@ -239,16 +258,60 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
                 const double t_round = iters * conc * m_us / kEff[t] + 1.5;
                 const double bytes = 4.0 * batch_count * ((double)M * K + (double)K * N + (double)M * N * (sp > 1 ? sp + 1.0 : 1.0));
                 const double l2_bytes = 4.0 * batch_count * (double)K * ((double)M * tn + (double)N * tm);
-                double est = std::max({rounds * t_round, bytes / 5.0e6, l2_bytes / 14.0e6}) + 3.0;
+                double est = std::max({rounds * t_round, bytes / 5.0e6, l2_bytes / 8.0e6}) + 3.0;
                 if (sp > 1) est += 5.0 + 4.0 * batch_count * (double)M * N * (sp + 1.0) / 6.0e6;
                 if (est < best) { best = est; tile = t; splits = sp; }
             }
         }
-        if (S.verbose) fprintf(stderr, "tenmo_hip gemm M=%lld N=%lld K=%lld batch=%lld -> tile %dx%d, %d K slice(s), est %.1f us\n",
-                               (long long)M, (long long)N, (long long)K, (long long)batch_count, kTiles[tile].bm, kTiles[tile].bn, splits, best);
+        // stream-K (persistent workgroups sharing tiles, see gemm_mfma.hpp): every CU gets the same
+        // number of K steps whatever the tile count, at the price of the fix-up traffic
+        if (S.force_streamk < 0 && am != KMAJOR_GEN && bm != KMAJOR_GEN) {
+            // Measured: the 128x128 tile with one workgroup per CU is the variant that wins; with many
+            // tiles per workgroup the classic launch is as full and shares operand panels in L2 better.
+            const int t = 1, wpc = 1;
+            const double tm = (double)((M + kTiles[t].bm - 1) / kTiles[t].bm), tn = (double)((N + kTiles[t].bn - 1) / kTiles[t].bn);
+            const double tiles = tm * tn * (double)batch_count, nks = std::ceil((double)K / GEMM_BK);
+            const double m_us = (kTiles[t].bm / 64) * (kTiles[t].bn / 64) * 8 * 64 / 2400.0;
+            const double wgs = cus * wpc;
+            if (tiles * nks >= wgs * 8 && tiles <= 3.0 * wgs) { // pieces of under eight K steps are all overhead
+                const double shared_tiles = std::min(2.0 * wgs, 2.0 * tiles);
+                const double fix = 2.0 * shared_tiles * kTiles[t].bm * kTiles[t].bn * 4.0 / 5.0e6;
+                const double est = tiles * nks / cus * m_us / kEff[t] + fix + 10.0;
+                if (est < 0.98 * best) { best_sk = est; sk_tile = t; sk_wpc = wpc; }
+            }
+        }
+        if (S.verbose) fprintf(stderr, "tenmo_hip gemm M=%lld N=%lld K=%lld batch=%lld -> tile %dx%d, %d K slice(s), est %.1f us%s\n",
+                               (long long)M, (long long)N, (long long)K, (long long)batch_count, kTiles[tile].bm, kTiles[tile].bn, splits, best,
+                               sk_wpc ? " (stream-K chosen instead)" : "");
     }
     if (S.force_tile >= 0 && S.force_tile < kNumTiles) tile = S.force_tile;
     if (S.force_splitk > 0) splits = S.force_splitk;
+    int streamk = S.force_streamk > 0 ? S.force_streamk : 0;
+    if (S.force_streamk < 0 && sk_wpc > 0 && S.force_tile < 0 && S.force_splitk <= 0) { streamk = sk_wpc; tile = sk_tile; }
+    if (streamk > 0 && tile <= 1 && am != KMAJOR_GEN && bm != KMAJOR_GEN) {
+        const int bmt = kTiles[tile].bm, bnt = kTiles[tile].bn;
+        g.tiles_m = (int32_t)((M + bmt - 1) / bmt);
+        g.tiles_n = (int32_t)((N + bnt - 1) / bnt);
+        g.k_splits = 1; g.k_per_split = K; g.partial = nullptr;
+        const int64_t tiles_total = (int64_t)g.tiles_m * g.tiles_n * batch_count;
+        StreamKArgs sk{};
+        sk.nks = (K + GEMM_BK - 1) / GEMM_BK;
+        sk.total = tiles_total * sk.nks;
+        const int64_t want = (int64_t)S.cus * std::min(streamk, tile == 0 ? 2 : 3);
+        int64_t per = (sk.total + want - 1) / want;
+        per = (per + 3) / 4 * 4; // no piece shorter than four K steps except at the end of K
+        sk.per_wg = per;
+        const int64_t wgs = (sk.total + per - 1) / per;
+        if (tiles_total <= 0x7fffffffLL && wgs >= 1) {
+            float* ws;
+            if (int rc = workspace((size_t)(2 * wgs) * bmt * bnt * sizeof(float), &ws)) return rc;
+            sk.partial = ws;
+            const bool need_fixup = per % sk.nks != 0;
+            if (S.verbose) fprintf(stderr, "tenmo_hip gemm stream-K: %lld workgroups x %lld K steps, %lld tiles of %dx%d\n", (long long)wgs, (long long)per, (long long)tiles_total, bmt, bnt);
+            if (tile == 0) return launch_streamk_tile<256, 128>(g, sk, (unsigned)wgs, tiles_total, need_fixup, am, bm);
+            return launch_streamk_tile<128, 128>(g, sk, (unsigned)wgs, tiles_total, need_fixup, am, bm);
+        }
+    }
     const int64_t nb = ((M + kTiles[tile].bm - 1) / kTiles[tile].bm) * ((N + kTiles[tile].bn - 1) / kTiles[tile].bn) * batch_count;
     g.k_splits = splits;
     g.k_per_split = K;
@@ -665,6 +728,7 @@ int tenmo_hip_init(int device_id) {
     HIP_TRY(hipMemcpy(S.one, &one, sizeof one, hipMemcpyHostToDevice));
     S.force_tile = env_int("TENMO_HIP_GEMM_TILE", -1);
     S.force_splitk = env_int("TENMO_HIP_GEMM_SPLITK", -1);
+    S.force_streamk = env_int("TENMO_HIP_GEMM_STREAMK", -1);
     S.verbose = env_int("TENMO_HIP_VERBOSE", 0);
     S.ready = true;
     return 0;
@@ -712,6 +776,7 @@ int tenmo_hip_set_tuning(const char* name, int value) {
     if (!name) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: null name");
     if (!strcmp(name, "gemm_tile")) { S.force_tile = value; return 0; }
     if (!strcmp(name, "gemm_splitk")) { S.force_splitk = value; return 0; }
+    if (!strcmp(name, "gemm_streamk")) { S.force_streamk = value; return 0; }
     if (!strcmp(name, "cols_wg_per_cu")) { S.cols_waves_per_cu = value > 0 ? value : 2; return 0; }
     return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: unknown knob '%s'", name);
 }

@@ -271,6 +271,48 @@ def test_column_sum(T):
     assert np.all(out.to_numpy() == 0)
 
 
+@pytest.mark.parametrize("tile", [0, 1])
+def test_stream_k(T, tile):
+    """Persistent stream-K launches: tiles shared between workgroups are summed by the fix-up kernel.
+    Shapes with fewer / more tiles than workgroups, ragged extents, K tails, transposed views, batches,
+    accumulate and the fused epilogue."""
+    L, lib = T.lib.load(), T.lib
+    rng = np.random.default_rng(53)
+    try:
+        L.tenmo_hip_set_tuning(b"gemm_tile", tile)
+        for wg_per_cu in (1, 2):
+            L.tenmo_hip_set_tuning(b"gemm_streamk", wg_per_cu)
+            for (bsz, m, k, n) in [(1, 768, 2000, 640), (1, 300, 4100, 200), (1, 2048, 512, 1536), (3, 260, 1000, 132), (1, 100, 64, 70), (1, 1500, 8192, 900)]:
+                a = rng.standard_normal((bsz, m, k), dtype=np.float32)
+                b = rng.standard_normal((k, n), dtype=np.float32)
+                ref = ref_matmul64(a, b)
+                A, B = T.Tensor.from_numpy(a), T.Tensor.from_numpy(b)
+                got = A.matmul(B, track_grad=False).to_numpy()
+                assert rel_fro(got, ref) <= RTOL_FRO, (tile, wg_per_cu, bsz, m, k, n)
+                # transposed views of both operands
+                At = T.Tensor.from_numpy(np.ascontiguousarray(a.transpose(0, 2, 1))).transpose()
+                Bt = T.Tensor.from_numpy(np.ascontiguousarray(b.T)).transpose()
+                got = At.matmul(Bt, track_grad=False).to_numpy()
+                assert rel_fro(got, ref) <= RTOL_FRO, (tile, wg_per_cu, bsz, m, k, n, "views")
+            # accumulate twice, then bias + ReLU through the fix-up
+            a = rng.standard_normal((700, 3000), dtype=np.float32)
+            b = rng.standard_normal((3000, 500), dtype=np.float32)
+            bias = rng.standard_normal(500).astype(np.float32)
+            A, B, Bi, out = T.Tensor.from_numpy(a), T.Tensor.from_numpy(b), T.Tensor.from_numpy(bias), T.Tensor.zeros(700, 500)
+            for _ in range(2):
+                lib.check(L.tenmo_hip_gemm_f32(A.buffer.data_ptr(), 0, 3000, 1, B.buffer.data_ptr(), 0, 500, 1, out.buffer.data_ptr(),
+                                               700, 500, 3000, 0, None, None, None, 1, 1))
+            assert rel_fro(out.to_numpy(), 2 * ref_matmul64(a, b)) <= RTOL_FRO
+            lib.check(L.tenmo_hip_gemm_epilogue_f32(A.buffer.data_ptr(), 0, 3000, 1, B.buffer.data_ptr(), 0, 500, 1, out.buffer.data_ptr(),
+                                                    700, 500, 3000, 0, None, None, None, Bi.buffer.data_ptr(), 1, None, 1))
+            z = ref_matmul64(a, b) + bias
+            near = np.abs(z) < 1e-3
+            assert rel_fro(np.where(near, 0, out.to_numpy()), np.where(near, 0, np.maximum(z, 0))) <= RTOL_FRO
+    finally:
+        L.tenmo_hip_set_tuning(b"gemm_tile", -1)
+        L.tenmo_hip_set_tuning(b"gemm_streamk", -1)
+
+
 def test_odd_strides_and_overlap(T, oracle):
     """Column stride 2, row stride 0 (broadcast rows), overlapping windows (tests/test_mmnd.mojo:143-175)."""
     rng = np.random.default_rng(23)
