@@ -2,17 +2,22 @@
 
     python -m tenmo_amd.build            # compile
 
-The library is built in-tree so that the copy of the tree that runs on the GPU machine carries it.
+The GEMM kernel is instantiated per workgroup tile in its own translation unit (``csrc/gemm_tiles.hip``
+compiled once per tile); the units are compiled in parallel and linked with the host side
+(``csrc/tenmo_hip.hip``).  The library is built in-tree so that the copy of the tree that runs on the
+GPU machine carries it.
 """
 from __future__ import annotations
 
 import os
 import subprocess
 import sys
+import tempfile
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
-SRC = os.path.join(HERE, "csrc", "tenmo_hip.hip")
+CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libtenmo_hip.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
@@ -22,25 +27,46 @@ FLAGS = [
     "-O3",
     "-std=c++17",
     "-fPIC",
-    "-shared",
     # packed fp32 instructions stay off: the compiler must not form v_pk_{add,mul,fma}_f32
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
     "-I", os.path.join(ROOT, "include"),
 ]
 
+# (rows, cols, part) units of the GEMM: part 0 = one workgroup per tile, 1 = the stream-K kernels
+TILES = [(256, 128, 0), (256, 128, 1), (128, 128, 0), (128, 128, 1), (64, 64, 0), (128, 64, 0), (64, 128, 0)]
+NOISE = "is not a recognized feature for this target"
+
+
+def _run(cmd):
+    res = subprocess.run(cmd, cwd=CSRC, capture_output=True, text=True)
+    err = "\n".join(l for l in res.stderr.splitlines() if NOISE not in l)
+    if res.returncode != 0:
+        raise RuntimeError("hipcc failed: " + " ".join(cmd) + "\n" + err)
+    return err
+
 
 def build(verbose: bool = False) -> str:
-    cmd = [HIPCC] + FLAGS + [SRC, "-o", LIB]
+    jobs = min(len(TILES) + 1, max(1, int(os.environ.get("MAX_JOBS", os.cpu_count() or 1))))
+    with tempfile.TemporaryDirectory(prefix="tenmo_hip_build_") as tmp:
+        units = [([os.path.join(CSRC, "tenmo_hip.hip")], os.path.join(tmp, "tenmo_hip.o"))]
+        for bm, bn, sk in TILES:
+            units.append(([f"-DTENMO_TILE_BM={bm}", f"-DTENMO_TILE_BN={bn}", f"-DTENMO_TILE_STREAMK={sk}",
+                           os.path.join(CSRC, "gemm_tiles.hip")], os.path.join(tmp, f"gemm_{bm}x{bn}_{sk}.o")))
+        cmds = [[HIPCC] + FLAGS + ["-c"] + src + ["-o", obj] for src, obj in units]
+        if verbose:
+            for c in cmds:
+                print(" ".join(c), flush=True)
+        with ThreadPoolExecutor(max_workers=jobs) as pool:
+            errs = list(pool.map(_run, cmds))
+        link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + [obj for _, obj in units] + ["-o", LIB]
+        if verbose:
+            print(" ".join(link), flush=True)
+        errs.append(_run(link))
     if verbose:
-        print(" ".join(cmd), flush=True)
-    res = subprocess.run(cmd, cwd=os.path.join(HERE, "csrc"), capture_output=True, text=True)
-    noise = "is not a recognized feature for this target"
-    err = "\n".join(l for l in res.stderr.splitlines() if noise not in l)
-    if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + err)
-    if verbose and err.strip():
-        print(err)
+        for e in errs:
+            if e.strip():
+                print(e)
     return LIB
 
 

@@ -209,4 +209,26 @@ __global__ void sgd_step_kernel(float* __restrict p, const float* __restrict g, 
     }
 }
 
+// Sums the k_splits partial results into C (plain or accumulating), slices in a fixed order, then
+// applies the fused epilogue.  One thread per output; eight slice loads in flight per thread.
+__global__ void splitk_reduce_kernel(const float* __restrict partial, float* __restrict C, int64_t n, int splits, int accumulate,
+                                     const float* __restrict bias, const float* __restrict mask, int relu, int64_t N) {
+    int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) {
+        float s = accumulate ? C[i] : 0.f;
+        int p = 0;
+        for (; p + 8 <= splits; p += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v[u] = partial[(int64_t)(p + u) * n + i];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) s += v[u];
+        }
+        for (; p < splits; ++p) s += partial[(int64_t)p * n + i];
+        if (bias || mask || relu) s = epilogue_value(s, bias, mask, relu, i, i % N);
+        C[i] = s;
+    }
+}
+
 } // namespace tenmo

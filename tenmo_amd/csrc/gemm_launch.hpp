@@ -1,0 +1,22 @@
+// Launchers of the GEMM kernel instantiations.  Each workgroup tile is compiled in its own
+// translation unit (gemm_tiles.hip, once per tile) so that the build runs them in parallel.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#include "gemm_mfma.hpp"
+
+namespace tenmo {
+
+// One workgroup per tile (grid.y = K slices).  false: no variant for these operand modes.
+bool launch_gemm_256x128(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream);
+bool launch_gemm_128x128(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream);
+bool launch_gemm_64x64(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream);
+bool launch_gemm_128x64(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream);
+bool launch_gemm_64x128(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream);
+
+// Stream-K: `wgs` persistent workgroups, then the fix-up over `tiles` tiles in `fix_parts` parts
+// each (0: no tile is shared, no fix-up).  Vector operand modes only.
+bool launch_streamk_256x128(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);
+bool launch_streamk_128x128(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);
+
+} // namespace tenmo

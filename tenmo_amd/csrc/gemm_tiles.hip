@@ -1,0 +1,44 @@
+// The instantiations of gemm_mfma_kernel (and, for the two large tiles, gemm_streamk_kernel) for ONE
+// workgroup tile, selected with -DTENMO_TILE_BM / -DTENMO_TILE_BN.  -DTENMO_TILE_STREAMK=0 compiles the
+// one-workgroup-per-tile kernels, =1 the stream-K kernels of that tile.  tenmo_amd/build.py compiles
+// this file once per (tile, part), in parallel.
+#include "gemm_launch.hpp"
+
+#ifndef TENMO_TILE_BM
+#error "compile with -DTENMO_TILE_BM=<rows> -DTENMO_TILE_BN=<cols>"
+#endif
+#define TENMO_PASTE3(a, b, c, d) a##b##c##d
+#define TENMO_NAME(prefix, bm, bn) TENMO_PASTE3(prefix, bm, x, bn)
+
+namespace tenmo {
+
+#if !TENMO_TILE_STREAMK
+bool TENMO_NAME(launch_gemm_, TENMO_TILE_BM, TENMO_TILE_BN)(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream) {
+    constexpr int BM = TENMO_TILE_BM, BN = TENMO_TILE_BN;
+#define TENMO_CASE(A_, B_)                                                                                     \
+    if (amode == A_ && bmode == B_) {                                                                          \
+        hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, A_, B_>), grid, dim3(GEMM_THREADS), 0, stream, g);        \
+        return true;                                                                                           \
+    }
+    TENMO_CASE(KMAJOR_VEC, KMAJOR_VEC) TENMO_CASE(KMAJOR_VEC, MNMAJOR_VEC) TENMO_CASE(KMAJOR_VEC, KMAJOR_GEN)
+    TENMO_CASE(MNMAJOR_VEC, KMAJOR_VEC) TENMO_CASE(MNMAJOR_VEC, MNMAJOR_VEC) TENMO_CASE(MNMAJOR_VEC, KMAJOR_GEN)
+    TENMO_CASE(KMAJOR_GEN, KMAJOR_VEC) TENMO_CASE(KMAJOR_GEN, MNMAJOR_VEC) TENMO_CASE(KMAJOR_GEN, KMAJOR_GEN)
+#undef TENMO_CASE
+    return false;
+}
+#else
+bool TENMO_NAME(launch_streamk_, TENMO_TILE_BM, TENMO_TILE_BN)(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles,
+                                                              unsigned fix_parts, int amode, int bmode, hipStream_t stream) {
+    constexpr int BM = TENMO_TILE_BM, BN = TENMO_TILE_BN;
+#define TENMO_CASE(A_, B_)                                                                                               \
+    if (amode == A_ && bmode == B_)                                                                                      \
+        hipLaunchKernelGGL((gemm_streamk_kernel<BM, BN, A_, B_>), dim3(wgs), dim3(GEMM_THREADS), 0, stream, g, sk);
+    TENMO_CASE(KMAJOR_VEC, KMAJOR_VEC) else TENMO_CASE(KMAJOR_VEC, MNMAJOR_VEC) else TENMO_CASE(MNMAJOR_VEC, KMAJOR_VEC) else TENMO_CASE(MNMAJOR_VEC, MNMAJOR_VEC)
+    else return false;
+#undef TENMO_CASE
+    if (fix_parts) hipLaunchKernelGGL((streamk_fixup_kernel<BM, BN>), dim3(tiles, fix_parts), dim3(256), 0, stream, g, sk);
+    return true;
+}
+#endif
+
+} // namespace tenmo

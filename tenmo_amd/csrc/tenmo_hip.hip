@@ -23,8 +23,8 @@
 
 #include "../../include/tenmo_hip.h"
 #include "cross_entropy.hpp"
+#include "gemm_launch.hpp"
 #include "elementwise.hpp"
-#include "gemm_mfma.hpp"
 #include "gemv.hpp"
 
 using namespace tenmo;
@@ -164,37 +164,6 @@ int operand_mode(int64_t row_stride, int64_t k_stride, int64_t rows, int64_t K) 
     return KMAJOR_GEN;
 }
 
-template <int BM, int BN, int AM, int BMo>
-void launch_gemm_variant(const GemmArgs& g, dim3 grid) {
-    hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, AM, BMo>), grid, dim3(GEMM_THREADS), 0, S.stream, g);
-}
-
-template <int BM, int BN>
-int launch_gemm_tile(const GemmArgs& g, dim3 grid, int am, int bm) {
-#define TENMO_CASE(A_, B_) if (am == A_ && bm == B_) { launch_gemm_variant<BM, BN, A_, B_>(g, grid); return 0; }
-    TENMO_CASE(KMAJOR_VEC, KMAJOR_VEC) TENMO_CASE(KMAJOR_VEC, MNMAJOR_VEC) TENMO_CASE(KMAJOR_VEC, KMAJOR_GEN)
-    TENMO_CASE(MNMAJOR_VEC, KMAJOR_VEC) TENMO_CASE(MNMAJOR_VEC, MNMAJOR_VEC) TENMO_CASE(MNMAJOR_VEC, KMAJOR_GEN)
-    TENMO_CASE(KMAJOR_GEN, KMAJOR_VEC) TENMO_CASE(KMAJOR_GEN, MNMAJOR_VEC) TENMO_CASE(KMAJOR_GEN, KMAJOR_GEN)
-#undef TENMO_CASE
-    return fail(TENMO_ERR_UNSUPPORTED, "no GEMM variant for operand modes %d/%d", am, bm);
-}
-
-// stream-K: persistent workgroups + fix-up of the shared tiles (vector operand modes only)
-template <int BM, int BN>
-int launch_streamk_tile(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, int64_t tiles_total, bool need_fixup, int am, int bm) {
-#define TENMO_CASE(A_, B_) if (am == A_ && bm == B_) { hipLaunchKernelGGL((gemm_streamk_kernel<BM, BN, A_, B_>), dim3(wgs), dim3(GEMM_THREADS), 0, S.stream, g, sk); }
-    TENMO_CASE(KMAJOR_VEC, KMAJOR_VEC) else TENMO_CASE(KMAJOR_VEC, MNMAJOR_VEC) else TENMO_CASE(MNMAJOR_VEC, KMAJOR_VEC) else TENMO_CASE(MNMAJOR_VEC, MNMAJOR_VEC)
-    else return fail(TENMO_ERR_UNSUPPORTED, "no stream-K variant for operand modes %d/%d", am, bm);
-#undef TENMO_CASE
-    if (need_fixup) {
-        // parts per tile: a power of two that brings the launch to a few workgroups per CU
-        unsigned parts = 1;
-        while (parts < 32 && (int64_t)tiles_total * parts < (int64_t)S.cus * 4) parts *= 2;
-        hipLaunchKernelGGL((streamk_fixup_kernel<BM, BN>), dim3((unsigned)tiles_total, parts), dim3(256), 0, S.stream, g, sk);
-    }
-    return 0;
-}
-
 struct TileShape { int bm, bn; };
 constexpr int kNumTiles = 5;
 const TileShape kTiles[kNumTiles] = {{256, 128}, {128, 128}, {64, 64}, {128, 64}, {64, 128}};
@@ -308,8 +277,12 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
             sk.partial = ws;
             const bool need_fixup = per % sk.nks != 0;
             if (S.verbose) fprintf(stderr, "tenmo_hip gemm stream-K: %lld workgroups x %lld K steps, %lld tiles of %dx%d\n", (long long)wgs, (long long)per, (long long)tiles_total, bmt, bnt);
-            if (tile == 0) return launch_streamk_tile<256, 128>(g, sk, (unsigned)wgs, tiles_total, need_fixup, am, bm);
-            return launch_streamk_tile<128, 128>(g, sk, (unsigned)wgs, tiles_total, need_fixup, am, bm);
+            // parts per shared tile in the fix-up: a power of two that brings it to a few workgroups per CU
+            unsigned parts = 0;
+            if (need_fixup) for (parts = 1; parts < 32 && tiles_total * parts < (int64_t)S.cus * 4; parts *= 2) {}
+            const bool ok = tile == 0 ? launch_streamk_256x128(g, sk, (unsigned)wgs, (unsigned)tiles_total, parts, am, bm, S.stream)
+                                      : launch_streamk_128x128(g, sk, (unsigned)wgs, (unsigned)tiles_total, parts, am, bm, S.stream);
+            return ok ? 0 : fail(TENMO_ERR_UNSUPPORTED, "no stream-K variant for operand modes %d/%d", am, bm);
         }
     }
     const int64_t nb = ((M + kTiles[tile].bm - 1) / kTiles[tile].bm) * ((N + kTiles[tile].bn - 1) / kTiles[tile].bn) * batch_count;
@@ -331,15 +304,15 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     g.tiles_n = (int32_t)((N + kTiles[tile].bn - 1) / kTiles[tile].bn);
     if (nb > 0x7fffffffLL) return fail(TENMO_ERR_UNSUPPORTED, "grid too large");
     dim3 grid((unsigned)nb, (unsigned)splits, 1);
-    int rc = 0;
+    bool ok = false;
     switch (tile) {
-        case 0: rc = launch_gemm_tile<256, 128>(g, grid, am, bm); break;
-        case 1: rc = launch_gemm_tile<128, 128>(g, grid, am, bm); break;
-        case 3: rc = launch_gemm_tile<128, 64>(g, grid, am, bm); break;
-        case 4: rc = launch_gemm_tile<64, 128>(g, grid, am, bm); break;
-        default: rc = launch_gemm_tile<64, 64>(g, grid, am, bm); break;
+        case 0: ok = launch_gemm_256x128(g, grid, am, bm, S.stream); break;
+        case 1: ok = launch_gemm_128x128(g, grid, am, bm, S.stream); break;
+        case 3: ok = launch_gemm_128x64(g, grid, am, bm, S.stream); break;
+        case 4: ok = launch_gemm_64x128(g, grid, am, bm, S.stream); break;
+        default: ok = launch_gemm_64x64(g, grid, am, bm, S.stream); break;
     }
-    if (rc) return rc;
+    if (!ok) return fail(TENMO_ERR_UNSUPPORTED, "no GEMM variant for operand modes %d/%d", am, bm);
     if (splits > 1) {
         const int64_t n = batch_count * M * N;
         hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
