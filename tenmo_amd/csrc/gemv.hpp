@@ -137,15 +137,55 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
     const int64_t k_end = min(g.k, k_begin + g.k_per_split);
     const bool full = (col0 + 3 * CSTEP < g.n);
     const bool any = (col0 < g.n);
+    // whether every lane of this wavefront has its four columns inside the row (wave-uniform)
+    const bool wave_full = (col0 + (63 - (t & 63)) * (ALIGNED ? 4 : 1) + 3 * CSTEP < g.n);
 
     f32x4 acc[R];
 #pragma unroll
     for (int r = 0; r < R; ++r) acc[r] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-    auto load4 = [&](const float* __restrict p) -> f32x4 {
+    auto load_full = [&](const float* __restrict p) -> f32x4 {
         if constexpr (ALIGNED) return __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(p));
         else return f32x4{__builtin_nontemporal_load(p), __builtin_nontemporal_load(p + CSTEP),
                           __builtin_nontemporal_load(p + 2 * CSTEP), __builtin_nontemporal_load(p + 3 * CSTEP)};
+    };
+    // Ragged wavefront (the row ends inside it): columns past the end are moved onto the last valid
+    // one, so the loads stay unconditional and as many are in flight as on the fast path; what they
+    // bring is never stored.
+    int64_t coff[4];
+#pragma unroll
+    for (int e = 0; e < 4; ++e) coff[e] = min(col0 + e * CSTEP, g.n - 1) - col0;
+    auto load_clamped = [&](const float* __restrict p) -> f32x4 {
+        return f32x4{__builtin_nontemporal_load(p + coff[0]), __builtin_nontemporal_load(p + coff[1]),
+                     __builtin_nontemporal_load(p + coff[2]), __builtin_nontemporal_load(p + coff[3])};
+    };
+    // U independent row loads in flight per lane; the last batch of a chunk re-reads row len-1 for
+    // the rows it lacks and drops them.
+    auto stream = [&](const float* __restrict p, int len, auto load4) {
+        constexpr int U = 8;
+        int kk = 0;
+        for (; kk + U <= len; kk += U) {
+            f32x4 m[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) m[u] = load4(p + (int64_t)(kk + u) * g.m_rs);
+            __builtin_amdgcn_sched_barrier(0); // all U loads are issued before the first use
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[r] += m[u] * xs[r][kk + u];
+        }
+        if (kk < len) {
+            f32x4 m[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) m[u] = load4(p + (int64_t)min(kk + u, len - 1) * g.m_rs);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (kk + u >= len) m[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[r] += m[u] * xs[r][kk + u]; // xs is zero past len
+            }
+        }
     };
 
     for (int64_t kc = k_begin; kc < k_end; kc += COLS_KCHUNK) {
@@ -156,36 +196,9 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
             xs[r][kk] = (r < g.rows && kk < len) ? Xb[(int64_t)r * g.x_rs + (kc + kk) * g.x_ks] : 0.f;
         }
         __syncthreads();
-        if (full) {
-            const float* __restrict p = Mb + kc * g.m_rs + col0;
-            int kk = 0;
-            constexpr int U = 8; // independent row loads in flight per lane
-            for (; kk + U <= len; kk += U) {
-                f32x4 m[U];
-#pragma unroll
-                for (int u = 0; u < U; ++u) m[u] = load4(p + (int64_t)(kk + u) * g.m_rs);
-#pragma unroll
-                for (int u = 0; u < U; ++u)
-#pragma unroll
-                    for (int r = 0; r < R; ++r) acc[r] += m[u] * xs[r][kk + u];
-            }
-            for (; kk < len; ++kk) {
-                const f32x4 m0 = load4(p + (int64_t)kk * g.m_rs);
-#pragma unroll
-                for (int r = 0; r < R; ++r) acc[r] += m0 * xs[r][kk];
-            }
-        } else if (any) {
-            for (int kk = 0; kk < len; ++kk) {
-                const float* p = Mb + (kc + kk) * g.m_rs + col0;
-                f32x4 m0 = {0.f, 0.f, 0.f, 0.f};
-                m0.x = p[0];
-                if (col0 + CSTEP < g.n) m0.y = p[CSTEP];
-                if (col0 + 2 * CSTEP < g.n) m0.z = p[2 * CSTEP];
-                if (col0 + 3 * CSTEP < g.n) m0.w = p[3 * CSTEP];
-#pragma unroll
-                for (int r = 0; r < R; ++r) acc[r] += m0 * xs[r][kk];
-            }
-        }
+        const float* __restrict p = Mb + kc * g.m_rs + col0;
+        if (wave_full) stream(p, len, load_full);
+        else if (any) stream(p, len, load_clamped);
     }
     if (!any) return;
     const bool to_partial = g.k_splits > 1;
@@ -204,6 +217,134 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
 #pragma unroll
             for (int e = 0; e < 4; ++e)
                 if (col0 + e * CSTEP < g.n) o[e * CSTEP] = accumulate ? o[e * CSTEP] + a[e] : a[e];
+        }
+    }
+}
+
+// ---- columns kernel for rows that do not start on 16-byte boundaries ---------------------------
+// Same job as cols_kernel, for a matrix whose first row IS 16-byte aligned but whose row pitch is
+// not a multiple of 4 floats (N = 50257): row r then starts m(r) = (r * pitch) % 4 elements past a
+// 16-byte boundary, and m depends only on r % 4.  Every lane still moves one ALIGNED 16-byte group
+// per row — the group that starts m(r) elements before its nominal columns — and keeps one
+// accumulator set per r % 4, so that a set always holds the same four columns.  At the end the four
+// sets are shifted back by their m through LDS and added.  Because a set's columns reach up to three
+// to the left of the nominal ones, a workgroup produces COLS_SHIFT_WIDTH = 1020 outputs from 1024
+// loaded columns.  The last row of the matrix is read element by element (an aligned group there
+// could end past the allocation); groups of other rows that run past the row end read the next
+// row's first elements, which are discarded.
+constexpr int COLS_SHIFT_WIDTH = COLS_THREADS * 4 - 4;
+
+template <int R>
+__global__ __launch_bounds__(COLS_THREADS) void cols_shift_kernel(const ColsArgs g) {
+    __shared__ float xs[R][COLS_KCHUNK];
+    __shared__ float outs[R][COLS_THREADS * 4 + 4];
+    const int t = threadIdx.x;
+    const int64_t block0 = (int64_t)blockIdx.x * COLS_SHIFT_WIDTH; // first output column of the workgroup
+    const int64_t batch = blockIdx.z;
+    int64_t x_off, m_off;
+    batch_offsets(g.batch, batch, x_off, m_off);
+    const float* __restrict Xb = g.X + x_off;
+    const float* __restrict Mb = g.Mx + m_off; // 16-byte aligned (the host checks)
+    const int64_t k_begin = (int64_t)blockIdx.y * g.k_per_split; // a multiple of 4
+    const int64_t k_end = min(g.k, k_begin + g.k_per_split);
+    const int64_t k_vec_end = min(k_end, g.k - 1);                // the matrix's last row is done apart
+    int mj[4]; // misalignment of the rows with r % 4 == j
+#pragma unroll
+    for (int j = 0; j < 4; ++j) mj[j] = (int)((j * (g.m_rs & 3)) & 3);
+
+    f32x4 acc[4][R];
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < R; ++r) acc[j][r] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // First column of this lane's group for class j.  A group that lies wholly beyond the row is
+    // moved back by whole groups onto the last one that starts inside it: the load stays unconditional
+    // and in bounds, and what it brings lands in output columns >= n, which are never stored.
+    int64_t c0[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        c0[j] = block0 - mj[j] + 4 * t;
+        if (c0[j] >= g.n) c0[j] -= 4 * ((c0[j] - g.n) / 4 + 1);
+    }
+
+    for (int64_t kc = k_begin; kc < k_end; kc += COLS_KCHUNK) {
+        const int len = (int)min((int64_t)COLS_KCHUNK, k_end - kc);
+        const int vlen = (int)max((int64_t)0, min((int64_t)len, k_vec_end - kc));
+        __syncthreads();
+        for (int idx = t; idx < R * COLS_KCHUNK; idx += COLS_THREADS) {
+            const int r = idx / COLS_KCHUNK, kk = idx % COLS_KCHUNK;
+            xs[r][kk] = (r < g.rows && kk < len) ? Xb[(int64_t)r * g.x_rs + (kc + kk) * g.x_ks] : 0.f;
+        }
+        __syncthreads();
+        int kk = 0;
+        constexpr int U = 8;
+        const float* __restrict pc = Mb + kc * g.m_rs;
+        for (; kk + U <= vlen; kk += U) { // kc + kk is a multiple of 4: row kk + u has class u % 4
+            f32x4 m[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+                m[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(pc + (int64_t)(kk + u) * g.m_rs + c0[u & 3]));
+            __builtin_amdgcn_sched_barrier(0); // all U loads are issued before the first use
+#pragma unroll
+            for (int u = 0; u < U; ++u)
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[u & 3][r] += m[u] * xs[r][kk + u];
+        }
+        if (kk < vlen) { // last batch of the chunk: the rows it lacks re-read the chunk's first row and are dropped
+            f32x4 m[U];
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const bool ok = kk + u < vlen;
+                m[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4*>(pc + (int64_t)(ok ? kk + u : 0) * g.m_rs + (ok ? c0[u & 3] : c0[0])));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                if (kk + u >= vlen) m[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int r = 0; r < R; ++r) acc[u & 3][r] += m[u] * xs[r][kk + u];
+            }
+        }
+        if (vlen < len) { // the matrix's last row: element by element, bounds-checked
+            const int kl = vlen;
+            const int j = (int)((kc + kl) & 3);
+            const float* __restrict row = pc + (int64_t)kl * g.m_rs;
+            const int64_t c = block0 - mj[j] + 4 * t;
+            f32x4 m0 = {0.f, 0.f, 0.f, 0.f};
+            if (c >= 0 && c < g.n) m0.x = row[c];
+            if (c + 1 >= 0 && c + 1 < g.n) m0.y = row[c + 1];
+            if (c + 2 >= 0 && c + 2 < g.n) m0.z = row[c + 2];
+            if (c + 3 >= 0 && c + 3 < g.n) m0.w = row[c + 3];
+#pragma unroll
+            for (int jj = 0; jj < 4; ++jj)
+                if (jj == j)
+#pragma unroll
+                    for (int r = 0; r < R; ++r) acc[jj][r] += m0 * xs[r][kl];
+        }
+    }
+    // shift the four sets back and add them: set j's element e of lane t is column block0 - mj + 4t + e
+    for (int idx = t; idx < R * (COLS_THREADS * 4 + 4); idx += COLS_THREADS) (&outs[0][0])[idx] = 0.f;
+    __syncthreads();
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+#pragma unroll
+        for (int r = 0; r < R; ++r) {
+            float* o = &outs[r][4 * t + 3 - mj[j]]; // local column + 3
+            o[0] += acc[j][r].x; o[1] += acc[j][r].y; o[2] += acc[j][r].z; o[3] += acc[j][r].w;
+        }
+        __syncthreads();
+    }
+    const bool to_partial = g.k_splits > 1;
+    float* __restrict ob = g.out + ((to_partial ? (int64_t)blockIdx.y * gridDim.z : 0) + batch) * g.rows * g.n;
+    const bool accumulate = g.accumulate && !to_partial;
+    for (int r = 0; r < R; ++r) {
+        if (r >= g.rows) break;
+        for (int c = t; c < COLS_SHIFT_WIDTH; c += COLS_THREADS) {
+            const int64_t col = block0 + c;
+            if (col < g.n) {
+                float* o = ob + (int64_t)r * g.n + col;
+                *o = accumulate ? *o + outs[r][c + 3] : outs[r][c + 3];
+            }
         }
     }
 }

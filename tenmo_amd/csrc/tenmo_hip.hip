@@ -334,6 +334,57 @@ bool cols_aligned(const ColsArgs& c) {
     return true;
 }
 
+// the first row of every batch is 16-byte aligned but the row pitch is not a multiple of 4 floats:
+// cols_shift_kernel keeps every load aligned (up to 4 left-operand rows)
+bool cols_shiftable(const ColsArgs& c) {
+    if ((uintptr_t)c.Mx % 16 != 0 || c.m_rs % 4 == 0 || c.m_rs < c.n || c.n < 4 || c.rows > 4) return false;
+    for (int d = 0; d < c.batch.rank; ++d) if (c.batch.b_str[d] % 4 != 0) return false;
+    return true;
+}
+
+template <int R>
+void launch_cols(const ColsArgs& c, dim3 grid, int variant) {
+    if (variant == 0) hipLaunchKernelGGL((cols_kernel<R, true>), grid, dim3(COLS_THREADS), 0, S.stream, c);
+    else if (variant == 2) hipLaunchKernelGGL((cols_kernel<R, false>), grid, dim3(COLS_THREADS), 0, S.stream, c);
+    else if constexpr (R <= 4) hipLaunchKernelGGL((cols_shift_kernel<R>), grid, dim3(COLS_THREADS), 0, S.stream, c);
+}
+
+// Runs the column-streaming product described by `c` (c.out is set here): picks the kernel variant,
+// cuts K into slices when the column blocks alone would not fill the chip, and adds the slices.
+int cols_run(ColsArgs c, int64_t batch_count, float* out, int accumulate) {
+    const int variant = cols_aligned(c) ? 0 : cols_shiftable(c) ? 1 : 2; // 16-byte loads / shifted sets / dword loads
+    const int64_t width = variant == 1 ? COLS_SHIFT_WIDTH : COLS_THREADS * 4;
+    const int64_t col_blocks = (c.n + width - 1) / width;
+    const int64_t K = c.k, R = c.rows;
+    int64_t splits = 1;
+    const int64_t want = (int64_t)S.cus * S.cols_waves_per_cu;
+    if (col_blocks * batch_count < want) splits = std::min<int64_t>((want + col_blocks * batch_count - 1) / (col_blocks * batch_count), (K + COLS_KSLICE_MIN - 1) / COLS_KSLICE_MIN);
+    splits = std::max<int64_t>(1, std::min<int64_t>(splits, 65535));
+    int64_t per = (K + splits - 1) / splits;
+    per = (per + COLS_KSLICE_MIN - 1) / COLS_KSLICE_MIN * COLS_KSLICE_MIN;
+    splits = (K + per - 1) / per;
+    c.k_splits = (int32_t)splits; c.k_per_split = per;
+    c.accumulate = accumulate;
+    float* target = out;
+    if (splits > 1) {
+        float* ws;
+        if (int rc = workspace((size_t)splits * batch_count * R * c.n * sizeof(float), &ws)) return rc;
+        target = ws;
+    }
+    c.out = target;
+    const dim3 grid((unsigned)col_blocks, (unsigned)splits, (unsigned)batch_count);
+    if (R <= 1) launch_cols<1>(c, grid, variant);
+    else if (R <= 2) launch_cols<2>(c, grid, variant);
+    else if (R <= 4) launch_cols<4>(c, grid, variant);
+    else launch_cols<8>(c, grid, variant);
+    if (splits > 1) {
+        const int64_t n = batch_count * R * c.n;
+        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
+                           target, out, n, (int)splits, accumulate, (const float*)nullptr, (const float*)nullptr, 0, (int64_t)1);
+    }
+    return 0;
+}
+
 // out[b][i] = sum_j Mat[b](i, j) * vec[b](j), i < n_out, j < n_red;  Mat(i,j) = Mx[i*out_s + j*red_s]
 int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* vec, int64_t v_s, float* out,
                     int64_t n_out, int64_t n_red, const BatchDesc& bd_mat_vec, int64_t batch_count, int accumulate) {
@@ -380,29 +431,7 @@ int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* 
         // in ColsArgs the X operand uses a_str and the matrix b_str: swap relative to (matrix, vector)
         c.batch = bd_mat_vec;
         for (int d = 0; d < MAX_BATCH_RANK; ++d) std::swap(c.batch.a_str[d], c.batch.b_str[d]);
-        const int64_t col_blocks = (n_out + COLS_THREADS * 4 - 1) / (COLS_THREADS * 4);
-        int64_t splits = 1;
-        const int64_t want = (int64_t)S.cus * S.cols_waves_per_cu;
-        if (col_blocks * batch_count < want) splits = std::min<int64_t>((want + col_blocks * batch_count - 1) / (col_blocks * batch_count), (n_red + COLS_KSLICE_MIN - 1) / COLS_KSLICE_MIN);
-        splits = std::max<int64_t>(1, std::min<int64_t>(splits, 65535));
-        int64_t per = (n_red + splits - 1) / splits;
-        per = (per + COLS_KSLICE_MIN - 1) / COLS_KSLICE_MIN * COLS_KSLICE_MIN;
-        splits = (n_red + per - 1) / per;
-        c.k_splits = (int32_t)splits; c.k_per_split = per;
-        float* target = out;
-        if (splits > 1) {
-            float* ws;
-            if (int rc = workspace((size_t)splits * batch_count * n_out * sizeof(float), &ws)) return rc;
-            target = ws;
-        }
-        c.out = target;
-        if (cols_aligned(c)) hipLaunchKernelGGL((cols_kernel<1, true>), dim3((unsigned)col_blocks, (unsigned)splits, (unsigned)batch_count), dim3(COLS_THREADS), 0, S.stream, c);
-        else hipLaunchKernelGGL((cols_kernel<1, false>), dim3((unsigned)col_blocks, (unsigned)splits, (unsigned)batch_count), dim3(COLS_THREADS), 0, S.stream, c);
-        if (splits > 1) {
-            const int64_t n = batch_count * n_out;
-            hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
-                               target, out, n, (int)splits, accumulate, (const float*)nullptr, (const float*)nullptr, 0, (int64_t)1);
-        }
+        if (int rc = cols_run(c, batch_count, out, accumulate)) return rc;
         return 0;
     }
     GemvArgs g{};
@@ -413,43 +442,12 @@ int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* 
 }
 
 // skinny GEMM: M <= 8 rows against a row-major B — the matrix is streamed once, like vm
-template <int R>
-void launch_cols(const ColsArgs& c, dim3 grid) {
-    if (cols_aligned(c)) hipLaunchKernelGGL((cols_kernel<R, true>), grid, dim3(COLS_THREADS), 0, S.stream, c);
-    else hipLaunchKernelGGL((cols_kernel<R, false>), grid, dim3(COLS_THREADS), 0, S.stream, c);
-}
-
 int skinny_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, int64_t b_rs, float* C,
                     int64_t M, int64_t N, int64_t K, const BatchDesc& bd, int64_t batch_count, int accumulate) {
     ColsArgs c{};
     c.X = A; c.Mx = B; c.x_rs = a_rs; c.x_ks = a_cs; c.m_rs = b_rs; c.k = K; c.n = N; c.rows = (int32_t)M; c.accumulate = accumulate;
     c.batch = bd;
-    const int64_t col_blocks = (N + COLS_THREADS * 4 - 1) / (COLS_THREADS * 4);
-    int64_t splits = 1;
-    const int64_t want = (int64_t)S.cus * S.cols_waves_per_cu;
-    if (col_blocks * batch_count < want) splits = std::min<int64_t>((want + col_blocks * batch_count - 1) / (col_blocks * batch_count), (K + COLS_KSLICE_MIN - 1) / COLS_KSLICE_MIN);
-    splits = std::max<int64_t>(1, std::min<int64_t>(splits, 65535));
-    int64_t per = (K + splits - 1) / splits;
-    per = (per + COLS_KSLICE_MIN - 1) / COLS_KSLICE_MIN * COLS_KSLICE_MIN;
-    splits = (K + per - 1) / per;
-    c.k_splits = (int32_t)splits; c.k_per_split = per;
-    float* target = C;
-    if (splits > 1) {
-        float* ws;
-        if (int rc = workspace((size_t)splits * batch_count * M * N * sizeof(float), &ws)) return rc;
-        target = ws;
-    }
-    c.out = target;
-    dim3 grid((unsigned)col_blocks, (unsigned)splits, (unsigned)batch_count);
-    if (M <= 1) launch_cols<1>(c, grid);
-    else if (M <= 2) launch_cols<2>(c, grid);
-    else if (M <= 4) launch_cols<4>(c, grid);
-    else launch_cols<8>(c, grid);
-    if (splits > 1) {
-        const int64_t n = batch_count * M * N;
-        hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
-                           target, C, n, (int)splits, accumulate, (const float*)nullptr, (const float*)nullptr, 0, (int64_t)1);
-    }
+    if (int rc = cols_run(c, batch_count, C, accumulate)) return rc;
     return 0;
 }
 

@@ -313,6 +313,38 @@ def test_stream_k(T, tile):
         L.tenmo_hip_set_tuning(b"gemm_streamk", -1)
 
 
+def test_columns_with_misaligned_row_pitch(T):
+    """vm and skinny products against a matrix whose row pitch is not a multiple of 4 floats (rows start
+    at every 16-byte phase): the shifted-accumulator kernel, its K slices, its last-row and edge handling,
+    batches, and the fall-backs (5..8 left rows, unaligned base)."""
+    rng = np.random.default_rng(59)
+    for (m, k, n) in [(1, 37, 4099), (1, 1000, 10007), (3, 768, 50257), (4, 129, 2051), (2, 64, 5001), (6, 200, 3001), (4, 5, 7), (1, 4097, 1021)]:
+        a = rng.standard_normal((m, k), dtype=np.float32)
+        b = rng.standard_normal((k, n), dtype=np.float32)
+        ref = ref_matmul64(a, b)
+        A, B = T.Tensor.from_numpy(a), T.Tensor.from_numpy(b)
+        if m == 1:
+            got = T.Tensor.from_numpy(a[0]).matmul(B, track_grad=False).to_numpy()      # vector x matrix
+            assert rel_fro(got, ref[0]) <= RTOL_FRO, ("vm", k, n)
+        got = A.matmul(B, track_grad=False).to_numpy()
+        assert rel_fro(got, ref) <= RTOL_FRO, (m, k, n)
+        # the same matrix one element into its storage: the base is no longer 16-byte aligned
+        store = np.zeros(k * n + 1, np.float32)
+        store[1:] = b.ravel()
+        Bo = T.Tensor.from_numpy(store).view((k, n), (n, 1), 1)
+        assert rel_fro(A.matmul(Bo, track_grad=False).to_numpy(), ref) <= RTOL_FRO, (m, k, n, "offset 1")
+        # padded rows (pitch n + 2)
+        padded = np.zeros((k, n + 2), np.float32)
+        padded[:, :n] = b
+        Bp = T.Tensor.from_numpy(padded.ravel()).view((k, n), (n + 2, 1), 0)
+        assert rel_fro(A.matmul(Bp, track_grad=False).to_numpy(), ref) <= RTOL_FRO, (m, k, n, "padded")
+    # batched right operand with an odd pitch and batch stride multiple of 4
+    a = rng.standard_normal((2, 768), dtype=np.float32)
+    b = rng.standard_normal((4, 768, 2503), dtype=np.float32)
+    got = T.Tensor.from_numpy(a).matmul(T.Tensor.from_numpy(b), track_grad=False).to_numpy()
+    assert rel_fro(got, ref_matmul64(a, b)) <= RTOL_FRO
+
+
 def test_odd_strides_and_overlap(T, oracle):
     """Column stride 2, row stride 0 (broadcast rows), overlapping windows (tests/test_mmnd.mojo:143-175)."""
     rng = np.random.default_rng(23)
