@@ -7,6 +7,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 #include "gemm_mfma.hpp"
 
 namespace tenmo {
@@ -28,69 +29,72 @@ struct GemvArgs {
 };
 
 // ---- rows kernel: unit stride along the reduction (row-major matrix . vector) ----------------
-// One wavefront owns R consecutive rows; its 64 lanes walk k in 16-byte steps, so every global
-// load instruction of a row is one contiguous 1 KiB burst.  R rows share each vector load.
+// WPR wavefronts (1 or 4) own one row and walk it in 16-byte steps per lane, UNROLL steps in flight:
+// the row is read as contiguous bursts of WPR x UNROLL KiB, which is what HBM streams best (several
+// rows per wavefront interleave short bursts of distant rows and lose 5-20%).  With WPR = 1 the four
+// wavefronts of a workgroup take four consecutive rows; WPR = 4 is for few, long rows.
 constexpr int MV_WAVES = 4;
-template <int R, int UNROLL>
+template <int WPR, int UNROLL, bool V_UNIT>
 __global__ __launch_bounds__(64 * MV_WAVES) void mv_rows_kernel(const GemvArgs g) {
+    static_assert(WPR == 1 || WPR == MV_WAVES, "one wavefront or the whole workgroup per row");
+    __shared__ float part[MV_WAVES];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t row0 = ((int64_t)blockIdx.x * MV_WAVES + wave) * R;
-    if (row0 >= g.rows) return;
+    const int64_t row = WPR == 1 ? (int64_t)blockIdx.x * MV_WAVES + wave : (int64_t)blockIdx.x;
+    if (row >= g.rows) return; // WPR == 4: uniform over the workgroup
     int64_t m_off, v_off;
     batch_offsets(g.batch, blockIdx.y, m_off, v_off);
-    const float* __restrict Mb = g.Mx + m_off;
+    const float* __restrict rowp = g.Mx + m_off + row * g.m_rs;
     const float* __restrict vb = g.v + v_off;
-
-    const float* rowp[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) rowp[r] = Mb + min(row0 + r, g.rows - 1) * g.m_rs; // clamped rows are discarded below
-
-    float acc[R];
-#pragma unroll
-    for (int r = 0; r < R; ++r) acc[r] = 0.f;
-
     const int64_t k = g.k;
-    const bool v_unit = (g.v_s == 1);
-    constexpr int STEP = 64 * 4;
-    int64_t kk = (int64_t)lane * 4;
-    // main loop: UNROLL independent 16-byte loads per row in flight
+    constexpr int STEP = 64 * WPR * 4;
+    int64_t kk = (int64_t)(WPR == 1 ? lane : threadIdx.x) * 4;
+    float acc = 0.f;
+
+    auto vec4 = [&](int64_t kx) -> f32x4 {
+        if constexpr (V_UNIT) return *reinterpret_cast<const f32x4_u*>(vb + kx);
+        else return f32x4{vb[kx * g.v_s], vb[(kx + 1) * g.v_s], vb[(kx + 2) * g.v_s], vb[(kx + 3) * g.v_s]};
+    };
+    auto fma4 = [&](const f32x4& m, const f32x4& x) {
+        acc = fmaf(m.x, x.x, acc); acc = fmaf(m.y, x.y, acc); acc = fmaf(m.z, x.z, acc); acc = fmaf(m.w, x.w, acc);
+    };
+    // main loop: UNROLL independent 16-byte loads in flight
     for (; kk + (int64_t)(UNROLL - 1) * STEP + 3 < k; kk += (int64_t)UNROLL * STEP) {
-        f32x4 mv[UNROLL][R], vv[UNROLL];
+        f32x4 m[UNROLL], x[UNROLL];
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) m[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(rowp + kk + (int64_t)u * STEP));
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) x[u] = vec4(kk + (int64_t)u * STEP);
+        __builtin_amdgcn_sched_barrier(0); // every load is issued before the first use
+#pragma unroll
+        for (int u = 0; u < UNROLL; ++u) fma4(m[u], x[u]);
+    }
+    { // the last, partial batch: whole groups of 4 that remain, still all in flight together
+        f32x4 m[UNROLL], x[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int64_t kx = kk + (int64_t)u * STEP;
-#pragma unroll
-            for (int r = 0; r < R; ++r) mv[u][r] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(rowp[r] + kx));
-            if (v_unit) vv[u] = *reinterpret_cast<const f32x4_u*>(vb + kx);
-            else vv[u] = f32x4{vb[kx * g.v_s], vb[(kx + 1) * g.v_s], vb[(kx + 2) * g.v_s], vb[(kx + 3) * g.v_s]};
+            m[u] = f32x4{0.f, 0.f, 0.f, 0.f}; x[u] = m[u];
+            if (kx + 3 < k) { m[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(rowp + kx)); x[u] = vec4(kx); }
         }
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u)
-#pragma unroll
-            for (int r = 0; r < R; ++r) {
-                acc[r] = fmaf(mv[u][r].x, vv[u].x, acc[r]);
-                acc[r] = fmaf(mv[u][r].y, vv[u].y, acc[r]);
-                acc[r] = fmaf(mv[u][r].z, vv[u].z, acc[r]);
-                acc[r] = fmaf(mv[u][r].w, vv[u].w, acc[r]);
-            }
+        for (int u = 0; u < UNROLL; ++u) fma4(m[u], x[u]);
     }
-    for (; kk < k; kk += STEP) {
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-            if (kk + e < k) {
-                const float x = vb[(kk + e) * g.v_s];
-#pragma unroll
-                for (int r = 0; r < R; ++r) acc[r] = fmaf(rowp[r][kk + e], x, acc[r]);
-            }
-        }
+    const int rest = (int)(k & 3); // the last k % 4 elements, one per lane
+    if ((WPR == 1 ? lane : (int)threadIdx.x) < rest) {
+        const int64_t kx = (k & ~(int64_t)3) + (WPR == 1 ? lane : (int)threadIdx.x);
+        acc = fmaf(rowp[kx], vb[kx * g.v_s], acc);
     }
+    float s = wave_sum(acc);
+    if constexpr (WPR > 1) {
+        if (lane == 0) part[wave] = s;
+        __syncthreads();
+        s = 0.f;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        const float s = wave_sum(acc[r]);
-        if (lane == 0 && row0 + r < g.rows) {
-            float* o = g.out + (int64_t)blockIdx.y * g.rows + row0 + r;
-            *o = g.accumulate ? *o + s : s;
-        }
+        for (int w = 0; w < MV_WAVES; ++w) s += part[w];
+    }
+    if (threadIdx.x == (WPR == 1 ? wave * 64 : 0)) {
+        float* o = g.out + (int64_t)blockIdx.y * g.rows + row;
+        *o = g.accumulate ? *o + s : s;
     }
 }
 
@@ -114,7 +118,7 @@ struct ColsArgs {
 };
 
 constexpr int COLS_THREADS = 256;
-constexpr int COLS_KCHUNK = 128; // k rows staged per LDS refill
+constexpr int COLS_STAGE_FLOATS = 2048; // R x (2048 / R) left-operand values are staged in LDS per refill
 constexpr int COLS_KSLICE_MIN = 32; // granularity of the K slices handed to workgroups
 
 // ALIGNED: every row of the matrix starts on a 16-byte boundary -> a lane owns 4 consecutive columns
@@ -123,6 +127,7 @@ constexpr int COLS_KSLICE_MIN = 32; // granularity of the K slices handed to wor
 // and uses dword loads, each still one contiguous 256-byte burst per wavefront.
 template <int R, bool ALIGNED>
 __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
+    constexpr int COLS_KCHUNK = COLS_STAGE_FLOATS / R; // k rows per LDS refill
     __shared__ float xs[R][COLS_KCHUNK];
     const int t = threadIdx.x;
     const int64_t col0 = (int64_t)blockIdx.x * COLS_THREADS * 4 + (ALIGNED ? 4 * t : t);
@@ -161,9 +166,9 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
     };
     // U independent row loads in flight per lane; the last batch of a chunk re-reads row len-1 for
     // the rows it lacks and drops them.
-    auto stream = [&](const float* __restrict p, int len, auto load4) {
-        constexpr int U = 8;
-        int kk = 0;
+    constexpr int U = R <= 2 ? 16 : 8;
+    auto stream = [&](const float* __restrict p, int first, int len, auto load4) { // rows [first, len), first % U == 0
+        int kk = first;
         for (; kk + U <= len; kk += U) {
             f32x4 m[U];
 #pragma unroll
@@ -183,10 +188,13 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
             for (int u = 0; u < U; ++u) {
                 if (kk + u >= len) m[u] = f32x4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-                for (int r = 0; r < R; ++r) acc[r] += m[u] * xs[r][kk + u]; // xs is zero past len
+                for (int r = 0; r < R; ++r) acc[r] += m[u] * xs[r][kk + u];
             }
         }
     };
+    // Workgroups start at different eighths of their K slices and wrap around: slices that lie a power
+    // of two apart in memory would otherwise walk the same memory channels in step.
+    const int rotation = (int)((blockIdx.y * 5 + blockIdx.x * 3) & 7);
 
     for (int64_t kc = k_begin; kc < k_end; kc += COLS_KCHUNK) {
         const int len = (int)min((int64_t)COLS_KCHUNK, k_end - kc);
@@ -197,8 +205,9 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
         }
         __syncthreads();
         const float* __restrict p = Mb + kc * g.m_rs + col0;
-        if (wave_full) stream(p, len, load_full);
-        else if (any) stream(p, len, load_clamped);
+        const int first = len >= 16 * U ? len / 8 * rotation / U * U : 0; // short slices are not worth a second ragged batch
+        if (wave_full) { stream(p, first, len, load_full); stream(p, 0, first, load_full); }
+        else if (any) { stream(p, first, len, load_clamped); stream(p, 0, first, load_clamped); }
     }
     if (!any) return;
     const bool to_partial = g.k_splits > 1;
@@ -236,6 +245,7 @@ constexpr int COLS_SHIFT_WIDTH = COLS_THREADS * 4 - 4;
 
 template <int R>
 __global__ __launch_bounds__(COLS_THREADS) void cols_shift_kernel(const ColsArgs g) {
+    constexpr int COLS_KCHUNK = COLS_STAGE_FLOATS / R; // k rows per LDS refill
     __shared__ float xs[R][COLS_KCHUNK];
     __shared__ float outs[R][COLS_THREADS * 4 + 4];
     const int t = threadIdx.x;

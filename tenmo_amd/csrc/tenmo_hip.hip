@@ -385,6 +385,13 @@ int cols_run(ColsArgs c, int64_t batch_count, float* out, int accumulate) {
     return 0;
 }
 
+template <int WPR, int UNROLL>
+void launch_rows(const GemvArgs& g, int64_t batch_count) {
+    const dim3 grid((unsigned)(WPR == 1 ? (g.rows + MV_WAVES - 1) / MV_WAVES : g.rows), (unsigned)batch_count);
+    if (g.v_s == 1) hipLaunchKernelGGL((mv_rows_kernel<WPR, UNROLL, true>), grid, dim3(64 * MV_WAVES), 0, S.stream, g);
+    else hipLaunchKernelGGL((mv_rows_kernel<WPR, UNROLL, false>), grid, dim3(64 * MV_WAVES), 0, S.stream, g);
+}
+
 // out[b][i] = sum_j Mat[b](i, j) * vec[b](j), i < n_out, j < n_red;  Mat(i,j) = Mx[i*out_s + j*red_s]
 int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* vec, int64_t v_s, float* out,
                     int64_t n_out, int64_t n_red, const BatchDesc& bd_mat_vec, int64_t batch_count, int accumulate) {
@@ -406,15 +413,9 @@ int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* 
             hipLaunchKernelGGL(mv_generic_kernel, dim3((unsigned)((n_out + 255) / 256), (unsigned)batch_count), dim3(256), 0, S.stream, g);
             return 0;
         }
-        // fewer rows per wavefront when the matrix is short, so the grid still covers the chip
-        const int64_t waves4 = (n_out + 3) / 4;
-        if (waves4 >= (int64_t)S.cus * 8) {
-            hipLaunchKernelGGL((mv_rows_kernel<4, 2>), dim3((unsigned)((n_out + 4 * MV_WAVES - 1) / (4 * MV_WAVES)), (unsigned)batch_count), dim3(64 * MV_WAVES), 0, S.stream, g);
-        } else if (n_out >= (int64_t)S.cus * 8) {
-            hipLaunchKernelGGL((mv_rows_kernel<2, 4>), dim3((unsigned)((n_out + 2 * MV_WAVES - 1) / (2 * MV_WAVES)), (unsigned)batch_count), dim3(64 * MV_WAVES), 0, S.stream, g);
-        } else {
-            hipLaunchKernelGGL((mv_rows_kernel<1, 4>), dim3((unsigned)((n_out + MV_WAVES - 1) / MV_WAVES), (unsigned)batch_count), dim3(64 * MV_WAVES), 0, S.stream, g);
-        }
+        // one wavefront per row; the whole workgroup per row when there are too few rows to cover the chip
+        if (n_out * batch_count < (int64_t)S.cus) launch_rows<MV_WAVES, 8>(g, batch_count);
+        else launch_rows<1, 8>(g, batch_count);
         return 0;
     }
     if (out_s == 1 || n_out == 1) {

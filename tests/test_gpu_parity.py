@@ -345,6 +345,33 @@ def test_columns_with_misaligned_row_pitch(T):
     assert rel_fro(got, ref_matmul64(a, b)) <= RTOL_FRO
 
 
+def test_column_kernels_reuse_workspace(T):
+    """The column-streaming kernels (vm, skinny) cut K into slices that go through the library's
+    workspace.  Same operand storage and workspace reused with new contents call after call, and `+=`."""
+    import torch
+    from tenmo_amd import _lib
+    L = _lib.load()
+    rng = np.random.default_rng(61)
+    for (m, k, n) in [(1, 4096, 4096), (4, 768, 50257), (3, 2000, 3000), (8, 1024, 2048), (1, 16384, 1024)]:
+        A = T.Tensor.from_numpy(np.zeros((m, k), np.float32))
+        B = T.Tensor.from_numpy(np.zeros((k, n), np.float32))
+        for rep in range(3):
+            a = rng.standard_normal((m, k), dtype=np.float32)
+            b = rng.standard_normal((k, n), dtype=np.float32)
+            A.buffer.storage.copy_(torch.from_numpy(a.ravel()))
+            B.buffer.storage.copy_(torch.from_numpy(b.ravel()))
+            got = A.matmul(B, track_grad=False).to_numpy()
+            assert rel_fro(got, ref_matmul64(a, b)) <= RTOL_FRO, (m, k, n, rep)
+    a = rng.standard_normal((1, 3000), dtype=np.float32)
+    b = rng.standard_normal((3000, 5000), dtype=np.float32)
+    c0 = rng.standard_normal((1, 5000), dtype=np.float32)
+    out = T.Tensor.from_numpy(c0.copy())
+    A, B = T.Tensor.from_numpy(a), T.Tensor.from_numpy(b)
+    _lib.check(L.tenmo_hip_gemm_f32(A.buffer.data_ptr(), 0, 3000, 1, B.buffer.data_ptr(), 0, 5000, 1, out.buffer.data_ptr(),
+                                    1, 5000, 3000, 0, None, None, None, 1, 1))
+    assert rel_fro(out.to_numpy(), c0.astype(np.float64) + ref_matmul64(a, b)) <= RTOL_FRO
+
+
 def test_odd_strides_and_overlap(T, oracle):
     """Column stride 2, row stride 0 (broadcast rows), overlapping windows (tests/test_mmnd.mojo:143-175)."""
     rng = np.random.default_rng(23)
