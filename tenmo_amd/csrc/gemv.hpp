@@ -29,72 +29,105 @@ struct GemvArgs {
 };
 
 // ---- rows kernel: unit stride along the reduction (row-major matrix . vector) ----------------
-// WPR wavefronts (1 or 4) own one row and walk it in 16-byte steps per lane, UNROLL steps in flight:
-// the row is read as contiguous bursts of WPR x UNROLL KiB, which is what HBM streams best (several
-// rows per wavefront interleave short bursts of distant rows and lose 5-20%).  With WPR = 1 the four
-// wavefronts of a workgroup take four consecutive rows; WPR = 4 is for few, long rows.
+// A unit of WPR wavefronts (1, or the 4 of a workgroup) owns RPW consecutive rows.  It walks the
+// reduction in batches of UNROLL 16-byte steps per lane: the vector's values of a batch are loaded
+// once into registers, then each of the RPW rows contributes one contiguous burst of WPR x UNROLL KiB
+// with all its loads in flight.  Measured on 16384^2 (fractions of the 8 TB/s HBM peak): workgroup
+// per 4 rows with the vector in registers 0.90; one row per unit 0.83-0.85 (the vector's loads then
+// compete with the matrix's); several rows interleaved load by load in one wavefront 0.65-0.80.
+// WPR = 1 is for rows too short to give four wavefronts a full batch each.
 constexpr int MV_WAVES = 4;
-template <int WPR, int UNROLL, bool V_UNIT>
+template <int WPR, int RPW, int UNROLL, bool V_UNIT>
 __global__ __launch_bounds__(64 * MV_WAVES) void mv_rows_kernel(const GemvArgs g) {
     static_assert(WPR == 1 || WPR == MV_WAVES, "one wavefront or the whole workgroup per row");
-    __shared__ float part[MV_WAVES];
+    __shared__ float part[MV_WAVES][RPW];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const int64_t row = WPR == 1 ? (int64_t)blockIdx.x * MV_WAVES + wave : (int64_t)blockIdx.x;
-    if (row >= g.rows) return; // WPR == 4: uniform over the workgroup
+    const int tid = WPR == 1 ? lane : (int)threadIdx.x;           // index inside the unit
+    const int64_t unit = WPR == 1 ? (int64_t)blockIdx.x * MV_WAVES + wave : (int64_t)blockIdx.x;
+    const int64_t row0 = unit * RPW;
+    if (row0 >= g.rows) return; // WPR == 4: uniform over the workgroup
     int64_t m_off, v_off;
     batch_offsets(g.batch, blockIdx.y, m_off, v_off);
-    const float* __restrict rowp = g.Mx + m_off + row * g.m_rs;
     const float* __restrict vb = g.v + v_off;
     const int64_t k = g.k;
     constexpr int STEP = 64 * WPR * 4;
-    int64_t kk = (int64_t)(WPR == 1 ? lane : threadIdx.x) * 4;
-    float acc = 0.f;
 
     auto vec4 = [&](int64_t kx) -> f32x4 {
         if constexpr (V_UNIT) return *reinterpret_cast<const f32x4_u*>(vb + kx);
         else return f32x4{vb[kx * g.v_s], vb[(kx + 1) * g.v_s], vb[(kx + 2) * g.v_s], vb[(kx + 3) * g.v_s]};
     };
-    auto fma4 = [&](const f32x4& m, const f32x4& x) {
-        acc = fmaf(m.x, x.x, acc); acc = fmaf(m.y, x.y, acc); acc = fmaf(m.z, x.z, acc); acc = fmaf(m.w, x.w, acc);
-    };
-    // main loop: UNROLL independent 16-byte loads in flight
-    for (; kk + (int64_t)(UNROLL - 1) * STEP + 3 < k; kk += (int64_t)UNROLL * STEP) {
-        f32x4 m[UNROLL], x[UNROLL];
+    const float* rowp[RPW]; // rows past the end repeat the last one; their sums are dropped
+    float acc[RPW];
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) m[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(rowp + kk + (int64_t)u * STEP));
+    for (int j = 0; j < RPW; ++j) { rowp[j] = g.Mx + m_off + min(row0 + j, g.rows - 1) * g.m_rs; acc[j] = 0.f; }
+    auto fma4 = [](float a, const f32x4& m, const f32x4& x) {
+        a = fmaf(m.x, x.x, a); a = fmaf(m.y, x.y, a); a = fmaf(m.z, x.z, a); return fmaf(m.w, x.w, a);
+    };
+
+    int64_t kk = (int64_t)tid * 4;
+    for (; kk + (int64_t)(UNROLL - 1) * STEP + 3 < k; kk += (int64_t)UNROLL * STEP) { // full batches
+        f32x4 x[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) x[u] = vec4(kk + (int64_t)u * STEP);
-        __builtin_amdgcn_sched_barrier(0); // every load is issued before the first use
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) fma4(m[u], x[u]);
+        for (int j = 0; j < RPW; ++j) {
+            f32x4 m[UNROLL];
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) m[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(rowp[j] + kk + (int64_t)u * STEP));
+            __builtin_amdgcn_sched_barrier(0); // every load of the row is issued before the first use
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) acc[j] = fma4(acc[j], m[u], x[u]);
+        }
     }
-    { // the last, partial batch: whole groups of 4 that remain, still all in flight together
-        f32x4 m[UNROLL], x[UNROLL];
+    if (__any(kk + 3 < k)) { // the last, partial batch: the whole groups of 4 that remain
+        f32x4 x[UNROLL];
+        bool ok[UNROLL];
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
             const int64_t kx = kk + (int64_t)u * STEP;
-            m[u] = f32x4{0.f, 0.f, 0.f, 0.f}; x[u] = m[u];
-            if (kx + 3 < k) { m[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(rowp + kx)); x[u] = vec4(kx); }
+            ok[u] = kx + 3 < k;
+            x[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+            if (ok[u]) x[u] = vec4(kx);
         }
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) fma4(m[u], x[u]);
-    }
-    const int rest = (int)(k & 3); // the last k % 4 elements, one per lane
-    if ((WPR == 1 ? lane : (int)threadIdx.x) < rest) {
-        const int64_t kx = (k & ~(int64_t)3) + (WPR == 1 ? lane : (int)threadIdx.x);
-        acc = fmaf(rowp[kx], vb[kx * g.v_s], acc);
-    }
-    float s = wave_sum(acc);
-    if constexpr (WPR > 1) {
-        if (lane == 0) part[wave] = s;
-        __syncthreads();
-        s = 0.f;
+        for (int j = 0; j < RPW; ++j) {
+            f32x4 m[UNROLL];
 #pragma unroll
-        for (int w = 0; w < MV_WAVES; ++w) s += part[w];
+            for (int u = 0; u < UNROLL; ++u) {
+                m[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+                if (ok[u]) m[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(rowp[j] + kk + (int64_t)u * STEP));
+            }
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < UNROLL; ++u) acc[j] = fma4(acc[j], m[u], x[u]);
+        }
     }
-    if (threadIdx.x == (WPR == 1 ? wave * 64 : 0)) {
-        float* o = g.out + (int64_t)blockIdx.y * g.rows + row;
-        *o = g.accumulate ? *o + s : s;
+    if (tid < (int)(k & 3)) { // the last k % 4 elements, one per lane
+        const int64_t kx = (k & ~(int64_t)3) + tid;
+        const float xe = vb[kx * g.v_s];
+#pragma unroll
+        for (int j = 0; j < RPW; ++j) acc[j] = fmaf(rowp[j][kx], xe, acc[j]);
+    }
+    float* __restrict ob = g.out + (int64_t)blockIdx.y * g.rows + row0;
+    if constexpr (WPR == 1) {
+#pragma unroll
+        for (int j = 0; j < RPW; ++j) {
+            const float s = wave_sum(acc[j]);
+            if (lane == 0 && row0 + j < g.rows) ob[j] = g.accumulate ? ob[j] + s : s;
+        }
+    } else {
+#pragma unroll
+        for (int j = 0; j < RPW; ++j) {
+            const float s = wave_sum(acc[j]);
+            if (lane == 0) part[wave][j] = s;
+        }
+        __syncthreads();
+        if (threadIdx.x < RPW && row0 + threadIdx.x < g.rows) {
+            float s = 0.f;
+#pragma unroll
+            for (int w = 0; w < MV_WAVES; ++w) s += part[w][threadIdx.x];
+            ob[threadIdx.x] = g.accumulate ? ob[threadIdx.x] + s : s;
+        }
     }
 }
 

@@ -385,11 +385,12 @@ int cols_run(ColsArgs c, int64_t batch_count, float* out, int accumulate) {
     return 0;
 }
 
-template <int WPR, int UNROLL>
+template <int WPR, int RPW, int UNROLL>
 void launch_rows(const GemvArgs& g, int64_t batch_count) {
-    const dim3 grid((unsigned)(WPR == 1 ? (g.rows + MV_WAVES - 1) / MV_WAVES : g.rows), (unsigned)batch_count);
-    if (g.v_s == 1) hipLaunchKernelGGL((mv_rows_kernel<WPR, UNROLL, true>), grid, dim3(64 * MV_WAVES), 0, S.stream, g);
-    else hipLaunchKernelGGL((mv_rows_kernel<WPR, UNROLL, false>), grid, dim3(64 * MV_WAVES), 0, S.stream, g);
+    const int64_t units = (g.rows + RPW - 1) / RPW;
+    const dim3 grid((unsigned)(WPR == 1 ? (units + MV_WAVES - 1) / MV_WAVES : units), (unsigned)batch_count);
+    if (g.v_s == 1) hipLaunchKernelGGL((mv_rows_kernel<WPR, RPW, UNROLL, true>), grid, dim3(64 * MV_WAVES), 0, S.stream, g);
+    else hipLaunchKernelGGL((mv_rows_kernel<WPR, RPW, UNROLL, false>), grid, dim3(64 * MV_WAVES), 0, S.stream, g);
 }
 
 // out[b][i] = sum_j Mat[b](i, j) * vec[b](j), i < n_out, j < n_red;  Mat(i,j) = Mx[i*out_s + j*red_s]
@@ -413,9 +414,14 @@ int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* 
             hipLaunchKernelGGL(mv_generic_kernel, dim3((unsigned)((n_out + 255) / 256), (unsigned)batch_count), dim3(256), 0, S.stream, g);
             return 0;
         }
-        // one wavefront per row; the whole workgroup per row when there are too few rows to cover the chip
-        if (n_out * batch_count < (int64_t)S.cus) launch_rows<MV_WAVES, 8>(g, batch_count);
-        else launch_rows<1, 8>(g, batch_count);
+        // long rows: the whole workgroup walks 4 rows (bursts of 32 KiB per row); shorter rows get shorter
+        // bursts and fewer rows per unit; rows under 2048 elements go one wavefront per unit
+        if (n_red >= 8192) {
+            if (n_out * batch_count >= 2 * (int64_t)S.cus) launch_rows<4, 4, 8>(g, batch_count);
+            else launch_rows<4, 1, 8>(g, batch_count);
+        } else if (n_red >= 2048) launch_rows<4, 2, 4>(g, batch_count);
+        else if (n_red >= 1024) launch_rows<1, 1, 8>(g, batch_count);
+        else launch_rows<1, 4, 4>(g, batch_count);
         return 0;
     }
     if (out_s == 1 || n_out == 1) {
