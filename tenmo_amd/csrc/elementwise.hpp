@@ -184,23 +184,38 @@ __global__ void sgd_step_kernel(float* __restrict p, const float* __restrict g, 
         f4* __restrict p4 = reinterpret_cast<f4*>(p);
         const f4* __restrict g4 = reinterpret_cast<const f4*>(g);
         f4* __restrict v4 = reinterpret_cast<f4*>(vel);
-        for (int64_t i = tid; i < n / 4; i += stride) {
-            const f4 pp = p4[i], gg = g4[i];
-            float pa[4] = {pp.x, pp.y, pp.z, pp.w};
-            const float ga[4] = {gg.x, gg.y, gg.z, gg.w};
-            if (vel) {
-                const f4 vv = v4[i];
-                float va[4] = {vv.x, vv.y, vv.z, vv.w};
+        constexpr int U = 4; // groups in flight per thread
+        const int64_t n4 = n / 4;
+        for (int64_t i0 = (int64_t)blockIdx.x * blockDim.x * U + threadIdx.x; i0 < n4; i0 += stride * U) {
+            f4 pp[U], gg[U], vv[U];
 #pragma unroll
-                for (int e = 0; e < 4; ++e) sgd_update(pa[e], ga[e], &va[e], lr, momentum, weight_decay);
-                const f4 vo = {va[0], va[1], va[2], va[3]};
-                v4[i] = vo;
-            } else {
-#pragma unroll
-                for (int e = 0; e < 4; ++e) sgd_update(pa[e], ga[e], nullptr, lr, momentum, weight_decay);
+            for (int u = 0; u < U; ++u) {
+                const int64_t i = i0 + (int64_t)u * blockDim.x;
+                pp[u] = f4{0.f, 0.f, 0.f, 0.f}; gg[u] = pp[u]; vv[u] = pp[u];
+                if (i < n4) {
+                    pp[u] = __builtin_nontemporal_load(p4 + i);
+                    gg[u] = __builtin_nontemporal_load(g4 + i);
+                    if (vel) vv[u] = __builtin_nontemporal_load(v4 + i);
+                }
             }
-            const f4 po = {pa[0], pa[1], pa[2], pa[3]};
-            p4[i] = po;
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int u = 0; u < U; ++u) {
+                const int64_t i = i0 + (int64_t)u * blockDim.x;
+                if (i >= n4) continue;
+                float pa[4] = {pp[u].x, pp[u].y, pp[u].z, pp[u].w};
+                const float ga[4] = {gg[u].x, gg[u].y, gg[u].z, gg[u].w};
+                if (vel) {
+                    float va[4] = {vv[u].x, vv[u].y, vv[u].z, vv[u].w};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) sgd_update(pa[e], ga[e], &va[e], lr, momentum, weight_decay);
+                    __builtin_nontemporal_store(f4{va[0], va[1], va[2], va[3]}, v4 + i);
+                } else {
+#pragma unroll
+                    for (int e = 0; e < 4; ++e) sgd_update(pa[e], ga[e], nullptr, lr, momentum, weight_decay);
+                }
+                __builtin_nontemporal_store(f4{pa[0], pa[1], pa[2], pa[3]}, p4 + i);
+            }
         }
         if (tid == 0)
             for (int64_t i = n / 4 * 4; i < n; ++i) sgd_update(p[i], g[i], vel ? vel + i : nullptr, lr, momentum, weight_decay);

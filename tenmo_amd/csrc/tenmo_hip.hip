@@ -902,8 +902,20 @@ int tenmo_hip_cross_entropy_backward_f32(const float* softmax, const void* targe
     a.softmax = softmax; a.target = target; a.upstream = upstream; a.grad = grad_logits;
     a.M = M; a.C = C; a.ignore_index = ignore_index; a.label_smoothing = label_smoothing;
     a.reduction = reduction; a.valid_count = valid_count; a.accumulate = accumulate ? 1 : 0;
+    if (C >= 4 && (uintptr_t)softmax % 16 == 0 && (uintptr_t)grad_logits % 16 == 0) {
+        // flat sweep: every group of four consecutive elements of the [M*C] array is one 16-byte access
+        constexpr int64_t per_block = CE_THREADS * 4 * 4; // elements per workgroup and pass
+        const int64_t blocks = std::max<int64_t>(1, std::min<int64_t>((M * C + per_block - 1) / per_block, (int64_t)S.cus * 16));
+        CeFlatSteps st{};
+        st.pass_rows = blocks * per_block / C; st.pass_cols = blocks * per_block % C;
+        st.unit_rows = CE_THREADS * 4 / C; st.unit_cols = CE_THREADS * 4 % C;
+        const dim3 grid((unsigned)blocks), block(CE_THREADS);
+        if (target_is_int64) hipLaunchKernelGGL(ce_backward_flat_kernel<int64_t>, grid, block, 0, S.stream, a, st);
+        else hipLaunchKernelGGL(ce_backward_flat_kernel<int32_t>, grid, block, 0, S.stream, a, st);
+        return finish(sync);
+    }
     // enough workgroups per row to fill the chip when there are few long rows
-    int64_t chunks = std::max<int64_t>(1, std::min<int64_t>((C + CE_THREADS * 8 - 1) / (CE_THREADS * 8), ((int64_t)S.cus * 8 + M - 1) / M));
+    int64_t chunks = std::max<int64_t>(1, std::min<int64_t>((C + CE_THREADS * 16 - 1) / (CE_THREADS * 16), ((int64_t)S.cus * 8 + M - 1) / M));
     if (M * chunks > 0x7fffffffLL) return fail(TENMO_ERR_UNSUPPORTED, "%s: grid too large", who);
     a.chunks = (int32_t)chunks;
     const dim3 grid((unsigned)(M * chunks)), block(CE_THREADS);
@@ -924,7 +936,7 @@ int tenmo_hip_sgd_step_f32(float* param, const float* grad, float* velocity, int
     if (n == 0) return 0;
     if (!param || !grad) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_sgd_step_f32: null pointer");
     const bool vec = (uintptr_t)param % 16 == 0 && (uintptr_t)grad % 16 == 0 && (uintptr_t)velocity % 16 == 0;
-    const int64_t work = vec ? (n + 3) / 4 : n;
+    const int64_t work = vec ? (n + 15) / 16 : n; // the vector path moves four groups of four per thread and pass
     const dim3 grid((unsigned)std::max<int64_t>(1, std::min<int64_t>((work + 255) / 256, (int64_t)S.cus * 16))), block(256);
     if (vec) hipLaunchKernelGGL(sgd_step_kernel<true>, grid, block, 0, S.stream, param, grad, velocity, n, lr, momentum, weight_decay);
     else hipLaunchKernelGGL(sgd_step_kernel<false>, grid, block, 0, S.stream, param, grad, velocity, n, lr, momentum, weight_decay);

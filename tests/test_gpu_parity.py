@@ -733,7 +733,7 @@ def test_cross_entropy_entries(T, oracle):
     L, lib = T.lib.load(), T.lib
     rng = np.random.default_rng(43)
     for M, Cn, ls, is64 in [(2, 3, 0.0, True), (64, 10, 0.0, False), (33, 17, 0.2, True), (5, 1000, 0.05, True),
-                            (7, 1001, 0.1, False), (300, 64, 0.0, True), (3, 50257, 0.1, True)]:
+                            (7, 1001, 0.1, False), (300, 64, 0.0, True), (3, 50257, 0.1, True), (2100, 8009, 0.1, True)]:
         x = (3 * rng.standard_normal((M, Cn))).astype(np.float32)
         t = rng.integers(0, Cn, M)
         t[rng.random(M) < 0.3] = -100
