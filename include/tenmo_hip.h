@@ -204,6 +204,16 @@ int tenmo_hip_cross_entropy_backward_f32(const float* softmax, const void* targe
                                          const float* upstream, int64_t M, int64_t C, int64_t ignore_index,
                                          float label_smoothing, int32_t reduction, int32_t valid_count,
                                          float* grad_logits, int32_t accumulate, int32_t sync);
+/* FusedIm2Col.forward — tenmo/cnn.mojo:308-507 (what Conv2dFused.invoke, :92-273, calls after it has
+ * padded the image): out[n, co, y, x] = bias[co] + sum over (ci, ky, kx) of
+ * padded_image[n, ci, y*stride + ky*dilation, x*stride + kx*dilation] * kernel[co, ci, ky, kx], with
+ * H_out = (H_pad - (KH + (KH-1)(dilation-1))) / stride + 1 and W_out likewise (:358-365).  All tensors
+ * dense: padded_image [N, C_in, H_pad, W_pad], kernel [C_out, C_in, KH, KW], bias [C_out] or NULL (the
+ * reference substitutes zeros, :128-131), out [N, C_out, H_out, W_out].  Runs as an implicit GEMM on
+ * the matrix-core kernel: the patch matrix is never materialised. */
+int tenmo_hip_conv2d_forward_f32(const float* padded_image, int64_t n_images, int64_t c_in, int64_t h_pad, int64_t w_pad,
+                                 const float* kernel, int64_t c_out, int64_t kh, int64_t kw, const float* bias,
+                                 int64_t stride, int64_t dilation, float* out, int32_t sync);
 /* SGDStep.launch_no_momentum / launch_momentum — tenmo/kernels/sgd_kernel.mojo:56-143 (CPU form:
  * tenmo/optim.mojo:93-160): g += weight_decay * p when weight_decay > 0; with velocity != NULL
  * v = momentum * v + g, p -= lr * v; else p -= lr * g. */

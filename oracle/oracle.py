@@ -87,6 +87,8 @@ def lib():
         L.oracle_cross_entropy_forward_f32.argtypes = [fp, i64p, C.c_int64, C.c_int64, C.c_int64, C.c_float, fp, fp, fp, i32p]
         L.oracle_cross_entropy_backward_f32.argtypes = [fp, i64p, fp, C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_int, C.c_int32, fp]
         L.oracle_sgd_step_f32.argtypes = [fp, fp, fp, C.c_int64, C.c_float, C.c_float, C.c_float]
+        L.oracle_conv2d_forward_f32.argtypes = [fp, C.c_int64, C.c_int64, C.c_int64, C.c_int64, fp, C.c_int64, C.c_int64, C.c_int64,
+                                                fp, C.c_int64, C.c_int64, fp]
         _lib = L
     return _lib
 
@@ -389,3 +391,49 @@ def sgd_step(param: np.ndarray, grad: np.ndarray, velocity: Optional[np.ndarray]
     fpp = C.POINTER(C.c_float)
     _check(lib().oracle_sgd_step_f32(param.ctypes.data_as(fpp), np.ascontiguousarray(grad).ctypes.data_as(fpp),
                                      velocity.ctypes.data_as(fpp) if velocity is not None else None, param.size, lr, momentum, weight_decay))
+
+
+def conv_padding(h_in: int, w_in: int, kh: int, kw: int, stride: int, dilation: int, padding) -> Tuple[int, int, int, int]:
+    """(top, bottom, left, right) zero padding as Conv2dFused.invoke derives it from its `padding` argument
+    — tenmo/cnn.mojo:183-222: "valid", "same", an int, a (height, width) pair or [(top, bottom), (left, right)]."""
+    dkh, dkw = kh + (kh - 1) * (dilation - 1), kw + (kw - 1) * (dilation - 1)
+    if padding == "valid":
+        return 0, 0, 0, 0
+    if padding == "same":
+        h_target, w_target = (h_in + stride - 1) // stride, (w_in + stride - 1) // stride
+        ph, pw = (h_target - 1) * stride + dkh - h_in, (w_target - 1) * stride + dkw - w_in
+        return ph // 2, ph - ph // 2, pw // 2, pw - pw // 2
+    if isinstance(padding, int):
+        return padding, padding, padding, padding
+    if isinstance(padding, tuple):
+        return padding[0], padding[0], padding[1], padding[1]
+    if isinstance(padding, list) and len(padding) == 2:
+        return padding[0][0], padding[0][1], padding[1][0], padding[1][1]
+    raise OracleError("Invalid padding type")
+
+
+def conv2d_forward(image: np.ndarray, kernel: np.ndarray, bias: Optional[np.ndarray] = None, stride: int = 1, dilation: int = 1,
+                   padding="valid") -> np.ndarray:
+    """Conv2dFused.forward (tenmo/cnn.mojo:92-273): zero-pad, then the fused im2col convolution (:308-507)."""
+    if image.ndim != 4 or kernel.ndim != 4:
+        raise OracleError("Image must be 4D: (N, C_in, H_in, W_in); kernel must be 4D: (C_out, C_in, KH, KW)")
+    n, c_in, h_in, w_in = image.shape
+    c_out, kc, kh, kw = kernel.shape
+    if kc != c_in:
+        raise OracleError("Kernel input channels must match input channels")
+    top, bottom, left, right = conv_padding(h_in, w_in, kh, kw, stride, dilation, padding)
+    padded = np.ascontiguousarray(np.pad(image.astype(np.float32), ((0, 0), (0, 0), (top, bottom), (left, right))))
+    dkh, dkw = kh + (kh - 1) * (dilation - 1), kw + (kw - 1) * (dilation - 1)
+    h_out, w_out = (padded.shape[2] - dkh) // stride + 1, (padded.shape[3] - dkw) // stride + 1
+    if h_out <= 0 or w_out <= 0:
+        raise OracleError("Invalid convolution parameters lead to non-positive output size")
+    out = np.empty((n, c_out, h_out, w_out), np.float32)
+    kern = np.ascontiguousarray(kernel, dtype=np.float32)
+    fpp = C.POINTER(C.c_float)
+    b = np.ascontiguousarray(bias, dtype=np.float32) if bias is not None else None
+    if b is not None and b.shape != (c_out,):
+        raise OracleError(f"Invalid bias tensor shape: {b.shape}. Should be (C_out,)")
+    _check(lib().oracle_conv2d_forward_f32(padded.ctypes.data_as(fpp), n, c_in, padded.shape[2], padded.shape[3], kern.ctypes.data_as(fpp),
+                                           c_out, kh, kw, b.ctypes.data_as(fpp) if b is not None else None, stride, dilation,
+                                           out.ctypes.data_as(fpp)))
+    return out

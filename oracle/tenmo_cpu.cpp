@@ -667,4 +667,33 @@ int oracle_sgd_step_f32(float* param, const float* grad, float* velocity, int64_
     return 0;
 }
 
+// Fused im2col + convolution + bias, FusedIm2Col.forward (tenmo/cnn.mojo:308-507), on an image that is
+// already padded (Conv2dFused.invoke pads first, :118-125, :229-235).  Per output position the sum starts
+// from the bias (:432, :479) and adds img * kernel over ci, then ky, then kx ascending (:435-470,
+// :481-498) in fp32; the reference's SIMD lanes run over output channels, which does not change the
+// order inside one output element.  Output sizes as in :358-365.
+int oracle_conv2d_forward_f32(const float* padded_image, int64_t n_images, int64_t c_in, int64_t h_pad, int64_t w_pad,
+                              const float* kernel, int64_t c_out, int64_t kh, int64_t kw, const float* bias,
+                              int64_t stride, int64_t dilation, float* out) {
+    if (c_in < 1 || c_out < 1 || kh < 1 || kw < 1 || stride < 1 || dilation < 1) return fail("conv2d: sizes, stride and dilation must be positive");
+    const int64_t dkh = kh + (kh - 1) * (dilation - 1), dkw = kw + (kw - 1) * (dilation - 1);
+    const int64_t h_out = (h_pad - dkh) / stride + 1, w_out = (w_pad - dkw) / stride + 1;
+    if (h_pad < dkh || w_pad < dkw || h_out <= 0 || w_out <= 0) return fail("conv2d: Invalid output dimensions");
+    for (int64_t n = 0; n < n_images; ++n)
+        for (int64_t y = 0; y < h_out; ++y)
+            for (int64_t x = 0; x < w_out; ++x)
+                for (int64_t co = 0; co < c_out; ++co) {
+                    float accum = bias ? bias[co] : 0.f;
+                    for (int64_t ci = 0; ci < c_in; ++ci)
+                        for (int64_t ky = 0; ky < kh; ++ky)
+                            for (int64_t kx = 0; kx < kw; ++kx) {
+                                const float img = padded_image[((n * c_in + ci) * h_pad + y * stride + ky * dilation) * w_pad + x * stride + kx * dilation];
+                                const float kv = kernel[((co * c_in + ci) * kh + ky) * kw + kx];
+                                accum += img * kv;
+                            }
+                    out[((n * c_out + co) * h_out + y) * w_out + x] = accum;
+                }
+    return 0;
+}
+
 } // extern "C"

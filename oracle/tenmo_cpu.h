@@ -100,6 +100,11 @@ int oracle_cross_entropy_backward_f32(const float* softmax, const int64_t* targe
 /* SGD step, tenmo/optim.mojo:93-160 */
 int oracle_sgd_step_f32(float* param, const float* grad, float* velocity, int64_t n, float lr, float momentum, float weight_decay);
 
+/* FusedIm2Col.forward on a padded image, tenmo/cnn.mojo:308-507 */
+int oracle_conv2d_forward_f32(const float* padded_image, int64_t n_images, int64_t c_in, int64_t h_pad, int64_t w_pad,
+                              const float* kernel, int64_t c_out, int64_t kh, int64_t kw, const float* bias,
+                              int64_t stride, int64_t dilation, float* out);
+
 #ifdef __cplusplus
 }
 #endif

@@ -246,4 +246,24 @@ __global__ void splitk_reduce_kernel(const float* __restrict partial, float* __r
     }
 }
 
+// Offset tables of the implicit im2col (tenmo/cnn.mojo:308-507 walks the same indices in loops):
+// patch element k = (ci, ky, kx) of output position p = (y, x) of one padded image [C_in, H_pad, W_pad]
+// lies at by_k[k] + by_pos[p] with
+//   by_k[k]   = ci*H_pad*W_pad + ky*dilation*W_pad + kx*dilation,   by_pos[p] = y*stride*W_pad + x*stride.
+struct ConvGeometry {
+    int32_t c_in, h_pad, w_pad, kh, kw, h_out, w_out, stride, dilation;
+};
+__global__ void conv_tables_kernel(const ConvGeometry c, int32_t* __restrict by_k, int32_t* __restrict by_pos) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    const int nk = c.c_in * c.kh * c.kw, np = c.h_out * c.w_out;
+    if (i < nk) {
+        const int ci = i / (c.kh * c.kw), r = i % (c.kh * c.kw), ky = r / c.kw, kx = r % c.kw;
+        by_k[i] = ci * c.h_pad * c.w_pad + ky * c.dilation * c.w_pad + kx * c.dilation;
+    }
+    if (i < np) {
+        const int y = i / c.w_out, x = i % c.w_out;
+        by_pos[i] = y * c.stride * c.w_pad + x * c.stride;
+    }
+}
+
 } // namespace tenmo

@@ -76,6 +76,11 @@ struct GemmArgs {
     const float* bias;    // + bias[col], or null                         (Linear: x.W + b)
     const float* mask;    // dense like C: result zeroed where mask <= 0, or null   (ReLU backward on dX)
     int32_t relu;         // max(.,0) after the bias                      (ReLU forward)
+    int32_t bias_rows;    // the bias is indexed by the row of C instead of the column (convolution: one per filter)
+    // Gathered B (implicit im2col): when set, B(n, k) = B[b_gather_row[n] + b_gather_k[k]] instead of
+    // B[k*b_rs + n*b_cs]; the operand then goes through the element-wise loader (KMAJOR_GEN).
+    const int32_t* b_gather_row; // [N]
+    const int32_t* b_gather_k;   // [K]
     BatchDesc batch;
 };
 
@@ -167,7 +172,8 @@ struct TileLoader {
     // register-staged loads with every element checked against the extents (edge tiles, K tail,
     // generic strides)
     __device__ __forceinline__ void load_checked(const float* __restrict base, int64_t rs, int64_t ks,
-                                                 int64_t row0, int64_t k0, int64_t R, int64_t K, int t) {
+                                                 int64_t row0, int64_t k0, int64_t R, int64_t K, int t,
+                                                 const int32_t* __restrict gather_row = nullptr, const int32_t* __restrict gather_k = nullptr) {
         if constexpr (MODE == KMAJOR_VEC) {
             const int kq = t & 3;
 #pragma unroll
@@ -211,7 +217,13 @@ struct TileLoader {
                 const int64_t row = row0 + (t >> 2) + 64 * i;
                 const int64_t k = k0 + 4 * kq;
                 f32x4 v = {0.f, 0.f, 0.f, 0.f};
-                if (row < R) {
+                if (row < R && gather_row) { // element (row, k) at base[gather_row[row] + gather_k[k]]
+                    const float* p = base + gather_row[row];
+                    if (k + 0 < K) v.x = p[gather_k[k]];
+                    if (k + 1 < K) v.y = p[gather_k[k + 1]];
+                    if (k + 2 < K) v.z = p[gather_k[k + 2]];
+                    if (k + 3 < K) v.w = p[gather_k[k + 3]];
+                } else if (row < R) {
                     const float* p = base + row * rs + k * ks;
                     if (k + 0 < K) v.x = p[0];
                     if (k + 1 < K) v.y = p[ks];
@@ -475,7 +487,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
     // ---- edge tiles, the K tail, generic strides: register-staged checked loads, two stages ----
     if (done < nk) {
         la.load_checked(Ab, a_row_s, a_k_s, m0, k_begin + done * GEMM_BK, g.M, k_end, t);
-        lb.load_checked(Bb, b_row_s, b_k_s, n0, k_begin + done * GEMM_BK, g.N, k_end, t);
+        lb.load_checked(Bb, b_row_s, b_k_s, n0, k_begin + done * GEMM_BK, g.N, k_end, t, g.b_gather_row, g.b_gather_k);
         la.store(stage0, t);
         lb.store(stage0 + A_FLOATS, t);
         __syncthreads();
@@ -486,7 +498,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
             if (more) {
                 const int64_t k0 = k_begin + (it + 1) * GEMM_BK;
                 la.load_checked(Ab, a_row_s, a_k_s, m0, k0, g.M, k_end, t);
-                lb.load_checked(Bb, b_row_s, b_k_s, n0, k0, g.N, k_end, t);
+                lb.load_checked(Bb, b_row_s, b_k_s, n0, k0, g.N, k_end, t, g.b_gather_row, g.b_gather_k);
             }
             compute(cur);
             if (more) {
@@ -514,7 +526,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
 #pragma unroll
                 for (int j = 0; j < NB; ++j) {
                     const int64_t col = n0 + wn * TN + tile_pos<BMODE, NB>(j, x);
-                    if (col < g.N) crow[col] = epilogue_value(acc[i][j][e], g.bias, mask, g.relu, row * g.N + col, col);
+                    if (col < g.N) crow[col] = epilogue_value(acc[i][j][e], g.bias, mask, g.relu, row * g.N + col, g.bias_rows ? row : col);
                 }
                 continue;
             }

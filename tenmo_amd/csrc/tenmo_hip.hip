@@ -67,6 +67,9 @@ struct State {
     size_t stage_bytes[3] = {0, 0, 0};
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
     float* one = nullptr; // device constant 1.0f: a stride-0 vector of ones for column sums
+    int32_t* conv_tables = nullptr;  // offset tables [C_in*KH*KW | H_out*W_out] of the last convolution geometry
+    size_t conv_tables_len = 0;      // capacity in entries
+    ConvGeometry conv_geometry{};    // the geometry the tables hold (c_in == 0: none)
     // tuning overrides (environment, read once): -1 = automatic
     int force_tile = -1;
     int force_splitk = -1;
@@ -173,6 +176,9 @@ struct Epilogue {
     const float* bias = nullptr; // + bias[col]
     const float* mask = nullptr; // dense like C: zero the result where mask <= 0
     int relu = 0;                // max(., 0) after the bias
+    int bias_rows = 0;           // bias[row] instead of bias[col]
+    const int32_t* gather_row = nullptr; // B gathered through offset tables (implicit im2col), see GemmArgs
+    const int32_t* gather_k = nullptr;
     bool any() const { return bias || mask || relu; }
 };
 
@@ -193,11 +199,12 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     g.a_rs = a_rs; g.a_cs = a_cs; g.b_rs = b_rs; g.b_cs = b_cs;
     g.M = M; g.N = N; g.K = K;
     g.accumulate = accumulate;
-    g.bias = ep.bias; g.mask = ep.mask; g.relu = ep.relu;
+    g.bias = ep.bias; g.mask = ep.mask; g.relu = ep.relu; g.bias_rows = ep.bias_rows;
+    g.b_gather_row = ep.gather_row; g.b_gather_k = ep.gather_k;
     g.batch = bd;
     g.batch_count = batch_count;
     const int am = operand_mode(a_rs, a_cs, M, K);
-    const int bm = operand_mode(b_cs, b_rs, N, K);
+    const int bm = ep.gather_row ? KMAJOR_GEN : operand_mode(b_cs, b_rs, N, K);
 
     // Pick the workgroup tile and the number of K slices with a small cost model of this chip
     // (constants fitted to measured launches on MI355X): per CU the matrix-pipe time is the sum over
@@ -217,7 +224,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
             const double tiles = tm * tn * (double)batch_count;
             const double m_us = (kTiles[t].bm / 64) * (kTiles[t].bn / 64) * 8 * 64 / 2400.0; // MFMA time of one K step of one wavefront
             for (int sp : kSplits) {
-                if (sp > 1 && (K / sp < 64 || (double)sp * batch_count * M * N * 4.0 > 1.0e9)) break;
+                if (sp > 1 && (K / sp < 64 || (double)sp * batch_count * M * N * 4.0 > 1.0e9 || ep.bias_rows)) break;
                 const double wgs = tiles * sp, slots = cus * kOcc[t];
                 // one round = every CU runs `conc` workgroups side by side; the dispatcher refills a CU
                 // only as slots free, so a partial extra round costs a whole one
@@ -254,7 +261,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
                                sk_wpc ? " (stream-K chosen instead)" : "");
     }
     if (S.force_tile >= 0 && S.force_tile < kNumTiles) tile = S.force_tile;
-    if (S.force_splitk > 0) splits = S.force_splitk;
+    if (S.force_splitk > 0 && !ep.bias_rows) splits = S.force_splitk; // the slice reduction applies the bias by column only
     int streamk = S.force_streamk > 0 ? S.force_streamk : 0;
     if (S.force_streamk < 0 && sk_wpc > 0 && S.force_tile < 0 && S.force_splitk <= 0) { streamk = sk_wpc; tile = sk_tile; }
     if (streamk > 0 && tile <= 1 && am != KMAJOR_GEN && bm != KMAJOR_GEN) {
@@ -720,6 +727,7 @@ int tenmo_hip_shutdown(void) {
     if (S.ws) (void)hipFree(S.ws);
     if (S.ws2) (void)hipFree(S.ws2);
     if (S.one) (void)hipFree(S.one);
+    if (S.conv_tables) (void)hipFree(S.conv_tables);
     for (int i = 0; i < 3; ++i) if (S.stage[i]) (void)hipFree(S.stage[i]);
     (void)hipEventDestroy(S.ev0);
     (void)hipEventDestroy(S.ev1);
@@ -927,6 +935,54 @@ int tenmo_hip_cross_entropy_backward_f32(const float* softmax, const void* targe
         if (vec) hipLaunchKernelGGL((ce_backward_kernel<int32_t, true>), grid, block, 0, S.stream, a);
         else hipLaunchKernelGGL((ce_backward_kernel<int32_t, false>), grid, block, 0, S.stream, a);
     }
+    return finish(sync);
+}
+
+int tenmo_hip_conv2d_forward_f32(const float* padded_image, int64_t n_images, int64_t c_in, int64_t h_pad, int64_t w_pad,
+                                 const float* kernel, int64_t c_out, int64_t kh, int64_t kw, const float* bias,
+                                 int64_t stride, int64_t dilation, float* out, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    const char* who = "tenmo_hip_conv2d_forward_f32";
+    if (n_images < 0 || c_in < 1 || c_out < 1 || kh < 1 || kw < 1 || h_pad < 1 || w_pad < 1)
+        return fail(TENMO_ERR_INVALID_SHAPE, "%s: image (N=%lld, C_in=%lld, %lldx%lld), kernel (C_out=%lld, %lldx%lld): sizes must be positive",
+                    who, (long long)n_images, (long long)c_in, (long long)h_pad, (long long)w_pad, (long long)c_out, (long long)kh, (long long)kw);
+    if (stride < 1 || dilation < 1) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: stride and dilation must be >= 1", who);
+    const int64_t dkh = kh + (kh - 1) * (dilation - 1), dkw = kw + (kw - 1) * (dilation - 1);
+    if (h_pad < dkh || w_pad < dkw) return fail(TENMO_ERR_INVALID_SHAPE, "%s: Invalid output dimensions (the dilated kernel %lldx%lld exceeds the padded image %lldx%lld)",
+                                                who, (long long)dkh, (long long)dkw, (long long)h_pad, (long long)w_pad);
+    const int64_t h_out = (h_pad - dkh) / stride + 1, w_out = (w_pad - dkw) / stride + 1;
+    const int64_t nk = c_in * kh * kw, np = h_out * w_out;
+    if (c_in * h_pad * w_pad > 0x7fffffffLL || nk > 0x7fffffffLL || np > 0x7fffffffLL)
+        return fail(TENMO_ERR_UNSUPPORTED, "%s: one image or one patch matrix dimension exceeds 2^31 elements", who);
+    if (n_images == 0) return 0;
+    if (!padded_image || !kernel || !out) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+
+    // offset tables of this geometry (rebuilt only when the geometry changes)
+    const ConvGeometry geo{(int32_t)c_in, (int32_t)h_pad, (int32_t)w_pad, (int32_t)kh, (int32_t)kw, (int32_t)h_out, (int32_t)w_out, (int32_t)stride, (int32_t)dilation};
+    const size_t need_len = (size_t)(nk + np);
+    if (need_len > S.conv_tables_len) {
+        if (S.conv_tables) {
+            HIP_TRY(hipStreamSynchronize(S.stream));
+            HIP_TRY(hipFree(S.conv_tables));
+            S.conv_tables = nullptr; S.conv_tables_len = 0;
+        }
+        HIP_TRY(hipMalloc(&S.conv_tables, need_len * sizeof(int32_t)));
+        S.conv_tables_len = need_len;
+        S.conv_geometry = ConvGeometry{};
+    }
+    int32_t* by_k = S.conv_tables;
+    int32_t* by_pos = S.conv_tables + nk;
+    if (memcmp(&geo, &S.conv_geometry, sizeof geo) != 0) {
+        const int64_t n = std::max(nk, np);
+        hipLaunchKernelGGL(conv_tables_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, S.stream, geo, by_k, by_pos);
+        S.conv_geometry = geo;
+    }
+    // per image: out[C_out, H_out*W_out] = kernel[C_out, C_in*KH*KW] . patches[C_in*KH*KW, H_out*W_out] + bias[row]
+    BatchDesc bd{};
+    bd.rank = 1; bd.shape[0] = n_images; bd.a_str[0] = 0; bd.b_str[0] = c_in * h_pad * w_pad;
+    Epilogue ep;
+    ep.bias = bias; ep.bias_rows = 1; ep.gather_row = by_pos; ep.gather_k = by_k;
+    if (int rc = gemm_dispatch(kernel, nk, 1, padded_image, 0, 0, out, c_out, np, nk, bd, n_images, 0, ep)) return rc;
     return finish(sync);
 }
 

@@ -51,3 +51,57 @@ def ce_reference64(logits, target, ignore_index=-100, ls=0.0):
     onehot[np.arange(M), t] = 1.0
     grad = (p - (1 - ls) * onehot - ls / C) * valid[:, None]
     return p, loss, grad
+
+
+def conv_case_tensors(case):
+    """image, kernel, bias (or None) and the keyword arguments of one `conv` case of the golden file."""
+    def tensor(spec):
+        if isinstance(spec, dict):
+            return np.full(spec["shape"], spec["fill"], np.float32)
+        return np.array(spec, np.float32)
+    if "image_per_batch_fill" in case:
+        image = np.empty(case["image_shape"], np.float32)
+        for b, v in enumerate(case["image_per_batch_fill"]):
+            image[b] = v
+    elif "image_arange" in case:
+        image = np.arange(int(np.prod(case["image_arange"])), dtype=np.float32).reshape(case["image_arange"])
+    else:
+        image = tensor(case["image"])
+    kernel = tensor(case["kernel"])
+    bias = np.array(case["bias"], np.float32) if "bias" in case else None
+    padding = case.get("padding", "valid")
+    if case.get("padding_kind") == "tuple":
+        padding = tuple(padding)
+    elif case.get("padding_kind") == "list":
+        padding = [tuple(p) for p in padding]
+    return image, kernel, bias, dict(stride=case.get("stride", 1), dilation=case.get("dilation", 1), padding=padding)
+
+
+def check_conv_case(case, out):
+    """Asserts what the reference's test asserts about the output of one `conv` case."""
+    name = case["name"]
+    if "expect_shape" in case:
+        assert list(out.shape) == case["expect_shape"], name
+    if "expect" in case:
+        assert np.allclose(out, np.array(case["expect"], np.float32), atol=1e-5), name
+    if "expect_all" in case:
+        assert np.all(out == case["expect_all"]), name
+    if "expect_planes" in case:
+        for co, v in enumerate(case["expect_planes"]):
+            assert np.all(out[0, co] == v), name
+    for n, co, y, x, v in case.get("expect_at", []):
+        assert abs(out[n, co, y, x] - v) <= 1e-5, name
+
+
+def conv_reference64(image, kernel, bias, stride, dilation, pads):
+    """Zero-padded cross-correlation in fp64 through numpy's sliding windows — shares nothing with the
+    loops of the CPU restatement.  pads = (top, bottom, left, right)."""
+    x = np.pad(image.astype(np.float64), ((0, 0), (0, 0), (pads[0], pads[1]), (pads[2], pads[3])))
+    kh, kw = kernel.shape[2:]
+    dkh, dkw = kh + (kh - 1) * (dilation - 1), kw + (kw - 1) * (dilation - 1)
+    win = np.lib.stride_tricks.sliding_window_view(x, (dkh, dkw), axis=(2, 3))       # [N, C, H', W', dkh, dkw]
+    win = win[:, :, ::stride, ::stride, ::dilation, ::dilation]                       # [N, C, Ho, Wo, kh, kw]
+    out = np.einsum("nchwij,ocij->nohw", win, kernel.astype(np.float64))
+    if bias is not None:
+        out = out + bias.astype(np.float64)[None, :, None, None]
+    return out

@@ -827,3 +827,57 @@ def test_sgd_entry(T, golden, oracle):
             assert np.allclose(V.cpu().numpy(), v_ref, rtol=1e-6, atol=1e-6)
     assert L.tenmo_hip_sgd_step_f32(None, G.data_ptr(), None, 4, 0.1, 0.0, 0.0, 1) == -3
     assert L.tenmo_hip_sgd_step_f32(None, None, None, 0, 0.1, 0.0, 0.0, 1) == 0
+
+
+def test_conv2d_forward(T, golden, oracle):
+    """Conv2dFused.forward through tenmo_hip_conv2d_forward_f32 (implicit GEMM): every forward case of
+    tests/test_cnn.mojo, then random shapes against the CPU restatement and an fp64 reference at the
+    matmul tolerance — channel counts either side of the 64-row tile, K = C_in*KH*KW not a multiple of 4
+    or 16, stride / dilation / padding of every kind, and the layer sizes of examples/mnist_conv."""
+    import ctypes as C
+    import torch
+    from helpers import check_conv_case, conv_case_tensors, conv_reference64
+    from tenmo_amd.cnn import Conv2dFused
+
+    for case in golden["conv"]["cases"]:
+        image, kernel, bias, kw = conv_case_tensors(case)
+        out = Conv2dFused.forward(T.Tensor.from_numpy(image), T.Tensor.from_numpy(kernel),
+                                  T.Tensor.from_numpy(bias) if bias is not None else None, **kw).to_numpy()
+        check_conv_case(case, out)
+    rng = np.random.default_rng(73)
+    for (n, ci, h, w, co, kh, kww, stride, dil, padding, with_bias) in [
+            (2, 3, 9, 11, 4, 3, 3, 1, 1, "valid", True), (1, 2, 8, 8, 3, 3, 2, 2, 1, "same", False),
+            (3, 1, 12, 7, 2, 2, 3, 1, 2, 1, True), (2, 4, 10, 10, 5, 3, 3, 2, 2, (2, 1), True),
+            (1, 3, 7, 9, 2, 1, 1, 1, 1, "valid", False), (2, 2, 6, 6, 3, 3, 3, 3, 1, [(1, 2), (0, 3)], True),
+            (64, 1, 28, 28, 16, 3, 3, 1, 1, "same", True), (16, 16, 14, 14, 32, 3, 3, 1, 1, "same", True),
+            (4, 3, 32, 32, 64, 5, 5, 1, 1, 2, True), (2, 64, 16, 16, 130, 3, 3, 2, 1, 1, True),
+            (1, 8, 40, 56, 96, 3, 3, 1, 2, "valid", False), (0, 3, 8, 8, 4, 3, 3, 1, 1, "valid", True)]:
+        image = rng.standard_normal((n, ci, h, w), dtype=np.float32)
+        kernel = rng.standard_normal((co, ci, kh, kww), dtype=np.float32)
+        bias = rng.standard_normal(co, dtype=np.float32) if with_bias else None
+        case = (n, ci, h, w, co, kh, kww, stride, dil, padding, with_bias)
+        got = Conv2dFused.forward(T.Tensor.from_numpy(image), T.Tensor.from_numpy(kernel),
+                                  T.Tensor.from_numpy(bias) if bias is not None else None, stride=stride, dilation=dil, padding=padding).to_numpy()
+        want = oracle.conv2d_forward(image, kernel, bias, stride=stride, dilation=dil, padding=padding)
+        assert got.shape == want.shape, case
+        if n == 0:
+            continue
+        ref = conv_reference64(image, kernel, bias, stride, dil, oracle.conv_padding(h, w, kh, kww, stride, dil, padding))
+        assert rel_fro(got, ref) <= RTOL_FRO, case
+        assert rel_fro(got, want) <= 2 * RTOL_FRO, case
+    # errors: the reference panics with these messages (cnn.mojo:167-176, :237-241, :132-137)
+    one = T.Tensor.ones(1, 1, 2, 2)
+    with pytest.raises(T.lib.TenmoHipError, match="4D"):
+        Conv2dFused.forward(T.Tensor.ones(1, 2, 2), one)
+    with pytest.raises(T.lib.TenmoHipError, match="input channels"):
+        Conv2dFused.forward(T.Tensor.ones(1, 2, 4, 4), one)
+    with pytest.raises(T.lib.TenmoHipError, match="non-positive output"):
+        Conv2dFused.forward(one, T.Tensor.ones(1, 1, 3, 3))
+    with pytest.raises(T.lib.TenmoHipError, match="bias"):
+        Conv2dFused.forward(T.Tensor.ones(1, 1, 4, 4), one, bias=T.Tensor.ones(2))
+    L = T.lib.load()
+    x = torch.ones(16, device="cuda")
+    assert L.tenmo_hip_conv2d_forward_f32(x.data_ptr(), 1, 1, 2, 2, x.data_ptr(), 1, 3, 3, None, 1, 1, x.data_ptr(), 1) == -2
+    assert b"Invalid output dimensions" in L.tenmo_hip_last_error()
+    assert L.tenmo_hip_conv2d_forward_f32(x.data_ptr(), 1, 1, 4, 4, x.data_ptr(), 1, 2, 2, None, 0, 1, x.data_ptr(), 1) == -3
+    assert L.tenmo_hip_conv2d_forward_f32(None, 1, 1, 4, 4, x.data_ptr(), 1, 2, 2, None, 1, 1, x.data_ptr(), 1) == -3

@@ -368,3 +368,37 @@ def test_sgd_oracle_is_pinned(golden, oracle):
     for want in g["expect_after_each"]:
         oracle.sgd_step(w, np.array(g["grad"], np.float32), v, g["lr"], momentum=g["momentum"])
         assert abs(w[0] - want) < 1e-6
+
+
+def test_conv_oracle_is_pinned(golden, oracle):
+    """The restatement of Conv2dFused.forward (tenmo/cnn.mojo:92-507) against every forward case of
+    tests/test_cnn.mojo that asserts values or shapes, then against two independent computations of a
+    zero-padded cross-correlation on random inputs: numpy sliding windows in fp64 and torch's conv2d in fp64
+    (a swapped kernel index, a wrong stride/dilation product or an off-by-one in the padding fails them)."""
+    import torch
+    from helpers import check_conv_case, conv_case_tensors, conv_reference64
+
+    for case in golden["conv"]["cases"]:
+        image, kernel, bias, kw = conv_case_tensors(case)
+        check_conv_case(case, oracle.conv2d_forward(image, kernel, bias, **kw))
+    rng = np.random.default_rng(71)
+    for (n, ci, h, w, co, kh, kww, stride, dil, padding, with_bias) in [
+            (2, 3, 9, 11, 4, 3, 3, 1, 1, "valid", True), (1, 2, 8, 8, 3, 3, 2, 2, 1, "same", False),
+            (3, 1, 12, 7, 2, 2, 3, 1, 2, 1, True), (2, 4, 10, 10, 5, 3, 3, 2, 2, (2, 1), True),
+            (1, 3, 7, 9, 2, 1, 1, 1, 1, "valid", False), (2, 2, 6, 6, 3, 3, 3, 3, 1, [(1, 2), (0, 3)], True)]:
+        image = rng.standard_normal((n, ci, h, w), dtype=np.float32)
+        kernel = rng.standard_normal((co, ci, kh, kww), dtype=np.float32)
+        bias = rng.standard_normal(co, dtype=np.float32) if with_bias else None
+        got = oracle.conv2d_forward(image, kernel, bias, stride=stride, dilation=dil, padding=padding)
+        pads = oracle.conv_padding(h, w, kh, kww, stride, dil, padding)
+        ref = conv_reference64(image, kernel, bias, stride, dil, pads)
+        assert got.shape == ref.shape and np.allclose(got, ref, rtol=1e-5, atol=1e-5), (n, ci, h, w, co, kh, kww, stride, dil, padding)
+        x = torch.nn.functional.pad(torch.from_numpy(image).double(), (pads[2], pads[3], pads[0], pads[1]))
+        tref = torch.nn.functional.conv2d(x, torch.from_numpy(kernel).double(), None if bias is None else torch.from_numpy(bias).double(),
+                                          stride=stride, dilation=dil).numpy()
+        assert np.allclose(got, tref, rtol=1e-5, atol=1e-5)
+    # error behaviour (cnn.mojo:167-176, :237-241)
+    with pytest.raises(oracle.OracleError):
+        oracle.conv2d_forward(np.ones((1, 2, 4, 4), np.float32), np.ones((1, 3, 2, 2), np.float32))
+    with pytest.raises(oracle.OracleError):
+        oracle.conv2d_forward(np.ones((1, 1, 2, 2), np.float32), np.ones((1, 1, 3, 3), np.float32))
