@@ -78,7 +78,8 @@ struct GemmArgs {
     int32_t relu;         // max(.,0) after the bias                      (ReLU forward)
     int32_t bias_rows;    // the bias is indexed by the row of C instead of the column (convolution: one per filter)
     // Gathered B (implicit im2col): when set, B(n, k) = B[b_gather_row[n] + b_gather_k[k]] instead of
-    // B[k*b_rs + n*b_cs]; the operand then goes through the element-wise loader (KMAJOR_GEN).
+    // B[k*b_rs + n*b_cs]; launched as an MN-major B, loaded through registers with 16-byte loads where
+    // four consecutive n are contiguous in memory.  b_gather_row must be strictly increasing.
     const int32_t* b_gather_row; // [N]
     const int32_t* b_gather_k;   // [K]
     BatchDesc batch;
@@ -199,7 +200,20 @@ struct TileLoader {
                 const int64_t k = k0 + c / QPR;
                 const int64_t row = row0 + 4 * (c % QPR);
                 f32x4 v = {0.f, 0.f, 0.f, 0.f};
-                if (k < K) {
+                if (k < K && gather_row) {
+                    // element (row, k) at base[gather_row[row] + gather_k[k]]; gather_row is increasing, so four
+                    // rows whose offsets span exactly 3 are contiguous in memory (one output row, stride 1)
+                    const float* pk = base + gather_k[k];
+                    if (row + 3 < R) {
+                        const int32_t o0 = gather_row[row], o3 = gather_row[row + 3];
+                        if (o3 - o0 == 3) v = *reinterpret_cast<const f32x4_u*>(pk + o0);
+                        else v = f32x4{pk[o0], pk[gather_row[row + 1]], pk[gather_row[row + 2]], pk[o3]};
+                    } else {
+                        if (row + 0 < R) v.x = pk[gather_row[row]];
+                        if (row + 1 < R) v.y = pk[gather_row[row + 1]];
+                        if (row + 2 < R) v.z = pk[gather_row[row + 2]];
+                    }
+                } else if (k < K) {
                     const float* p = base + k * ks + row;
                     if (row + 3 < R) v = *reinterpret_cast<const f32x4_u*>(p);
                     else {
@@ -217,13 +231,7 @@ struct TileLoader {
                 const int64_t row = row0 + (t >> 2) + 64 * i;
                 const int64_t k = k0 + 4 * kq;
                 f32x4 v = {0.f, 0.f, 0.f, 0.f};
-                if (row < R && gather_row) { // element (row, k) at base[gather_row[row] + gather_k[k]]
-                    const float* p = base + gather_row[row];
-                    if (k + 0 < K) v.x = p[gather_k[k]];
-                    if (k + 1 < K) v.y = p[gather_k[k + 1]];
-                    if (k + 2 < K) v.z = p[gather_k[k + 2]];
-                    if (k + 3 < K) v.w = p[gather_k[k + 3]];
-                } else if (row < R) {
+                if (row < R) {
                     const float* p = base + row * rs + k * ks;
                     if (k + 0 < K) v.x = p[0];
                     if (k + 1 < K) v.y = p[ks];
@@ -388,7 +396,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
         const int64_t a_pitch = AMODE == KMAJOR_VEC ? a_row_s : a_k_s, b_pitch = BMODE == KMAJOR_VEC ? b_row_s : b_k_s;
         const bool a_ok = ((m0 + BM <= g.M) || AMODE == KMAJOR_VEC || (g.M % 4 == 0 && g.M >= 4)) && a_pitch >= 0 && a_pitch <= LA::MAX_DIRECT_PITCH;
         const bool b_ok = ((n0 + BN <= g.N) || BMODE == KMAJOR_VEC || (g.N % 4 == 0 && g.N >= 4)) && b_pitch >= 0 && b_pitch <= LB::MAX_DIRECT_PITCH;
-        const int64_t nfast = (a_ok && b_ok) ? (k_end - k_begin) / GEMM_BK : 0;
+        const int64_t nfast = (a_ok && b_ok && !g.b_gather_row) ? (k_end - k_begin) / GEMM_BK : 0; // a gathered B is register-staged
         if (nfast > 0) {
             constexpr int NLA = LA::NCH, NL = LA::NCH + LB::NCH;  // direct loads per wave per K step
             constexpr int PA = frag_parts<AMODE, MB>(), PB = frag_parts<BMODE, NB>(); // LDS reads per chunk
@@ -522,36 +530,37 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
             const int64_t row = m0 + wm * TM + tile_pos<AMODE, MB>(i, ip);
             if (row >= g.M) continue;
             float* crow = dst.base + (row - dst.row0) * dst.ld - dst.col0;
-            if (fused) { // rare enough to stay scalar
+            float val[NB]; // the finished sums of this row, fused epilogue applied (never combined with accumulate)
 #pragma unroll
-                for (int j = 0; j < NB; ++j) {
+            for (int j = 0; j < NB; ++j) {
+                val[j] = acc[i][j][e];
+                if (fused) {
                     const int64_t col = n0 + wn * TN + tile_pos<BMODE, NB>(j, x);
-                    if (col < g.N) crow[col] = epilogue_value(acc[i][j][e], g.bias, mask, g.relu, row * g.N + col, g.bias_rows ? row : col);
+                    if (col < g.N) val[j] = epilogue_value(val[j], g.bias, mask, g.relu, row * g.N + col, g.bias_rows ? row : col);
                 }
-                continue;
             }
             if constexpr (BMODE == MNMAJOR_VEC && NB > 1) {
                 const int64_t col = n0 + wn * TN + NB * x;
                 if (col + NB <= g.N) {
                     if constexpr (NB == 4) {
-                        f32x4 v = {acc[i][0][e], acc[i][1][e], acc[i][2][e], acc[i][3][e]};
+                        f32x4 v = {val[0], val[1], val[2], val[3]};
                         if (accumulate) v += *reinterpret_cast<const f32x4_u*>(crow + col);
                         *reinterpret_cast<f32x4_u*>(crow + col) = v;
                     } else {
-                        f32x2 v = {acc[i][0][e], acc[i][1][e]};
+                        f32x2 v = {val[0], val[1]};
                         if (accumulate) v += *reinterpret_cast<const f32x2_u*>(crow + col);
                         *reinterpret_cast<f32x2_u*>(crow + col) = v;
                     }
                 } else {
 #pragma unroll
                     for (int j = 0; j < NB; ++j)
-                        if (col + j < g.N) crow[col + j] = accumulate ? crow[col + j] + acc[i][j][e] : acc[i][j][e];
+                        if (col + j < g.N) crow[col + j] = accumulate ? crow[col + j] + val[j] : val[j];
                 }
             } else {
 #pragma unroll
                 for (int j = 0; j < NB; ++j) {
                     const int64_t col = n0 + wn * TN + tile_pos<BMODE, NB>(j, x);
-                    if (col < g.N) crow[col] = accumulate ? crow[col] + acc[i][j][e] : acc[i][j][e];
+                    if (col < g.N) crow[col] = accumulate ? crow[col] + val[j] : val[j];
                 }
             }
         }

@@ -204,7 +204,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     g.batch = bd;
     g.batch_count = batch_count;
     const int am = operand_mode(a_rs, a_cs, M, K);
-    const int bm = ep.gather_row ? KMAJOR_GEN : operand_mode(b_cs, b_rs, N, K);
+    const int bm = ep.gather_row ? MNMAJOR_VEC : operand_mode(b_cs, b_rs, N, K);
 
     // Pick the workgroup tile and the number of K slices with a small cost model of this chip
     // (constants fitted to measured launches on MI355X): per CU the matrix-pipe time is the sum over
@@ -241,7 +241,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         }
         // stream-K (persistent workgroups sharing tiles, see gemm_mfma.hpp): every CU gets the same
         // number of K steps whatever the tile count, at the price of the fix-up traffic
-        if (S.force_streamk < 0 && am != KMAJOR_GEN && bm != KMAJOR_GEN) {
+        if (S.force_streamk < 0 && am != KMAJOR_GEN && bm != KMAJOR_GEN && !ep.gather_row) {
             // Measured: the 128x128 tile with one workgroup per CU is the variant that wins; with many
             // tiles per workgroup the classic launch is as full and shares operand panels in L2 better.
             const int t = 1, wpc = 1;
@@ -264,7 +264,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     if (S.force_splitk > 0 && !ep.bias_rows) splits = S.force_splitk; // the slice reduction applies the bias by column only
     int streamk = S.force_streamk > 0 ? S.force_streamk : 0;
     if (S.force_streamk < 0 && sk_wpc > 0 && S.force_tile < 0 && S.force_splitk <= 0) { streamk = sk_wpc; tile = sk_tile; }
-    if (streamk > 0 && tile <= 1 && am != KMAJOR_GEN && bm != KMAJOR_GEN) {
+    if (streamk > 0 && tile <= 1 && am != KMAJOR_GEN && bm != KMAJOR_GEN && !ep.gather_row) {
         const int bmt = kTiles[tile].bm, bnt = kTiles[tile].bn;
         g.tiles_m = (int32_t)((M + bmt - 1) / bmt);
         g.tiles_n = (int32_t)((N + bnt - 1) / bnt);
