@@ -109,3 +109,22 @@ def test_blas_handle_load_failure_is_recorded(tmp_path):
     assert not h.is_initialized() and "Failed to load" in h.error()
     with pytest.raises(RuntimeError):
         h.matmul(np.zeros((2, 2), np.float32), np.zeros((2, 2), np.float32))
+
+
+def test_conv_padding_parse_matches_reference_shapes(golden):
+    """Host-side padding parse of the Conv2dFused mirror (tenmo/cnn.mojo:183-222) against the output shapes
+    asserted by tests/test_cnn.mojo; no GPU call is made."""
+    from helpers import conv_case_tensors
+    from tenmo_amd.cnn import parse_padding
+
+    for case in golden["conv"]["cases"]:
+        if "expect_shape" not in case and "expect" not in case:
+            continue
+        image, kernel, _, kw = conv_case_tensors(case)
+        kh, kww = kernel.shape[2:]
+        top, bottom, left, right = parse_padding(image.shape[2], image.shape[3], kh, kww, kw["stride"], kw["dilation"], kw["padding"])
+        dkh, dkw = kh + (kh - 1) * (kw["dilation"] - 1), kww + (kww - 1) * (kw["dilation"] - 1)
+        h_out = (image.shape[2] + top + bottom - dkh) // kw["stride"] + 1
+        w_out = (image.shape[3] + left + right - dkw) // kw["stride"] + 1
+        want = case.get("expect_shape") or list(__import__("numpy").array(case["expect"]).shape)
+        assert [image.shape[0], kernel.shape[0], h_out, w_out] == want, case["name"]
