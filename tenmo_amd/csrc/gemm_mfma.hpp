@@ -170,6 +170,71 @@ struct TileLoader {
         asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(lane_off[j]), "s"(src) : "memory");
     }
 
+    // ---- register-staged path (generic strides, gathered operands, ragged MN-major tiles) --------
+    // Per-thread source of chunk i as a 32-bit element offset from the operand's base, fixed for the
+    // whole tile: the K loop only adds the step's offset.  Rows past the extent R are clamped onto the
+    // last valid row (K-major forms: their products are never stored); an MN-major chunk moves 4 rows at
+    // once and cannot be clamped, so `staged_ok` is false for a tile that has such a chunk — or whose
+    // offsets do not fit 31 bits — and that tile takes the checked loads.
+    // (Only the two vector forms take it: issuing a generic operand's 8-16 element loads together costs
+    // 20-35 more registers, which spills next to the 256x128 accumulators and lowers the occupancy of
+    // the 128-row tiles; measured slower than the checked loads, which issue one chunk at a time.)
+    static constexpr bool STAGED_FAST = MODE != KMAJOR_GEN;
+    uint32_t soff[NCH];
+    uint32_t vec_mask;     // gathered MN-major: bit i = the 4 rows of chunk i are contiguous in memory
+    bool staged_ok;
+
+    __device__ __forceinline__ void init_staged(int64_t rs, int64_t ks, int64_t row0, int64_t R, int t, const int32_t* __restrict gather_row) {
+        vec_mask = ~0u;
+        if constexpr (!STAGED_FAST) {
+            staged_ok = false;
+        } else if constexpr (MODE == MNMAJOR_VEC) {
+            staged_ok = row0 + ROWS <= R && R <= 0x7fffffffLL; // uniform over the workgroup
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                const int64_t row = row0 + 4 * ((t + GEMM_THREADS * i) % QPR);
+                soff[i] = (uint32_t)row;
+                if (staged_ok && gather_row) {
+                    const int32_t o0 = gather_row[row];
+                    if (gather_row[row + 3] - o0 != 3) vec_mask &= ~(1u << i); // offsets increase: a span of 3 means contiguous
+                    soff[i] = (uint32_t)o0;
+                }
+            }
+        } else {
+            staged_ok = rs >= 0 && (R - 1) * rs + 16 <= 0x7fffffffLL;
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) soff[i] = (uint32_t)(min(row0 + (t >> 2) + 64 * i, R - 1) * rs + 4 * (t & 3));
+        }
+    }
+
+    // One whole K step (k0 .. k0+15 all valid), no bounds checks.
+    __device__ __forceinline__ void load_staged(const float* __restrict base, int64_t ks, int64_t row0, int64_t k0,
+                                                const int32_t* __restrict gather_row, const int32_t* __restrict gather_k, int t) {
+        if constexpr (!STAGED_FAST) {
+            return;
+        } else if constexpr (MODE == KMAJOR_VEC) {
+            const float* __restrict b0 = base + k0;
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) r[i] = *reinterpret_cast<const f32x4_u*>(b0 + soff[i]);
+        } else if constexpr (MODE == MNMAJOR_VEC) {
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) {
+                const int64_t k = k0 + (t + GEMM_THREADS * i) / QPR;
+                if (gather_row) {
+                    const float* pk = base + gather_k[k] + soff[i];
+                    if (vec_mask >> i & 1) r[i] = *reinterpret_cast<const f32x4_u*>(pk);
+                    else {
+                        const int64_t row = row0 + 4 * ((t + GEMM_THREADS * i) % QPR);
+                        const int32_t o0 = gather_row[row];
+                        r[i] = f32x4{pk[0], pk[gather_row[row + 1] - o0], pk[gather_row[row + 2] - o0], pk[gather_row[row + 3] - o0]};
+                    }
+                } else {
+                    r[i] = *reinterpret_cast<const f32x4_u*>(base + k * ks + soff[i]);
+                }
+            }
+        }
+    }
+
     // register-staged loads with every element checked against the extents (edge tiles, K tail,
     // generic strides)
     __device__ __forceinline__ void load_checked(const float* __restrict base, int64_t rs, int64_t ks,
@@ -494,8 +559,22 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
 
     // ---- edge tiles, the K tail, generic strides: register-staged checked loads, two stages ----
     if (done < nk) {
-        la.load_checked(Ab, a_row_s, a_k_s, m0, k_begin + done * GEMM_BK, g.M, k_end, t);
-        lb.load_checked(Bb, b_row_s, b_k_s, n0, k_begin + done * GEMM_BK, g.N, k_end, t, g.b_gather_row, g.b_gather_k);
+        constexpr bool STAGED_FAST = TileLoader<BM, AMODE>::STAGED_FAST && TileLoader<BN, BMODE>::STAGED_FAST;
+        if constexpr (STAGED_FAST) {
+            la.init_staged(a_row_s, a_k_s, m0, g.M, t, nullptr);
+            lb.init_staged(b_row_s, b_k_s, n0, g.N, t, g.b_gather_row);
+        }
+        // a whole K step goes through the unchecked loads; the K tail and ragged MN-major tiles through the checked ones
+        auto load_a = [&](int64_t k0) {
+            if (STAGED_FAST && la.staged_ok && k0 + GEMM_BK <= k_end) la.load_staged(Ab, a_k_s, m0, k0, nullptr, nullptr, t);
+            else la.load_checked(Ab, a_row_s, a_k_s, m0, k0, g.M, k_end, t);
+        };
+        auto load_b = [&](int64_t k0) {
+            if (STAGED_FAST && lb.staged_ok && k0 + GEMM_BK <= k_end) lb.load_staged(Bb, b_k_s, n0, k0, g.b_gather_row, g.b_gather_k, t);
+            else lb.load_checked(Bb, b_row_s, b_k_s, n0, k0, g.N, k_end, t, g.b_gather_row, g.b_gather_k);
+        };
+        load_a(k_begin + done * GEMM_BK);
+        load_b(k_begin + done * GEMM_BK);
         la.store(stage0, t);
         lb.store(stage0 + A_FLOATS, t);
         __syncthreads();
@@ -505,8 +584,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
             const bool more = (it + 1 < nk);
             if (more) {
                 const int64_t k0 = k_begin + (it + 1) * GEMM_BK;
-                la.load_checked(Ab, a_row_s, a_k_s, m0, k0, g.M, k_end, t);
-                lb.load_checked(Bb, b_row_s, b_k_s, n0, k0, g.N, k_end, t, g.b_gather_row, g.b_gather_k);
+                load_a(k0);
+                load_b(k0);
             }
             compute(cur);
             if (more) {
