@@ -886,6 +886,36 @@ int tenmo_hip_cross_entropy_forward_f32(const float* logits, const void* target,
             const dim3 grid((unsigned)((M + 127) / 128)), block(128);
             if (target_is_int64) hipLaunchKernelGGL(ce_forward_rows_kernel<int64_t>, grid, block, 0, S.stream, a);
             else hipLaunchKernelGGL(ce_forward_rows_kernel<int32_t>, grid, block, 0, S.stream, a);
+        } else if ((uintptr_t)logits % 4 == 0 &&
+                   (softmax_out ? (C >= 40000 && (uintptr_t)softmax_out % 16 == 0 && (uintptr_t)logits % 16 == 0) : C >= 256)) {
+            // streaming form: row statistics (max, 1/sum, loss) in one read-only pass, then the softmax as a flat
+            // sweep.  Always when only the loss is wanted (2x faster than holding the row in registers); with the
+            // softmax for the longest rows, where the two passes together beat the register-resident single pass
+            CeRowStats* stats = nullptr;
+            if (softmax_out) {
+                float* ws;
+                if (int rc = workspace((size_t)M * sizeof(CeRowStats), &ws)) return rc;
+                stats = reinterpret_cast<CeRowStats*>(ws);
+            }
+            if (M > 0x7fffffffLL) return fail(TENMO_ERR_UNSUPPORTED, "%s: grid too large", who);
+            const bool i64 = target_is_int64 != 0;
+            if (C >= 8192) { // the whole workgroup on one row
+                const dim3 grid((unsigned)M), block(CE_THREADS);
+                if (i64) hipLaunchKernelGGL((ce_stats_kernel<int64_t, CE_THREADS / 64, 8>), grid, block, 0, S.stream, a, stats);
+                else hipLaunchKernelGGL((ce_stats_kernel<int32_t, CE_THREADS / 64, 8>), grid, block, 0, S.stream, a, stats);
+            } else { // a wavefront per row
+                const dim3 grid((unsigned)((M + CE_THREADS / 64 - 1) / (CE_THREADS / 64))), block(CE_THREADS);
+                if (i64) hipLaunchKernelGGL((ce_stats_kernel<int64_t, 1, 4>), grid, block, 0, S.stream, a, stats);
+                else hipLaunchKernelGGL((ce_stats_kernel<int32_t, 1, 4>), grid, block, 0, S.stream, a, stats);
+            }
+            if (softmax_out) {
+                constexpr int64_t per_block = CE_THREADS * 4 * 4; // elements per workgroup and pass
+                const int64_t blocks = std::max<int64_t>(1, std::min<int64_t>((M * C + per_block - 1) / per_block, (int64_t)S.cus * 16));
+                CeFlatSteps st{};
+                st.pass_rows = blocks * per_block / C; st.pass_cols = blocks * per_block % C;
+                st.unit_rows = CE_THREADS * 4 / C; st.unit_cols = CE_THREADS * 4 % C;
+                hipLaunchKernelGGL(ce_softmax_flat_kernel, dim3((unsigned)blocks), dim3(CE_THREADS), 0, S.stream, logits, softmax_out, stats, M, C, st);
+            }
         } else {
             // 16-byte accesses need the two arrays congruent modulo 16 bytes (then their rows are too)
             const bool vec = (uintptr_t)logits % 4 == 0 && (!softmax_out || (uintptr_t)softmax_out % 16 == (uintptr_t)logits % 16);

@@ -724,16 +724,18 @@ def test_mlp_graph_replay_matches_eager(T, oracle):
 
 @pytest.mark.gpu
 def test_cross_entropy_entries(T, oracle):
-    """tenmo_hip_cross_entropy_forward_f32 / _backward_f32 against the CPU restatement: thread-per-row
-    and workgroup-per-row kernels, aligned and unaligned rows, int64 and int32 targets, ignore_index,
-    label smoothing, the three reductions, accumulate."""
+    """tenmo_hip_cross_entropy_forward_f32 / _backward_f32 against the CPU restatement: thread-per-row,
+    register-resident and streaming (row statistics + flat softmax sweep, wavefront or workgroup per row)
+    forward kernels, aligned and unaligned rows, int64 and int32 targets, ignore_index, label smoothing,
+    the three reductions, accumulate."""
     import ctypes as C
     import torch
 
     L, lib = T.lib.load(), T.lib
     rng = np.random.default_rng(43)
     for M, Cn, ls, is64 in [(2, 3, 0.0, True), (64, 10, 0.0, False), (33, 17, 0.2, True), (5, 1000, 0.05, True),
-                            (7, 1001, 0.1, False), (300, 64, 0.0, True), (3, 50257, 0.1, True), (2100, 8009, 0.1, True)]:
+                            (7, 1001, 0.1, False), (300, 64, 0.0, True), (3, 50257, 0.1, True), (2100, 8009, 0.1, True),
+                            (37, 9001, 0.05, False), (130, 40003, 0.0, True), (3, 70001, 0.1, True)]:
         x = (3 * rng.standard_normal((M, Cn))).astype(np.float32)
         t = rng.integers(0, Cn, M)
         t[rng.random(M) < 0.3] = -100
@@ -754,8 +756,10 @@ def test_cross_entropy_entries(T, oracle):
         assert np.allclose(sm.cpu().numpy(), p64, rtol=1e-5, atol=1e-7), case
         assert np.allclose(rows.cpu().numpy(), loss64, rtol=1e-5, atol=1e-5), case
         assert np.allclose(sm.cpu().numpy(), sm_ref, rtol=2e-4, atol=1e-7), case
-        assert np.allclose(rows.cpu().numpy(), rows_ref, rtol=1e-5, atol=1e-5), case
-        assert abs(float(total.item()) - total_ref) <= 1e-5 * max(1.0, abs(total_ref)), case
+        loose = 1e-5 if Cn <= 60000 else 5e-5  # the restatement's serial fp32 sums over 70001 classes are off by 1e-5 themselves
+        assert np.allclose(rows.cpu().numpy(), rows_ref, rtol=loose, atol=1e-5), case
+        assert abs(float(total.item()) - total_ref) <= loose * max(1.0, abs(total_ref)), case
+        assert abs(float(total.item()) - float(np.sum(loss64))) <= 1e-5 * max(1.0, abs(float(np.sum(loss64)))), case
         # a softmax buffer that is not congruent with the logits modulo 16 bytes takes the element-wise path
         sm_odd = torch.empty(M * Cn + 1, dtype=torch.float32, device="cuda")
         lib.check(L.tenmo_hip_cross_entropy_forward_f32(X.data_ptr(), Tg.data_ptr(), 1 if is64 else 0, M, Cn, -100, ls,
