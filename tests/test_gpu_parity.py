@@ -885,3 +885,115 @@ def test_conv2d_forward(T, golden, oracle):
     assert b"Invalid output dimensions" in L.tenmo_hip_last_error()
     assert L.tenmo_hip_conv2d_forward_f32(x.data_ptr(), 1, 1, 4, 4, x.data_ptr(), 1, 2, 2, None, 0, 1, x.data_ptr(), 1) == -3
     assert L.tenmo_hip_conv2d_forward_f32(None, 1, 1, 4, 4, x.data_ptr(), 1, 2, 2, None, 1, 1, x.data_ptr(), 1) == -3
+
+
+def _random_matrix_view(rng, rows, cols, layout, pad):
+    """A rows x cols matrix inside a larger storage: row-major, column-major (a transposed view) or both
+    strides > 1, with a padded pitch and a small offset.  Returns (device storage, offset, rs, cs, numpy copy)."""
+    import torch
+    off = int(rng.integers(0, 5))
+    if layout == "row":
+        rs, cs = cols + pad, 1
+        n = off + rows * rs + 8
+    elif layout == "col":
+        rs, cs = 1, rows + pad
+        n = off + cols * cs + 8
+    else:
+        cs = int(rng.integers(2, 4))
+        rs = cols * cs + pad
+        n = off + rows * rs + 8
+    st = rng.standard_normal(n).astype(np.float32)
+    a = np.lib.stride_tricks.as_strided(st[off:], (rows, cols), (4 * rs, 4 * cs)).copy()
+    return torch.from_numpy(st).cuda(), off, rs, cs, a
+
+
+def test_randomized_gemm_views(T):
+    """Seeded sweep of tenmo_hip_gemm_f32: random shapes (ragged against every tile), operand layouts, padded
+    pitches, offsets, accumulate, and forced tile / split-K / stream-K choices, against fp64."""
+    import torch
+    L = T.lib.load()
+    rng = np.random.default_rng(101)
+    try:
+        for case in range(160):
+            big = rng.random() < 0.25
+            M, N, K = (int(rng.integers(1, 700 if big else 200)), int(rng.integers(1, 700 if big else 200)), int(rng.integers(1, 900 if big else 150)))
+            if rng.random() < 0.15:
+                K, M, N = int(rng.integers(1000, 5000)), int(rng.integers(1, 130)), int(rng.integers(1, 130))
+            la, lb = rng.choice(["row", "col", "gen"], p=[0.45, 0.4, 0.15]), rng.choice(["row", "col", "gen"], p=[0.45, 0.4, 0.15])
+            pa, pb = int(rng.choice([0, 0, 1, 3, 4, 8])), int(rng.choice([0, 0, 1, 3, 4, 8]))
+            tile, sk, stk = int(rng.choice([-1, -1, 0, 1, 2, 3, 4])), int(rng.choice([-1, -1, -1, 1, 2, 3])), int(rng.choice([-1, -1, -1, 0, 1, 2]))
+            acc = int(rng.random() < 0.3)
+            A, ao, ars, acs, a = _random_matrix_view(rng, M, K, la, pa)
+            B, bo, brs, bcs, b = _random_matrix_view(rng, K, N, lb, pb)
+            c0 = rng.standard_normal((M, N)).astype(np.float32)
+            Cd = torch.from_numpy(c0.copy()).cuda()
+            L.tenmo_hip_set_tuning(b"gemm_tile", tile)
+            L.tenmo_hip_set_tuning(b"gemm_splitk", sk)
+            L.tenmo_hip_set_tuning(b"gemm_streamk", stk)
+            desc = (case, M, N, K, str(la), str(lb), pa, pb, ao, bo, tile, sk, stk, acc)
+            T.lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), ao, ars, acs, B.data_ptr(), bo, brs, bcs, Cd.data_ptr(), M, N, K, 0, None, None, None, acc, 1))
+            ref = a.astype(np.float64) @ b.astype(np.float64) + (c0 if acc else 0)
+            assert rel_fro(Cd.cpu().numpy(), ref) <= RTOL_FRO, desc
+    finally:
+        for knob in (b"gemm_tile", b"gemm_splitk", b"gemm_streamk"):
+            L.tenmo_hip_set_tuning(knob, -1)
+
+
+def test_randomized_mv_vm_skinny_views(T):
+    """Seeded sweep of the view-level mv / vm / skinny / broadcast-batched entries: random sizes, transposed
+    storage, padded pitches, offsets and batch shapes, against fp64; the element after the result must stay
+    untouched."""
+    import ctypes as C
+    import torch
+    L, lib = T.lib.load(), T.lib
+    rng = np.random.default_rng(103)
+
+    def mk(shape, transpose_last=False, pad=0, off=0):
+        shape = tuple(shape)
+        sshape = shape[:-2] + (shape[-1], shape[-2]) if transpose_last and len(shape) >= 2 else shape
+        pshape = sshape[:-1] + (sshape[-1] + pad,)
+        st = rng.standard_normal(int(np.prod(pshape)) + off + 4).astype(np.float32)
+        strides = [1]
+        for d in reversed(pshape[1:]):
+            strides.insert(0, strides[0] * d)
+        arr = np.lib.stride_tricks.as_strided(st[off:], sshape, tuple(4 * x for x in strides))
+        vshape, vstr = list(sshape), list(strides)
+        if transpose_last and len(shape) >= 2:
+            vstr[-1], vstr[-2] = vstr[-2], vstr[-1]
+            vshape[-1], vshape[-2] = vshape[-2], vshape[-1]
+            arr = np.swapaxes(arr, -1, -2)
+        dev = torch.from_numpy(st).cuda()
+        return dev, lib.make_view(dev.data_ptr(), off, vshape, vstr), arr.copy()
+
+    for case in range(120):
+        kind = str(rng.choice(["mv", "vm", "skinny", "bmm"]))
+        pad, off, tr = int(rng.choice([0, 0, 1, 2, 3, 4])), int(rng.choice([0, 0, 1, 2, 4])), bool(rng.random() < 0.4)
+        bshape = tuple(int(rng.integers(1, 4)) for _ in range(int(rng.choice([0, 0, 1, 2]))))
+        if kind == "mv":
+            R, K = int(rng.integers(1, 3000)), int(rng.integers(1, 5000))
+            if rng.random() < 0.2:
+                R, K = int(rng.integers(1, 40)), int(rng.integers(5000, 70000))
+            d1, v1, a = mk(bshape + (R, K), tr, pad, off)
+            d2, v2, b = mk((K,), False, 0, int(rng.choice([0, 1])))
+            ref, fn = np.einsum("...rk,k->...r", a.astype(np.float64), b.astype(np.float64)), L.tenmo_hip_matrix_vector_nd
+        elif kind == "vm":
+            K, N = int(rng.integers(1, 3000)), int(rng.integers(1, 6000))
+            d1, v1, a = mk((K,), False, 0, int(rng.choice([0, 1])))
+            d2, v2, b = mk(bshape + (K, N), tr, pad, off)
+            ref, fn = np.einsum("k,...kn->...n", a.astype(np.float64), b.astype(np.float64)), L.tenmo_hip_vector_matmul_nd
+        elif kind == "skinny":
+            M, K, N = int(rng.integers(1, 9)), int(rng.integers(1, 1500)), int(rng.integers(2048, 9000))
+            d1, v1, a = mk((M, K), bool(rng.random() < 0.3), 0, 0)
+            d2, v2, b = mk(bshape + (K, N), False, pad, off)
+            ref, fn = a.astype(np.float64) @ b.astype(np.float64), L.tenmo_hip_matmul_nd
+        else:
+            M, K, N = int(rng.integers(1, 150)), int(rng.integers(1, 200)), int(rng.integers(1, 150))
+            ba = tuple(1 if rng.random() < 0.3 else x for x in bshape)
+            d1, v1, a = mk(ba + (M, K), bool(rng.random() < 0.4), pad, off)
+            d2, v2, b = mk(bshape + (K, N), tr, 0, 0)
+            ref, fn = a.astype(np.float64) @ b.astype(np.float64), L.tenmo_hip_matmul_nd
+        out = torch.full((int(np.prod(ref.shape)) + 1,), 7.0, device="cuda")
+        desc = (case, kind, a.shape, b.shape, tr, pad, off)
+        lib.check(fn(C.byref(v1), C.byref(v2), out.data_ptr(), 1))
+        assert rel_fro(out[:-1].cpu().numpy().reshape(ref.shape), ref) <= RTOL_FRO, desc
+        assert float(out[-1]) == 7.0, desc
