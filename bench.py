@@ -28,9 +28,9 @@ PEAK_FP32_MFMA_TFLOPS = 157.3  # 256 CU x 2.4 GHz x 256 flop/clk/CU
 PEAK_HBM_GBPS = 8000.0
 
 # Bytes moved between L2 and the memory fabric per 8192^3 launch, from two rocprofv3 --pmc runs
-# (FETCH_SIZE 4.50e6 KiB scaled by 2.0, WRITE_SIZE 2.621e5 KiB scaled by 1.0; the scale factors are
+# (FETCH_SIZE 2.965e6 KiB scaled by 2.0, WRITE_SIZE 2.621e5 KiB scaled by 1.0; the scale factors are
 # what the same counters read for a plain 1 GiB copy).  Only valid for the default size.
-MEASURED_TRAFFIC_BYTES = 9.5e9
+MEASURED_TRAFFIC_BYTES = 6.3e9
 
 
 def main() -> int:

@@ -375,9 +375,7 @@ __device__ __forceinline__ void bare_barrier() {
 
 // position of tile number `tid` (0 .. tiles_m*tiles_n-1) in the tile grid.
 // Workgroup ids are dealt round-robin to the 8 XCDs (checked with HW_REG_XCC_ID), so with groups
-// of 8 tile-rows each XCD keeps one tile-row of A hot in its L2 and streams B past it.  Giving
-// each XCD a compact 8x8 block of tiles instead was measured: 1.8x the L2-miss traffic (a tall A
-// panel at a power-of-two row pitch thrashes a few L2 sets) and up to 4 % slower.
+// of 8 tile-rows each XCD keeps one tile-row of A hot in its L2 and streams B past it.
 __device__ __forceinline__ void tile_coords(const GemmArgs& g, int64_t tid, int64_t& tile_m, int64_t& tile_n) {
     constexpr int GROUP_M = 8;
     const int64_t per_group = (int64_t)GROUP_M * g.tiles_n;
@@ -385,6 +383,28 @@ __device__ __forceinline__ void tile_coords(const GemmArgs& g, int64_t tid, int6
     const int64_t gsz = min((int64_t)g.tiles_m - first_m, (int64_t)GROUP_M);
     tile_m = first_m + (tid % per_group) % gsz;
     tile_n = (tid % per_group) / gsz;
+}
+
+// The same for the one-workgroup-per-tile launch of the 256x128 tile, whose 64 resident workgroups per
+// XCD (2 per CU) then form one block of 2 x 32 (or 4 x 16) tiles: the XCD's L2 fetches 2 (4) panels of A
+// and 32 (16) of B per round instead of 1 and 64.  Measured at 8192^3: L2-miss traffic 9.2 GB -> 5.9 GB
+// (6.2 GB for 4 x 16), run time unchanged (the kernel is bound by the matrix pipe); an 8 x 8 block has
+// the least traffic on paper but measured 11.5 GB — eight A panels at a power-of-two row pitch thrash a
+// few L2 sets.  Tile grids that do not divide into such blocks keep the order above.
+template <int BM, int BN>
+__device__ __forceinline__ void tile_coords_blocked(const GemmArgs& g, int64_t tid, int64_t& tile_m, int64_t& tile_n) {
+    if constexpr (BM == 256 && BN == 128) {
+        const int rn = g.tiles_n % 32 == 0 ? 32 : 16, rm = 64 / rn;
+        const int64_t bm_count = g.tiles_m / rm, bn_count = g.tiles_n / rn;
+        if (g.tiles_m % rm == 0 && g.tiles_n % rn == 0 && (bm_count * bn_count) % 8 == 0) {
+            const int64_t xcd = tid % 8, j = tid / 8, round = j / 64, q = j % 64;
+            const int64_t block = round * 8 + xcd; // the 8 XCDs work on 8 neighbouring blocks at a time
+            tile_m = (block / bn_count) * rm + q % rm;
+            tile_n = (block % bn_count) * rn + q / rm;
+            return;
+        }
+    }
+    tile_coords(g, tid, tile_m, tile_n);
 }
 
 // where a finished tile goes: element (row, col) of the product is written to
@@ -661,7 +681,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     const int64_t pid = blockIdx.x;
     const int64_t batch = pid / tiles;
     int64_t tile_m, tile_n;
-    tile_coords(g, pid % tiles, tile_m, tile_n);
+    tile_coords_blocked<BM, BN>(g, pid % tiles, tile_m, tile_n);
 
     int64_t k_begin = 0, k_end = g.K;
     TileDest dst;

@@ -997,3 +997,28 @@ def test_randomized_mv_vm_skinny_views(T):
         lib.check(fn(C.byref(v1), C.byref(v2), out.data_ptr(), 1))
         assert rel_fro(out[:-1].cpu().numpy().reshape(ref.shape), ref) <= RTOL_FRO, desc
         assert float(out[-1]) == 7.0, desc
+
+
+def test_blocked_tile_order(T):
+    """The 256x128 tile's one-workgroup-per-tile launch walks tile grids that divide into 2x32 / 4x16 blocks
+    per XCD in block order: every tile must still be computed exactly once (shapes whose grids do and do not
+    divide, with K slices and batches on top)."""
+    import torch
+    L = T.lib.load()
+    rng = np.random.default_rng(107)
+    try:
+        L.tenmo_hip_set_tuning(b"gemm_tile", 0)
+        L.tenmo_hip_set_tuning(b"gemm_streamk", 0)
+        for (M, N, K, sk, nb) in [(512, 32768, 40, 1, 1), (8192, 6144, 24, 1, 1), (1024, 16384, 130, 2, 1), (512, 8192, 33, 1, 4), (768, 32768, 17, 1, 1), (4096, 4096, 16, 1, 1)]:
+            L.tenmo_hip_set_tuning(b"gemm_splitk", sk)
+            a = rng.standard_normal((nb, M, K), dtype=np.float32)
+            b = rng.standard_normal((K, N), dtype=np.float32)
+            A, B = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+            Cd = torch.empty((nb, M, N), dtype=torch.float32, device="cuda")
+            T.lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, K, 1, B.data_ptr(), 0, N, 1, Cd.data_ptr(), M, N, K,
+                                             1, T.lib.i64([nb]), T.lib.i64([M * K]), T.lib.i64([0]), 0, 1))
+            ref = a.astype(np.float64) @ b.astype(np.float64)
+            assert rel_fro(Cd.cpu().numpy(), ref) <= RTOL_FRO, (M, N, K, sk, nb)
+    finally:
+        for knob in (b"gemm_tile", b"gemm_splitk", b"gemm_streamk"):
+            L.tenmo_hip_set_tuning(knob, -1)
