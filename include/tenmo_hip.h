@@ -214,6 +214,23 @@ int tenmo_hip_cross_entropy_backward_f32(const float* softmax, const void* targe
 int tenmo_hip_conv2d_forward_f32(const float* padded_image, int64_t n_images, int64_t c_in, int64_t h_pad, int64_t w_pad,
                                  const float* kernel, int64_t c_out, int64_t kh, int64_t kw, const float* bias,
                                  int64_t stride, int64_t dilation, float* out, int32_t sync);
+/* FusedCol2ImBackward.backward — tenmo/cnn.mojo:546-948: the three gradients of the fused convolution
+ * for the upstream gradient grad_out [N, C_out, H_out, W_out]; each output pointer may be NULL (that
+ * parent does not require a gradient):
+ *   grad_bias[co]               = sum over (n, y, x) of grad_out                      (:669-713)
+ *   grad_kernel[co, ci, ky, kx] = sum over (n, y, x) of grad_out[n, co, y, x] *
+ *                                 padded_image[n, ci, y*stride + ky*dilation, x*stride + kx*dilation]   (:716-815)
+ *   grad_padded_image[n, ci, y*stride + ky*dilation, x*stride + kx*dilation] += kernel[co, ci, ky, kx] *
+ *                                 grad_out[n, co, y, x]   over all (co, ky, kx, y, x)   (:818-948)
+ * accumulate != 0 adds into the three outputs (the reference's update_grad(AddTensor), :607-650) instead
+ * of overwriting them.  The gradient is with respect to the PADDED image, as in the reference (its Pad
+ * operator's backward removes the border).  All three run on the matrix-core GEMM: the kernel gradient
+ * with the patches gathered (no patch matrix), the image gradient as a stride-1 convolution of the
+ * spread-out upstream gradient with the reversed kernel. */
+int tenmo_hip_conv2d_backward_f32(const float* padded_image, int64_t n_images, int64_t c_in, int64_t h_pad, int64_t w_pad,
+                                  const float* kernel, int64_t c_out, int64_t kh, int64_t kw, int64_t stride, int64_t dilation,
+                                  const float* grad_out, float* grad_padded_image, float* grad_kernel, float* grad_bias,
+                                  int32_t accumulate, int32_t sync);
 /* SGDStep.launch_no_momentum / launch_momentum — tenmo/kernels/sgd_kernel.mojo:56-143 (CPU form:
  * tenmo/optim.mojo:93-160): g += weight_decay * p when weight_decay > 0; with velocity != NULL
  * v = momentum * v + g, p -= lr * v; else p -= lr * g. */

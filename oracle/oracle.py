@@ -87,6 +87,8 @@ def lib():
         L.oracle_cross_entropy_forward_f32.argtypes = [fp, i64p, C.c_int64, C.c_int64, C.c_int64, C.c_float, fp, fp, fp, i32p]
         L.oracle_cross_entropy_backward_f32.argtypes = [fp, i64p, fp, C.c_int64, C.c_int64, C.c_int64, C.c_float, C.c_int, C.c_int32, fp]
         L.oracle_sgd_step_f32.argtypes = [fp, fp, fp, C.c_int64, C.c_float, C.c_float, C.c_float]
+        L.oracle_conv2d_backward_f32.argtypes = [fp, C.c_int64, C.c_int64, C.c_int64, C.c_int64, fp, C.c_int64, C.c_int64, C.c_int64,
+                                                 C.c_int64, C.c_int64, fp, fp, fp, fp]
         L.oracle_conv2d_forward_f32.argtypes = [fp, C.c_int64, C.c_int64, C.c_int64, C.c_int64, fp, C.c_int64, C.c_int64, C.c_int64,
                                                 fp, C.c_int64, C.c_int64, fp]
         _lib = L
@@ -437,3 +439,20 @@ def conv2d_forward(image: np.ndarray, kernel: np.ndarray, bias: Optional[np.ndar
                                            c_out, kh, kw, b.ctypes.data_as(fpp) if b is not None else None, stride, dilation,
                                            out.ctypes.data_as(fpp)))
     return out
+
+
+def conv2d_backward(image: np.ndarray, kernel: np.ndarray, grad_out: np.ndarray, stride: int = 1, dilation: int = 1, padding="valid"):
+    """(grad_image, grad_kernel, grad_bias) of Conv2dFused for the upstream gradient `grad_out`: the fused backward
+    on the padded image (tenmo/cnn.mojo:546-948), then the border removed as the Pad operator's backward does."""
+    n, c_in, h_in, w_in = image.shape
+    c_out, _, kh, kw = kernel.shape
+    top, bottom, left, right = conv_padding(h_in, w_in, kh, kw, stride, dilation, padding)
+    padded = np.ascontiguousarray(np.pad(image.astype(np.float32), ((0, 0), (0, 0), (top, bottom), (left, right))))
+    kern = np.ascontiguousarray(kernel, dtype=np.float32)
+    go = np.ascontiguousarray(grad_out, dtype=np.float32)
+    g_pad, g_k, g_b = np.empty_like(padded), np.empty_like(kern), np.empty(c_out, np.float32)
+    fpp = C.POINTER(C.c_float)
+    _check(lib().oracle_conv2d_backward_f32(padded.ctypes.data_as(fpp), n, c_in, padded.shape[2], padded.shape[3], kern.ctypes.data_as(fpp),
+                                            c_out, kh, kw, stride, dilation, go.ctypes.data_as(fpp),
+                                            g_pad.ctypes.data_as(fpp), g_k.ctypes.data_as(fpp), g_b.ctypes.data_as(fpp)))
+    return g_pad[:, :, top:top + h_in, left:left + w_in].copy(), g_k, g_b

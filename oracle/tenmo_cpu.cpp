@@ -696,4 +696,55 @@ int oracle_conv2d_forward_f32(const float* padded_image, int64_t n_images, int64
     return 0;
 }
 
+// The three gradients of the fused convolution, FusedCol2ImBackward (tenmo/cnn.mojo:546-948), for the upstream
+// gradient grad_out [N, C_out, H_out, W_out]; a null output is skipped.  Bias: the sum over (n, y, x) per channel
+// (:669-713).  Kernel: grad_out viewed [C_out, N*H_out*W_out] times the patch matrix (:716-815; the reference
+// builds the patches and calls Tensor.matmul — here the same sums in the order n, y, x).  Padded image: the
+// scatter loop of :818-948 in its order (n, y, x, co, ci, ky, kx), with its skip of zero upstream values.
+int oracle_conv2d_backward_f32(const float* padded_image, int64_t n_images, int64_t c_in, int64_t h_pad, int64_t w_pad,
+                               const float* kernel, int64_t c_out, int64_t kh, int64_t kw, int64_t stride, int64_t dilation,
+                               const float* grad_out, float* grad_padded_image, float* grad_kernel, float* grad_bias) {
+    if (c_in < 1 || c_out < 1 || kh < 1 || kw < 1 || stride < 1 || dilation < 1) return fail("conv2d backward: sizes, stride and dilation must be positive");
+    const int64_t dkh = kh + (kh - 1) * (dilation - 1), dkw = kw + (kw - 1) * (dilation - 1);
+    if (h_pad < dkh || w_pad < dkw) return fail("conv2d backward: Invalid output dimensions");
+    const int64_t h_out = (h_pad - dkh) / stride + 1, w_out = (w_pad - dkw) / stride + 1;
+    auto go = [&](int64_t n, int64_t co, int64_t y, int64_t x) { return grad_out[((n * c_out + co) * h_out + y) * w_out + x]; };
+    if (grad_bias)
+        for (int64_t co = 0; co < c_out; ++co) {
+            float acc = 0.f;
+            for (int64_t n = 0; n < n_images; ++n)
+                for (int64_t y = 0; y < h_out; ++y)
+                    for (int64_t x = 0; x < w_out; ++x) acc += go(n, co, y, x);
+            grad_bias[co] = acc;
+        }
+    if (grad_kernel)
+        for (int64_t co = 0; co < c_out; ++co)
+            for (int64_t ci = 0; ci < c_in; ++ci)
+                for (int64_t ky = 0; ky < kh; ++ky)
+                    for (int64_t kx = 0; kx < kw; ++kx) {
+                        float acc = 0.f;
+                        for (int64_t n = 0; n < n_images; ++n)
+                            for (int64_t y = 0; y < h_out; ++y)
+                                for (int64_t x = 0; x < w_out; ++x)
+                                    acc += go(n, co, y, x) * padded_image[((n * c_in + ci) * h_pad + y * stride + ky * dilation) * w_pad + x * stride + kx * dilation];
+                        grad_kernel[((co * c_in + ci) * kh + ky) * kw + kx] = acc;
+                    }
+    if (grad_padded_image) {
+        for (int64_t i = 0; i < n_images * c_in * h_pad * w_pad; ++i) grad_padded_image[i] = 0.f;
+        for (int64_t n = 0; n < n_images; ++n)
+            for (int64_t y = 0; y < h_out; ++y)
+                for (int64_t x = 0; x < w_out; ++x)
+                    for (int64_t co = 0; co < c_out; ++co) {
+                        const float g = go(n, co, y, x);
+                        if (g == 0.f) continue;
+                        for (int64_t ci = 0; ci < c_in; ++ci)
+                            for (int64_t ky = 0; ky < kh; ++ky)
+                                for (int64_t kx = 0; kx < kw; ++kx)
+                                    grad_padded_image[((n * c_in + ci) * h_pad + y * stride + ky * dilation) * w_pad + x * stride + kx * dilation] +=
+                                        g * kernel[((co * c_in + ci) * kh + ky) * kw + kx];
+                    }
+    }
+    return 0;
+}
+
 } // extern "C"

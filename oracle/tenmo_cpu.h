@@ -105,6 +105,11 @@ int oracle_conv2d_forward_f32(const float* padded_image, int64_t n_images, int64
                               const float* kernel, int64_t c_out, int64_t kh, int64_t kw, const float* bias,
                               int64_t stride, int64_t dilation, float* out);
 
+/* FusedCol2ImBackward: bias, kernel and padded-image gradients, tenmo/cnn.mojo:546-948 */
+int oracle_conv2d_backward_f32(const float* padded_image, int64_t n_images, int64_t c_in, int64_t h_pad, int64_t w_pad,
+                               const float* kernel, int64_t c_out, int64_t kh, int64_t kw, int64_t stride, int64_t dilation,
+                               const float* grad_out, float* grad_padded_image, float* grad_kernel, float* grad_bias);
+
 #ifdef __cplusplus
 }
 #endif

@@ -82,6 +82,8 @@ SIGNATURES = {
                                                        C.c_int32, C.c_int32, _ptr, C.c_int32, C.c_int32]),
     "tenmo_hip_conv2d_forward_f32": (C.c_int, [_ptr, C.c_int64, C.c_int64, C.c_int64, C.c_int64, _ptr, C.c_int64, C.c_int64, C.c_int64,
                                                _ptr, C.c_int64, C.c_int64, _ptr, C.c_int32]),
+    "tenmo_hip_conv2d_backward_f32": (C.c_int, [_ptr, C.c_int64, C.c_int64, C.c_int64, C.c_int64, _ptr, C.c_int64, C.c_int64, C.c_int64,
+                                                C.c_int64, C.c_int64, _ptr, _ptr, _ptr, _ptr, C.c_int32, C.c_int32]),
     "tenmo_hip_sgd_step_f32": (C.c_int, [_ptr, _ptr, _ptr, C.c_int64, C.c_float, C.c_float, C.c_float, C.c_int32]),
     "cblas_sgemm": (None, [C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_int, C.c_float, _ptr, C.c_int,
                            _ptr, C.c_int, C.c_float, _ptr, C.c_int]),

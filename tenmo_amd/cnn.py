@@ -4,8 +4,9 @@ The reference's layer parses ``padding`` ("valid", "same", int, (h, w) pair, [(t
 cnn.mojo:183-222), zero-pads the image with its ``Pad`` operator (:229-235) and hands the padded image to
 the fused im2col kernel (``FusedIm2Col.forward``, :308-507).  The same split is kept here: the padding is a
 device-side copy (plumbing, ``torch.nn.functional.pad``), the convolution itself runs in the library as an
-implicit GEMM on the matrix-core kernel.  Forward only: the reference's backward (``FusedCol2ImBackward``,
-cnn.mojo:546-950) is not part of this build; its kernel gradient is a plain ``Tensor.matmul`` (:799).
+implicit GEMM on the matrix-core kernel.  ``Conv2dFused.backward`` is ``FusedCol2ImBackward`` (cnn.mojo:546-948)
+through ``tenmo_hip_conv2d_backward_f32`` followed by the removal of the padding border (the ``Pad`` operator's
+backward); it is a plain function here, not wired into the autograd mirror of ``tensor.py``.
 """
 from __future__ import annotations
 
@@ -82,3 +83,32 @@ class Conv2dFused:
         if not sync:
             check(L.tenmo_hip_sync())  # `img` (a temporary when padded) must outlive the launch
         return Tensor(out)
+
+    @staticmethod
+    def backward(image: Tensor, kernel: Tensor, grad_out: Tensor, stride: int = 1, dilation: int = 1, padding: Padding = "valid",
+                 need_image: bool = True, need_kernel: bool = True, need_bias: bool = True):
+        """(grad_image, grad_kernel, grad_bias) for the upstream gradient of ``forward``'s output; entries not needed are None."""
+        n, c_in, h_in, w_in = image.shape()
+        c_out, _, kh, kw = kernel.shape()
+        top, bottom, left, right = parse_padding(h_in, w_in, kh, kw, stride, dilation, padding)
+        h_pad, w_pad = h_in + top + bottom, w_in + left + right
+        for t, who in ((image, "image"), (kernel, "kernel"), (grad_out, "grad_out")):
+            if not t.buffer.is_contiguous():
+                raise TenmoHipError(-4, f"Conv2dFused.backward: {who} must be contiguous")
+        _lib.init()
+        img = image.buffer.storage[image.buffer.offset:image.buffer.offset + n * c_in * h_in * w_in].view(n, c_in, h_in, w_in)
+        if top or bottom or left or right:
+            img = torch.nn.functional.pad(img, (left, right, top, bottom)).contiguous()
+        g_pad = NDBuffer.empty((n, c_in, h_pad, w_pad)) if need_image else None
+        g_k = NDBuffer.empty((c_out, c_in, kh, kw)) if need_kernel else None
+        g_b = NDBuffer.empty((c_out,)) if need_bias else None
+        L = _lib.load()
+        check(L.tenmo_hip_conv2d_backward_f32(img.data_ptr(), n, c_in, h_pad, w_pad, kernel.buffer.data_ptr() + 4 * kernel.buffer.offset,
+                                              c_out, kh, kw, stride, dilation, grad_out.buffer.data_ptr() + 4 * grad_out.buffer.offset,
+                                              g_pad.data_ptr() if g_pad else None, g_k.data_ptr() if g_k else None,
+                                              g_b.data_ptr() if g_b else None, 0, 1))
+        g_img = None
+        if g_pad is not None:  # Pad backward: drop the border
+            inner = g_pad.storage[:n * c_in * h_pad * w_pad].view(n, c_in, h_pad, w_pad)[:, :, top:top + h_in, left:left + w_in].contiguous()
+            g_img = Tensor(NDBuffer(inner.view(-1), (n, c_in, h_in, w_in)))
+        return g_img, Tensor(g_k) if g_k else None, Tensor(g_b) if g_b else None

@@ -266,4 +266,31 @@ __global__ void conv_tables_kernel(const ConvGeometry c, int32_t* __restrict by_
     }
 }
 
+// Upstream gradient [planes, h_out, w_out] spread out for the input-gradient convolution: element (y, x) goes
+// to (off_y + y*stride, off_x + x*stride) of a zero-filled [planes, h_dst, w_dst] array.
+__global__ void conv_dilate_pad_kernel(const float* __restrict src, float* __restrict dst, int64_t planes, int h_out, int w_out,
+                                       int h_dst, int w_dst, int stride, int off_y, int off_x) {
+    const int64_t total = planes * h_dst * w_dst;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int xx = (int)(i % w_dst), yy = (int)((i / w_dst) % h_dst);
+        const int64_t plane = i / ((int64_t)w_dst * h_dst);
+        const int ry = yy - off_y, rx = xx - off_x;
+        float v = 0.f;
+        if (ry >= 0 && rx >= 0 && ry % stride == 0 && rx % stride == 0) {
+            const int y = ry / stride, x = rx / stride;
+            if (y < h_out && x < w_out) v = src[(plane * h_out + y) * w_out + x];
+        }
+        dst[i] = v;
+    }
+}
+
+// kernel [c_out, c_in, kh, kw] -> [c_in, c_out, kh, kw] with both spatial axes reversed
+__global__ void conv_flip_kernel(const float* __restrict src, float* __restrict dst, int c_out, int c_in, int kh, int kw) {
+    const int total = c_out * c_in * kh * kw;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= total) return;
+    const int kx = i % kw, ky = (i / kw) % kh, co = (i / (kw * kh)) % c_out, ci = i / (kw * kh * c_out);
+    dst[i] = src[((co * c_in + ci) * kh + (kh - 1 - ky)) * kw + (kw - 1 - kx)];
+}
+
 } // namespace tenmo

@@ -968,27 +968,11 @@ int tenmo_hip_cross_entropy_backward_f32(const float* softmax, const void* targe
     return finish(sync);
 }
 
-int tenmo_hip_conv2d_forward_f32(const float* padded_image, int64_t n_images, int64_t c_in, int64_t h_pad, int64_t w_pad,
-                                 const float* kernel, int64_t c_out, int64_t kh, int64_t kw, const float* bias,
-                                 int64_t stride, int64_t dilation, float* out, int32_t sync) {
-    if (int rc = ensure_ready()) return rc;
-    const char* who = "tenmo_hip_conv2d_forward_f32";
-    if (n_images < 0 || c_in < 1 || c_out < 1 || kh < 1 || kw < 1 || h_pad < 1 || w_pad < 1)
-        return fail(TENMO_ERR_INVALID_SHAPE, "%s: image (N=%lld, C_in=%lld, %lldx%lld), kernel (C_out=%lld, %lldx%lld): sizes must be positive",
-                    who, (long long)n_images, (long long)c_in, (long long)h_pad, (long long)w_pad, (long long)c_out, (long long)kh, (long long)kw);
-    if (stride < 1 || dilation < 1) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: stride and dilation must be >= 1", who);
-    const int64_t dkh = kh + (kh - 1) * (dilation - 1), dkw = kw + (kw - 1) * (dilation - 1);
-    if (h_pad < dkh || w_pad < dkw) return fail(TENMO_ERR_INVALID_SHAPE, "%s: Invalid output dimensions (the dilated kernel %lldx%lld exceeds the padded image %lldx%lld)",
-                                                who, (long long)dkh, (long long)dkw, (long long)h_pad, (long long)w_pad);
-    const int64_t h_out = (h_pad - dkh) / stride + 1, w_out = (w_pad - dkw) / stride + 1;
-    const int64_t nk = c_in * kh * kw, np = h_out * w_out;
-    if (c_in * h_pad * w_pad > 0x7fffffffLL || nk > 0x7fffffffLL || np > 0x7fffffffLL)
-        return fail(TENMO_ERR_UNSUPPORTED, "%s: one image or one patch matrix dimension exceeds 2^31 elements", who);
-    if (n_images == 0) return 0;
-    if (!padded_image || !kernel || !out) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
-
-    // offset tables of this geometry (rebuilt only when the geometry changes)
-    const ConvGeometry geo{(int32_t)c_in, (int32_t)h_pad, (int32_t)w_pad, (int32_t)kh, (int32_t)kw, (int32_t)h_out, (int32_t)w_out, (int32_t)stride, (int32_t)dilation};
+// out[n, c_out, h_out, w_out] (+)= conv(padded_image, kernel) + bias as an implicit GEMM per image:
+// out[C_out, H_out*W_out] = kernel[C_out, C_in*KH*KW] . patches[C_in*KH*KW, H_out*W_out] + bias[row].
+// Sizes are validated by the callers.  The offset tables are rebuilt only when the geometry changes.
+static int conv_tables(const ConvGeometry& geo, int32_t** by_k, int32_t** by_pos) {
+    const int64_t nk = (int64_t)geo.c_in * geo.kh * geo.kw, np = (int64_t)geo.h_out * geo.w_out;
     const size_t need_len = (size_t)(nk + np);
     if (need_len > S.conv_tables_len) {
         if (S.conv_tables) {
@@ -1000,19 +984,119 @@ int tenmo_hip_conv2d_forward_f32(const float* padded_image, int64_t n_images, in
         S.conv_tables_len = need_len;
         S.conv_geometry = ConvGeometry{};
     }
-    int32_t* by_k = S.conv_tables;
-    int32_t* by_pos = S.conv_tables + nk;
+    *by_k = S.conv_tables;
+    *by_pos = S.conv_tables + nk;
     if (memcmp(&geo, &S.conv_geometry, sizeof geo) != 0) {
         const int64_t n = std::max(nk, np);
-        hipLaunchKernelGGL(conv_tables_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, S.stream, geo, by_k, by_pos);
+        hipLaunchKernelGGL(conv_tables_kernel, dim3((unsigned)((n + 255) / 256)), dim3(256), 0, S.stream, geo, *by_k, *by_pos);
         S.conv_geometry = geo;
     }
-    // per image: out[C_out, H_out*W_out] = kernel[C_out, C_in*KH*KW] . patches[C_in*KH*KW, H_out*W_out] + bias[row]
+    return 0;
+}
+
+static int conv_forward_impl(const float* padded_image, int64_t n_images, const ConvGeometry& geo, const float* kernel, int64_t c_out,
+                             const float* bias, float* out, int accumulate) {
+    int32_t *by_k, *by_pos;
+    if (int rc = conv_tables(geo, &by_k, &by_pos)) return rc;
+    const int64_t nk = (int64_t)geo.c_in * geo.kh * geo.kw, np = (int64_t)geo.h_out * geo.w_out;
     BatchDesc bd{};
-    bd.rank = 1; bd.shape[0] = n_images; bd.a_str[0] = 0; bd.b_str[0] = c_in * h_pad * w_pad;
+    bd.rank = 1; bd.shape[0] = n_images; bd.a_str[0] = 0; bd.b_str[0] = (int64_t)geo.c_in * geo.h_pad * geo.w_pad;
     Epilogue ep;
     ep.bias = bias; ep.bias_rows = 1; ep.gather_row = by_pos; ep.gather_k = by_k;
-    if (int rc = gemm_dispatch(kernel, nk, 1, padded_image, 0, 0, out, c_out, np, nk, bd, n_images, 0, ep)) return rc;
+    return gemm_dispatch(kernel, nk, 1, padded_image, 0, 0, out, c_out, np, nk, bd, n_images, accumulate, ep);
+}
+
+// shared argument checks of the two convolution entries; fills `geo`
+static int conv_check(const char* who, int64_t n_images, int64_t c_in, int64_t h_pad, int64_t w_pad, int64_t c_out, int64_t kh, int64_t kw,
+                      int64_t stride, int64_t dilation, ConvGeometry* geo) {
+    if (n_images < 0 || c_in < 1 || c_out < 1 || kh < 1 || kw < 1 || h_pad < 1 || w_pad < 1)
+        return fail(TENMO_ERR_INVALID_SHAPE, "%s: image (N=%lld, C_in=%lld, %lldx%lld), kernel (C_out=%lld, %lldx%lld): sizes must be positive",
+                    who, (long long)n_images, (long long)c_in, (long long)h_pad, (long long)w_pad, (long long)c_out, (long long)kh, (long long)kw);
+    if (stride < 1 || dilation < 1) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: stride and dilation must be >= 1", who);
+    const int64_t dkh = kh + (kh - 1) * (dilation - 1), dkw = kw + (kw - 1) * (dilation - 1);
+    if (h_pad < dkh || w_pad < dkw) return fail(TENMO_ERR_INVALID_SHAPE, "%s: Invalid output dimensions (the dilated kernel %lldx%lld exceeds the padded image %lldx%lld)",
+                                                who, (long long)dkh, (long long)dkw, (long long)h_pad, (long long)w_pad);
+    const int64_t h_out = (h_pad - dkh) / stride + 1, w_out = (w_pad - dkw) / stride + 1;
+    // the input-gradient pass convolves an array of (h_pad + dkh - 1) x (w_pad + dkw - 1) per channel: bound that one too
+    if (std::max(c_in, c_out) * (h_pad + dkh) * (w_pad + dkw) > 0x7fffffffLL || c_in * kh * kw > 0x7fffffffLL || c_out * kh * kw > 0x7fffffffLL)
+        return fail(TENMO_ERR_UNSUPPORTED, "%s: one image or one patch matrix dimension exceeds 2^31 elements", who);
+    *geo = ConvGeometry{(int32_t)c_in, (int32_t)h_pad, (int32_t)w_pad, (int32_t)kh, (int32_t)kw, (int32_t)h_out, (int32_t)w_out, (int32_t)stride, (int32_t)dilation};
+    return 0;
+}
+
+int tenmo_hip_conv2d_forward_f32(const float* padded_image, int64_t n_images, int64_t c_in, int64_t h_pad, int64_t w_pad,
+                                 const float* kernel, int64_t c_out, int64_t kh, int64_t kw, const float* bias,
+                                 int64_t stride, int64_t dilation, float* out, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    const char* who = "tenmo_hip_conv2d_forward_f32";
+    ConvGeometry geo;
+    if (int rc = conv_check(who, n_images, c_in, h_pad, w_pad, c_out, kh, kw, stride, dilation, &geo)) return rc;
+    if (n_images == 0) return 0;
+    if (!padded_image || !kernel || !out) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: null pointer", who);
+    if (int rc = conv_forward_impl(padded_image, n_images, geo, kernel, c_out, bias, out, 0)) return rc;
+    return finish(sync);
+}
+
+int tenmo_hip_conv2d_backward_f32(const float* padded_image, int64_t n_images, int64_t c_in, int64_t h_pad, int64_t w_pad,
+                                  const float* kernel, int64_t c_out, int64_t kh, int64_t kw, int64_t stride, int64_t dilation,
+                                  const float* grad_out, float* grad_padded_image, float* grad_kernel, float* grad_bias,
+                                  int32_t accumulate, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    const char* who = "tenmo_hip_conv2d_backward_f32";
+    ConvGeometry geo;
+    if (int rc = conv_check(who, n_images, c_in, h_pad, w_pad, c_out, kh, kw, stride, dilation, &geo)) return rc;
+    if (n_images == 0) return 0;
+    if (!grad_out) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: null upstream gradient", who);
+    if (grad_kernel && !padded_image) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: the kernel gradient needs the padded image", who);
+    if (grad_padded_image && !kernel) return fail(TENMO_ERR_INVALID_ARGUMENT, "%s: the image gradient needs the kernel", who);
+    const int64_t np = (int64_t)geo.h_out * geo.w_out, nk = c_in * kh * kw;
+    const int acc = accumulate ? 1 : 0;
+    BatchDesc one_batch{};
+    for (int d = 0; d < MAX_BATCH_RANK; ++d) one_batch.shape[d] = 1;
+
+    if (grad_bias) { // sums over (n, y, x) per output channel: row sums of [N*C_out, H_out*W_out], then column sums over N
+        if (n_images == 1) {
+            if (int rc = matvec_dispatch(grad_out, np, 1, S.one, 0, grad_bias, c_out, np, one_batch, 1, acc)) return rc;
+        } else {
+            float* rows;
+            if (int rc = workspace2((size_t)(n_images * c_out) * sizeof(float), &rows)) return rc;
+            if (int rc = matvec_dispatch(grad_out, np, 1, S.one, 0, rows, n_images * c_out, np, one_batch, 1, 0)) return rc;
+            if (int rc = matvec_dispatch(rows, 1, c_out, S.one, 0, grad_bias, c_out, n_images, one_batch, 1, acc)) return rc;
+        }
+    }
+    if (grad_kernel) { // per image grad_out[C_out, P] . patches^T[P, C_in*KH*KW] (the patches gathered), summed over the images
+        int32_t *by_k, *by_pos;
+        if (int rc = conv_tables(geo, &by_k, &by_pos)) return rc;
+        BatchDesc bd{};
+        bd.rank = 1; bd.shape[0] = n_images; bd.a_str[0] = c_out * np; bd.b_str[0] = c_in * h_pad * w_pad;
+        Epilogue ep;
+        ep.gather_row = by_k; ep.gather_k = by_pos; // B(n = patch element, k = position)
+        if (n_images == 1) {
+            if (int rc = gemm_dispatch(grad_out, np, 1, padded_image, 0, 0, grad_kernel, c_out, nk, np, bd, 1, acc, ep)) return rc;
+        } else {
+            float* per_image;
+            if (int rc = workspace2((size_t)(n_images * c_out * nk) * sizeof(float), &per_image)) return rc;
+            if (int rc = gemm_dispatch(grad_out, np, 1, padded_image, 0, 0, per_image, c_out, nk, np, bd, n_images, 0, ep)) return rc;
+            if (int rc = matvec_dispatch(per_image, 1, c_out * nk, S.one, 0, grad_kernel, c_out * nk, n_images, one_batch, 1, acc)) return rc;
+        }
+    }
+    if (grad_padded_image) {
+        // The scatter of the reference's loop (cnn.mojo:818-948) as a gather: a stride-1 convolution, same dilation, of the
+        // upstream gradient spread out by `stride` and zero-padded by the dilated kernel size - 1, with the kernel's
+        // channel axes swapped and its spatial axes reversed.
+        const int64_t dkh = kh + (kh - 1) * (dilation - 1), dkw = kw + (kw - 1) * (dilation - 1);
+        const int64_t h_dst = h_pad + dkh - 1, w_dst = w_pad + dkw - 1;
+        const int64_t spread_len = n_images * c_out * h_dst * w_dst, flip_len = c_out * nk;
+        float* buf;
+        if (int rc = workspace2((size_t)(spread_len + flip_len) * sizeof(float), &buf)) return rc;
+        float* spread = buf;
+        float* flipped = buf + spread_len;
+        hipLaunchKernelGGL(conv_dilate_pad_kernel, dim3((unsigned)std::min<int64_t>((spread_len + 255) / 256, (int64_t)S.cus * 32)), dim3(256), 0, S.stream,
+                           grad_out, spread, n_images * c_out, (int)geo.h_out, (int)geo.w_out, (int)h_dst, (int)w_dst, (int)stride, (int)(dkh - 1), (int)(dkw - 1));
+        hipLaunchKernelGGL(conv_flip_kernel, dim3((unsigned)((flip_len + 255) / 256)), dim3(256), 0, S.stream, kernel, flipped, (int)c_out, (int)c_in, (int)kh, (int)kw);
+        const ConvGeometry back{(int32_t)c_out, (int32_t)h_dst, (int32_t)w_dst, (int32_t)kh, (int32_t)kw, (int32_t)h_pad, (int32_t)w_pad, 1, (int32_t)dilation};
+        if (int rc = conv_forward_impl(spread, n_images, back, flipped, c_in, nullptr, grad_padded_image, acc)) return rc;
+    }
     return finish(sync);
 }
 

@@ -105,3 +105,30 @@ def conv_reference64(image, kernel, bias, stride, dilation, pads):
     if bias is not None:
         out = out + bias.astype(np.float64)[None, :, None, None]
     return out
+
+
+def check_conv_backward_case(case, grad_image, grad_kernel, grad_bias):
+    """Asserts what the reference's test asserts about the gradients of one `conv.backward_cases` entry."""
+    name = case["name"]
+    if "grad_image" in case:
+        assert np.array_equal(grad_image, np.array(case["grad_image"], np.float32)), name
+    if "grad_kernel" in case:
+        assert np.array_equal(grad_kernel, np.array(case["grad_kernel"], np.float32)), name
+    if "grad_kernel_every_filter_channel" in case:
+        want = np.array(case["grad_kernel_every_filter_channel"], np.float32)
+        assert all(np.array_equal(grad_kernel[co, ci], want) for co in range(grad_kernel.shape[0]) for ci in range(grad_kernel.shape[1])), name
+    if "grad_bias" in case:
+        assert np.allclose(grad_bias, np.array(case["grad_bias"], np.float32), atol=1e-5), name
+    if "grad_image_shape" in case:
+        assert list(grad_image.shape) == case["grad_image_shape"] and list(grad_kernel.shape) == case["grad_kernel_shape"], name
+
+
+def conv_backward_reference64(image, kernel, grad_out, stride, dilation, pads):
+    """Gradients of the zero-padded cross-correlation by torch autograd in fp64 (independent of the restated loops)."""
+    import torch
+    x = torch.from_numpy(image).double().requires_grad_(True)
+    k = torch.from_numpy(kernel).double().requires_grad_(True)
+    b = torch.zeros(kernel.shape[0], dtype=torch.float64, requires_grad=True)
+    y = torch.nn.functional.conv2d(torch.nn.functional.pad(x, (pads[2], pads[3], pads[0], pads[1])), k, b, stride=stride, dilation=dilation)
+    y.backward(torch.from_numpy(grad_out).double())
+    return x.grad.numpy(), k.grad.numpy(), b.grad.numpy()

@@ -1022,3 +1022,56 @@ def test_blocked_tile_order(T):
     finally:
         for knob in (b"gemm_tile", b"gemm_splitk", b"gemm_streamk"):
             L.tenmo_hip_set_tuning(knob, -1)
+
+
+def test_conv2d_backward(T, golden, oracle):
+    """FusedCol2ImBackward through tenmo_hip_conv2d_backward_f32: the gradients asserted in tests/test_cnn.mojo,
+    then random layers against the CPU restatement and torch autograd in fp64 (stride, dilation, all padding
+    forms, one and many images, channel counts around the tile sizes), NULL outputs and accumulate."""
+    import torch
+    from helpers import check_conv_backward_case, conv_backward_reference64, conv_case_tensors
+    from tenmo_amd.cnn import Conv2dFused
+
+    def run(image, kernel, up, **kw):
+        gi, gk, gb = Conv2dFused.backward(T.Tensor.from_numpy(image), T.Tensor.from_numpy(kernel), T.Tensor.from_numpy(up), **kw)
+        return gi.to_numpy(), gk.to_numpy(), gb.to_numpy()
+
+    for case in golden["conv"]["backward_cases"]:
+        image, kernel, _, kw = conv_case_tensors(case)
+        up = conv_case_tensors({"image": case["upstream"], "kernel": case["kernel"]})[0]
+        check_conv_backward_case(case, *run(image, kernel, up, **kw))
+    rng = np.random.default_rng(83)
+    for (n, ci, h, w, co, kh, kww, stride, dil, padding) in [
+            (2, 3, 9, 11, 4, 3, 3, 1, 1, "valid"), (1, 2, 8, 8, 3, 3, 2, 2, 1, "same"), (3, 1, 12, 7, 2, 2, 3, 1, 2, 1),
+            (2, 4, 10, 10, 5, 3, 3, 2, 2, (2, 1)), (1, 3, 7, 9, 2, 1, 1, 1, 1, "valid"), (2, 2, 6, 6, 3, 3, 3, 3, 1, [(1, 2), (0, 3)]),
+            (32, 1, 28, 28, 16, 3, 3, 1, 1, "same"), (8, 16, 14, 14, 32, 3, 3, 1, 1, "same"), (2, 70, 12, 12, 130, 3, 3, 2, 1, 1),
+            (1, 8, 20, 36, 96, 5, 5, 1, 1, "valid")]:
+        image = rng.standard_normal((n, ci, h, w), dtype=np.float32)
+        kernel = rng.standard_normal((co, ci, kh, kww), dtype=np.float32)
+        out_shape = oracle.conv2d_forward(image, kernel, None, stride=stride, dilation=dil, padding=padding).shape
+        up = rng.standard_normal(out_shape, dtype=np.float32)
+        case = (n, ci, h, w, co, kh, kww, stride, dil, padding)
+        got = run(image, kernel, up, stride=stride, dilation=dil, padding=padding)
+        want = oracle.conv2d_backward(image, kernel, up, stride=stride, dilation=dil, padding=padding)
+        ref = conv_backward_reference64(image, kernel, up, stride, dil, oracle.conv_padding(h, w, kh, kww, stride, dil, padding))
+        for g, o, r, what in zip(got, want, ref, ("image", "kernel", "bias")):
+            assert g.shape == r.shape, (what, case)
+            assert rel_fro(g, r) <= RTOL_FRO, (what, case)
+            assert rel_fro(g, o) <= 3 * RTOL_FRO, (what, case)
+    # NULL outputs are skipped; accumulate adds into what is there
+    L = T.lib.load()
+    n, ci, h, w, co, k = 3, 4, 9, 9, 6, 3
+    image = rng.standard_normal((n, ci, h, w), dtype=np.float32)
+    kernel = rng.standard_normal((co, ci, k, k), dtype=np.float32)
+    up = rng.standard_normal((n, co, h - k + 1, w - k + 1), dtype=np.float32)
+    gi_ref, gk_ref, gb_ref = oracle.conv2d_backward(image, kernel, up)
+    X, K, U = torch.from_numpy(image).cuda(), torch.from_numpy(kernel).cuda(), torch.from_numpy(up).cuda()
+    gk = torch.ones_like(K)
+    gb = torch.full((co,), 2.0, device="cuda")
+    gi = torch.full_like(X, 3.0)
+    T.lib.check(L.tenmo_hip_conv2d_backward_f32(X.data_ptr(), n, ci, h, w, K.data_ptr(), co, k, k, 1, 1, U.data_ptr(), None, gk.data_ptr(), None, 1, 1))
+    assert rel_fro(gk.cpu().numpy(), gk_ref + 1.0) <= RTOL_FRO and float(gb[0]) == 2.0 and float(gi.flatten()[0]) == 3.0
+    T.lib.check(L.tenmo_hip_conv2d_backward_f32(None, n, ci, h, w, K.data_ptr(), co, k, k, 1, 1, U.data_ptr(), gi.data_ptr(), None, gb.data_ptr(), 1, 1))
+    assert rel_fro(gi.cpu().numpy(), gi_ref + 3.0) <= RTOL_FRO and rel_fro(gb.cpu().numpy(), gb_ref + 2.0) <= RTOL_FRO
+    assert L.tenmo_hip_conv2d_backward_f32(None, n, ci, h, w, K.data_ptr(), co, k, k, 1, 1, U.data_ptr(), None, gk.data_ptr(), None, 0, 1) == -3
+    assert L.tenmo_hip_conv2d_backward_f32(X.data_ptr(), n, ci, h, w, K.data_ptr(), co, k, k, 1, 1, None, None, gk.data_ptr(), None, 0, 1) == -3

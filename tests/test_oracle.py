@@ -402,3 +402,27 @@ def test_conv_oracle_is_pinned(golden, oracle):
         oracle.conv2d_forward(np.ones((1, 2, 4, 4), np.float32), np.ones((1, 3, 2, 2), np.float32))
     with pytest.raises(oracle.OracleError):
         oracle.conv2d_forward(np.ones((1, 1, 2, 2), np.float32), np.ones((1, 1, 3, 3), np.float32))
+
+
+def test_conv_backward_oracle_is_pinned(golden, oracle):
+    """The restated FusedCol2ImBackward (tenmo/cnn.mojo:546-948) against the gradients asserted in
+    tests/test_cnn.mojo and against torch autograd in fp64 on random cases with stride, dilation and every
+    padding form (a flipped kernel index or a stride/dilation mix-up in the scatter fails these)."""
+    from helpers import check_conv_backward_case, conv_backward_reference64, conv_case_tensors
+
+    for case in golden["conv"]["backward_cases"]:
+        image, kernel, _, kw = conv_case_tensors(case)
+        up = conv_case_tensors({"image": case["upstream"], "kernel": case["kernel"]})[0]
+        check_conv_backward_case(case, *oracle.conv2d_backward(image, kernel, up, **kw))
+    rng = np.random.default_rng(79)
+    for (n, ci, h, w, co, kh, kww, stride, dil, padding) in [
+            (2, 3, 9, 11, 4, 3, 3, 1, 1, "valid"), (1, 2, 8, 8, 3, 3, 2, 2, 1, "same"), (3, 1, 12, 7, 2, 2, 3, 1, 2, 1),
+            (2, 4, 10, 10, 5, 3, 3, 2, 2, (2, 1)), (1, 3, 7, 9, 2, 1, 1, 1, 1, "valid"), (2, 2, 6, 6, 3, 3, 3, 3, 1, [(1, 2), (0, 3)])]:
+        image = rng.standard_normal((n, ci, h, w), dtype=np.float32)
+        kernel = rng.standard_normal((co, ci, kh, kww), dtype=np.float32)
+        out_shape = oracle.conv2d_forward(image, kernel, None, stride=stride, dilation=dil, padding=padding).shape
+        up = rng.standard_normal(out_shape, dtype=np.float32)
+        got = oracle.conv2d_backward(image, kernel, up, stride=stride, dilation=dil, padding=padding)
+        want = conv_backward_reference64(image, kernel, up, stride, dil, oracle.conv_padding(h, w, kh, kww, stride, dil, padding))
+        for g, r, what in zip(got, want, ("image", "kernel", "bias")):
+            assert g.shape == r.shape and np.allclose(g, r, rtol=1e-4, atol=1e-4), (what, n, ci, h, w, co, kh, kww, stride, dil, padding)
