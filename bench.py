@@ -41,6 +41,8 @@ def main() -> int:
     ap.add_argument("--size", type=int, default=8192, help="M=N=K of the square GEMM (default: the headline size)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the mv/vm and MLP-step side measurements")
+    ap.add_argument("--adjacent", action="store_true",
+                    help="also time the adjacent operators (cross-entropy, SGD step, convolution) into `extra`; off by default")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy, the known-size kernel against which FETCH_SIZE/WRITE_SIZE are scaled")
     args = ap.parse_args()
@@ -132,6 +134,8 @@ def main() -> int:
     extra = {}
     if not args.no_extra:
         extra.update(side_measurements(L, _lib, torch, np))
+    if args.adjacent:
+        extra.update(adjacent_operators(L, _lib, torch))
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_gemm_baseline(A, B, S, np)
         if not args.no_extra:
@@ -172,6 +176,59 @@ def side_measurements(L, _lib, torch, np):
         res["%s_16384_us" % nm] = round(ms * 1e3, 2)
         res["%s_16384_gbps" % nm] = round(gbps, 1)
         res["%s_16384_frac_hbm_peak" % nm] = round(gbps / PEAK_HBM_GBPS, 4)
+    return res
+
+
+def adjacent_operators(L, _lib, torch):
+    """Cross-entropy over GPT-2-sized logits, an SGD step on 2^28 parameters and one convolution layer, forward and
+    backward: microseconds per call and fractions of the HBM peak on algorithmic bytes (TFLOP/s for the convolution)."""
+    res = {}
+    M, Cn = 8192, 50257
+    x = torch.randn(M, Cn, device="cuda")
+    t = torch.randint(0, Cn, (M,), device="cuda")
+    sm = torch.empty_like(x)
+    rows = torch.empty(M, device="cuda")
+    tot = torch.zeros(1, device="cuda")
+    val = torch.zeros(1, dtype=torch.int32, device="cuda")
+    up = torch.ones(1, device="cuda")
+    fwd = lambda soft: _lib.check(L.tenmo_hip_cross_entropy_forward_f32(x.data_ptr(), t.data_ptr(), 1, M, Cn, -100, 0.0, soft, rows.data_ptr(),
+                                                                        tot.data_ptr(), val.data_ptr(), 0))
+    by = M * Cn * 4.0
+    ms = hip_time(L, _lib, lambda: fwd(None), 10)
+    res["ce_8192x50257_loss_only_us"] = round(ms * 1e3, 1)
+    res["ce_8192x50257_loss_only_frac_hbm_peak"] = round(by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 3)
+    ms = hip_time(L, _lib, lambda: fwd(sm.data_ptr()), 10)
+    res["ce_8192x50257_forward_us"] = round(ms * 1e3, 1)
+    res["ce_8192x50257_forward_frac_hbm_peak"] = round(2 * by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 3)
+    g = x  # the logits are no longer needed: their storage takes the gradient
+    ms = hip_time(L, _lib, lambda: _lib.check(L.tenmo_hip_cross_entropy_backward_f32(sm.data_ptr(), t.data_ptr(), 1, up.data_ptr(), M, Cn, -100, 0.0, 2, M,
+                                                                                     g.data_ptr(), 0, 0)), 10)
+    res["ce_8192x50257_backward_us"] = round(ms * 1e3, 1)
+    res["ce_8192x50257_backward_frac_hbm_peak"] = round(2 * by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 3)
+    del x, sm, g
+    n = 1 << 28
+    p = torch.randn(n, device="cuda")
+    gr = torch.randn(n, device="cuda")
+    ms = hip_time(L, _lib, lambda: _lib.check(L.tenmo_hip_sgd_step_f32(p.data_ptr(), gr.data_ptr(), None, n, 0.01, 0.0, 0.0, 0)), 10)
+    res["sgd_2p28_us"] = round(ms * 1e3, 1)
+    res["sgd_2p28_frac_hbm_peak"] = round(12.0 * n / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 3)
+    del p, gr
+    nb, ci, h, w, co, k = 128, 64, 34, 34, 128, 3
+    img = torch.randn(nb, ci, h, w, device="cuda")
+    ker = torch.randn(co, ci, k, k, device="cuda")
+    bias = torch.randn(co, device="cuda")
+    ho, wo = h - k + 1, w - k + 1
+    out = torch.empty(nb, co, ho, wo, device="cuda")
+    flop = 2.0 * nb * co * ho * wo * ci * k * k
+    ms = hip_time(L, _lib, lambda: _lib.check(L.tenmo_hip_conv2d_forward_f32(img.data_ptr(), nb, ci, h, w, ker.data_ptr(), co, k, k, bias.data_ptr(), 1, 1,
+                                                                             out.data_ptr(), 0)), 10)
+    res["conv_128x64x34x34_k3_to_128_forward_us"] = round(ms * 1e3, 1)
+    res["conv_128x64x34x34_k3_to_128_forward_tflops"] = round(flop / (ms * 1e-3) / 1e12, 1)
+    gi, gk, gb = torch.empty_like(img), torch.empty_like(ker), torch.empty_like(bias)
+    ms = hip_time(L, _lib, lambda: _lib.check(L.tenmo_hip_conv2d_backward_f32(img.data_ptr(), nb, ci, h, w, ker.data_ptr(), co, k, k, 1, 1, out.data_ptr(),
+                                                                              gi.data_ptr(), gk.data_ptr(), gb.data_ptr(), 0, 0)), 10)
+    res["conv_128x64x34x34_k3_to_128_backward_us"] = round(ms * 1e3, 1)
+    res["conv_128x64x34x34_k3_to_128_backward_tflops"] = round(2 * flop / (ms * 1e-3) / 1e12, 1)
     return res
 
 
