@@ -84,6 +84,45 @@ __global__ void outer_add_kernel(const OuterArgs g) {
     }
 }
 
+// The same with four consecutive j per thread (q_s == 1, J % 4 == 0, grad 16-byte aligned): 16-byte loads of q and of
+// the gradient, four groups in flight, streaming stores — the update is a read-modify-write sweep over the gradient.
+__global__ __launch_bounds__(256) void outer_add_vec_kernel(const OuterArgs g) {
+    typedef float f4 __attribute__((ext_vector_type(4)));
+    typedef float f4u __attribute__((ext_vector_type(4), aligned(4)));
+    constexpr int U = 4;
+    const int64_t J4 = g.J / 4, total4 = g.parent_batch * g.I * J4;
+    f4* __restrict grad4 = reinterpret_cast<f4*>(g.grad);
+    for (int64_t i0 = (int64_t)blockIdx.x * 256 * U + threadIdx.x; i0 < total4; i0 += (int64_t)gridDim.x * 256 * U) {
+        f4 old[U], acc[U];
+        bool ok[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int64_t idx = i0 + (int64_t)u * 256;
+            ok[u] = idx < total4;
+            acc[u] = f4{0.f, 0.f, 0.f, 0.f}; old[u] = acc[u];
+            if (!ok[u]) continue;
+            old[u] = __builtin_nontemporal_load(grad4 + idx);
+            const int64_t j = 4 * (idx % J4), i = (idx / J4) % g.I;
+            int64_t pb = idx / (J4 * g.I);
+            int64_t pbase = 0, qbase = 0;
+            for (int d = g.rank - 1; d >= 0; --d) {
+                if (g.kept[d]) { const int64_t c = pb % g.shape[d]; pb /= g.shape[d]; pbase += c * g.p_str[d]; qbase += c * g.q_str[d]; }
+            }
+            for (int64_t r = 0; r < g.reduced_total; ++r) {
+                int64_t rr = r, po = pbase, qo = qbase;
+                for (int d = g.rank - 1; d >= 0; --d) {
+                    if (!g.kept[d]) { const int64_t c = rr % g.shape[d]; rr /= g.shape[d]; po += c * g.p_str[d]; qo += c * g.q_str[d]; }
+                }
+                const f4 qv = *reinterpret_cast<const f4u*>(g.q + qo + j);
+                acc[u] += g.p[po + i * g.p_s] * qv;
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+            if (ok[u]) __builtin_nontemporal_store(old[u] + acc[u], grad4 + (i0 + (int64_t)u * 256));
+    }
+}
+
 __global__ void fill_kernel(float* p, int64_t n, float value) {
     for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (int64_t)gridDim.x * blockDim.x) p[i] = value;
 }

@@ -1252,7 +1252,12 @@ static int outer_grad(const float* p, int64_t p_s, const int64_t* p_bstr, const 
     o.reduced_total = red_total;
     const int64_t total = kept_total * I * J;
     if (total == 0) return 0;
-    hipLaunchKernelGGL(outer_add_kernel, dim3((unsigned)std::min<int64_t>((total + 255) / 256, 65535)), dim3(256), 0, S.stream, o);
+    if (q_s == 1 && J % 4 == 0 && (uintptr_t)grad % 16 == 0) {
+        const int64_t blocks = std::max<int64_t>(1, std::min<int64_t>((total / 4 + 1023) / 1024, (int64_t)S.cus * 16));
+        hipLaunchKernelGGL(outer_add_vec_kernel, dim3((unsigned)blocks), dim3(256), 0, S.stream, o);
+    } else {
+        hipLaunchKernelGGL(outer_add_kernel, dim3((unsigned)std::min<int64_t>((total + 255) / 256, 65535)), dim3(256), 0, S.stream, o);
+    }
     return 0;
 }
 
