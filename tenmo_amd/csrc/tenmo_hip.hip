@@ -622,7 +622,10 @@ int reduce_to_parent(const float* full, const Geometry& g, const tenmo_view* par
     r.reduced_total = red_total;
     const int64_t total = kept_total * r.inner;
     if (total == 0) return 0;
-    hipLaunchKernelGGL(broadcast_reduce_add_kernel, dim3((unsigned)std::min<int64_t>((total + 255) / 256, 65535)), dim3(256), 0, S.stream, r);
+    if (r.inner % 4 == 0 && (uintptr_t)r.src % 16 == 0 && (uintptr_t)r.dst % 16 == 0)
+        hipLaunchKernelGGL(broadcast_reduce_add_vec_kernel, dim3((unsigned)std::min<int64_t>((total / 4 + 255) / 256, 65535)), dim3(256), 0, S.stream, r);
+    else
+        hipLaunchKernelGGL(broadcast_reduce_add_kernel, dim3((unsigned)std::min<int64_t>((total + 255) / 256, 65535)), dim3(256), 0, S.stream, r);
     return 0;
 }
 
