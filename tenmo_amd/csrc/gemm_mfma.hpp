@@ -593,26 +593,83 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
             if (STAGED_FAST && lb.staged_ok && k0 + GEMM_BK <= k_end) lb.load_staged(Bb, b_k_s, n0, k0, g.b_gather_row, g.b_gather_k, t);
             else lb.load_checked(Bb, b_row_s, b_k_s, n0, k0, g.N, k_end, t, g.b_gather_row, g.b_gather_k);
         };
-        load_a(k_begin + done * GEMM_BK);
-        load_b(k_begin + done * GEMM_BK);
-        la.store(stage0, t);
-        lb.store(stage0 + A_FLOATS, t);
-        __syncthreads();
-        for (int64_t it = done; it < nk; ++it) {
-            float* cur = ((it - done) & 1) ? stage1 : stage0;
-            float* nxt = ((it - done) & 1) ? stage0 : stage1;
-            const bool more = (it + 1 < nk);
-            if (more) {
-                const int64_t k0 = k_begin + (it + 1) * GEMM_BK;
-                load_a(k0);
-                load_b(k0);
-            }
-            compute(cur);
-            if (more) {
-                la.store(nxt, t);
-                lb.store(nxt + A_FLOATS, t);
+        if constexpr (BM * BN <= 128 * 128 && STAGED_FAST) {
+            // Two LDS stages; the barrier sits in the middle of a step (as in the direct ring): behind the first half's
+            // MFMAs the operand fetch of the second half, then the next step's registers go to the other stage, barrier,
+            // and behind the second half's MFMAs the operand fetch of the next step's first half.
+            constexpr int PA2 = frag_parts<AMODE, MB>(), PB2 = frag_parts<BMODE, NB>();
+            constexpr int NMFMA2 = 4 * MB * NB;
+            constexpr int PER_SLOT2 = (PA2 + PB2 + NMFMA2 - 1) / NMFMA2;
+            auto fetch2 = [&](const float* st, int kc, float (&fa)[MB][4], float (&fb)[NB][4], int p) {
+                if (p < PA2) load_fragment_part<BM, AMODE, MB>(st, wm * TM, kc, lane, fa, p);
+                else if (p < PA2 + PB2) load_fragment_part<BN, BMODE, NB>(st + A_FLOATS, wn * TN, kc, lane, fb, p - PA2);
+            };
+            auto mfma2 = [&](const float (&fa)[MB][4], const float (&fb)[NB][4], auto&& slot) {
+                int n = 0;
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+#pragma unroll
+                    for (int i = 0; i < MB; ++i)
+#pragma unroll
+                        for (int j = 0; j < NB; ++j) {
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+                            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                            for (int u = 0; u < PER_SLOT2; ++u) slot(n * PER_SLOT2 + u);
+                            __builtin_amdgcn_sched_barrier(0);
+                            ++n;
+                        }
+            };
+            float ga0[MB][4], gb0[NB][4], ga1[MB][4], gb1[NB][4];
+            load_a(k_begin + done * GEMM_BK);
+            load_b(k_begin + done * GEMM_BK);
+            la.store(stage0, t);
+            lb.store(stage0 + A_FLOATS, t);
+            __syncthreads();
+            load_fragments<BM, AMODE, MB>(stage0, wm * TM, 0, lane, ga0);
+            load_fragments<BN, BMODE, NB>(stage0 + A_FLOATS, wn * TN, 0, lane, gb0);
+            for (int64_t it = done; it < nk; ++it) {
+                float* cur = ((it - done) & 1) ? stage1 : stage0;
+                float* nxt = ((it - done) & 1) ? stage0 : stage1;
+                const bool more = (it + 1 < nk);
+                if (more) {
+                    const int64_t k0 = k_begin + (it + 1) * GEMM_BK;
+                    load_a(k0);
+                    load_b(k0);
+                }
+                mfma2(ga0, gb0, [&](int p) { fetch2(cur, 1, ga1, gb1, p); });
+                if (more) {
+                    la.store(nxt, t);
+                    lb.store(nxt + A_FLOATS, t);
+                    __syncthreads();
+                }
+                mfma2(ga1, gb1, [&](int p) { if (more) fetch2(nxt, 0, ga0, gb0, p); });
             }
             __syncthreads();
+        } else { // plain two-stage loop: the 256x128 accumulators leave no registers for a second set of operand fragments,
+                 // and the element loads of a generic operand need the whole step to land (measured 15 % slower with the
+                 // barrier mid-step)
+            load_a(k_begin + done * GEMM_BK);
+            load_b(k_begin + done * GEMM_BK);
+            la.store(stage0, t);
+            lb.store(stage0 + A_FLOATS, t);
+            __syncthreads();
+            for (int64_t it = done; it < nk; ++it) {
+                float* cur = ((it - done) & 1) ? stage1 : stage0;
+                float* nxt = ((it - done) & 1) ? stage0 : stage1;
+                const bool more = (it + 1 < nk);
+                if (more) {
+                    const int64_t k0 = k_begin + (it + 1) * GEMM_BK;
+                    load_a(k0);
+                    load_b(k0);
+                }
+                compute(cur);
+                if (more) {
+                    la.store(nxt, t);
+                    lb.store(nxt + A_FLOATS, t);
+                }
+                __syncthreads();
+            }
         }
     }
 
