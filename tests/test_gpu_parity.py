@@ -1075,3 +1075,39 @@ def test_conv2d_backward(T, golden, oracle):
     assert rel_fro(gi.cpu().numpy(), gi_ref + 3.0) <= RTOL_FRO and rel_fro(gb.cpu().numpy(), gb_ref + 2.0) <= RTOL_FRO
     assert L.tenmo_hip_conv2d_backward_f32(None, n, ci, h, w, K.data_ptr(), co, k, k, 1, 1, U.data_ptr(), None, gk.data_ptr(), None, 0, 1) == -3
     assert L.tenmo_hip_conv2d_backward_f32(X.data_ptr(), n, ci, h, w, K.data_ptr(), co, k, k, 1, 1, None, None, gk.data_ptr(), None, 0, 1) == -3
+
+
+def test_zz_shutdown_and_reinit(T):
+    """tenmo_hip_shutdown releases the library's stream and scratch; after tenmo_hip_init everything works again and
+    gives the same results (split-K workspace, column-kernel partial sums and the convolution tables are re-grown)."""
+    import torch
+    L = T.lib.load()
+    rng = np.random.default_rng(109)
+    a = rng.standard_normal((96, 4000), dtype=np.float32)
+    b = rng.standard_normal((4000, 80), dtype=np.float32)
+    img = rng.standard_normal((2, 3, 10, 10), dtype=np.float32)
+    ker = rng.standard_normal((5, 3, 3, 3), dtype=np.float32)
+    A, B, X, K = (torch.from_numpy(v).cuda() for v in (a, b, img, ker))
+
+    def run():
+        out = torch.empty((96, 80), device="cuda")
+        L.tenmo_hip_set_tuning(b"gemm_splitk", 4)
+        try:
+            T.lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, 4000, 1, B.data_ptr(), 0, 80, 1, out.data_ptr(), 96, 80, 4000, 0, None, None, None, 0, 1))
+        finally:
+            L.tenmo_hip_set_tuning(b"gemm_splitk", -1)
+        vm = torch.empty(80, device="cuda")
+        T.lib.check(L.tenmo_hip_vm_f32(A.data_ptr(), 0, 1, B.data_ptr(), 0, 80, 1, vm.data_ptr(), 4000, 80, 0, None, None, None, 0, 1))
+        conv = torch.empty((2, 5, 8, 8), device="cuda")
+        T.lib.check(L.tenmo_hip_conv2d_forward_f32(X.data_ptr(), 2, 3, 10, 10, K.data_ptr(), 5, 3, 3, None, 1, 1, conv.data_ptr(), 1))
+        return out.cpu().numpy(), vm.cpu().numpy(), conv.cpu().numpy()
+
+    before = run()
+    assert rel_fro(before[0], ref_matmul64(a, b)) <= RTOL_FRO
+    assert L.tenmo_hip_shutdown() == 0
+    assert L.tenmo_hip_sync() == -1 and b"not initialised" in L.tenmo_hip_last_error()
+    assert L.tenmo_hip_shutdown() == 0  # idempotent
+    assert L.tenmo_hip_init(0) == 0
+    after = run()
+    for x, y in zip(before, after):
+        assert np.array_equal(x, y)
