@@ -93,11 +93,17 @@ __device__ __forceinline__ float epilogue_value(float v, const float* __restrict
     return v;
 }
 
+// The batch index and every batch dimension are below 2^31 (the host refuses larger grids), so the
+// mixed-radix decode runs in 32-bit arithmetic: a 64-bit division costs a workgroup hundreds of
+// instructions before its first load.
 __device__ __forceinline__ void batch_offsets(const BatchDesc& bd, int64_t b, int64_t& a_off, int64_t& b_off) {
     a_off = 0; b_off = 0;
+    uint32_t rest = (uint32_t)b;
     for (int d = bd.rank - 1; d >= 0; --d) {
-        int64_t c = b % bd.shape[d];
-        b /= bd.shape[d];
+        const uint32_t extent = (uint32_t)bd.shape[d];
+        const uint32_t q = rest / extent;
+        const int64_t c = rest - q * extent;
+        rest = q;
         a_off += c * bd.a_str[d];
         b_off += c * bd.b_str[d];
     }
@@ -376,13 +382,18 @@ __device__ __forceinline__ void bare_barrier() {
 // position of tile number `tid` (0 .. tiles_m*tiles_n-1) in the tile grid.
 // Workgroup ids are dealt round-robin to the 8 XCDs (checked with HW_REG_XCC_ID), so with groups
 // of 8 tile-rows each XCD keeps one tile-row of A hot in its L2 and streams B past it.
-__device__ __forceinline__ void tile_coords(const GemmArgs& g, int64_t tid, int64_t& tile_m, int64_t& tile_n) {
-    constexpr int GROUP_M = 8;
-    const int64_t per_group = (int64_t)GROUP_M * g.tiles_n;
-    const int64_t first_m = (tid / per_group) * GROUP_M;
-    const int64_t gsz = min((int64_t)g.tiles_m - first_m, (int64_t)GROUP_M);
-    tile_m = first_m + (tid % per_group) % gsz;
-    tile_n = (tid % per_group) / gsz;
+__device__ __forceinline__ void tile_coords(const GemmArgs& g, int64_t tile_id, int64_t& tile_m, int64_t& tile_n) {
+    // tile ids are below 2^31: 32-bit divisions (a 64-bit one costs hundreds of instructions)
+    constexpr uint32_t GROUP_M = 8;
+    const uint32_t tid = (uint32_t)tile_id;
+    const uint64_t per_group64 = (uint64_t)GROUP_M * (uint32_t)g.tiles_n;
+    const uint32_t per_group = per_group64 > 0xffffffffull ? 0xffffffffu : (uint32_t)per_group64; // clamped: then group 0 holds every tile
+    const uint32_t group = tid / per_group, in_group = tid - group * per_group;
+    const uint32_t first_m = group * GROUP_M;
+    const uint32_t gsz = min((uint32_t)g.tiles_m - first_m, GROUP_M);
+    const uint32_t col = in_group / gsz;
+    tile_m = first_m + (in_group - col * gsz);
+    tile_n = col;
 }
 
 // The same for the one-workgroup-per-tile launch of the 256x128 tile, whose 64 resident workgroups per
@@ -394,13 +405,15 @@ __device__ __forceinline__ void tile_coords(const GemmArgs& g, int64_t tid, int6
 template <int BM, int BN>
 __device__ __forceinline__ void tile_coords_blocked(const GemmArgs& g, int64_t tid, int64_t& tile_m, int64_t& tile_n) {
     if constexpr (BM == 256 && BN == 128) {
-        const int rn = g.tiles_n % 32 == 0 ? 32 : 16, rm = 64 / rn;
-        const int64_t bm_count = g.tiles_m / rm, bn_count = g.tiles_n / rn;
+        const uint32_t rn = g.tiles_n % 32 == 0 ? 32 : 16, rm = 64 / rn; // powers of two
+        const uint32_t bm_count = (uint32_t)g.tiles_m / rm, bn_count = (uint32_t)g.tiles_n / rn;
         if (g.tiles_m % rm == 0 && g.tiles_n % rn == 0 && (bm_count * bn_count) % 8 == 0) {
-            const int64_t xcd = tid % 8, j = tid / 8, round = j / 64, q = j % 64;
-            const int64_t block = round * 8 + xcd; // the 8 XCDs work on 8 neighbouring blocks at a time
-            tile_m = (block / bn_count) * rm + q % rm;
-            tile_n = (block % bn_count) * rn + q / rm;
+            const uint32_t t32 = (uint32_t)tid;
+            const uint32_t xcd = t32 % 8, j = t32 / 8, round = j / 64, q = j % 64;
+            const uint32_t block = round * 8 + xcd; // the 8 XCDs work on 8 neighbouring blocks at a time
+            const uint32_t block_m = block / bn_count;
+            tile_m = block_m * rm + q % rm;
+            tile_n = (block - block_m * bn_count) * rn + q / rm;
             return;
         }
     }
@@ -734,11 +747,12 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
     __shared__ __attribute__((aligned(1024))) float stage2[DIRECT ? STAGE_FLOATS : 4];
 
-    const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-    const int64_t pid = blockIdx.x;
-    const int64_t batch = pid / tiles;
+    const uint32_t tiles = (uint32_t)g.tiles_m * (uint32_t)g.tiles_n; // the grid, batches included, is below 2^31
+    const uint32_t pid = blockIdx.x;
+    const uint32_t batch32 = pid / tiles;
+    const int64_t batch = batch32;
     int64_t tile_m, tile_n;
-    tile_coords_blocked<BM, BN>(g, pid % tiles, tile_m, tile_n);
+    tile_coords_blocked<BM, BN>(g, pid - batch32 * tiles, tile_m, tile_n);
 
     int64_t k_begin = 0, k_end = g.K;
     TileDest dst;
