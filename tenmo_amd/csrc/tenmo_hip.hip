@@ -230,15 +230,17 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
             for (int sp : kSplits) {
                 if (sp > 1 && (K / sp < 64 || (double)sp * batch_count * M * N * 4.0 > 1.0e9 || ep.bias_rows)) break;
                 const double wgs = tiles * sp, slots = cus * kOcc[t];
-                // one round = every CU runs `conc` workgroups side by side; the dispatcher refills a CU
-                // only as slots free, so a partial extra round costs a whole one
-                const double rounds = wgs <= slots ? 1.0 : std::ceil(wgs / slots);
-                const double conc = wgs <= slots ? std::ceil(wgs / cus) : kOcc[t];
+                // one round = every CU runs `conc` workgroups side by side.  After the full rounds the rest
+                // runs with fewer workgroups per CU, each of them faster for it; the rounds do not end in
+                // step, which costs a quarter of a round where a partial one follows full ones.
                 const double iters = std::ceil((double)K / sp / GEMM_BK);
-                const double t_round = iters * conc * m_us / kEff[t] + 1.5;
+                auto round_us = [&](double conc) { return iters * conc * m_us / kEff[t] + 1.5; };
+                const double full = std::floor(wgs / slots), rest = wgs - full * slots;
+                double t_rounds = full * round_us(kOcc[t]);
+                if (rest > 0) t_rounds += round_us(std::ceil(rest / cus)) + (full > 0 ? 0.25 * round_us(kOcc[t]) : 0.0);
                 const double bytes = 4.0 * batch_count * ((double)M * K + (double)K * N + (double)M * N * (sp > 1 ? sp + 1.0 : 1.0));
                 const double l2_bytes = 4.0 * batch_count * (double)K * ((double)M * tn + (double)N * tm);
-                double est = std::max({rounds * t_round, bytes / 5.0e6, l2_bytes / 8.0e6}) + 3.0;
+                double est = std::max({t_rounds, bytes / 5.0e6, l2_bytes / 8.0e6}) + 3.0;
                 if (sp > 1) est += 5.0 + 4.0 * batch_count * (double)M * N * (sp + 1.0) / 6.0e6;
                 if (est < best) { best = est; tile = t; splits = sp; }
             }
