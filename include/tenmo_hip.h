@@ -66,7 +66,7 @@ int tenmo_hip_set_stream(void* hip_stream);
 int tenmo_hip_device_info(int* compute_units, char* name, int name_len);
 /* Overrides of the automatic kernel selection, for measurement: "gemm_tile" (0: 256x128, 1: 128x128,
  * 2: 64x64, 3: 128x64, 4: 64x128 workgroup tile; -1 automatic), "gemm_splitk" (number of K slices;
- * -1 automatic), "gemm_streamk" (n > 0: persistent stream-K launch with n workgroups per CU for the
+ * -1 automatic), "gemm_streamk" (n > 0: persistent stream-K launch with n workgroups per CU, at most two, for the
  * 256x128 / 128x128 tiles, 0: never, -1 automatic) and "cols_wg_per_cu" (workgroups per CU the
  * column-streaming kernel aims for).  The
  * environment variables TENMO_HIP_GEMM_TILE / TENMO_HIP_GEMM_SPLITK / TENMO_HIP_GEMM_STREAMK set the same at init.

@@ -770,17 +770,21 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
 }
 
 // ---- stream-K --------------------------------------------------------------------------------
-// The launch's work is cut into K steps ("iterations": tile-major, K-minor, batches outermost) and
-// every workgroup of a persistent grid takes an equal contiguous run of them, so the chip stays
-// full whatever the tile count.  A workgroup whose run covers a whole tile stores it as usual; the
-// pieces of a tile that is shared between workgroups go to compact partial tiles (two slots per
-// workgroup: slot 2w for a piece that starts inside the tile, 2w+1 for one that starts at its
-// beginning) and streamk_fixup_kernel adds them in workgroup order — deterministic, no spinning.
+// A persistent grid.  The first `dp_tiles` tiles (a multiple of the grid size) are taken whole, one
+// per workgroup and round: workgroup w works on tile round * grid + w, so the workgroups that run side
+// by side work on neighbouring tiles and share operand panels in L2, exactly as in the one-tile-per-
+// workgroup launch.  The work of the remaining tiles is cut into K steps ("iterations": tile-major,
+// K-minor) and every workgroup takes an equal contiguous run of them, so the chip stays full whatever
+// the tile count.  A workgroup whose run covers a whole tile stores it as usual; the pieces of a tile
+// that is shared between workgroups go to compact partial tiles (two slots per workgroup: slot 2w for
+// a piece that starts inside the tile, 2w+1 for one that starts at its beginning) and
+// streamk_fixup_kernel adds them in workgroup order — deterministic, no spinning.
 struct StreamKArgs {
-    int64_t total;   // iterations in the launch = tiles * nks
-    int64_t per_wg;  // iterations per workgroup
-    int64_t nks;     // K steps per tile
-    float* partial;  // [2 * workgroups][BM * BN]
+    int64_t dp_tiles; // tiles (batches included) stored whole, round-robin over the grid
+    int64_t total;    // iterations of the shared part = (tiles - dp_tiles) * nks
+    int64_t per_wg;   // iterations per workgroup
+    int64_t nks;      // K steps per tile
+    float* partial;   // [2 * workgroups][BM * BN]
 };
 
 template <int BM, int BN, int AMODE, int BMODE>
@@ -790,16 +794,31 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_streamk_kernel(const Gem
     __shared__ __attribute__((aligned(1024))) float stage0[STAGE_FLOATS];
     __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
     __shared__ __attribute__((aligned(1024))) float stage2[DIRECT ? STAGE_FLOATS : 4];
-    const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
+    const uint32_t tiles = (uint32_t)g.tiles_m * (uint32_t)g.tiles_n; // tile ids, batches included, are below 2^31
     const int64_t w = blockIdx.x;
+    uint32_t whole = blockIdx.x; // next tile of the data-parallel part
     int64_t it = w * sk.per_wg;
     const int64_t end = min(sk.total, it + sk.per_wg);
-    while (it < end) {
-        const int64_t gt = it / sk.nks, k0 = it % sk.nks;
-        const int64_t k1 = min(sk.nks, k0 + (end - it));
-        const int64_t batch = gt / tiles;
+    for (;;) { // one call site for gemm_tile: the function is large
+        uint32_t gt;
+        int64_t k0, k1;
+        const bool is_whole = whole < (uint32_t)sk.dp_tiles;
+        if (is_whole) {
+            gt = whole; k0 = 0; k1 = sk.nks;
+            whole += gridDim.x;
+        } else if (it < end) {
+            const int64_t st = it / sk.nks; // shared tile number
+            k0 = it - st * sk.nks;
+            k1 = min(sk.nks, k0 + (end - it));
+            gt = (uint32_t)(sk.dp_tiles + st);
+            it += k1 - k0;
+        } else {
+            break;
+        }
+        const uint32_t batch32 = gt / tiles;
+        const int64_t batch = batch32;
         int64_t tile_m, tile_n;
-        tile_coords(g, gt % tiles, tile_m, tile_n);
+        tile_coords_blocked<BM, BN>(g, gt - batch32 * tiles, tile_m, tile_n); // one numbering for both parts and the fix-up
         TileDest dst;
         if (k0 == 0 && k1 == sk.nks) {
             dst.base = g.C + batch * g.M * g.N; dst.ld = g.N; dst.row0 = 0; dst.col0 = 0;
@@ -810,23 +829,22 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_streamk_kernel(const Gem
             dst.accumulate = false; dst.fused = false;
         }
         gemm_tile<BM, BN, AMODE, BMODE>(g, stage0, stage1, stage2, batch, tile_m, tile_n, k0 * GEMM_BK, min(g.K, k1 * GEMM_BK), dst);
-        it += k1 - k0;
     }
 }
 
 // A tile that was shared between workgroups is the sum of their partial tiles (ascending workgroup
-// order), finished with accumulate / the fused epilogue.  blockIdx.x = tile, blockIdx.y = one of
-// gridDim.y equal parts of the tile, so that a launch with few tiles still fills the chip.
+// order), finished with accumulate / the fused epilogue.  blockIdx.x = shared tile, blockIdx.y = one
+// of gridDim.y equal parts of the tile, so that a launch with few tiles still fills the chip.
 template <int BM, int BN>
 __global__ void streamk_fixup_kernel(const GemmArgs g, const StreamKArgs sk) {
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
-    const int64_t gt = blockIdx.x;
-    const int64_t it0 = gt * sk.nks, it1 = it0 + sk.nks;
+    const int64_t gt = sk.dp_tiles + blockIdx.x;
+    const int64_t it0 = (int64_t)blockIdx.x * sk.nks, it1 = it0 + sk.nks;
     const int64_t w_first = it0 / sk.per_wg, w_last = (it1 - 1) / sk.per_wg;
     if (w_first == w_last) return; // one workgroup had the whole tile and stored it
     const int64_t batch = gt / tiles;
     int64_t tile_m, tile_n;
-    tile_coords(g, gt % tiles, tile_m, tile_n);
+    tile_coords_blocked<BM, BN>(g, gt % tiles, tile_m, tile_n);
     float* __restrict Cb = g.C + batch * g.M * g.N;
     const float* __restrict mask = g.mask ? g.mask + batch * g.M * g.N : nullptr;
     const bool fused = g.bias != nullptr || g.mask != nullptr || g.relu != 0;

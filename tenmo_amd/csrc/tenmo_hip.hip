@@ -182,6 +182,17 @@ struct Epilogue {
     bool any() const { return bias || mask || relu; }
 };
 
+// Stream-K launch of `tiles` tiles of `nks` K steps on `wgs` persistent workgroups: `whole_rounds` rounds of
+// whole tiles (one per workgroup and round), then `shared` tiles whose K steps are spread evenly.  The shared
+// part gives every workgroup at least eight K steps where the tile count allows: a shorter piece is all
+// prologue and epilogue, so one round of whole tiles goes into the shared part instead.
+void streamk_partition(int64_t tiles, int64_t nks, int64_t wgs, int64_t* whole_rounds, int64_t* shared) {
+    int64_t full = tiles / wgs, rest = tiles - full * wgs;
+    if (rest > 0 && rest * nks < 8 * wgs && full > 0) { --full; rest += wgs; }
+    *whole_rounds = full;
+    *shared = rest;
+}
+
 int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, int64_t b_rs, int64_t b_cs, float* C,
                   int64_t M, int64_t N, int64_t K, const BatchDesc& bd, int64_t batch_count, int accumulate, const Epilogue& ep = Epilogue()) {
     if (M == 0 || N == 0 || batch_count == 0) return 0;
@@ -245,21 +256,27 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
                 if (est < best) { best = est; tile = t; splits = sp; }
             }
         }
-        // stream-K (persistent workgroups sharing tiles, see gemm_mfma.hpp): every CU gets the same
-        // number of K steps whatever the tile count, at the price of the fix-up traffic
+        // stream-K (persistent workgroups: rounds of whole tiles, then the K steps of the remaining tiles
+        // spread evenly, see gemm_mfma.hpp): no partial last round, at the price of the fix-up traffic
         if (S.force_streamk < 0 && am != KMAJOR_GEN && bm != KMAJOR_GEN && !ep.gather_row) {
-            // Measured: the 128x128 tile with one workgroup per CU is the variant that wins; with many
-            // tiles per workgroup the classic launch is as full and shares operand panels in L2 better.
-            const int t = 1, wpc = 1;
-            const double tm = (double)((M + kTiles[t].bm - 1) / kTiles[t].bm), tn = (double)((N + kTiles[t].bn - 1) / kTiles[t].bn);
-            const double tiles = tm * tn * (double)batch_count, nks = std::ceil((double)K / GEMM_BK);
-            const double m_us = (kTiles[t].bm / 64) * (kTiles[t].bn / 64) * 8 * 64 / 2400.0;
-            const double wgs = cus * wpc;
-            if (tiles * nks >= wgs * 8 && tiles <= 3.0 * wgs) { // pieces of under eight K steps are all overhead
-                const double shared_tiles = std::min(2.0 * wgs, 2.0 * tiles);
-                const double fix = 2.0 * shared_tiles * kTiles[t].bm * kTiles[t].bn * 4.0 / 5.0e6;
-                const double est = tiles * nks / cus * m_us / kEff[t] + fix + 10.0;
-                if (est < 0.98 * best) { best_sk = est; sk_tile = t; sk_wpc = wpc; }
+            // Measured: 128x128 wins, with one workgroup per CU while there are at most two tiles per CU and with two
+            // beyond (three do not fit its registers); 256x128 with two per CU comes within 1-2 % at large sizes.
+            for (int t = 1; t >= 0; --t) {
+                const int64_t tiles = ((M + kTiles[t].bm - 1) / kTiles[t].bm) * ((N + kTiles[t].bn - 1) / kTiles[t].bn) * batch_count;
+                const int wpc = (t == 0 || tiles >= 2 * (int64_t)S.cus) ? 2 : 1;
+                const int64_t nks = (K + GEMM_BK - 1) / GEMM_BK, wgs = (int64_t)S.cus * wpc;
+                int64_t whole_rounds, shared;
+                streamk_partition(tiles, nks, wgs, &whole_rounds, &shared);
+                if (shared == 0 || shared * nks < wgs * 8) continue; // nothing to share / pieces of under eight K steps are all overhead
+                // with fewer tiles than workgroups only 128x128 at one workgroup per CU wins; with rounds of whole tiles a
+                // short K loses (measured at K = 768: -10 % to +2 %, against +5 to +16 % from K = 2560 up)
+                if (whole_rounds == 0 ? (t != 1 || wpc != 1) : nks < 64) continue;
+                const double m_us = (kTiles[t].bm / 64) * (kTiles[t].bn / 64) * 8 * 64 / 2400.0;
+                const double step_us = wpc * m_us / kEff[t]; // one K step of every workgroup of a CU
+                const double pieces = (double)std::min(2 * wgs, 2 * shared);
+                const double fix = 2.0 * pieces * kTiles[t].bm * kTiles[t].bn * 4.0 / 5.0e6;
+                const double est = whole_rounds * (nks * step_us + 1.5) + (double)shared * nks / wgs * step_us + fix + 10.0;
+                if (est < 0.98 * best && est < best_sk) { best_sk = est; sk_tile = t; sk_wpc = wpc; }
             }
         }
         if (S.verbose) fprintf(stderr, "tenmo_hip gemm M=%lld N=%lld K=%lld batch=%lld -> tile %dx%d, %d K slice(s), est %.1f us%s\n",
@@ -278,23 +295,28 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         const int64_t tiles_total = (int64_t)g.tiles_m * g.tiles_n * batch_count;
         StreamKArgs sk{};
         sk.nks = (K + GEMM_BK - 1) / GEMM_BK;
-        sk.total = tiles_total * sk.nks;
-        const int64_t want = (int64_t)S.cus * std::min(streamk, tile == 0 ? 2 : 3);
-        int64_t per = (sk.total + want - 1) / want;
+        const int64_t want = (int64_t)S.cus * std::min(streamk, 2); // the registers of both kernels allow two workgroups per CU
+        int64_t whole_rounds, shared;
+        streamk_partition(tiles_total, sk.nks, want, &whole_rounds, &shared);
+        sk.dp_tiles = whole_rounds * want;
+        sk.total = shared * sk.nks;
+        int64_t per = std::max<int64_t>((sk.total + want - 1) / want, 1);
         per = (per + 3) / 4 * 4; // no piece shorter than four K steps except at the end of K
         sk.per_wg = per;
-        const int64_t wgs = (sk.total + per - 1) / per;
+        // every workgroup of the grid takes whole tiles; with none of those, only the workgroups that get a run
+        const int64_t wgs = whole_rounds > 0 ? want : (sk.total + per - 1) / per;
         if (tiles_total <= 0x7fffffffLL && wgs >= 1) {
             float* ws;
             if (int rc = workspace((size_t)(2 * wgs) * bmt * bnt * sizeof(float), &ws)) return rc;
             sk.partial = ws;
-            const bool need_fixup = per % sk.nks != 0;
-            if (S.verbose) fprintf(stderr, "tenmo_hip gemm stream-K: %lld workgroups x %lld K steps, %lld tiles of %dx%d\n", (long long)wgs, (long long)per, (long long)tiles_total, bmt, bnt);
+            const bool need_fixup = shared > 0 && per % sk.nks != 0;
+            if (S.verbose) fprintf(stderr, "tenmo_hip gemm stream-K: %lld workgroups, %lld whole tiles each, then %lld K steps each of %lld shared tiles of %dx%d\n",
+                                   (long long)wgs, (long long)whole_rounds, (long long)per, (long long)shared, bmt, bnt);
             // parts per shared tile in the fix-up: a power of two that brings it to a few workgroups per CU
             unsigned parts = 0;
-            if (need_fixup) for (parts = 1; parts < 32 && tiles_total * parts < (int64_t)S.cus * 4; parts *= 2) {}
-            const bool ok = tile == 0 ? launch_streamk_256x128(g, sk, (unsigned)wgs, (unsigned)tiles_total, parts, am, bm, S.stream)
-                                      : launch_streamk_128x128(g, sk, (unsigned)wgs, (unsigned)tiles_total, parts, am, bm, S.stream);
+            if (need_fixup) for (parts = 1; parts < 32 && shared * parts < (int64_t)S.cus * 4; parts *= 2) {}
+            const bool ok = tile == 0 ? launch_streamk_256x128(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream)
+                                      : launch_streamk_128x128(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream);
             return ok ? 0 : fail(TENMO_ERR_UNSUPPORTED, "no stream-K variant for operand modes %d/%d", am, bm);
         }
     }

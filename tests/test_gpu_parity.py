@@ -274,7 +274,8 @@ def test_column_sum(T):
 @pytest.mark.parametrize("tile", [0, 1])
 def test_stream_k(T, tile):
     """Persistent stream-K launches: tiles shared between workgroups are summed by the fix-up kernel.
-    Shapes with fewer / more tiles than workgroups, ragged extents, K tails, transposed views, batches,
+    Shapes with fewer tiles than workgroups, with rounds of whole tiles ahead of the shared ones (one
+    matrix and batched), with whole rounds only, ragged extents, K tails, transposed views, batches,
     accumulate and the fused epilogue."""
     L, lib = T.lib.load(), T.lib
     rng = np.random.default_rng(53)
@@ -282,7 +283,8 @@ def test_stream_k(T, tile):
         L.tenmo_hip_set_tuning(b"gemm_tile", tile)
         for wg_per_cu in (1, 2):
             L.tenmo_hip_set_tuning(b"gemm_streamk", wg_per_cu)
-            for (bsz, m, k, n) in [(1, 768, 2000, 640), (1, 300, 4100, 200), (1, 2048, 512, 1536), (3, 260, 1000, 132), (1, 100, 64, 70), (1, 1500, 8192, 900)]:
+            for (bsz, m, k, n) in [(1, 768, 2000, 640), (1, 300, 4100, 200), (1, 2048, 512, 1536), (3, 260, 1000, 132), (1, 100, 64, 70), (1, 1500, 8192, 900),
+                                      (1, 2304, 400, 2432), (4, 2300, 400, 2432), (1, 2304, 100, 2432), (1, 4096, 48, 4096)]:
                 a = rng.standard_normal((bsz, m, k), dtype=np.float32)
                 b = rng.standard_normal((k, n), dtype=np.float32)
                 ref = ref_matmul64(a, b)
