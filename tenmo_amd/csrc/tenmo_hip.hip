@@ -268,9 +268,14 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
                 int64_t whole_rounds, shared;
                 streamk_partition(tiles, nks, wgs, &whole_rounds, &shared);
                 if (shared == 0 || shared * nks < wgs * 8) continue; // nothing to share / pieces of under eight K steps are all overhead
-                // with fewer tiles than workgroups only 128x128 at one workgroup per CU wins; with rounds of whole tiles a
-                // short K loses (measured at K = 768: -10 % to +2 %, against +5 to +16 % from K = 2560 up)
-                if (whole_rounds == 0 ? (t != 1 || wpc != 1) : nks < 64) continue;
+                // with fewer tiles than workgroups only 128x128 at one workgroup per CU wins; with rounds of whole tiles and a
+                // short K the shared part must be small (measured at K = 768: -10 % with a third of the tiles shared, +5 %
+                // with 2 %; from K = 2560 up +5 to +18 % whatever the share)
+                if (whole_rounds == 0 ? (t != 1 || wpc != 1) : (nks < 64 && shared * 10 > tiles)) continue;
+                // 16-byte loads from rows that are not 16-byte aligned are slow enough to be the bound, and one workgroup
+                // per CU hides them badly (measured [2048,50257].[50257,768]: 118 against 126 TFLOP/s with K slices)
+                const int64_t a_pitch = am == KMAJOR_VEC ? a_rs : a_cs, b_pitch = bm == KMAJOR_VEC ? b_cs : b_rs;
+                if (wpc == 1 && ((M > 1 && K > 1 && a_pitch % 4 != 0) || (N > 1 && K > 1 && b_pitch % 4 != 0))) continue;
                 const double m_us = (kTiles[t].bm / 64) * (kTiles[t].bn / 64) * 8 * 64 / 2400.0;
                 const double step_us = wpc * m_us / kEff[t]; // one K step of every workgroup of a CU
                 const double pieces = (double)std::min(2 * wgs, 2 * shared);
@@ -279,6 +284,14 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
                 if (est < 0.98 * best && est < best_sk) { best_sk = est; sk_tile = t; sk_wpc = wpc; }
             }
         }
+        // A product with K <= 128 and a large result is bound by its stores, which the model does not rank: all tiles
+        // sit on the same byte floor.  Measured there (K = 32 .. 128, results of 64 MB and more, one matrix and batches),
+        // the small tiles win — more workgroups per CU overlap one's stores with another's loads: 64x64 for a K-major B
+        // (8192x8192x64: 112 us against 135 with 256x128; attention Q.K^T 179 against 202), 64x128 for an MN-major B
+        // (110 against 116).
+        if (K <= 128 && splits == 1 && sk_wpc == 0 && !ep.gather_row && am != KMAJOR_GEN && bm != KMAJOR_GEN &&
+            ((M + 63) / 64) * ((N + 63) / 64) * batch_count >= 2048)
+            tile = bm == KMAJOR_VEC ? 2 : 4;
         if (S.verbose) fprintf(stderr, "tenmo_hip gemm M=%lld N=%lld K=%lld batch=%lld -> tile %dx%d, %d K slice(s), est %.1f us%s\n",
                                (long long)M, (long long)N, (long long)K, (long long)batch_count, kTiles[tile].bm, kTiles[tile].bn, splits, best,
                                sk_wpc ? " (stream-K chosen instead)" : "");
