@@ -1079,6 +1079,42 @@ def test_conv2d_backward(T, golden, oracle):
     assert L.tenmo_hip_conv2d_backward_f32(X.data_ptr(), n, ci, h, w, K.data_ptr(), co, k, k, 1, 1, None, None, gk.data_ptr(), None, 0, 1) == -3
 
 
+def test_products_with_more_than_2_31_elements(T):
+    """Results and operands with more than 2^31 elements: element offsets must be 64-bit everywhere.  The
+    inputs are small integers, so every product is exact in fp32 and the check is equality: a GEMM whose
+    result has 46400^2 elements, a batched one with 40 x 8192^2, mv and vm over a [65536, 40000] matrix."""
+    import torch
+    L = T.lib.load()
+    gen = torch.Generator(device="cuda").manual_seed(5)
+    ints = lambda *shape: torch.randint(-3, 4, shape, generator=gen, device="cuda").float()
+    K = 16
+    M = N = 46400
+    A, B = ints(M, K), ints(K, N)
+    Cd = torch.empty((M, N), dtype=torch.float32, device="cuda")
+    T.lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, K, 1, B.data_ptr(), 0, N, 1, Cd.data_ptr(), M, N, K, 0, None, None, None, 0, 1))
+    for r0 in range(0, M, 5800): # reference in slabs of rows: fp32 sums of small integers are exact in any order
+        assert torch.equal(Cd[r0:r0 + 5800], A[r0:r0 + 5800] @ B), ("gemm", r0)
+    del Cd
+    nb, M, N = 40, 8192, 8192
+    A, B = ints(nb, M, K), ints(K, N)
+    Cd = torch.empty((nb, M, N), dtype=torch.float32, device="cuda")
+    T.lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, K, 1, B.data_ptr(), 0, N, 1, Cd.data_ptr(), M, N, K,
+                                     1, T.lib.i64([nb]), T.lib.i64([M * K]), T.lib.i64([0]), 0, 1))
+    for b in range(nb):
+        assert torch.equal(Cd[b], A[b] @ B), ("batched gemm", b)
+    del Cd, A, B
+    rows, cols = 65536, 40000
+    Mx, x, y = ints(rows, cols), ints(cols), ints(rows)
+    out = torch.empty(rows, dtype=torch.float32, device="cuda")
+    T.lib.check(L.tenmo_hip_mv_f32(Mx.data_ptr(), 0, cols, 1, x.data_ptr(), 0, 1, out.data_ptr(), rows, cols, 0, None, None, None, 0, 1))
+    ref = torch.cat([Mx[r0:r0 + 8192].double() @ x.double() for r0 in range(0, rows, 8192)])
+    assert torch.equal(out.double(), ref), "mv"
+    out = torch.empty(cols, dtype=torch.float32, device="cuda")
+    T.lib.check(L.tenmo_hip_vm_f32(y.data_ptr(), 0, 1, Mx.data_ptr(), 0, cols, 1, out.data_ptr(), rows, cols, 0, None, None, None, 0, 1))
+    ref = sum(y[r0:r0 + 8192].double() @ Mx[r0:r0 + 8192].double() for r0 in range(0, rows, 8192))
+    assert torch.equal(out.double(), ref), "vm"
+
+
 def test_zz_shutdown_and_reinit(T):
     """tenmo_hip_shutdown releases the library's stream and scratch; after tenmo_hip_init everything works again and
     gives the same results (split-K workspace, column-kernel partial sums and the convolution tables are re-grown)."""
