@@ -34,7 +34,7 @@ FLAGS = [
 ]
 
 # (rows, cols, part) units of the GEMM: part 0 = one workgroup per tile, 1 = the stream-K kernels
-TILES = [(256, 128, 0), (256, 128, 1), (128, 128, 0), (128, 128, 1), (64, 64, 0), (128, 64, 0), (64, 128, 0)]
+TILES = [(256, 128, 0), (256, 128, 1), (128, 128, 0), (128, 128, 1), (64, 64, 0), (64, 64, 1), (128, 64, 0), (128, 64, 1), (64, 128, 0)]
 NOISE = "is not a recognized feature for this target"
 
 

@@ -18,5 +18,7 @@ bool launch_gemm_64x128(const GemmArgs& g, dim3 grid, int amode, int bmode, hipS
 // each (0: no tile is shared, no fix-up).  Vector operand modes only.
 bool launch_streamk_256x128(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);
 bool launch_streamk_128x128(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);
+bool launch_streamk_128x64(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);
+bool launch_streamk_64x64(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);
 
 } // namespace tenmo

@@ -787,8 +787,9 @@ struct StreamKArgs {
     float* partial;   // [2 * workgroups][BM * BN]
 };
 
+// (the small tiles must keep to the registers of four workgroups per CU, as their one-tile-per-workgroup kernels do)
 template <int BM, int BN, int AMODE, int BMODE>
-__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_streamk_kernel(const GemmArgs g, const StreamKArgs sk) {
+__global__ __launch_bounds__(GEMM_THREADS, (BM * BN <= 128 * 64 ? 4 : 2)) void gemm_streamk_kernel(const GemmArgs g, const StreamKArgs sk) {
     constexpr int STAGE_FLOATS = (BM + BN) * GEMM_BK;
     constexpr bool DIRECT = (AMODE != KMAJOR_GEN) && (BMODE != KMAJOR_GEN);
     __shared__ __attribute__((aligned(1024))) float stage0[STAGE_FLOATS];
@@ -875,7 +876,7 @@ __global__ void streamk_fixup_kernel(const GemmArgs g, const StreamKArgs sk) {
             const int64_t i = row * g.N + col + q;
             float o = v[q];
             if (g.accumulate) o += Cb[i];
-            if (fused) o = epilogue_value(o, g.bias, mask, g.relu, i, col + q);
+            if (fused) o = epilogue_value(o, g.bias, mask, g.relu, i, g.bias_rows ? row : col + q);
             Cb[i] = o;
         }
     }

@@ -1,4 +1,4 @@
-// The instantiations of gemm_mfma_kernel (and, for the two large tiles, gemm_streamk_kernel) for ONE
+// The instantiations of gemm_mfma_kernel (and, for four of the tiles, gemm_streamk_kernel) for ONE
 // workgroup tile, selected with -DTENMO_TILE_BM / -DTENMO_TILE_BN.  -DTENMO_TILE_STREAMK=0 compiles the
 // one-workgroup-per-tile kernels, =1 the stream-K kernels of that tile.  tenmo_amd/build.py compiles
 // this file once per (tile, part), in parallel.

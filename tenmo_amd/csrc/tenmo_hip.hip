@@ -171,6 +171,9 @@ struct TileShape { int bm, bn; };
 constexpr int kNumTiles = 5;
 const TileShape kTiles[kNumTiles] = {{256, 128}, {128, 128}, {64, 64}, {128, 64}, {64, 128}};
 
+const double kOccupancy[kNumTiles] = {2, 3, 6, 4, 4}; // resident workgroups per CU of each tile's kernel (LDS / VGPR limits)
+const int kStreamKOccupancy[kNumTiles] = {2, 2, 4, 4, 0}; // the same for the stream-K kernels (more registers; none for 64x128)
+
 // what the GEMM store does besides writing the sums (all optional)
 struct Epilogue {
     const float* bias = nullptr; // + bias[col]
@@ -225,7 +228,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     int sk_tile = 0, sk_wpc = 0;
     double best_sk = 1e300;
     {
-        static const double kOcc[kNumTiles] = {2, 3, 6, 4, 4};             // resident workgroups per CU (LDS / VGPR limits)
+        const double* kOcc = kOccupancy;
         static const double kEff[kNumTiles] = {0.96, 0.93, 0.84, 0.90, 0.90}; // matrix-pipe efficiency of the K loop
         static const int kSplits[] = {1, 2, 3, 4, 6, 8, 12, 16, 24, 32};
         const double cus = (double)S.cus;
@@ -258,20 +261,26 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         }
         // stream-K (persistent workgroups: rounds of whole tiles, then the K steps of the remaining tiles
         // spread evenly, see gemm_mfma.hpp): no partial last round, at the price of the fix-up traffic
-        if (S.force_streamk < 0 && am != KMAJOR_GEN && bm != KMAJOR_GEN && !ep.gather_row) {
+        if (S.force_streamk < 0 && am != KMAJOR_GEN && bm != KMAJOR_GEN) {
             // Measured: 128x128 wins, with one workgroup per CU while there are at most two tiles per CU and with two
             // beyond (three do not fit its registers); 256x128 with two per CU comes within 1-2 % at large sizes.
-            for (int t = 1; t >= 0; --t) {
+            // A gathered operand keeps its tile (see above) at that tile's resident workgroups per CU.
+            const int gather_tile = M > 64 ? 3 : 2;
+            for (int t = ep.gather_row ? gather_tile : 1; t >= 0; --t) {
                 const int64_t tiles = ((M + kTiles[t].bm - 1) / kTiles[t].bm) * ((N + kTiles[t].bn - 1) / kTiles[t].bn) * batch_count;
-                const int wpc = (t == 0 || tiles >= 2 * (int64_t)S.cus) ? 2 : 1;
+                const int wpc = ep.gather_row ? kStreamKOccupancy[t] : (t == 0 || tiles >= 2 * (int64_t)S.cus) ? 2 : 1;
                 const int64_t nks = (K + GEMM_BK - 1) / GEMM_BK, wgs = (int64_t)S.cus * wpc;
                 int64_t whole_rounds, shared;
                 streamk_partition(tiles, nks, wgs, &whole_rounds, &shared);
-                if (shared == 0 || shared * nks < wgs * 8) continue; // nothing to share / pieces of under eight K steps are all overhead
+                const bool last = ep.gather_row != nullptr; // one candidate only
+                if (shared == 0 || shared * nks < wgs * 8) { if (last) break; continue; } // nothing to share / pieces of under eight K steps are all overhead
                 // with fewer tiles than workgroups only 128x128 at one workgroup per CU wins; with rounds of whole tiles and a
                 // short K the shared part must be small (measured at K = 768: -10 % with a third of the tiles shared, +5 %
                 // with 2 %; from K = 2560 up +5 to +18 % whatever the share)
-                if (whole_rounds == 0 ? (t != 1 || wpc != 1) : (nks < 64 && shared * 10 > tiles)) continue;
+                if (!ep.gather_row && (whole_rounds == 0 ? (t != 1 || wpc != 1) : (nks < 64 && shared * 10 > tiles))) continue;
+                // gathered: measured on convolution layers, 128x64 gains 5-8 % from K = 1024 up while the tiles make at most
+                // two rounds, and loses 9 % at three (its stream-K kernel spills a few registers) and with a short K; 64x64 loses
+                if (ep.gather_row && (t != 3 || nks < 64 || whole_rounds > 1)) break;
                 // 16-byte loads from rows that are not 16-byte aligned are slow enough to be the bound, and one workgroup
                 // per CU hides them badly (measured [2048,50257].[50257,768]: 118 against 126 TFLOP/s with K slices)
                 const int64_t a_pitch = am == KMAJOR_VEC ? a_rs : a_cs, b_pitch = bm == KMAJOR_VEC ? b_cs : b_rs;
@@ -282,6 +291,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
                 const double fix = 2.0 * pieces * kTiles[t].bm * kTiles[t].bn * 4.0 / 5.0e6;
                 const double est = whole_rounds * (nks * step_us + 1.5) + (double)shared * nks / wgs * step_us + fix + 10.0;
                 if (est < 0.98 * best && est < best_sk) { best_sk = est; sk_tile = t; sk_wpc = wpc; }
+                if (last) break;
             }
         }
         // A product with K <= 128 and a large result is bound by its stores, which the model does not rank: all tiles
@@ -300,7 +310,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     if (S.force_splitk > 0 && !ep.bias_rows) splits = S.force_splitk; // the slice reduction applies the bias by column only
     int streamk = S.force_streamk > 0 ? S.force_streamk : 0;
     if (S.force_streamk < 0 && sk_wpc > 0 && S.force_tile < 0 && S.force_splitk <= 0) { streamk = sk_wpc; tile = sk_tile; }
-    if (streamk > 0 && tile <= 1 && am != KMAJOR_GEN && bm != KMAJOR_GEN && !ep.gather_row) {
+    if (streamk > 0 && tile <= 3 && am != KMAJOR_GEN && bm != KMAJOR_GEN && (!ep.gather_row || tile >= 2)) {
         const int bmt = kTiles[tile].bm, bnt = kTiles[tile].bn;
         g.tiles_m = (int32_t)((M + bmt - 1) / bmt);
         g.tiles_n = (int32_t)((N + bnt - 1) / bnt);
@@ -308,7 +318,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         const int64_t tiles_total = (int64_t)g.tiles_m * g.tiles_n * batch_count;
         StreamKArgs sk{};
         sk.nks = (K + GEMM_BK - 1) / GEMM_BK;
-        const int64_t want = (int64_t)S.cus * std::min(streamk, 2); // the registers of both kernels allow two workgroups per CU
+        const int64_t want = (int64_t)S.cus * std::min(streamk, kStreamKOccupancy[tile]); // every workgroup of the grid must be resident
         int64_t whole_rounds, shared;
         streamk_partition(tiles_total, sk.nks, want, &whole_rounds, &shared);
         sk.dp_tiles = whole_rounds * want;
@@ -328,8 +338,10 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
             // parts per shared tile in the fix-up: a power of two that brings it to a few workgroups per CU
             unsigned parts = 0;
             if (need_fixup) for (parts = 1; parts < 32 && shared * parts < (int64_t)S.cus * 4; parts *= 2) {}
-            const bool ok = tile == 0 ? launch_streamk_256x128(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream)
-                                      : launch_streamk_128x128(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream);
+            const bool ok = tile == 0   ? launch_streamk_256x128(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream)
+                            : tile == 1 ? launch_streamk_128x128(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream)
+                            : tile == 2 ? launch_streamk_64x64(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream)
+                                        : launch_streamk_128x64(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream);
             return ok ? 0 : fail(TENMO_ERR_UNSUPPORTED, "no stream-K variant for operand modes %d/%d", am, bm);
         }
     }

@@ -271,7 +271,7 @@ def test_column_sum(T):
     assert np.all(out.to_numpy() == 0)
 
 
-@pytest.mark.parametrize("tile", [0, 1])
+@pytest.mark.parametrize("tile", [0, 1, 2, 3])
 def test_stream_k(T, tile):
     """Persistent stream-K launches: tiles shared between workgroups are summed by the fix-up kernel.
     Shapes with fewer tiles than workgroups, with rounds of whole tiles ahead of the shared ones (one
@@ -281,7 +281,7 @@ def test_stream_k(T, tile):
     rng = np.random.default_rng(53)
     try:
         L.tenmo_hip_set_tuning(b"gemm_tile", tile)
-        for wg_per_cu in (1, 2):
+        for wg_per_cu in ((1, 2) if tile <= 1 else (1, 4)):
             L.tenmo_hip_set_tuning(b"gemm_streamk", wg_per_cu)
             for (bsz, m, k, n) in [(1, 768, 2000, 640), (1, 300, 4100, 200), (1, 2048, 512, 1536), (3, 260, 1000, 132), (1, 100, 64, 70), (1, 1500, 8192, 900),
                                       (1, 2304, 400, 2432), (4, 2300, 400, 2432), (1, 2304, 100, 2432), (1, 4096, 48, 4096)]:
@@ -1024,6 +1024,40 @@ def test_blocked_tile_order(T):
     finally:
         for knob in (b"gemm_tile", b"gemm_splitk", b"gemm_streamk"):
             L.tenmo_hip_set_tuning(knob, -1)
+
+
+def test_conv2d_stream_k(T, oracle):
+    """The convolution's gathered products through the persistent stream-K launch (rounds of whole tiles, then
+    tiles shared between workgroups and summed by the fix-up, which also adds the per-channel bias): forward and
+    the three gradients of layers with fewer and more tiles than workgroups, both gather tiles."""
+    import torch
+    from helpers import conv_backward_reference64
+    from tenmo_amd.cnn import Conv2dFused
+    L = T.lib.load()
+    rng = np.random.default_rng(131)
+    try:
+        for tile in (2, 3):
+            L.tenmo_hip_set_tuning(b"gemm_tile", tile)
+            L.tenmo_hip_set_tuning(b"gemm_streamk", 4)
+            for (n, ci, h, w, co, k, stride) in [(2, 8, 20, 20, 70, 3, 1), (40, 16, 36, 36, 150, 3, 1), (3, 40, 30, 30, 24, 5, 2)]:
+                image = rng.standard_normal((n, ci, h, w), dtype=np.float32)
+                kernel = rng.standard_normal((co, ci, k, k), dtype=np.float32)
+                bias = rng.standard_normal(co, dtype=np.float32)
+                case = (tile, n, ci, h, w, co, k, stride)
+                got = Conv2dFused.forward(T.Tensor.from_numpy(image), T.Tensor.from_numpy(kernel), T.Tensor.from_numpy(bias), stride=stride).to_numpy()
+                pads = oracle.conv_padding(h, w, k, k, stride, 1, "valid")
+                ref = torch.nn.functional.conv2d(torch.from_numpy(image).double(), torch.from_numpy(kernel).double(),
+                                                 torch.from_numpy(bias).double(), stride=stride).numpy()
+                assert rel_fro(got, ref) <= RTOL_FRO, case
+                up = rng.standard_normal(got.shape, dtype=np.float32)
+                gi, gk, gb = Conv2dFused.backward(T.Tensor.from_numpy(image), T.Tensor.from_numpy(kernel), T.Tensor.from_numpy(up), stride=stride)
+                ri, rk, rb = conv_backward_reference64(image, kernel, up, stride, 1, pads)
+                assert rel_fro(gi.to_numpy(), ri) <= RTOL_FRO, case + ("image",)
+                assert rel_fro(gk.to_numpy(), rk) <= RTOL_FRO, case + ("kernel",)
+                assert rel_fro(gb.to_numpy(), rb) <= RTOL_FRO, case + ("bias",)
+    finally:
+        L.tenmo_hip_set_tuning(b"gemm_tile", -1)
+        L.tenmo_hip_set_tuning(b"gemm_streamk", -1)
 
 
 def test_conv2d_backward(T, golden, oracle):
