@@ -356,13 +356,30 @@ __global__ void conv_dilate_pad_kernel(const float* __restrict src, float* __res
     }
 }
 
-// kernel [c_out, c_in, kh, kw] -> [c_in, c_out, kh, kw] with both spatial axes reversed
-__global__ void conv_flip_kernel(const float* __restrict src, float* __restrict dst, int c_out, int c_in, int kh, int kw) {
-    const int total = c_out * c_in * kh * kw;
+// kernel [c_out, c_in, kh, kw] -> [c_in, c_out, th, tw]: channel axes swapped, and of each spatial axis the taps
+// last, last - step, last - 2*step, ... (th / tw of them).  th = kh, tw = kw, last = kh-1 / kw-1, step = 1 is the
+// whole kernel with both spatial axes reversed.
+__global__ void conv_flip_taps_kernel(const float* __restrict src, float* __restrict dst, int c_out, int c_in, int kh, int kw,
+                                      int th, int tw, int last_y, int last_x, int step) {
+    const int total = c_out * c_in * th * tw;
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= total) return;
-    const int kx = i % kw, ky = (i / kw) % kh, co = (i / (kw * kh)) % c_out, ci = i / (kw * kh * c_out);
-    dst[i] = src[((co * c_in + ci) * kh + (kh - 1 - ky)) * kw + (kw - 1 - kx)];
+    const int tx = i % tw, ty = (i / tw) % th, co = (i / (tw * th)) % c_out, ci = i / (tw * th * c_out);
+    dst[i] = src[((co * c_in + ci) * kh + (last_y - ty * step)) * kw + (last_x - tx * step)];
+}
+
+// dst[plane, py + stride*i, px + stride*j] (+)= src[plane, i, j] for i < hs, j < ws: one phase of a strided image
+// gradient put in place.  src == nullptr writes zeros (a phase no kernel tap reaches).
+__global__ void conv_scatter_phase_kernel(const float* __restrict src, float* __restrict dst, int64_t planes, int h, int w, int hs, int ws,
+                                          int py, int px, int stride, int accumulate) {
+    const int64_t total = planes * hs * ws;
+    for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (int64_t)gridDim.x * blockDim.x) {
+        const int j = (int)(i % ws), r = (int)((i / ws) % hs);
+        const int64_t plane = i / ((int64_t)ws * hs);
+        float* d = dst + (plane * h + py + (int64_t)stride * r) * w + px + (int64_t)stride * j;
+        const float v = src ? src[i] : 0.f;
+        *d = accumulate ? *d + v : v;
+    }
 }
 
 } // namespace tenmo

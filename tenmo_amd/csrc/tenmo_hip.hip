@@ -12,6 +12,7 @@
 #include <hip/hip_runtime.h>
 
 #include <algorithm>
+#include <numeric>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -73,6 +74,7 @@ struct State {
     // tuning overrides (environment, read once): -1 = automatic
     int force_tile = -1;
     int force_splitk = -1;
+    int force_conv_phases = -1; // strided image gradient phase by phase: -1 automatic (large layers), 0 never, 1 always
     int force_streamk = -1;    // -1 automatic, 0 never, n > 0: stream-K with n workgroups per CU
     int verbose = 0;
     int cols_waves_per_cu = 2; // target workgroups per CU of the column-streaming kernels (long K slices stream best)
@@ -248,7 +250,11 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
                 // runs with fewer workgroups per CU, each of them faster for it; the rounds do not end in
                 // step, which costs a quarter of a round where a partial one follows full ones.
                 const double iters = std::ceil((double)K / sp / GEMM_BK);
-                auto round_us = [&](double conc) { return iters * conc * m_us / kEff[t] + 1.5; };
+                // a gathered operand is loaded through a table lookup and registers, one K step ahead only: a workgroup
+                // cannot finish a step in less than about 1.4 us however few share the CU (measured: 256 workgroups of
+                // 128 steps 200 us), so a launch with few tiles is better cut into K slices
+                const double step_floor = ep.gather_row ? 1.4 : 0.0;
+                auto round_us = [&](double conc) { return iters * std::max(conc * m_us / kEff[t], step_floor) + 1.5; };
                 const double full = std::floor(wgs / slots), rest = wgs - full * slots;
                 double t_rounds = full * round_us(kOcc[t]);
                 if (rest > 0) t_rounds += round_us(std::ceil(rest / cus)) + (full > 0 ? 0.25 * round_us(kOcc[t]) : 0.0);
@@ -819,6 +825,7 @@ int tenmo_hip_set_tuning(const char* name, int value) {
     if (!strcmp(name, "gemm_tile")) { S.force_tile = value; return 0; }
     if (!strcmp(name, "gemm_splitk")) { S.force_splitk = value; return 0; }
     if (!strcmp(name, "gemm_streamk")) { S.force_streamk = value; return 0; }
+    if (!strcmp(name, "conv_phases")) { S.force_conv_phases = value; return 0; }
     if (!strcmp(name, "cols_wg_per_cu")) { S.cols_waves_per_cu = value > 0 ? value : 2; return 0; }
     return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: unknown knob '%s'", name);
 }
@@ -1136,7 +1143,63 @@ int tenmo_hip_conv2d_backward_f32(const float* padded_image, int64_t n_images, i
             if (int rc = matvec_dispatch(per_image, 1, c_out * nk, S.one, 0, grad_kernel, c_out * nk, n_images, one_batch, 1, acc)) return rc;
         }
     }
-    if (grad_padded_image) {
+    const bool by_phase = stride > 1 && (S.force_conv_phases >= 0 ? S.force_conv_phases != 0
+                                                                     : (double)n_images * c_in * c_out * kh * kw * h_pad * w_pad >= 5.0e8);
+    if (grad_padded_image && by_phase) {
+        // Strided layer: the image gradient phase by phase.  The input positions (y, x) with y % stride = py and
+        // x % stride = px are reached only by the kernel taps with ky*dilation = py and kx*dilation = px modulo the stride,
+        // each from the upstream element ((y - ky*dilation) / stride, ...): a stride-1 convolution of the upstream gradient
+        // (zero-padded, not spread out) with those taps reversed, whose result goes to every stride-th position.  All
+        // phases together do the multiply-adds of the forward pass; the single convolution below does stride^2 times as
+        // many, most of them with the zeros between the spread-out elements.  (Small layers keep it: fewer launches.)
+        const int64_t g = std::gcd(stride, dilation), tap_step = stride / g, tap_dil = dilation / g;
+        struct Axis { int64_t first, count, last, amax, size; }; // taps ky = first + i*tap_step; amax = upstream offset of the last tap
+        auto axis = [&](int64_t phase, int64_t ksize, int64_t extent, int64_t out_extent) {
+            Axis a{-1, 0, -1, 0, 0};
+            for (int64_t k = 0; k < ksize; ++k)
+                if ((k * dilation - phase) % stride == 0) { if (a.first < 0) a.first = k; a.last = k; ++a.count; }
+            a.size = phase < extent ? (extent - phase + stride - 1) / stride : 0;
+            if (a.count) a.amax = (a.last * dilation - phase) / stride;
+            (void)out_extent;
+            return a;
+        };
+        int64_t max_src = 0, max_out = 0;
+        for (int64_t py = 0; py < stride; ++py)
+            for (int64_t px = 0; px < stride; ++px) {
+                const Axis ay = axis(py, kh, h_pad, geo.h_out), ax = axis(px, kw, w_pad, geo.w_out);
+                if (!ay.count || !ax.count || !ay.size || !ax.size) continue;
+                max_src = std::max(max_src, n_images * c_out * (ay.size + (ay.count - 1) * tap_dil) * (ax.size + (ax.count - 1) * tap_dil));
+                max_out = std::max(max_out, n_images * c_in * ay.size * ax.size);
+            }
+        const int64_t flip_len = c_out * c_in * kh * kw;
+        float* buf = nullptr;
+        if (max_src > 0)
+            if (int rc = workspace2((size_t)(max_src + max_out + flip_len) * sizeof(float), &buf)) return rc;
+        float *padded = buf, *phase_out = buf + max_src, *taps = buf + max_src + max_out;
+        for (int64_t py = 0; py < stride; ++py)
+            for (int64_t px = 0; px < stride; ++px) {
+                const Axis ay = axis(py, kh, h_pad, geo.h_out), ax = axis(px, kw, w_pad, geo.w_out);
+                if (!ay.size || !ax.size) continue;
+                const int64_t planes = n_images * c_in, out_len = planes * ay.size * ax.size;
+                const dim3 sgrid((unsigned)std::min<int64_t>((out_len + 255) / 256, (int64_t)S.cus * 32));
+                if (!ay.count || !ax.count) { // no tap reaches this phase: its gradient is zero
+                    if (!acc) hipLaunchKernelGGL(conv_scatter_phase_kernel, sgrid, dim3(256), 0, S.stream, (const float*)nullptr, grad_padded_image, planes,
+                                                 (int)h_pad, (int)w_pad, (int)ay.size, (int)ax.size, (int)py, (int)px, (int)stride, 0);
+                    continue;
+                }
+                const int64_t h_src = ay.size + (ay.count - 1) * tap_dil, w_src = ax.size + (ax.count - 1) * tap_dil;
+                const int64_t src_len = n_images * c_out * h_src * w_src, taps_len = c_out * c_in * ay.count * ax.count;
+                hipLaunchKernelGGL(conv_dilate_pad_kernel, dim3((unsigned)std::min<int64_t>((src_len + 255) / 256, (int64_t)S.cus * 32)), dim3(256), 0, S.stream,
+                                   grad_out, padded, n_images * c_out, (int)geo.h_out, (int)geo.w_out, (int)h_src, (int)w_src, 1, (int)ay.amax, (int)ax.amax);
+                hipLaunchKernelGGL(conv_flip_taps_kernel, dim3((unsigned)((taps_len + 255) / 256)), dim3(256), 0, S.stream, kernel, taps, (int)c_out, (int)c_in,
+                                   (int)kh, (int)kw, (int)ay.count, (int)ax.count, (int)ay.last, (int)ax.last, (int)tap_step);
+                const ConvGeometry back{(int32_t)c_out, (int32_t)h_src, (int32_t)w_src, (int32_t)ay.count, (int32_t)ax.count,
+                                        (int32_t)ay.size, (int32_t)ax.size, 1, (int32_t)tap_dil};
+                if (int rc = conv_forward_impl(padded, n_images, back, taps, c_in, nullptr, phase_out, 0)) return rc;
+                hipLaunchKernelGGL(conv_scatter_phase_kernel, sgrid, dim3(256), 0, S.stream, (const float*)phase_out, grad_padded_image, planes,
+                                   (int)h_pad, (int)w_pad, (int)ay.size, (int)ax.size, (int)py, (int)px, (int)stride, acc);
+            }
+    } else if (grad_padded_image) {
         // The scatter of the reference's loop (cnn.mojo:818-948) as a gather: a stride-1 convolution, same dilation, of the
         // upstream gradient spread out by `stride` and zero-padded by the dilated kernel size - 1, with the kernel's
         // channel axes swapped and its spatial axes reversed.
@@ -1149,7 +1212,8 @@ int tenmo_hip_conv2d_backward_f32(const float* padded_image, int64_t n_images, i
         float* flipped = buf + spread_len;
         hipLaunchKernelGGL(conv_dilate_pad_kernel, dim3((unsigned)std::min<int64_t>((spread_len + 255) / 256, (int64_t)S.cus * 32)), dim3(256), 0, S.stream,
                            grad_out, spread, n_images * c_out, (int)geo.h_out, (int)geo.w_out, (int)h_dst, (int)w_dst, (int)stride, (int)(dkh - 1), (int)(dkw - 1));
-        hipLaunchKernelGGL(conv_flip_kernel, dim3((unsigned)((flip_len + 255) / 256)), dim3(256), 0, S.stream, kernel, flipped, (int)c_out, (int)c_in, (int)kh, (int)kw);
+        hipLaunchKernelGGL(conv_flip_taps_kernel, dim3((unsigned)((flip_len + 255) / 256)), dim3(256), 0, S.stream, kernel, flipped, (int)c_out, (int)c_in,
+                           (int)kh, (int)kw, (int)kh, (int)kw, (int)(kh - 1), (int)(kw - 1), 1);
         const ConvGeometry back{(int32_t)c_out, (int32_t)h_dst, (int32_t)w_dst, (int32_t)kh, (int32_t)kw, (int32_t)h_pad, (int32_t)w_pad, 1, (int32_t)dilation};
         if (int rc = conv_forward_impl(spread, n_images, back, flipped, c_in, nullptr, grad_padded_image, acc)) return rc;
     }

@@ -1060,6 +1060,48 @@ def test_conv2d_stream_k(T, oracle):
         L.tenmo_hip_set_tuning(b"gemm_streamk", -1)
 
 
+def test_conv2d_strided_image_gradient_by_phase(T, oracle):
+    """The image gradient of a strided convolution computed phase by phase (one small stride-1 convolution per
+    residue of the input position modulo the stride) against torch autograd in fp64 and the CPU restatement:
+    strides 2-4 with dilations 1-3, kernels smaller than the stride (phases no tap reaches), 1x1 kernels, image
+    sizes that leave a remainder, accumulate; the same cases through the single-convolution form must agree."""
+    from helpers import conv_backward_reference64
+    from tenmo_amd.cnn import Conv2dFused
+    L = T.lib.load()
+    rng = np.random.default_rng(151)
+    cases = [(2, 3, 11, 12, 4, 3, 3, 2, 1), (1, 2, 9, 9, 3, 3, 3, 3, 1), (2, 2, 14, 13, 3, 3, 3, 2, 2), (1, 3, 17, 15, 2, 3, 2, 2, 3),
+             (2, 1, 12, 12, 2, 2, 2, 4, 1), (1, 2, 10, 10, 2, 1, 1, 2, 1), (3, 4, 16, 16, 5, 5, 5, 3, 2), (2, 70, 19, 19, 66, 3, 3, 2, 1),
+             (1, 2, 13, 11, 2, 4, 3, 4, 3), (2, 2, 8, 8, 2, 3, 3, 6, 1)]
+    try:
+        for (n, ci, h, w, co, kh, kw, stride, dil) in cases:
+            image = rng.standard_normal((n, ci, h, w), dtype=np.float32)
+            kernel = rng.standard_normal((co, ci, kh, kw), dtype=np.float32)
+            ho, wo = (h - (kh + (kh - 1) * (dil - 1))) // stride + 1, (w - (kw + (kw - 1) * (dil - 1))) // stride + 1
+            up = rng.standard_normal((n, co, ho, wo), dtype=np.float32)
+            ri, rk, rb = conv_backward_reference64(image, kernel, up, stride, dil, (0, 0, 0, 0))
+            want = oracle.conv2d_backward(image, kernel, up, stride=stride, dilation=dil, padding="valid")[0]
+            got = {}
+            for phases in (1, 0):
+                L.tenmo_hip_set_tuning(b"conv_phases", phases)
+                gi, gk, gb = Conv2dFused.backward(T.Tensor.from_numpy(image), T.Tensor.from_numpy(kernel), T.Tensor.from_numpy(up), stride=stride, dilation=dil)
+                got[phases] = gi.to_numpy()
+                case = (phases, n, ci, h, w, co, kh, kw, stride, dil)
+                assert rel_fro(got[phases], ri) <= RTOL_FRO, case
+                assert rel_fro(got[phases], want) <= 2 * RTOL_FRO, case
+                assert rel_fro(gk.to_numpy(), rk) <= RTOL_FRO, case
+            assert rel_fro(got[1], got[0]) <= RTOL_FRO
+            # accumulate: gradient added onto what the buffer holds
+            L.tenmo_hip_set_tuning(b"conv_phases", 1)
+            import torch
+            X, K, U = (torch.from_numpy(a).cuda() for a in (image, kernel, up))
+            G = torch.ones((n, ci, h, w), dtype=torch.float32, device="cuda")
+            T.lib.check(L.tenmo_hip_conv2d_backward_f32(X.data_ptr(), n, ci, h, w, K.data_ptr(), co, kh, kw, stride, dil, U.data_ptr(),
+                                                        G.data_ptr(), None, None, 1, 1))
+            assert rel_fro(G.cpu().numpy(), ri + 1.0) <= RTOL_FRO, ("accumulate",) + case
+    finally:
+        L.tenmo_hip_set_tuning(b"conv_phases", -1)
+
+
 def test_conv2d_backward(T, golden, oracle):
     """FusedCol2ImBackward through tenmo_hip_conv2d_backward_f32: the gradients asserted in tests/test_cnn.mojo,
     then random layers against the CPU restatement and torch autograd in fp64 (stride, dilation, all padding
