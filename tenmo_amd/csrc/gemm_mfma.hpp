@@ -598,15 +598,86 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
             lb.init_staged(b_row_s, b_k_s, n0, g.N, t, g.b_gather_row);
         }
         // a whole K step goes through the unchecked loads; the K tail and ragged MN-major tiles through the checked ones
-        auto load_a = [&](int64_t k0) {
-            if (STAGED_FAST && la.staged_ok && k0 + GEMM_BK <= k_end) la.load_staged(Ab, a_k_s, m0, k0, nullptr, nullptr, t);
-            else la.load_checked(Ab, a_row_s, a_k_s, m0, k0, g.M, k_end, t);
+        auto load_a_into = [&](TileLoader<BM, AMODE>& l, int64_t k0) {
+            if (STAGED_FAST && l.staged_ok && k0 + GEMM_BK <= k_end) l.load_staged(Ab, a_k_s, m0, k0, nullptr, nullptr, t);
+            else l.load_checked(Ab, a_row_s, a_k_s, m0, k0, g.M, k_end, t);
         };
-        auto load_b = [&](int64_t k0) {
-            if (STAGED_FAST && lb.staged_ok && k0 + GEMM_BK <= k_end) lb.load_staged(Bb, b_k_s, n0, k0, g.b_gather_row, g.b_gather_k, t);
-            else lb.load_checked(Bb, b_row_s, b_k_s, n0, k0, g.N, k_end, t, g.b_gather_row, g.b_gather_k);
+        auto load_b_into = [&](TileLoader<BN, BMODE>& l, int64_t k0) {
+            if (STAGED_FAST && l.staged_ok && k0 + GEMM_BK <= k_end) l.load_staged(Bb, b_k_s, n0, k0, g.b_gather_row, g.b_gather_k, t);
+            else l.load_checked(Bb, b_row_s, b_k_s, n0, k0, g.N, k_end, t, g.b_gather_row, g.b_gather_k);
         };
-        if constexpr (BM * BN <= 128 * 128 && STAGED_FAST) {
+        auto load_a = [&](int64_t k0) { load_a_into(la, k0); };
+        auto load_b = [&](int64_t k0) { load_b_into(lb, k0); };
+        if constexpr (BM * BN <= 64 * 64 && STAGED_FAST) {
+            // (64x64 only: the second register set costs the 128x64 tile a resident workgroup per CU, measured a loss there)
+            // Two LDS stages and two sets of staging registers: the loads of step it+2 are issued at the top of step it
+            // and go to LDS in the middle of step it+1, so that they have a step and a half to land (a gathered operand
+            // needs a table lookup and then the load: with one set, in flight for half a step only, the small tiles were
+            // bound by that latency).  The barrier sits in the middle of a step as in the direct ring: behind the first
+            // half's MFMAs the operand fetch of the second half, then the next step's registers go to the other stage,
+            // barrier, and behind the second half's MFMAs the operand fetch of the next step's first half.
+            constexpr int PA2 = frag_parts<AMODE, MB>(), PB2 = frag_parts<BMODE, NB>();
+            constexpr int NMFMA2 = 4 * MB * NB;
+            constexpr int PER_SLOT2 = (PA2 + PB2 + NMFMA2 - 1) / NMFMA2;
+            auto fetch2 = [&](const float* st, int kc, float (&fa)[MB][4], float (&fb)[NB][4], int p) {
+                if (p < PA2) load_fragment_part<BM, AMODE, MB>(st, wm * TM, kc, lane, fa, p);
+                else if (p < PA2 + PB2) load_fragment_part<BN, BMODE, NB>(st + A_FLOATS, wn * TN, kc, lane, fb, p - PA2);
+            };
+            auto mfma2 = [&](const float (&fa)[MB][4], const float (&fb)[NB][4], auto&& slot) {
+                int n = 0;
+#pragma unroll
+                for (int s = 0; s < 4; ++s)
+#pragma unroll
+                    for (int i = 0; i < MB; ++i)
+#pragma unroll
+                        for (int j = 0; j < NB; ++j) {
+                            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[i][s], fb[j][s], acc[i][j], 0, 0, 0);
+                            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                            for (int u = 0; u < PER_SLOT2; ++u) slot(n * PER_SLOT2 + u);
+                            __builtin_amdgcn_sched_barrier(0);
+                            ++n;
+                        }
+            };
+            TileLoader<BM, AMODE> la2; // the same per-thread offsets, a second set of staging registers
+            TileLoader<BN, BMODE> lb2;
+            la2.init_staged(a_row_s, a_k_s, m0, g.M, t, nullptr);
+            lb2.init_staged(b_row_s, b_k_s, n0, g.N, t, g.b_gather_row);
+            float ga0[MB][4], gb0[NB][4], ga1[MB][4], gb1[NB][4];
+            const int64_t kb = k_begin + done * GEMM_BK;
+            load_a_into(la, kb);
+            load_b_into(lb, kb);
+            la.store(stage0, t);
+            lb.store(stage0 + A_FLOATS, t);
+            if (done + 1 < nk) { load_a_into(la, kb + GEMM_BK); load_b_into(lb, kb + GEMM_BK); } // step 1 into the first set
+            __syncthreads();
+            load_fragments<BM, AMODE, MB>(stage0, wm * TM, 0, lane, ga0);
+            load_fragments<BN, BMODE, NB>(stage0 + A_FLOATS, wn * TN, 0, lane, gb0);
+            // one K step: `held` holds step it+1 (loaded a step ago), `ahead` receives step it+2
+            auto step = [&](TileLoader<BM, AMODE>& a_held, TileLoader<BN, BMODE>& b_held, TileLoader<BM, AMODE>& a_ahead, TileLoader<BN, BMODE>& b_ahead,
+                            float* cur, float* nxt, int64_t it) {
+                const bool more = it + 1 < nk;
+                if (it + 2 < nk) {
+                    const int64_t k0 = k_begin + (it + 2) * GEMM_BK;
+                    load_a_into(a_ahead, k0);
+                    load_b_into(b_ahead, k0);
+                }
+                mfma2(ga0, gb0, [&](int p) { fetch2(cur, 1, ga1, gb1, p); });
+                if (more) {
+                    a_held.store(nxt, t);
+                    b_held.store(nxt + A_FLOATS, t);
+                    __syncthreads();
+                }
+                mfma2(ga1, gb1, [&](int p) { if (more) fetch2(nxt, 0, ga0, gb0, p); });
+            };
+            int64_t it = done;
+            for (; it + 1 < nk; it += 2) {
+                step(la, lb, la2, lb2, stage0, stage1, it);
+                step(la2, lb2, la, lb, stage1, stage0, it + 1);
+            }
+            if (it < nk) step(la, lb, la2, lb2, stage0, stage1, it);
+            __syncthreads();
+        } else if constexpr (BM * BN <= 128 * 128 && STAGED_FAST) {
             // Two LDS stages; the barrier sits in the middle of a step (as in the direct ring): behind the first half's
             // MFMAs the operand fetch of the second half, then the next step's registers go to the other stage, barrier,
             // and behind the second half's MFMAs the operand fetch of the next step's first half.
