@@ -1180,16 +1180,16 @@ int tenmo_hip_conv2d_backward_f32(const float* padded_image, int64_t n_images, i
             for (int64_t px = 0; px < stride; ++px) {
                 const Axis ay = axis(py, kh, h_pad, geo.h_out), ax = axis(px, kw, w_pad, geo.w_out);
                 if (!ay.size || !ax.size) continue;
-                const int64_t planes = n_images * c_in, out_len = planes * ay.size * ax.size;
-                const dim3 sgrid((unsigned)std::min<int64_t>((out_len + 255) / 256, (int64_t)S.cus * 32));
+                const int64_t planes = n_images * c_in;
+                const dim3 sgrid((unsigned)std::min<int64_t>(planes, (int64_t)S.cus * 32)); // a workgroup per plane
                 if (!ay.count || !ax.count) { // no tap reaches this phase: its gradient is zero
                     if (!acc) hipLaunchKernelGGL(conv_scatter_phase_kernel, sgrid, dim3(256), 0, S.stream, (const float*)nullptr, grad_padded_image, planes,
                                                  (int)h_pad, (int)w_pad, (int)ay.size, (int)ax.size, (int)py, (int)px, (int)stride, 0);
                     continue;
                 }
                 const int64_t h_src = ay.size + (ay.count - 1) * tap_dil, w_src = ax.size + (ax.count - 1) * tap_dil;
-                const int64_t src_len = n_images * c_out * h_src * w_src, taps_len = c_out * c_in * ay.count * ax.count;
-                hipLaunchKernelGGL(conv_dilate_pad_kernel, dim3((unsigned)std::min<int64_t>((src_len + 255) / 256, (int64_t)S.cus * 32)), dim3(256), 0, S.stream,
+                const int64_t taps_len = c_out * c_in * ay.count * ax.count;
+                hipLaunchKernelGGL(conv_dilate_pad_kernel, dim3((unsigned)std::min<int64_t>(n_images * c_out, (int64_t)S.cus * 32)), dim3(256), 0, S.stream,
                                    grad_out, padded, n_images * c_out, (int)geo.h_out, (int)geo.w_out, (int)h_src, (int)w_src, 1, (int)ay.amax, (int)ax.amax);
                 hipLaunchKernelGGL(conv_flip_taps_kernel, dim3((unsigned)((taps_len + 255) / 256)), dim3(256), 0, S.stream, kernel, taps, (int)c_out, (int)c_in,
                                    (int)kh, (int)kw, (int)ay.count, (int)ax.count, (int)ay.last, (int)ax.last, (int)tap_step);
@@ -1210,7 +1210,7 @@ int tenmo_hip_conv2d_backward_f32(const float* padded_image, int64_t n_images, i
         if (int rc = workspace2((size_t)(spread_len + flip_len) * sizeof(float), &buf)) return rc;
         float* spread = buf;
         float* flipped = buf + spread_len;
-        hipLaunchKernelGGL(conv_dilate_pad_kernel, dim3((unsigned)std::min<int64_t>((spread_len + 255) / 256, (int64_t)S.cus * 32)), dim3(256), 0, S.stream,
+        hipLaunchKernelGGL(conv_dilate_pad_kernel, dim3((unsigned)std::min<int64_t>(n_images * c_out, (int64_t)S.cus * 32)), dim3(256), 0, S.stream,
                            grad_out, spread, n_images * c_out, (int)geo.h_out, (int)geo.w_out, (int)h_dst, (int)w_dst, (int)stride, (int)(dkh - 1), (int)(dkw - 1));
         hipLaunchKernelGGL(conv_flip_taps_kernel, dim3((unsigned)((flip_len + 255) / 256)), dim3(256), 0, S.stream, kernel, flipped, (int)c_out, (int)c_in,
                            (int)kh, (int)kw, (int)kh, (int)kw, (int)(kh - 1), (int)(kw - 1), 1);
