@@ -78,8 +78,9 @@ struct GemmArgs {
     int32_t relu;         // max(.,0) after the bias                      (ReLU forward)
     int32_t bias_rows;    // the bias is indexed by the row of C instead of the column (convolution: one per filter)
     // Gathered B (implicit im2col): when set, B(n, k) = B[b_gather_row[n] + b_gather_k[k]] instead of
-    // B[k*b_rs + n*b_cs]; launched as an MN-major B, loaded through registers with 16-byte loads where
-    // four consecutive n are contiguous in memory.  b_gather_row must be strictly increasing.
+    // B[k*b_rs + n*b_cs]; loaded through registers.  Launched as an MN-major B it takes 16-byte loads where four
+    // consecutive n are contiguous in memory (b_gather_row strictly increasing), launched as a K-major B where
+    // four consecutive k are (b_gather_k strictly increasing).
     const int32_t* b_gather_row; // [N]
     const int32_t* b_gather_k;   // [K]
     BatchDesc batch;
@@ -206,6 +207,10 @@ struct TileLoader {
                     soff[i] = (uint32_t)o0;
                 }
             }
+        } else if (gather_row) { // K-major gather: element (row, k) at base[gather_row[row] + gather_k[k]], rows clamped
+            staged_ok = true;
+#pragma unroll
+            for (int i = 0; i < NCH; ++i) soff[i] = (uint32_t)gather_row[min(row0 + (t >> 2) + 64 * i, R - 1)];
         } else {
             staged_ok = rs >= 0 && (R - 1) * rs + 16 <= 0x7fffffffLL;
 #pragma unroll
@@ -219,6 +224,22 @@ struct TileLoader {
         if constexpr (!STAGED_FAST) {
             return;
         } else if constexpr (MODE == KMAJOR_VEC) {
+            if (gather_row) {
+                // this thread's four k of the step; gather_k is increasing, so a span of 3 means contiguous in memory
+                const int32_t* __restrict gk = gather_k + k0 + 4 * (t & 3);
+                const int32_t g0 = gk[0], g1 = gk[1], g2 = gk[2], g3 = gk[3];
+                if (g3 - g0 == 3) {
+#pragma unroll
+                    for (int i = 0; i < NCH; ++i) r[i] = *reinterpret_cast<const f32x4_u*>(base + soff[i] + g0);
+                } else {
+#pragma unroll
+                    for (int i = 0; i < NCH; ++i) {
+                        const float* __restrict p = base + soff[i];
+                        r[i] = f32x4{p[g0], p[g1], p[g2], p[g3]};
+                    }
+                }
+                return;
+            }
             const float* __restrict b0 = base + k0;
 #pragma unroll
             for (int i = 0; i < NCH; ++i) r[i] = *reinterpret_cast<const f32x4_u*>(b0 + soff[i]);
@@ -253,7 +274,13 @@ struct TileLoader {
                 const int64_t row = row0 + (t >> 2) + 64 * i;
                 const int64_t k = k0 + 4 * kq;
                 f32x4 v = {0.f, 0.f, 0.f, 0.f};
-                if (row < R) {
+                if (row < R && gather_row) { // K-major gather, element by element
+                    const float* p = base + gather_row[row];
+                    if (k + 0 < K) v.x = p[gather_k[k]];
+                    if (k + 1 < K) v.y = p[gather_k[k + 1]];
+                    if (k + 2 < K) v.z = p[gather_k[k + 2]];
+                    if (k + 3 < K) v.w = p[gather_k[k + 3]];
+                } else if (row < R) {
                     const float* p = base + row * rs + k;
                     if (k + 3 < K) v = *reinterpret_cast<const f32x4_u*>(p);
                     else {

@@ -184,6 +184,7 @@ struct Epilogue {
     int bias_rows = 0;           // bias[row] instead of bias[col]
     const int32_t* gather_row = nullptr; // B gathered through offset tables (implicit im2col), see GemmArgs
     const int32_t* gather_k = nullptr;
+    bool gather_kmajor = false;          // the gathered B is contiguous along k (16-byte loads along k) rather than along n
     bool any() const { return bias || mask || relu; }
 };
 
@@ -220,7 +221,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     g.batch = bd;
     g.batch_count = batch_count;
     const int am = operand_mode(a_rs, a_cs, M, K);
-    const int bm = ep.gather_row ? MNMAJOR_VEC : operand_mode(b_cs, b_rs, N, K);
+    const int bm = ep.gather_row ? (ep.gather_kmajor ? KMAJOR_VEC : MNMAJOR_VEC) : operand_mode(b_cs, b_rs, N, K);
 
     // Pick the workgroup tile and the number of K slices with a small cost model of this chip
     // (constants fitted to measured launches on MI355X): per CU the matrix-pipe time is the sum over
@@ -1134,6 +1135,7 @@ int tenmo_hip_conv2d_backward_f32(const float* padded_image, int64_t n_images, i
         bd.rank = 1; bd.shape[0] = n_images; bd.a_str[0] = c_out * np; bd.b_str[0] = c_in * h_pad * w_pad;
         Epilogue ep;
         ep.gather_row = by_k; ep.gather_k = by_pos; // B(n = patch element, k = position)
+        ep.gather_kmajor = stride == 1;             // neighbouring positions of an output row are neighbours in the image
         if (n_images == 1) {
             if (int rc = gemm_dispatch(grad_out, np, 1, padded_image, 0, 0, grad_kernel, c_out, nk, np, bd, 1, acc, ep)) return rc;
         } else {
