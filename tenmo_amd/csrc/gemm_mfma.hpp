@@ -77,6 +77,9 @@ struct GemmArgs {
     const float* mask;    // dense like C: result zeroed where mask <= 0, or null   (ReLU backward on dX)
     int32_t relu;         // max(.,0) after the bias                      (ReLU forward)
     int32_t bias_rows;    // the bias is indexed by the row of C instead of the column (convolution: one per filter)
+    float* colsum;        // [batch][N] or null: receives the column sums of the finished C (after the epilogue above); only for
+                          // a launch whose tile holds every row (tiles_m == 1), one K slice, one of the tiles up to 128x64
+                          // (the bias gradient of a hidden layer, out of the GEMM that produces that layer's gradient)
     // Gathered B (implicit im2col): when set, B(n, k) = B[b_gather_row[n] + b_gather_k[k]] instead of
     // B[k*b_rs + n*b_cs]; loaded through registers.  Launched as an MN-major B it takes 16-byte loads where four
     // consecutive n are contiguous in memory (b_gather_row strictly increasing), launched as a K-major B where
@@ -789,6 +792,11 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
     const bool fused = dst.fused && (g.bias != nullptr || g.mask != nullptr || g.relu != 0);
     const float* __restrict mask = g.mask ? g.mask + batch * g.M * g.N : nullptr;
     const int h = lane >> 5, x = lane & 31;
+    constexpr bool COLSUM = BM * BN <= 128 * 64; // the larger tiles have no registers to spare for it
+    const bool colsum = COLSUM && g.colsum != nullptr && dst.fused;
+    float cs[NB]; // this lane's part of the column sums
+#pragma unroll
+    for (int j = 0; j < NB; ++j) cs[j] = 0.f;
 #pragma unroll
     for (int i = 0; i < MB; ++i) {
 #pragma unroll
@@ -805,6 +813,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
                     const int64_t col = n0 + wn * TN + tile_pos<BMODE, NB>(j, x);
                     if (col < g.N) val[j] = epilogue_value(val[j], g.bias, mask, g.relu, row * g.N + col, g.bias_rows ? row : col);
                 }
+                if constexpr (COLSUM) { if (colsum) cs[j] += val[j]; }
             }
             if constexpr (BMODE == MNMAJOR_VEC && NB > 1) {
                 const int64_t col = n0 + wn * TN + NB * x;
@@ -828,6 +837,25 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
                 for (int j = 0; j < NB; ++j) {
                     const int64_t col = n0 + wn * TN + tile_pos<BMODE, NB>(j, x);
                     if (col < g.N) crow[col] = accumulate ? crow[col] + val[j] : val[j];
+                }
+            }
+        }
+    }
+    if constexpr (COLSUM) {
+        if (colsum) { // uniform over the workgroup; the LDS stages are free: every wave has left the K loop
+            float* red = stage0;
+#pragma unroll
+            for (int j = 0; j < NB; ++j) cs[j] += __shfl_xor(cs[j], 32); // the two halves of a wavefront hold different rows
+            if (wm == 1 && h == 0) {
+#pragma unroll
+                for (int j = 0; j < NB; ++j) red[wn * TN + tile_pos<BMODE, NB>(j, x)] = cs[j];
+            }
+            __syncthreads();
+            if (wm == 0 && h == 0) {
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
+                    const int local = wn * TN + tile_pos<BMODE, NB>(j, x);
+                    if (n0 + local < g.N) g.colsum[batch * g.N + n0 + local] = cs[j] + red[local];
                 }
             }
         }

@@ -185,7 +185,8 @@ struct Epilogue {
     const int32_t* gather_row = nullptr; // B gathered through offset tables (implicit im2col), see GemmArgs
     const int32_t* gather_k = nullptr;
     bool gather_kmajor = false;          // the gathered B is contiguous along k (16-byte loads along k) rather than along n
-    bool any() const { return bias || mask || relu; }
+    float* colsum = nullptr;             // [batch][N]: also write the column sums of the result (needs M <= 128, see GemmArgs)
+    bool any() const { return bias || mask || relu || colsum; }
 };
 
 // Stream-K launch of `tiles` tiles of `nks` K steps on `wgs` persistent workgroups: `whole_rounds` rounds of
@@ -218,6 +219,8 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     g.accumulate = accumulate;
     g.bias = ep.bias; g.mask = ep.mask; g.relu = ep.relu; g.bias_rows = ep.bias_rows;
     g.b_gather_row = ep.gather_row; g.b_gather_k = ep.gather_k;
+    g.colsum = ep.colsum;
+    if (ep.colsum && (M > 128 || accumulate)) return fail(TENMO_ERR_UNSUPPORTED, "column sums in the GEMM store need M <= 128 and no accumulate");
     g.batch = bd;
     g.batch_count = batch_count;
     const int am = operand_mode(a_rs, a_cs, M, K);
@@ -241,11 +244,12 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
             // gradients), the 128x64 tile wins there by 10-40 % over the larger ones, whose staging registers crowd the
             // accumulators, and 64x64 when there are at most 64 rows
             if (ep.gather_row && t != (M > 64 ? 3 : 2)) continue;
+            if (ep.colsum && (t < 2 || kTiles[t].bm < M)) continue; // one tile must hold every row, and only the small tiles sum columns
             const double tm = (double)((M + kTiles[t].bm - 1) / kTiles[t].bm), tn = (double)((N + kTiles[t].bn - 1) / kTiles[t].bn);
             const double tiles = tm * tn * (double)batch_count;
             const double m_us = (kTiles[t].bm / 64) * (kTiles[t].bn / 64) * 8 * 64 / 2400.0; // MFMA time of one K step of one wavefront
             for (int sp : kSplits) {
-                if (sp > 1 && (K / sp < 64 || (double)sp * batch_count * M * N * 4.0 > 1.0e9 || ep.bias_rows)) break;
+                if (sp > 1 && (K / sp < 64 || (double)sp * batch_count * M * N * 4.0 > 1.0e9 || ep.bias_rows || ep.colsum)) break;
                 const double wgs = tiles * sp, slots = cus * kOcc[t];
                 // one round = every CU runs `conc` workgroups side by side.  After the full rounds the rest
                 // runs with fewer workgroups per CU, each of them faster for it; the rounds do not end in
@@ -268,7 +272,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         }
         // stream-K (persistent workgroups: rounds of whole tiles, then the K steps of the remaining tiles
         // spread evenly, see gemm_mfma.hpp): no partial last round, at the price of the fix-up traffic
-        if (S.force_streamk < 0 && am != KMAJOR_GEN && bm != KMAJOR_GEN) {
+        if (S.force_streamk < 0 && am != KMAJOR_GEN && bm != KMAJOR_GEN && !ep.colsum) {
             // Measured: 128x128 wins, with one workgroup per CU while there are at most two tiles per CU and with two
             // beyond (three do not fit its registers); 256x128 with two per CU comes within 1-2 % at large sizes.
             // A gathered operand keeps its tile (see above) at that tile's resident workgroups per CU.
@@ -306,16 +310,16 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         // the small tiles win — more workgroups per CU overlap one's stores with another's loads: 64x64 for a K-major B
         // (8192x8192x64: 112 us against 135 with 256x128; attention Q.K^T 179 against 202), 64x128 for an MN-major B
         // (110 against 116).
-        if (K <= 128 && splits == 1 && sk_wpc == 0 && !ep.gather_row && am != KMAJOR_GEN && bm != KMAJOR_GEN &&
+        if (K <= 128 && splits == 1 && sk_wpc == 0 && !ep.gather_row && !ep.colsum && am != KMAJOR_GEN && bm != KMAJOR_GEN &&
             ((M + 63) / 64) * ((N + 63) / 64) * batch_count >= 2048)
             tile = bm == KMAJOR_VEC ? 2 : 4;
         if (S.verbose) fprintf(stderr, "tenmo_hip gemm M=%lld N=%lld K=%lld batch=%lld -> tile %dx%d, %d K slice(s), est %.1f us%s\n",
                                (long long)M, (long long)N, (long long)K, (long long)batch_count, kTiles[tile].bm, kTiles[tile].bn, splits, best,
                                sk_wpc ? " (stream-K chosen instead)" : "");
     }
-    if (S.force_tile >= 0 && S.force_tile < kNumTiles) tile = S.force_tile;
-    if (S.force_splitk > 0 && !ep.bias_rows) splits = S.force_splitk; // the slice reduction applies the bias by column only
-    int streamk = S.force_streamk > 0 ? S.force_streamk : 0;
+    if (S.force_tile >= 0 && S.force_tile < kNumTiles && !(ep.colsum && (S.force_tile < 2 || kTiles[S.force_tile].bm < M))) tile = S.force_tile;
+    if (S.force_splitk > 0 && !ep.bias_rows && !ep.colsum) splits = S.force_splitk; // the slice reduction applies the bias by column only
+    int streamk = S.force_streamk > 0 && !ep.colsum ? S.force_streamk : 0;
     if (S.force_streamk < 0 && sk_wpc > 0 && S.force_tile < 0 && S.force_splitk <= 0) { streamk = sk_wpc; tile = sk_tile; }
     if (streamk > 0 && tile <= 3 && am != KMAJOR_GEN && bm != KMAJOR_GEN && (!ep.gather_row || tile >= 2)) {
         const int bmt = kTiles[tile].bm, bnt = kTiles[tile].bn;
@@ -1622,8 +1626,11 @@ static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int6
         const int64_t I = m->dims[l], O = m->dims[l + 1];
         const float* in = l == 0 ? x : m->act[l - 1];
         const float* gl = m->grad[l];
+        const bool from_gemm = B <= 128; // hidden layers: summed in the store of the GEMM that produced this gradient (below)
         if (one_block && l == L - 1) {
             // done by the cross-entropy launch
+        } else if (from_gemm && l < L - 1) {
+            // done by the dX product of layer l+1
         } else if (B * O >= (int64_t)1 << 18) { // large: stream the gradient once at HBM rate
             if (int rc = matvec_dispatch(gl, 1, O, S.one, 0, m->db[l], O, B, bd, 1, 0)) return rc;
         } else {
@@ -1634,6 +1641,7 @@ static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int6
         if (l > 0) { // dX = g . W^T(view)  (tenmo/matmul.mojo:36-38); the network input needs no gradient (:34)
             Epilogue ep; // ReLU backward in the GEMM store: zero where the forward activation was not positive
             ep.mask = m->act[l - 1];
+            if (from_gemm) ep.colsum = m->db[l - 1]; // bias gradient of layer l-1 = column sums of its (masked) gradient
             if (int rc = gemm_dispatch(gl, O, 1, m->W[l], 1, O, m->grad[l - 1], B, I, O, bd, 1, 0, ep)) return rc;
         }
     }

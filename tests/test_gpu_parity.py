@@ -689,6 +689,18 @@ def test_mlp_loss_curve_tracks_cpu(T, oracle):
     for l in range(2):
         (dWg, dbg), (dWc, dbc) = gpu.grads(l), cpu.grads(l)
         assert rel_fro(dWg, dWc) <= 1e-4 and rel_fro(dbg, dbc) <= 1e-4
+    # batches up to 128 rows: the hidden layers' bias gradients come out of the store of the GEMM that produces their
+    # gradient (ragged widths, 65..128 rows take the 128-row tile)
+    for batch, dims in ((100, [50, 70, 33, 6]), (128, [20, 200, 64, 130, 4]), (7, [9, 5, 3])):
+        Ws, bs = R.xavier_mlp(dims, seed + 2)
+        gpu, cpu = MLP(dims, Ws, bs, batch), oracle.MLP(dims, Ws, bs, batch)
+        for step in range(4):
+            x = rs.standard_normal((batch, dims[0])).astype(np.float32)
+            y = rs.integers(0, dims[-1], batch).astype(np.int32)
+            assert abs(gpu.step(x, y, 0.05) - cpu.step(x, y, 0.05)) <= 1e-4, (batch, step)
+        for l in range(len(dims) - 1):
+            (dWg, dbg), (dWc, dbc) = gpu.grads(l), cpu.grads(l)
+            assert rel_fro(dWg, dWc) <= 1e-4 and rel_fro(dbg, dbc) <= 1e-4, (batch, l)
     # cross-entropy vector of the reference: uniform logits -> -log(1/3)
     m = MLP([2, 3], [np.zeros((2, 3), np.float32)], [np.ones(3, np.float32)], 2)
     assert abs(m.step(np.ones((2, 2), np.float32), np.asarray([0, 1], np.int32), 0.0) - 1.0986122886681098) < 1e-6
