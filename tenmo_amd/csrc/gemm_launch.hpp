@@ -14,6 +14,10 @@ bool launch_gemm_64x64(const GemmArgs& g, dim3 grid, int amode, int bmode, hipSt
 bool launch_gemm_128x64(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream);
 bool launch_gemm_64x128(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream);
 
+// Two products with the 64x64 tile in one launch (count0 / count1 workgroups).  false: no variant for these operand modes.
+bool launch_gemm_pair_64x64(const GemmArgs& g0, const GemmArgs& g1, unsigned count0, unsigned count1, int amode0, int bmode0, int amode1, int bmode1,
+                            hipStream_t stream);
+
 // Stream-K: `wgs` persistent workgroups, then the fix-up over `tiles` tiles in `fix_parts` parts
 // each (0: no tile is shared, no fix-up).  Vector operand modes only.
 bool launch_streamk_256x128(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);

@@ -862,19 +862,10 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
     }
 }
 
-// One workgroup per tile (and per K slice when g.k_splits > 1).
+// One workgroup per tile (and per K slice when g.k_splits > 1): tile number `pid` (batches included) and K slice `slice`.
 template <int BM, int BN, int AMODE, int BMODE>
-__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmArgs g) {
-    constexpr int STAGE_FLOATS = (BM + BN) * GEMM_BK;
-    constexpr bool DIRECT = (AMODE != KMAJOR_GEN) && (BMODE != KMAJOR_GEN);
-    // three separate objects: the compiler can then tell that a direct load into one stage does
-    // not alias the operand fetch from another
-    __shared__ __attribute__((aligned(1024))) float stage0[STAGE_FLOATS];
-    __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
-    __shared__ __attribute__((aligned(1024))) float stage2[DIRECT ? STAGE_FLOATS : 4];
-
+__device__ __forceinline__ void gemm_workgroup(const GemmArgs& g, float* stage0, float* stage1, float* stage2, uint32_t pid, uint32_t slice) {
     const uint32_t tiles = (uint32_t)g.tiles_m * (uint32_t)g.tiles_n; // the grid, batches included, is below 2^31
-    const uint32_t pid = blockIdx.x;
     const uint32_t batch32 = pid / tiles;
     const int64_t batch = batch32;
     int64_t tile_m, tile_n;
@@ -884,15 +875,40 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     TileDest dst;
     dst.ld = g.N; dst.row0 = 0; dst.col0 = 0;
     if (g.k_splits > 1) { // partial sums of this K slice; the slice reduction finishes them
-        k_begin = (int64_t)blockIdx.y * g.k_per_split;
+        k_begin = (int64_t)slice * g.k_per_split;
         k_end = min(g.K, k_begin + g.k_per_split);
-        dst.base = g.partial + ((int64_t)blockIdx.y * g.batch_count + batch) * g.M * g.N;
+        dst.base = g.partial + ((int64_t)slice * g.batch_count + batch) * g.M * g.N;
         dst.accumulate = false; dst.fused = false;
     } else {
         dst.base = g.C + batch * g.M * g.N;
         dst.accumulate = g.accumulate != 0; dst.fused = true;
     }
     gemm_tile<BM, BN, AMODE, BMODE>(g, stage0, stage1, stage2, batch, tile_m, tile_n, k_begin, k_end, dst);
+}
+
+template <int BM, int BN, int AMODE, int BMODE>
+__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmArgs g) {
+    constexpr int STAGE_FLOATS = (BM + BN) * GEMM_BK;
+    constexpr bool DIRECT = (AMODE != KMAJOR_GEN) && (BMODE != KMAJOR_GEN);
+    // three separate objects: the compiler can then tell that a direct load into one stage does
+    // not alias the operand fetch from another
+    __shared__ __attribute__((aligned(1024))) float stage0[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage2[DIRECT ? STAGE_FLOATS : 4];
+    gemm_workgroup<BM, BN, AMODE, BMODE>(g, stage0, stage1, stage2, blockIdx.x, blockIdx.y);
+}
+
+// Two independent products in one launch (both with one K slice and vector operand forms): workgroups below `first_count`
+// work on g0, the others on g1.  For small products that a dependent-launch latency of about 5 us each would dominate
+// (the weight gradient of a layer and the gradient passed to the layer below both consume the same upstream gradient).
+template <int BM, int BN, int AMODE0, int BMODE0, int AMODE1, int BMODE1>
+__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_pair_kernel(const GemmArgs g0, const GemmArgs g1, uint32_t first_count) {
+    constexpr int STAGE_FLOATS = (BM + BN) * GEMM_BK;
+    __shared__ __attribute__((aligned(1024))) float stage0[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage2[STAGE_FLOATS];
+    if (blockIdx.x < first_count) gemm_workgroup<BM, BN, AMODE0, BMODE0>(g0, stage0, stage1, stage2, blockIdx.x, 0);
+    else gemm_workgroup<BM, BN, AMODE1, BMODE1>(g1, stage0, stage1, stage2, blockIdx.x - first_count, 0);
 }
 
 // ---- stream-K --------------------------------------------------------------------------------

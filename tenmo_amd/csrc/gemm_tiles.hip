@@ -26,6 +26,16 @@ bool TENMO_NAME(launch_gemm_, TENMO_TILE_BM, TENMO_TILE_BN)(const GemmArgs& g, d
 #undef TENMO_CASE
     return false;
 }
+#if TENMO_TILE_BM == 64 && TENMO_TILE_BN == 64
+bool launch_gemm_pair_64x64(const GemmArgs& g0, const GemmArgs& g1, unsigned count0, unsigned count1, int amode0, int bmode0, int amode1, int bmode1,
+                            hipStream_t stream) {
+    // the one combination in use: X^T(view).G beside G.W^T(view)
+    if (amode0 != MNMAJOR_VEC || bmode0 != MNMAJOR_VEC || amode1 != KMAJOR_VEC || bmode1 != KMAJOR_VEC) return false;
+    hipLaunchKernelGGL((gemm_pair_kernel<64, 64, MNMAJOR_VEC, MNMAJOR_VEC, KMAJOR_VEC, KMAJOR_VEC>), dim3(count0 + count1), dim3(GEMM_THREADS), 0, stream,
+                       g0, g1, count0);
+    return true;
+}
+#endif
 #else
 bool TENMO_NAME(launch_streamk_, TENMO_TILE_BM, TENMO_TILE_BN)(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles,
                                                               unsigned fix_parts, int amode, int bmode, hipStream_t stream) {

@@ -519,6 +519,35 @@ int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* 
     return 0;
 }
 
+// Two small products in ONE launch of the 64x64 tile (no batches, one K slice each); `ep1` belongs to the second.
+// Returns 1 when the pair form does not apply (sizes, operand forms): the caller then launches them one by one.
+int gemm_pair_dispatch(const float* A0, int64_t a0_rs, int64_t a0_cs, const float* B0, int64_t b0_rs, int64_t b0_cs, float* C0, int64_t M0, int64_t N0, int64_t K0,
+                       const float* A1, int64_t a1_rs, int64_t a1_cs, const float* B1, int64_t b1_rs, int64_t b1_cs, float* C1, int64_t M1, int64_t N1, int64_t K1,
+                       const Epilogue& ep1) {
+    if (S.force_tile >= 0 || S.force_splitk > 0 || S.force_streamk > 0) return 1; // overrides apply to single launches
+    if (M0 < 1 || N0 < 1 || K0 < 1 || M1 < 1 || N1 < 1 || K1 < 1 || ep1.gather_row || ep1.bias_rows) return 1;
+    if (ep1.colsum && M1 > 64) return 1;
+    auto fill = [](GemmArgs& g, const float* A, int64_t a_rs, int64_t a_cs, const float* B, int64_t b_rs, int64_t b_cs, float* C, int64_t M, int64_t N, int64_t K) {
+        g.A = A; g.B = B; g.C = C;
+        g.a_rs = a_rs; g.a_cs = a_cs; g.b_rs = b_rs; g.b_cs = b_cs;
+        g.M = M; g.N = N; g.K = K;
+        g.tiles_m = (int32_t)((M + 63) / 64); g.tiles_n = (int32_t)((N + 63) / 64);
+        g.k_splits = 1; g.k_per_split = K; g.batch_count = 1;
+        g.batch.rank = 0;
+        for (int d = 0; d < MAX_BATCH_RANK; ++d) g.batch.shape[d] = 1;
+    };
+    GemmArgs g0{}, g1{};
+    fill(g0, A0, a0_rs, a0_cs, B0, b0_rs, b0_cs, C0, M0, N0, K0);
+    fill(g1, A1, a1_rs, a1_cs, B1, b1_rs, b1_cs, C1, M1, N1, K1);
+    g1.bias = ep1.bias; g1.mask = ep1.mask; g1.relu = ep1.relu; g1.colsum = ep1.colsum;
+    const int64_t c0 = (int64_t)g0.tiles_m * g0.tiles_n, c1 = (int64_t)g1.tiles_m * g1.tiles_n;
+    // small products only: beyond a few workgroups per CU each product fills the chip by itself and wants its own tile choice
+    if (c0 + c1 > (int64_t)S.cus * 2 || K0 > 4096 || K1 > 4096) return 1;
+    const bool ok = launch_gemm_pair_64x64(g0, g1, (unsigned)c0, (unsigned)c1, operand_mode(a0_rs, a0_cs, M0, K0), operand_mode(b0_cs, b0_rs, N0, K0),
+                                           operand_mode(a1_rs, a1_cs, M1, K1), operand_mode(b1_cs, b1_rs, N1, K1), S.stream);
+    return ok ? 0 : 1;
+}
+
 // skinny GEMM: M <= 8 rows against a row-major B — the matrix is streamed once, like vm
 int skinny_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, int64_t b_rs, float* C,
                     int64_t M, int64_t N, int64_t K, const BatchDesc& bd, int64_t batch_count, int accumulate) {
@@ -1637,12 +1666,20 @@ static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int6
             hipLaunchKernelGGL(column_sum_kernel, dim3((unsigned)((O + 63) / 64)), dim3(64), 0, S.stream, gl, B, O, m->db[l]);
         }
         // dW = in^T(view) . g        (tenmo/matmul.mojo:46-48)
-        if (int rc = gemm_dispatch(in, 1, I, gl, O, 1, m->dW[l], I, O, B, bd, 1, 0)) return rc;
-        if (l > 0) { // dX = g . W^T(view)  (tenmo/matmul.mojo:36-38); the network input needs no gradient (:34)
-            Epilogue ep; // ReLU backward in the GEMM store: zero where the forward activation was not positive
+        // dX = g . W^T(view)         (tenmo/matmul.mojo:36-38); the network input needs no gradient (:34)
+        Epilogue ep; // ReLU backward in the GEMM store: zero where the forward activation was not positive
+        if (l > 0) {
             ep.mask = m->act[l - 1];
             if (from_gemm) ep.colsum = m->db[l - 1]; // bias gradient of layer l-1 = column sums of its (masked) gradient
-            if (int rc = gemm_dispatch(gl, O, 1, m->W[l], 1, O, m->grad[l - 1], B, I, O, bd, 1, 0, ep)) return rc;
+        }
+        // both consume the same upstream gradient and are independent: one launch for the two when they are small
+        int paired = 1;
+        if (l > 0) paired = gemm_pair_dispatch(in, 1, I, gl, O, 1, m->dW[l], I, O, B, gl, O, 1, m->W[l], 1, O, m->grad[l - 1], B, I, O, ep);
+        if (paired < 0) return paired;
+        if (paired != 0) {
+            if (int rc = gemm_dispatch(in, 1, I, gl, O, 1, m->dW[l], I, O, B, bd, 1, 0)) return rc;
+            if (l > 0)
+                if (int rc = gemm_dispatch(gl, O, 1, m->W[l], 1, O, m->grad[l - 1], B, I, O, bd, 1, 0, ep)) return rc;
         }
     }
     // every parameter tensor in one launch
