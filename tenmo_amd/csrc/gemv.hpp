@@ -428,6 +428,31 @@ __global__ __launch_bounds__(DOT_THREADS) void dot_partial_kernel(const float* _
     if (threadIdx.x == 0) partial[blockIdx.x] = s;
 }
 
+// Unit strides: 16-byte streaming loads, U groups of each vector in flight per thread, every workgroup side by side in one
+// window that moves through the arrays (the element-at-a-time kernel above reaches 4 TB/s on 2 GB; this form 6.5+).
+// The n % 4 last elements are added by the first threads of workgroup 0.  Fixed partition: the result is deterministic.
+template <int U>
+__global__ __launch_bounds__(DOT_THREADS) void dot_partial_vec_kernel(const float* __restrict a, const float* __restrict b, int64_t n, float* __restrict partial) {
+    const int64_t n4 = n / 4, stride = (int64_t)gridDim.x * DOT_THREADS;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    int64_t i = (int64_t)blockIdx.x * DOT_THREADS + threadIdx.x;
+    for (; i + (U - 1) * stride < n4; i += U * stride) {
+        f32x4 x[U], y[U];
+#pragma unroll
+        for (int u = 0; u < U; ++u) x[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(a) + i + u * stride);
+#pragma unroll
+        for (int u = 0; u < U; ++u) y[u] = __builtin_nontemporal_load(reinterpret_cast<const f32x4_u*>(b) + i + u * stride);
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int u = 0; u < U; ++u) acc += x[u] * y[u];
+    }
+    for (; i < n4; i += stride) acc += reinterpret_cast<const f32x4_u*>(a)[i] * reinterpret_cast<const f32x4_u*>(b)[i];
+    float s = (acc.x + acc.y) + (acc.z + acc.w);
+    if (blockIdx.x == 0 && 4 * n4 + threadIdx.x < n) s = fmaf(a[4 * n4 + threadIdx.x], b[4 * n4 + threadIdx.x], s);
+    s = block_sum(s);
+    if (threadIdx.x == 0) partial[blockIdx.x] = s;
+}
+
 __global__ __launch_bounds__(DOT_THREADS) void dot_final_kernel(const float* __restrict partial, int nparts, float* __restrict out) {
     float acc = 0.f;
     for (int i = threadIdx.x; i < nparts; i += DOT_THREADS) acc += partial[i];

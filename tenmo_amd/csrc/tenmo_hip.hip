@@ -1274,10 +1274,12 @@ int tenmo_hip_dot_f32(const float* a, int64_t a_off, int64_t a_s, const float* b
     if (n < 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_dot_f32: negative length");
     if (int rc = need(out, true, "tenmo_hip_dot_f32", "result pointer")) return rc;
     if ((!a || !b) && n > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_dot_f32: null operand");
-    const int parts = (int)std::max<int64_t>(1, std::min<int64_t>((n + DOT_THREADS * 8 - 1) / (DOT_THREADS * 8), 1024));
+    const bool vec = a_s == 1 && b_s == 1 && n >= 4096; // 16-byte loads (alignment of 4 bytes is enough for them)
+    const int parts = (int)std::max<int64_t>(1, std::min<int64_t>((n + DOT_THREADS * 8 - 1) / (DOT_THREADS * 8), vec ? (int64_t)S.cus * 8 : 1024));
     float* ws;
     if (int rc = workspace(parts * sizeof(float), &ws)) return rc;
-    hipLaunchKernelGGL(dot_partial_kernel, dim3(parts), dim3(DOT_THREADS), 0, S.stream, a + a_off, a_s, b + b_off, b_s, n, ws);
+    if (vec) hipLaunchKernelGGL(dot_partial_vec_kernel<4>, dim3(parts), dim3(DOT_THREADS), 0, S.stream, a + a_off, b + b_off, n, ws);
+    else hipLaunchKernelGGL(dot_partial_kernel, dim3(parts), dim3(DOT_THREADS), 0, S.stream, a + a_off, a_s, b + b_off, b_s, n, ws);
     hipLaunchKernelGGL(dot_final_kernel, dim3(1), dim3(DOT_THREADS), 0, S.stream, ws, parts, out);
     return finish(sync);
 }

@@ -558,6 +558,16 @@ def test_dot(T, oracle):
         got = float(T.Tensor.from_numpy(a).matmul(T.Tensor.from_numpy(b), track_grad=False).to_numpy())
         ref = float(np.dot(a.astype(np.float64), b.astype(np.float64)))
         assert abs(got - ref) <= 1e-5 * max(1.0, np.linalg.norm(a) * np.linalg.norm(b)), n
+    # the streaming form (unit strides, 16-byte loads): every alignment of the two vectors, lengths with a remainder, strides
+    import torch
+    L = T.lib.load()
+    big_a, big_b = rng.standard_normal(2_100_000, dtype=np.float32), rng.standard_normal(2_100_000, dtype=np.float32)
+    Ad, Bd, out = torch.from_numpy(big_a).cuda(), torch.from_numpy(big_b).cuda(), torch.zeros(1, device="cuda")
+    for (ao, bo, n, sa, sb) in [(0, 0, 2_097_152, 1, 1), (1, 0, 2_000_003, 1, 1), (2, 3, 1_999_998, 1, 1), (3, 1, 4097, 1, 1), (0, 0, 4096, 1, 1),
+                                (5, 7, 500_001, 2, 1), (0, 1, 300_000, 3, 2)]:
+        T.lib.check(L.tenmo_hip_dot_f32(Ad.data_ptr(), ao, sa, Bd.data_ptr(), bo, sb, n, out.data_ptr(), 1))
+        av, bv = big_a[ao:ao + n * sa:sa].astype(np.float64), big_b[bo:bo + n * sb:sb].astype(np.float64)
+        assert abs(float(out) - float(av @ bv)) <= 1e-5 * np.linalg.norm(av) * np.linalg.norm(bv), (ao, bo, n, sa, sb)
     a = np.arange(1, 8, dtype=np.float32)
     A, B = T.Tensor.from_numpy(a, True), T.Tensor.from_numpy(2 * a, True)
     out = A.dot(B)
