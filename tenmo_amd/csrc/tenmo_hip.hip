@@ -297,7 +297,10 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
                 const int64_t a_pitch = am == KMAJOR_VEC ? a_rs : a_cs, b_pitch = bm == KMAJOR_VEC ? b_cs : b_rs;
                 if (wpc == 1 && ((M > 1 && K > 1 && a_pitch % 4 != 0) || (N > 1 && K > 1 && b_pitch % 4 != 0))) continue;
                 const double m_us = (kTiles[t].bm / 64) * (kTiles[t].bn / 64) * 8 * 64 / 2400.0;
-                const double step_us = wpc * m_us / kEff[t]; // one K step of every workgroup of a CU
+                // one K step of every workgroup of a CU.  The 256x128 stream-K kernel spills a few registers: up to about a
+                // thousand of its tiles the 128x128 one at two per CU is 2-4 % ahead (3072^3 .. 5120^3), beyond that 256x128
+                // is level or ahead (6144^3 .. 10240^3: the smaller tile's operand traffic starts to count)
+                const double step_us = wpc * m_us / (t == 0 && tiles <= 1024 ? kEff[1] : kEff[t]);
                 const double pieces = (double)std::min(2 * wgs, 2 * shared);
                 const double fix = 2.0 * pieces * kTiles[t].bm * kTiles[t].bn * 4.0 / 5.0e6;
                 const double est = whole_rounds * (nks * step_us + 1.5) + (double)shared * nks / wgs * step_us + fix + 10.0;
