@@ -24,6 +24,19 @@ def numpy_view(t):
     return np.lib.stride_tricks.as_strided(st[t.get("offset", 0):], tuple(t["shape"]), tuple(4 * s for s in strides_of(t))).copy()
 
 
+def scatter_to_storage(t, grad):
+    """Gradient of a view scattered (added) onto the storage behind it: what the reference's view backward
+    leaves in the base tensor's gradbox.  Overlapping strides add up."""
+    st = np.zeros(len(t["storage"]), np.float64)
+    idx = np.full(tuple(t["shape"]), t.get("offset", 0), np.int64)
+    for ax, (n, s) in enumerate(zip(t["shape"], strides_of(t))):
+        shape = [1] * len(t["shape"])
+        shape[ax] = n
+        idx = idx + (np.arange(n, dtype=np.int64) * s).reshape(shape)
+    np.add.at(st, idx.ravel(), np.asarray(grad, np.float64).ravel())
+    return st
+
+
 def rel_fro(x, ref):
     x = np.asarray(x, np.float64)
     ref = np.asarray(ref, np.float64)

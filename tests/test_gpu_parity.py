@@ -9,7 +9,7 @@ import ctypes as C
 import numpy as np
 import pytest
 
-from helpers import RTOL_FRO, ce_reference64, numpy_view, ref_matmul64, rel_fro, storage_of, strides_of
+from helpers import RTOL_FRO, ce_reference64, numpy_view, ref_matmul64, rel_fro, scatter_to_storage, storage_of, strides_of
 
 pytestmark = pytest.mark.gpu
 
@@ -61,12 +61,19 @@ def test_golden_forward_and_backward(T, golden):
         out = A.matmul(B, mode=mode[c["op"]])
         if "expect" in c:
             np.testing.assert_allclose(out.to_numpy(), np.asarray(c["expect"], np.float32), rtol=1e-5, atol=1e-8, err_msg=c["name"])
-        if "grad_A" in c or "grad_B" in c:
+        if "expect_shape" in c:
+            assert list(out.shape()) == c["expect_shape"], c["name"]
+        if any(k in c for k in ("grad_A", "grad_B", "base_grad_A", "base_grad_B")):
             out.backward(1.0)  # loss = out.sum(); loss.backward()
             if "grad_A" in c:
                 np.testing.assert_allclose(A.grad(), np.asarray(c["grad_A"], np.float32), rtol=1e-5, err_msg=c["name"] + " grad_A")
             if "grad_B" in c:
                 np.testing.assert_allclose(B.grad(), np.asarray(c["grad_B"], np.float32), rtol=1e-5, err_msg=c["name"] + " grad_B")
+            # gradients asserted on the tensor behind a view: the view-shaped gradient scattered onto its storage
+            if "base_grad_A" in c:
+                np.testing.assert_allclose(scatter_to_storage(c["A"], A.grad()), c["base_grad_A"], rtol=1e-5, err_msg=c["name"] + " base_grad_A")
+            if "base_grad_B" in c:
+                np.testing.assert_allclose(scatter_to_storage(c["B"], B.grad()), c["base_grad_B"], rtol=1e-5, err_msg=c["name"] + " base_grad_B")
 
 
 def test_closed_forms(T, golden):

@@ -3,7 +3,7 @@ vectors, fp64 brute force, closed forms and algebraic invariants.  Runs without 
 import numpy as np
 import pytest
 
-from helpers import ce_reference64, numpy_view, ref_matmul64, rel_fro, storage_of, strides_of
+from helpers import ce_reference64, numpy_view, ref_matmul64, rel_fro, scatter_to_storage, storage_of, strides_of
 
 
 def _view(O, t):
@@ -24,12 +24,14 @@ def test_golden_forward(golden, oracle):
             got = O.dot(A, B)
         if "expect" in c:
             np.testing.assert_allclose(got, np.asarray(c["expect"], np.float32), rtol=1e-5, atol=1e-8, err_msg=c["name"])
+        if "expect_shape" in c:
+            assert list(np.shape(got)) == c["expect_shape"], c["name"]
 
 
 def test_golden_backward(golden, oracle):
     O = oracle
     for c in golden["cases"]:
-        if "grad_A" not in c and "grad_B" not in c:
+        if not any(k in c for k in ("grad_A", "grad_B", "base_grad_A", "base_grad_B")):
             continue
         A, B = _view(O, c["A"]), _view(O, c["B"])
         if c["op"] == "mm":
@@ -43,6 +45,11 @@ def test_golden_backward(golden, oracle):
             np.testing.assert_allclose(gA, np.asarray(c["grad_A"], np.float32), rtol=1e-5, err_msg=c["name"] + " grad_A")
         if "grad_B" in c:
             np.testing.assert_allclose(gB, np.asarray(c["grad_B"], np.float32), rtol=1e-5, err_msg=c["name"] + " grad_B")
+        # gradients asserted on the tensor behind a view: the view-shaped gradient scattered onto its storage
+        if "base_grad_A" in c:
+            np.testing.assert_allclose(scatter_to_storage(c["A"], gA), c["base_grad_A"], rtol=1e-5, err_msg=c["name"] + " base_grad_A")
+        if "base_grad_B" in c:
+            np.testing.assert_allclose(scatter_to_storage(c["B"], gB), c["base_grad_B"], rtol=1e-5, err_msg=c["name"] + " base_grad_B")
 
 
 @pytest.mark.parametrize("width", [0, 16, 8, 1])
