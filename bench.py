@@ -43,6 +43,8 @@ def main() -> int:
     ap.add_argument("--no-extra", action="store_true", help="skip the mv/vm and MLP-step side measurements")
     ap.add_argument("--adjacent", action="store_true",
                     help="also time the adjacent operators (cross-entropy, SGD step, convolution) into `extra`; off by default")
+    ap.add_argument("--attention", action="store_true",
+                    help="also time the attention-shaped batched products (Q.K^T, P.V, P^T.dO, Q^T.dS at [8,12,1024,64]) into `extra`; off by default")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy, the known-size kernel against which FETCH_SIZE/WRITE_SIZE are scaled")
     args = ap.parse_args()
@@ -136,6 +138,8 @@ def main() -> int:
         extra.update(side_measurements(L, _lib, torch, np))
     if args.adjacent:
         extra.update(adjacent_operators(L, _lib, torch))
+    if args.attention:
+        extra.update(attention_products(L, _lib, torch))
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_gemm_baseline(A, B, S, np)
         if not args.no_extra:
@@ -176,6 +180,40 @@ def side_measurements(L, _lib, torch, np):
         res["%s_16384_us" % nm] = round(ms * 1e3, 2)
         res["%s_16384_gbps" % nm] = round(gbps, 1)
         res["%s_16384_frac_hbm_peak" % nm] = round(gbps / PEAK_HBM_GBPS, 4)
+    return res
+
+
+def attention_products(L, _lib, torch):
+    """The broadcast-batched products of attention at Q, K, V = [8, 12, 1024, 64]: S = Q.K^T (K as a transposed view),
+    O = P.V, dV = P^T.dO and Q^T.dS, each 12.88 GFLOP and 453 MB of algorithmic traffic; time, TFLOP/s and the
+    relative Frobenius error of one batch against fp64."""
+    Bn, H, T, D = 8, 12, 1024, 64
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(64)
+    Q, K, V = (torch.randn((Bn, H, T, D), generator=gen, device="cuda", dtype=torch.float32) for _ in range(3))
+    S = torch.empty((Bn, H, T, T), device="cuda", dtype=torch.float32)
+    O = torch.empty((Bn, H, T, D), device="cuda", dtype=torch.float32)
+    O2 = torch.empty((Bn, H, D, T), device="cuda", dtype=torch.float32)
+    bs, st, pst = (Bn, H), (H * T * D, T * D), (H * T * T, T * T)
+
+    def gemm(A, B, Cc, M, N, Kk, a_rs, a_cs, b_rs, b_cs, ab, bb):
+        _lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, a_rs, a_cs, B.data_ptr(), 0, b_rs, b_cs, Cc.data_ptr(), M, N, Kk,
+                                        2, _lib.i64(bs), _lib.i64(ab), _lib.i64(bb), 0, 0))
+
+    cases = (
+        ("qkt", lambda: gemm(Q, K, S, T, T, D, D, 1, 1, D, st, st), lambda: (S[1, 2], Q[1, 2].double() @ K[1, 2].double().T)),
+        ("pv", lambda: gemm(S, V, O, T, D, T, T, 1, D, 1, pst, st), lambda: (O[1, 2], S[1, 2].double() @ V[1, 2].double())),
+        ("ptdo", lambda: gemm(S, V, O, T, D, T, 1, T, D, 1, pst, st), lambda: (O[1, 2], S[1, 2].double().T @ V[1, 2].double())),
+        ("qtds", lambda: gemm(Q, S, O2, D, T, T, 1, D, T, 1, st, pst), lambda: (O2[1, 2], Q[1, 2].double().T @ S[1, 2].double())),
+    )
+    flop = 96 * 2.0 * T * T * D
+    res = {}
+    for nm, fn, check in cases:
+        ms = hip_time(L, _lib, fn, 20)
+        got, ref = check()
+        res["attn_%s_us" % nm] = round(ms * 1e3, 1)
+        res["attn_%s_tflops" % nm] = round(flop / (ms * 1e-3) / 1e12, 1)
+        res["attn_%s_rel_err" % nm] = float((got.double() - ref).norm() / ref.norm())
     return res
 
 

@@ -47,12 +47,13 @@ def _run(cmd):
 
 
 def build(verbose: bool = False) -> str:
-    jobs = min(len(TILES) + 1, max(1, int(os.environ.get("MAX_JOBS", os.cpu_count() or 1))))
+    jobs = min(len(TILES) + 2, max(1, int(os.environ.get("MAX_JOBS", os.cpu_count() or 1))))
     with tempfile.TemporaryDirectory(prefix="tenmo_hip_build_") as tmp:
         units = [([os.path.join(CSRC, "tenmo_hip.hip")], os.path.join(tmp, "tenmo_hip.o"))]
         for bm, bn, sk in TILES:
             units.append(([f"-DTENMO_TILE_BM={bm}", f"-DTENMO_TILE_BN={bn}", f"-DTENMO_TILE_STREAMK={sk}",
                            os.path.join(CSRC, "gemm_tiles.hip")], os.path.join(tmp, f"gemm_{bm}x{bn}_{sk}.o")))
+        units.append(([os.path.join(CSRC, "gemm_smallk.hip")], os.path.join(tmp, "gemm_smallk.o")))
         cmds = [[HIPCC] + FLAGS + ["-c"] + src + ["-o", obj] for src, obj in units]
         if verbose:
             for c in cmds:

@@ -76,6 +76,7 @@ struct State {
     int force_splitk = -1;
     int force_conv_phases = -1; // strided image gradient phase by phase: -1 automatic (large layers), 0 never, 1 always
     int force_streamk = -1;    // -1 automatic, 0 never, n > 0: stream-K with n workgroups per CU
+    int force_smallk = -1;     // -1 automatic, 0 never, 1: the short-reduction kernel wherever it can run
     int verbose = 0;
     int cols_waves_per_cu = 2; // target workgroups per CU of the column-streaming kernels (long K slices stream best)
 };
@@ -319,6 +320,23 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         if (S.verbose) fprintf(stderr, "tenmo_hip gemm M=%lld N=%lld K=%lld batch=%lld -> tile %dx%d, %d K slice(s), est %.1f us%s\n",
                                (long long)M, (long long)N, (long long)K, (long long)batch_count, kTiles[tile].bm, kTiles[tile].bn, splits, best,
                                sk_wpc ? " (stream-K chosen instead)" : "");
+    }
+    // Short reduction with both operands K-major and a plain (or accumulating) store: the persistent whole-K-in-LDS
+    // kernel, which loads its next tile before it stores this one (gemm_smallk.hip).  Automatic where the launch is
+    // store-bound as above and every workgroup gets several tiles.
+    {
+        const int64_t tm = (M + 63) / 64, tn = (N + 63) / 64, tiles64 = tm * tn * batch_count;
+        const bool can = am == KMAJOR_VEC && bm == KMAJOR_VEC && a_cs == 1 && b_rs == 1 && K % GEMM_BK == 0 && K <= 64 && !ep.any() && !ep.gather_row &&
+                         !ep.colsum && a_rs >= 0 && a_rs <= (int64_t(1) << 21) && b_cs >= 0 && b_cs <= (int64_t(1) << 21) && N < (int64_t(1) << 29) &&
+                         tiles64 <= 0x7fffffffLL;
+        const bool want = S.force_smallk > 0 || (S.force_smallk < 0 && S.force_tile < 0 && S.force_splitk <= 0 && S.force_streamk <= 0 &&
+                                                  splits == 1 && sk_wpc == 0 && tiles64 >= 2048);
+        if (can && want) {
+            g.tiles_m = (int32_t)tm; g.tiles_n = (int32_t)tn;
+            g.k_splits = 1; g.k_per_split = K; g.partial = nullptr;
+            if (S.verbose) fprintf(stderr, "tenmo_hip gemm: short-reduction kernel, %lld tiles of 64x64\n", (long long)tiles64);
+            if (launch_gemm_smallk_64x64(g, (unsigned)S.cus, (unsigned)tiles64, S.force_smallk != 2, S.stream)) return 0;
+        }
     }
     if (S.force_tile >= 0 && S.force_tile < kNumTiles && !(ep.colsum && (S.force_tile < 2 || kTiles[S.force_tile].bm < M))) tile = S.force_tile;
     if (S.force_splitk > 0 && !ep.bias_rows && !ep.colsum) splits = S.force_splitk; // the slice reduction applies the bias by column only
@@ -813,6 +831,7 @@ int tenmo_hip_init(int device_id) {
     S.force_tile = env_int("TENMO_HIP_GEMM_TILE", -1);
     S.force_splitk = env_int("TENMO_HIP_GEMM_SPLITK", -1);
     S.force_streamk = env_int("TENMO_HIP_GEMM_STREAMK", -1);
+    S.force_smallk = env_int("TENMO_HIP_GEMM_SMALLK", -1);
     S.verbose = env_int("TENMO_HIP_VERBOSE", 0);
     S.ready = true;
     return 0;
@@ -862,6 +881,7 @@ int tenmo_hip_set_tuning(const char* name, int value) {
     if (!strcmp(name, "gemm_tile")) { S.force_tile = value; return 0; }
     if (!strcmp(name, "gemm_splitk")) { S.force_splitk = value; return 0; }
     if (!strcmp(name, "gemm_streamk")) { S.force_streamk = value; return 0; }
+    if (!strcmp(name, "gemm_smallk")) { S.force_smallk = value; return 0; }
     if (!strcmp(name, "conv_phases")) { S.force_conv_phases = value; return 0; }
     if (!strcmp(name, "cols_wg_per_cu")) { S.cols_waves_per_cu = value > 0 ? value : 2; return 0; }
     return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: unknown knob '%s'", name);

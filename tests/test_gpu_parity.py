@@ -140,6 +140,36 @@ def test_ragged_tiles_and_k_slices(T, oracle, tile):
         L.tenmo_hip_set_tuning(b"gemm_splitk", -1)
 
 
+@pytest.mark.parametrize("smallk", [1, 0])
+def test_short_reduction_kernel(T, smallk):
+    """C (+)= A . B^T(view) with K a multiple of 16 up to 64 through the kernel-level entry point: the persistent
+    short-reduction kernel forced on (and, as the control, off), over whole and ragged tiles, batches, a
+    broadcast B, fewer tiles than workgroups and more, with and without accumulation; against fp64."""
+    import torch
+    L, lib = T.lib.load(), T.lib
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(23)
+    cases = [((), 64, 64, 16, 0), ((), 128, 192, 64, 0), ((3,), 100, 130, 32, 0), ((2, 3), 257, 65, 64, 1), ((2,), 333, 777, 48, 1),
+             ((), 1000, 1000, 48, 0), ((7,), 1, 1, 16, 0), ((2,), 512, 512, 64, 1), ((9,), 1024, 1024, 64, 0), ((40,), 320, 192, 32, 1),
+             ((3, 2), 640, 320, 96, 0)]  # (the last one has K > 64: the ordinary kernel either way)
+    try:
+        L.tenmo_hip_set_tuning(b"gemm_smallk", smallk)
+        for bshape, M, N, K, acc in cases:
+            for bcast in (False, True):
+                A = torch.randn((*bshape, M, K), generator=gen, device="cuda")
+                Bt = torch.randn((*((1,) * len(bshape) if bcast else bshape), N, K), generator=gen, device="cuda")
+                Cc = torch.randn((*bshape, M, N), generator=gen, device="cuda")
+                ref = A.double() @ Bt.double().transpose(-1, -2) + (Cc.double() if acc else 0)
+                ab = [A.stride(i) for i in range(len(bshape))]
+                bb = [0 if bcast else Bt.stride(i) for i in range(len(bshape))]
+                lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, K, 1, Bt.data_ptr(), 0, 1, K, Cc.data_ptr(), M, N, K, len(bshape),
+                                               lib.i64(bshape), lib.i64(ab), lib.i64(bb), acc, 1))
+                err = float((Cc.double() - ref).norm() / ref.norm())
+                assert err <= RTOL_FRO, (smallk, bshape, M, N, K, acc, bcast, err)
+    finally:
+        L.tenmo_hip_set_tuning(b"gemm_smallk", -1)
+
+
 def test_raw_abi_arguments(T):
     """Argument checking of the kernel-level entry points (status codes + messages, nothing launched)."""
     L, lib = T.lib.load(), T.lib
