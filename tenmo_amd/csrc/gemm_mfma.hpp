@@ -416,6 +416,22 @@ __device__ __forceinline__ void tile_coords(const GemmArgs& g, int64_t tile_id, 
     // tile ids are below 2^31: 32-bit divisions (a 64-bit one costs hundreds of instructions)
     constexpr uint32_t GROUP_M = 8;
     const uint32_t tid = (uint32_t)tile_id;
+    // Fewer than 8 tile-rows: the tiles of one column block all go to the same XCD (ids that are equal mod 8), so
+    // that a panel of B is fetched from memory by one L2 instead of by up to `tiles_m` of them (A, with so few
+    // rows, is small).  The columns beyond the last multiple of 8 keep the plain column-major order.
+    if ((uint32_t)g.tiles_m < GROUP_M && g.tiles_m > 1) {
+        const uint32_t gsz = (uint32_t)g.tiles_m, cols8 = (uint32_t)g.tiles_n & ~7u, main_tiles = gsz * cols8;
+        if (tid < main_tiles) {
+            const uint32_t xcd = tid % 8, j = tid / 8, c = j / gsz;
+            tile_m = j - c * gsz;
+            tile_n = c * 8 + xcd;
+        } else {
+            const uint32_t r = tid - main_tiles, c = r / gsz;
+            tile_m = r - c * gsz;
+            tile_n = cols8 + c;
+        }
+        return;
+    }
     const uint64_t per_group64 = (uint64_t)GROUP_M * (uint32_t)g.tiles_n;
     const uint32_t per_group = per_group64 > 0xffffffffull ? 0xffffffffu : (uint32_t)per_group64; // clamped: then group 0 holds every tile
     const uint32_t group = tid / per_group, in_group = tid - group * per_group;
