@@ -882,10 +882,21 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
 template <int BM, int BN, int AMODE, int BMODE>
 __device__ __forceinline__ void gemm_workgroup(const GemmArgs& g, float* stage0, float* stage1, float* stage2, uint32_t pid, uint32_t slice) {
     const uint32_t tiles = (uint32_t)g.tiles_m * (uint32_t)g.tiles_n; // the grid, batches included, is below 2^31
-    const uint32_t batch32 = pid / tiles;
-    const int64_t batch = batch32;
+    uint32_t batch32;
     int64_t tile_m, tile_n;
-    tile_coords_blocked<BM, BN>(g, pid - batch32 * tiles, tile_m, tile_n);
+    // With 8 or more batches each XCD (workgroup id mod 8) takes whole batches, so that a batch's operands are
+    // fetched by one L2 only (attention P.V: V is otherwise read by all eight); the batches beyond the last
+    // multiple of 8 keep the plain order.
+    const uint32_t by_xcd = ((uint32_t)g.batch_count & ~7u) * tiles;
+    if (pid < by_xcd) {
+        const uint32_t xcd = pid % 8, j = pid / 8, bl = j / tiles;
+        batch32 = bl * 8 + xcd;
+        tile_coords(g, j - bl * tiles, tile_m, tile_n);
+    } else {
+        batch32 = pid / tiles;
+        tile_coords_blocked<BM, BN>(g, pid - batch32 * tiles, tile_m, tile_n);
+    }
+    const int64_t batch = batch32;
 
     int64_t k_begin = 0, k_end = g.K;
     TileDest dst;
