@@ -317,6 +317,14 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         if (K <= 128 && splits == 1 && sk_wpc == 0 && !ep.gather_row && !ep.colsum && am != KMAJOR_GEN && bm != KMAJOR_GEN &&
             ((M + 63) / 64) * ((N + 63) / 64) * batch_count >= 2048)
             tile = bm == KMAJOR_VEC ? 2 : 4;
+        // A short reduction (K <= 512) into a large result whose 256x128 or 128x128 tiles do not even fill one round: the
+        // model underrates what the few large workgroups lose to their prologue and to storing 64-128 KB each with
+        // nothing beside them.  Measured ([256,192..512].[.,50000], [512,256].[256,16384], [1024,256].[256,8192], both
+        // layouts of B): 128x64 is 11-16 % faster there and within 3 % of the best tile.
+        else if (K <= 512 && tile <= 1 && splits == 1 && sk_wpc == 0 && !ep.gather_row && !ep.colsum && am != KMAJOR_GEN && bm != KMAJOR_GEN &&
+                 (double)batch_count * M * N * 4.0 >= 16.0e6 &&
+                 ((M + kTiles[tile].bm - 1) / kTiles[tile].bm) * ((N + kTiles[tile].bn - 1) / kTiles[tile].bn) * batch_count < (int64_t)(S.cus * kOccupancy[tile]))
+            tile = 3;
         if (S.verbose) fprintf(stderr, "tenmo_hip gemm M=%lld N=%lld K=%lld batch=%lld -> tile %dx%d, %d K slice(s), est %.1f us%s\n",
                                (long long)M, (long long)N, (long long)K, (long long)batch_count, kTiles[tile].bm, kTiles[tile].bn, splits, best,
                                sk_wpc ? " (stream-K chosen instead)" : "");
