@@ -45,7 +45,7 @@ __global__ __launch_bounds__(SMALLK_THREADS, WGS_PER_CU) void gemm_smallk_kernel
     const uint32_t per_xcd = gridDim.x / xcds, xcd = blockIdx.x % xcds;
     auto tile_at = [&](uint32_t q) { // q = position in this XCD's sequence; increasing in q; >= total_tiles: done
         const uint32_t c = q / chunk;
-        const uint64_t tl = (uint64_t)(c * xcds + xcd) * chunk + (q - c * chunk);
+        const uint64_t tl = ((uint64_t)c * xcds + xcd) * chunk + (q - c * chunk);
         return (uint32_t)std::min<uint64_t>(tl, total_tiles);
     };
     uint32_t q = blockIdx.x / xcds;
