@@ -26,17 +26,52 @@ namespace tenmo {
 
 constexpr int SMALLK_THREADS = 512; // four computing wavefronts and four loading ones
 
-template <int NK, int WGS_PER_CU, bool ACC>
-__global__ __launch_bounds__(SMALLK_THREADS, WGS_PER_CU) void gemm_smallk_kernel(const GemmArgs g, const uint32_t total_tiles, const uint32_t xcds, const uint32_t chunk) {
+// AMODE / BMODE: KMAJOR_VEC or MNMAJOR_VEC (the LDS layouts and loaders of gemm_mfma.hpp).  NK = K steps of 16 that
+// cover K; `col_major`: tiles are numbered column block by column block (few tile-rows: see the launcher).
+// TileLoader::load_direct (one 16-row / 4-k part `part` of the tile at K offset koff) for the lanes with `ok` only:
+// the others neither read memory nor write LDS.  The execution mask is narrowed inside the assembly block, because
+// under a divergent branch the compiler no longer keeps the block's scalar operands in scalar registers.
+template <class Loader>
+__device__ __forceinline__ void load_direct_where(const Loader& l, float* lds, int64_t koff, int part, bool ok) {
+    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
+    const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + part * 1024);
+    const float* src = l.origin + koff * l.kstep;
+    const uint32_t pred = ok ? 1u : 0u;
+    uint64_t saved_exec;
+    asm volatile("s_mov_b32 m0, %1\n\t"
+                 "s_mov_b64 %0, exec\n\t"
+                 "v_cmp_ne_u32_e32 vcc, 0, %4\n\t"
+                 "s_and_b64 exec, exec, vcc\n\t"
+                 "global_load_lds_dwordx4 %2, %3\n\t"
+                 "s_mov_b64 exec, %0"
+                 : "=&s"(saved_exec)
+                 : "s"(dst), "v"(l.lane_off[0]), "s"(src), "v"(pred)
+                 : "memory", "vcc");
+}
+
+template <int AMODE, int BMODE, int NK, int WGS_PER_CU, bool ACC>
+__global__ __launch_bounds__(SMALLK_THREADS, WGS_PER_CU) void gemm_smallk_kernel(const GemmArgs g, const uint32_t total_tiles, const uint32_t xcds, const uint32_t chunk,
+                                                                                 const int col_major) {
     constexpr int BM = 64, BN = 64;
     constexpr int A_FLOATS = BM * GEMM_BK, STAGE = (BM + BN) * GEMM_BK;
-    using LA = TileLoader<BM, KMAJOR_VEC>;
-    using LB = TileLoader<BN, KMAJOR_VEC>;
-    static_assert(LA::NCH == 1 && LB::NCH == 1, "one direct load per operand, 16 rows and K step");
+    using LA = TileLoader<BM, AMODE>;
+    using LB = TileLoader<BN, BMODE>;
+    static_assert(LA::NCH == 1 && LB::NCH == 1, "one direct load per operand, quarter tile and K step");
     __shared__ __attribute__((aligned(1024))) float panel0[STAGE * NK];
     __shared__ __attribute__((aligned(1024))) float panel1[STAGE * NK];
 
     const int t = threadIdx.x, lane = t & 63, wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    // K not a multiple of 16: the loads of the last K step skip what lies beyond K (a K-major operand in 16-byte
+    // chunks: the host admits K % 4 == 0 only), and those places of the panels, which no load ever writes, are
+    // zeroed once here.
+    const int k_tail = (int)g.K - (NK - 1) * GEMM_BK; // valid k of the last step, 1..16
+    if (k_tail < GEMM_BK) {
+        for (int i = t * 4; i < STAGE * NK; i += SMALLK_THREADS * 4) {
+            *reinterpret_cast<f32x4*>(panel0 + i) = f32x4{0.f, 0.f, 0.f, 0.f};
+            *reinterpret_cast<f32x4*>(panel1 + i) = f32x4{0.f, 0.f, 0.f, 0.f};
+        }
+        __syncthreads();
+    }
     const uint32_t tiles_n = (uint32_t)g.tiles_n, tiles_per_batch = (uint32_t)g.tiles_m * tiles_n;
     // Which tiles this workgroup takes.  Workgroup ids are dealt round-robin to the `xcds` XCDs (8, or 1 for a plain
     // round-robin over the grid); the workgroups of one XCD walk `chunk` consecutive tiles together (one batch),
@@ -57,17 +92,28 @@ __global__ __launch_bounds__(SMALLK_THREADS, WGS_PER_CU) void gemm_smallk_kernel
         return tile < total_tiles;
     };
     // tiles are numbered row by row inside a batch: workgroups side by side share the A rows and stream B
+    const uint32_t tiles_m = (uint32_t)g.tiles_m;
     auto tile_coords3 = [&](uint32_t tl, uint32_t& b, int64_t& m0, int64_t& n0) {
         b = tl / tiles_per_batch;
-        const uint32_t r = tl - b * tiles_per_batch, tm = r / tiles_n;
+        const uint32_t r = tl - b * tiles_per_batch;
+        uint32_t tm, tn;
+        if (col_major) { tn = r / tiles_m; tm = r - tn * tiles_m; }
+        else { tm = r / tiles_n; tn = r - tm * tiles_n; }
         m0 = (int64_t)tm * BM;
-        n0 = (int64_t)(r - tm * tiles_n) * BN;
+        n0 = (int64_t)tn * BN;
     };
 
     if (wave >= 4) {
         // ---- a loading wavefront: one of the four 16-row parts of the ordinary tile loader ----
         // (one wavefront for the whole panel was measured at about 110 ns per 1 KiB load: far too slow)
         const int w = wave - 4;
+        // k (within a K step) of this lane's 16 bytes, as the loaders lay them out: a K-major load moves 4 consecutive k
+        // of one row (chunk (lane & 3) ^ ((lane >> 4) & 3), the swizzle), an MN-major load one k of 4 rows
+        auto last_ok = [&](int mode) {
+            if (mode == KMAJOR_VEC) return 4 * ((lane & 3) ^ ((lane >> 4) & 3)) + 4 <= k_tail;
+            return 4 * w + lane / 16 < k_tail;
+        };
+        const bool a_last_ok = last_ok(AMODE), b_last_ok = last_ok(BMODE);
         auto issue_tile = [&](float* panel, uint32_t tl) {
             uint32_t b;
             int64_t m0, n0, a_boff, b_boff;
@@ -75,13 +121,16 @@ __global__ __launch_bounds__(SMALLK_THREADS, WGS_PER_CU) void gemm_smallk_kernel
             batch_offsets(g.batch, b, a_boff, b_boff);
             LA la;
             LB lb;
-            la.init_direct(g.A + a_boff, g.a_rs, 1, m0, 0, g.M, lane, w);
-            lb.init_direct(g.B + b_boff, g.b_cs, 1, n0, 0, g.N, lane, w);
+            la.init_direct(g.A + a_boff, g.a_rs, g.a_cs, m0, 0, g.M, lane, w);
+            lb.init_direct(g.B + b_boff, g.b_cs, g.b_rs, n0, 0, g.N, lane, w);
 #pragma unroll
-            for (int it = 0; it < NK; ++it) {
+            for (int it = 0; it < NK - 1; ++it) {
                 la.load_direct(panel + it * STAGE, (int64_t)it * GEMM_BK, w, 0);
                 lb.load_direct(panel + it * STAGE + A_FLOATS, (int64_t)it * GEMM_BK, w, 0);
             }
+            // the last step: this lane's part of it may lie beyond K
+            load_direct_where(la, panel + (NK - 1) * STAGE, (int64_t)(NK - 1) * GEMM_BK, w, a_last_ok);
+            load_direct_where(lb, panel + (NK - 1) * STAGE + A_FLOATS, (int64_t)(NK - 1) * GEMM_BK, w, b_last_ok);
         };
         issue_tile(panel0, tile);
         for (;;) {
@@ -125,14 +174,14 @@ __global__ __launch_bounds__(SMALLK_THREADS, WGS_PER_CU) void gemm_smallk_kernel
 #pragma unroll
         for (int e = 0; e < 16; ++e) acc[e] = 0.f;
         float fa[2][1][4], fb[2][1][4];
-        load_fragments<BM, KMAJOR_VEC, 1>(panel, wm * 32, 0, lane, fa[0]);
-        load_fragments<BN, KMAJOR_VEC, 1>(panel + A_FLOATS, wn * 32, 0, lane, fb[0]);
+        load_fragments<BM, AMODE, 1>(panel, wm * 32, 0, lane, fa[0]);
+        load_fragments<BN, BMODE, 1>(panel + A_FLOATS, wn * 32, 0, lane, fb[0]);
 #pragma unroll
         for (int c = 0; c < 2 * NK; ++c) { // 8-wide chunks of K; the operand fetch runs one chunk ahead
             if (c + 1 < 2 * NK) {
                 const float* st = panel + ((c + 1) >> 1) * STAGE;
-                load_fragments<BM, KMAJOR_VEC, 1>(st, wm * 32, (c + 1) & 1, lane, fa[(c + 1) & 1]);
-                load_fragments<BN, KMAJOR_VEC, 1>(st + A_FLOATS, wn * 32, (c + 1) & 1, lane, fb[(c + 1) & 1]);
+                load_fragments<BM, AMODE, 1>(st, wm * 32, (c + 1) & 1, lane, fa[(c + 1) & 1]);
+                load_fragments<BN, BMODE, 1>(st + A_FLOATS, wn * 32, (c + 1) & 1, lane, fb[(c + 1) & 1]);
             }
 #pragma unroll
             for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[c & 1][0][s], fb[c & 1][0][s], acc, 0, 0, 0);
@@ -154,29 +203,58 @@ __global__ __launch_bounds__(SMALLK_THREADS, WGS_PER_CU) void gemm_smallk_kernel
     }
 }
 
-bool launch_gemm_smallk_64x64(const GemmArgs& g, unsigned cus, unsigned total_tiles, bool by_batch, hipStream_t stream) {
-    const int nk = (int)(g.K / GEMM_BK);
-    if (g.K % GEMM_BK != 0 || nk < 1 || nk > 4 || total_tiles == 0) return false;
-    // LDS per workgroup: two panels of 8 KiB per K step
-#define TENMO_SMALLK(NK_, WPC_)                                                                                                     \
-    {                                                                                                                               \
-        const unsigned wgs = std::min(total_tiles, cus * WPC_);                                                                     \
-        const unsigned per_batch = (unsigned)g.tiles_m * (unsigned)g.tiles_n;                                                       \
-        const bool xcd_order = by_batch && wgs % 8 == 0 && total_tiles / per_batch >= 8;                                            \
-        const unsigned xcds = xcd_order ? 8 : 1, chunk = xcd_order ? per_batch : 1;                                                 \
-        if (g.accumulate)                                                                                                           \
-            hipLaunchKernelGGL((gemm_smallk_kernel<NK_, WPC_, true>), dim3(wgs), dim3(SMALLK_THREADS), 0, stream, g, total_tiles, xcds, chunk);  \
-        else                                                                                                                        \
-            hipLaunchKernelGGL((gemm_smallk_kernel<NK_, WPC_, false>), dim3(wgs), dim3(SMALLK_THREADS), 0, stream, g, total_tiles, xcds, chunk); \
+namespace {
+
+struct SmallkLaunch {
+    unsigned cus, total_tiles;
+    bool by_batch;
+    hipStream_t stream;
+};
+
+template <int AMODE, int BMODE, int NK, int WPC>
+void launch_smallk(const GemmArgs& g, const SmallkLaunch& l) {
+    const unsigned wgs = std::min(l.total_tiles, l.cus * WPC);
+    const unsigned per_batch = (unsigned)g.tiles_m * (unsigned)g.tiles_n;
+    // With 8 or more batches the workgroups of an XCD take whole batches; else, with fewer than 8 tile-rows, whole
+    // column blocks (tiles numbered column block by column block): a panel of B is then fetched by one L2.
+    unsigned xcds = 1, chunk = 1;
+    int col_major = 0;
+    if (wgs % 8 == 0) {
+        if (l.by_batch && l.total_tiles / per_batch >= 8) { xcds = 8; chunk = per_batch; }
+        else if (l.by_batch && g.tiles_m < 8 && g.tiles_n >= 64) { xcds = 8; chunk = (unsigned)g.tiles_m; col_major = 1; }
     }
+    if (g.accumulate)
+        hipLaunchKernelGGL((gemm_smallk_kernel<AMODE, BMODE, NK, WPC, true>), dim3(wgs), dim3(SMALLK_THREADS), 0, l.stream, g, l.total_tiles, xcds, chunk, col_major);
+    else
+        hipLaunchKernelGGL((gemm_smallk_kernel<AMODE, BMODE, NK, WPC, false>), dim3(wgs), dim3(SMALLK_THREADS), 0, l.stream, g, l.total_tiles, xcds, chunk, col_major);
+}
+
+// LDS per workgroup: two panels of 8 KiB per K step
+template <int AMODE, int BMODE>
+bool launch_smallk_modes(const GemmArgs& g, int nk, const SmallkLaunch& l) {
     switch (nk) {
-        case 1: TENMO_SMALLK(1, 4); break;
-        case 2: TENMO_SMALLK(2, 4); break;
-        case 3: TENMO_SMALLK(3, 2); break;
-        default: TENMO_SMALLK(4, 2); break;
+        case 1: launch_smallk<AMODE, BMODE, 1, 4>(g, l); return true;
+        case 2: launch_smallk<AMODE, BMODE, 2, 4>(g, l); return true;
+        case 3: launch_smallk<AMODE, BMODE, 3, 2>(g, l); return true;
+        case 4: launch_smallk<AMODE, BMODE, 4, 2>(g, l); return true;
+        case 5: launch_smallk<AMODE, BMODE, 5, 1>(g, l); return true;
+        case 6: launch_smallk<AMODE, BMODE, 6, 1>(g, l); return true;
+        case 7: launch_smallk<AMODE, BMODE, 7, 1>(g, l); return true;
+        default: return false;
     }
-#undef TENMO_SMALLK
-    return true;
+}
+
+} // namespace
+
+bool launch_gemm_smallk_64x64(const GemmArgs& g, int amode, int bmode, unsigned cus, unsigned total_tiles, bool by_batch, hipStream_t stream) {
+    const int nk = (int)((g.K + GEMM_BK - 1) / GEMM_BK);
+    if (nk < 1 || nk > 7 || total_tiles == 0) return false;
+    const SmallkLaunch l{cus, total_tiles, by_batch, stream};
+    if (amode == KMAJOR_VEC && bmode == KMAJOR_VEC) return launch_smallk_modes<KMAJOR_VEC, KMAJOR_VEC>(g, nk, l);
+    if (amode == KMAJOR_VEC && bmode == MNMAJOR_VEC) return launch_smallk_modes<KMAJOR_VEC, MNMAJOR_VEC>(g, nk, l);
+    if (amode == MNMAJOR_VEC && bmode == KMAJOR_VEC) return launch_smallk_modes<MNMAJOR_VEC, KMAJOR_VEC>(g, nk, l);
+    if (amode == MNMAJOR_VEC && bmode == MNMAJOR_VEC) return launch_smallk_modes<MNMAJOR_VEC, MNMAJOR_VEC>(g, nk, l);
+    return false;
 }
 
 } // namespace tenmo

@@ -329,21 +329,28 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
                                (long long)M, (long long)N, (long long)K, (long long)batch_count, kTiles[tile].bm, kTiles[tile].bn, splits, best,
                                sk_wpc ? " (stream-K chosen instead)" : "");
     }
-    // Short reduction with both operands K-major and a plain (or accumulating) store: the persistent whole-K-in-LDS
-    // kernel, which loads its next tile before it stores this one (gemm_smallk.hip).  Automatic where the launch is
-    // store-bound as above and every workgroup gets several tiles.
+    // Short reduction, vector operand forms and a plain (or accumulating) store: the persistent whole-K-in-LDS kernel
+    // (gemm_smallk.hip).  Automatic for K <= 64 where the launch is store-bound as above and every workgroup gets several
+    // tiles (measured: 8192x8192xK, K = 32 / 64, every operand layout 76-115 -> 60-93 us; [256,64].[64,50000] 27 -> 21 us;
+    // K = 96 .. 112, one workgroup per CU: level with the ordinary kernel, so those only when forced).
     {
         const int64_t tm = (M + 63) / 64, tn = (N + 63) / 64, tiles64 = tm * tn * batch_count;
-        const bool can = am == KMAJOR_VEC && bm == KMAJOR_VEC && a_cs == 1 && b_rs == 1 && K % GEMM_BK == 0 && K <= 64 && !ep.any() && !ep.gather_row &&
-                         !ep.colsum && a_rs >= 0 && a_rs <= (int64_t(1) << 21) && b_cs >= 0 && b_cs <= (int64_t(1) << 21) && N < (int64_t(1) << 29) &&
-                         tiles64 <= 0x7fffffffLL;
+        // what the direct loads need: a K-major operand a row pitch below 2^21 and, when K is no multiple of 16, K % 4 == 0
+        // (it moves 4 consecutive k at a time); an MN-major one a k pitch below 2^25 and an extent divisible by 4
+        auto operand_ok = [&](int mode, int64_t row_s, int64_t k_s, int64_t extent) {
+            if (mode == KMAJOR_VEC) return k_s == 1 && row_s >= 0 && row_s <= (int64_t(1) << 21) && (K % GEMM_BK == 0 || K % 4 == 0);
+            if (mode == MNMAJOR_VEC) return row_s == 1 && k_s >= 0 && k_s <= (int64_t(1) << 25) && extent % 4 == 0 && extent >= 4;
+            return false;
+        };
+        const bool can = K >= 1 && K <= 112 && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum &&
+                         N < (int64_t(1) << 29) && tiles64 <= 0x7fffffffLL;
         const bool want = S.force_smallk > 0 || (S.force_smallk < 0 && S.force_tile < 0 && S.force_splitk <= 0 && S.force_streamk <= 0 &&
-                                                  splits == 1 && sk_wpc == 0 && tiles64 >= 2048);
+                                                  splits == 1 && sk_wpc == 0 && tiles64 >= 2048 && K <= 64);
         if (can && want) {
             g.tiles_m = (int32_t)tm; g.tiles_n = (int32_t)tn;
             g.k_splits = 1; g.k_per_split = K; g.partial = nullptr;
             if (S.verbose) fprintf(stderr, "tenmo_hip gemm: short-reduction kernel, %lld tiles of 64x64\n", (long long)tiles64);
-            if (launch_gemm_smallk_64x64(g, (unsigned)S.cus, (unsigned)tiles64, S.force_smallk != 2, S.stream)) return 0;
+            if (launch_gemm_smallk_64x64(g, am, bm, (unsigned)S.cus, (unsigned)tiles64, S.force_smallk != 2, S.stream)) return 0;
         }
     }
     if (S.force_tile >= 0 && S.force_tile < kNumTiles && !(ep.colsum && (S.force_tile < 2 || kTiles[S.force_tile].bm < M))) tile = S.force_tile;
