@@ -25,7 +25,7 @@ bool launch_streamk_128x128(const GemmArgs& g, const StreamKArgs& sk, unsigned w
 bool launch_streamk_128x64(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);
 bool launch_streamk_64x64(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);
 
-// Short reduction (K up to 112), vector operand modes, plain or accumulating store: persistent workgroups that hold a
+// Short reduction (K up to 64), vector operand modes, plain or accumulating store: persistent workgroups that hold a
 // whole tile's operands in LDS, loaded one tile ahead by wavefronts of their own (gemm_smallk.hip).  `total_tiles` =
 // batches x 64x64 tiles (g.tiles_m, g.tiles_n set for that tile).  The caller has checked what the direct loads need
 // (pitches, an MN-major extent divisible by 4, K % 4 == 0 for a K-major operand when K is no multiple of 16).

@@ -237,9 +237,6 @@ bool launch_smallk_modes(const GemmArgs& g, int nk, const SmallkLaunch& l) {
         case 2: launch_smallk<AMODE, BMODE, 2, 4>(g, l); return true;
         case 3: launch_smallk<AMODE, BMODE, 3, 2>(g, l); return true;
         case 4: launch_smallk<AMODE, BMODE, 4, 2>(g, l); return true;
-        case 5: launch_smallk<AMODE, BMODE, 5, 1>(g, l); return true;
-        case 6: launch_smallk<AMODE, BMODE, 6, 1>(g, l); return true;
-        case 7: launch_smallk<AMODE, BMODE, 7, 1>(g, l); return true;
         default: return false;
     }
 }
@@ -248,7 +245,7 @@ bool launch_smallk_modes(const GemmArgs& g, int nk, const SmallkLaunch& l) {
 
 bool launch_gemm_smallk_64x64(const GemmArgs& g, int amode, int bmode, unsigned cus, unsigned total_tiles, bool by_batch, hipStream_t stream) {
     const int nk = (int)((g.K + GEMM_BK - 1) / GEMM_BK);
-    if (nk < 1 || nk > 7 || total_tiles == 0) return false;
+    if (nk < 1 || nk > 4 || total_tiles == 0) return false; // (more K steps: one workgroup per CU, no gain; not instantiated)
     const SmallkLaunch l{cus, total_tiles, by_batch, stream};
     if (amode == KMAJOR_VEC && bmode == KMAJOR_VEC) return launch_smallk_modes<KMAJOR_VEC, KMAJOR_VEC>(g, nk, l);
     if (amode == KMAJOR_VEC && bmode == MNMAJOR_VEC) return launch_smallk_modes<KMAJOR_VEC, MNMAJOR_VEC>(g, nk, l);

@@ -332,7 +332,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     // Short reduction, vector operand forms and a plain (or accumulating) store: the persistent whole-K-in-LDS kernel
     // (gemm_smallk.hip).  Automatic for K <= 64 where the launch is store-bound as above and every workgroup gets several
     // tiles (measured: 8192x8192xK, K = 32 / 64, every operand layout 76-115 -> 60-93 us; [256,64].[64,50000] 27 -> 21 us;
-    // K = 96 .. 112, one workgroup per CU: level with the ordinary kernel, so those only when forced).
+    // K = 96 .. 112, one workgroup per CU, measured level with the ordinary kernel: not built).
     {
         const int64_t tm = (M + 63) / 64, tn = (N + 63) / 64, tiles64 = tm * tn * batch_count;
         // what the direct loads need: a K-major operand a row pitch below 2^21 and, when K is no multiple of 16, K % 4 == 0
@@ -342,7 +342,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
             if (mode == MNMAJOR_VEC) return row_s == 1 && k_s >= 0 && k_s <= (int64_t(1) << 25) && extent % 4 == 0 && extent >= 4;
             return false;
         };
-        const bool can = K >= 1 && K <= 112 && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum &&
+        const bool can = K >= 1 && K <= 64 && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum &&
                          N < (int64_t(1) << 29) && tiles64 <= 0x7fffffffLL;
         const bool want = S.force_smallk > 0 || (S.force_smallk < 0 && S.force_tile < 0 && S.force_splitk <= 0 && S.force_streamk <= 0 &&
                                                   splits == 1 && sk_wpc == 0 && tiles64 >= 2048 && K <= 64);
