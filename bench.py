@@ -8,15 +8,25 @@ C = A.B with M = N = K = 8192 (the size the headline metric is quoted on), opera
 HBM before the timed region.  Prints ONE JSON line with the whole-job throughput in TFLOP/s,
 the roofline of the dominant kernel (fp32 MFMA peak 157.3 TFLOP/s) measured with HIP events on the
 stream the kernel runs on, and a CPU baseline (the C++ restatement of the reference's CPU matmul,
-timed on this host's cores on a bounded sample of the same workload).  The `extra` object carries
-the other headline figures: mv / vm bandwidth at 16384^2 and the MLP training step in ms on GPU
-and CPU.
+timed on this host's cores on a bounded sample of the same workload).
+
+`extra.rows` carries one entry per product of every benchmark configuration — the square sweep with
+a row-major and a transposed-view A, the attention-shaped batched products and their gradients, the
+broadcast-batched case with its backward, the GPT-2-shaped linear layers (forward, dX, dW), mv, vm,
+the skinny product and the CBOW logits with their gradient: microseconds per launch (HIP events,
+median of three groups of back-to-back launches after a warm-up), TFLOP/s and GB/s on the
+algorithmic flop and bytes, the roof that bounds it (the larger of flop / 157.3 TFLOP/s and
+bytes / 8 TB/s), the fraction of that roof, and the relative Frobenius error of the whole result
+against fp64.  Products whose operands and result would fit the chip's 256 MB memory-side cache are
+timed over several copies of their buffers in rotation, so that every launch reads from HBM.
+`extra` also holds the MLP training step in ms on GPU and CPU and the shader clock under load.
 """
 from __future__ import annotations
 
 import argparse
 import ctypes as C
 import json
+import math
 import os
 import sys
 import time
@@ -26,11 +36,23 @@ sys.path.insert(0, ROOT)
 
 PEAK_FP32_MFMA_TFLOPS = 157.3  # 256 CU x 2.4 GHz x 256 flop/clk/CU
 PEAK_HBM_GBPS = 8000.0
+MALL_BYTES = 256e6             # memory-side cache: a working set below this would be served from it
 
-# Bytes moved between L2 and the memory fabric per 8192^3 launch, from two rocprofv3 --pmc runs
-# (FETCH_SIZE 2.965e6 KiB scaled by 2.0, WRITE_SIZE 2.621e5 KiB scaled by 1.0; the scale factors are
-# what the same counters read for a plain 1 GiB copy).  Only valid for the default size.
-MEASURED_TRAFFIC_BYTES = 6.3e9
+# HBM bytes per 8192^3 launch of the headline kernel = FETCH_SIZE x its copy-calibration factor +
+# WRITE_SIZE x its factor, read from the two counter summaries under profiles/ (None when absent)
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "gemm_mfma_256x128_square8192.md")
+
+
+def measured_traffic_bytes():
+    """`traffic_bytes_per_launch: <number>` line of the committed counter summary for the headline kernel."""
+    try:
+        with open(TRAFFIC_PROFILE) as f:
+            for line in f:
+                if line.lower().startswith("traffic_bytes_per_launch:"):
+                    return float(line.split(":", 1)[1].split()[0])
+    except OSError:
+        pass
+    return None
 
 
 def main() -> int:
@@ -40,11 +62,10 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=3)
     ap.add_argument("--size", type=int, default=8192, help="M=N=K of the square GEMM (default: the headline size)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
-    ap.add_argument("--no-extra", action="store_true", help="skip the mv/vm and MLP-step side measurements")
+    ap.add_argument("--no-extra", action="store_true", help="skip the per-configuration rows and the MLP-step measurement")
+    ap.add_argument("--rows", default="", help="comma-separated substrings: only the rows whose name contains one of them")
     ap.add_argument("--adjacent", action="store_true",
                     help="also time the adjacent operators (cross-entropy, SGD step, convolution) into `extra`; off by default")
-    ap.add_argument("--attention", action="store_true",
-                    help="also time the attention-shaped batched products (Q.K^T, P.V, P^T.dO, Q^T.dS at [8,12,1024,64]) into `extra`; off by default")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy, the known-size kernel against which FETCH_SIZE/WRITE_SIZE are scaled")
     args = ap.parse_args()
@@ -105,12 +126,12 @@ def main() -> int:
     flop = 2.0 * S * S * S
     value = flop / (wall_ms * 1e-3) / 1e12
     achieved = flop / (kernel_ms * 1e-3) / 1e12
+    # shader clock under a full matrix-core load, right behind the timed launches
+    mhz = C.c_float()
+    _lib.check(L.tenmo_hip_clock_probe(50000, C.byref(mhz)))
 
-    # accuracy gate on the timed result: sampled rows against fp64
-    rows = torch.tensor([0, S // 3, S - 1], device="cuda")
-    ref = (A[rows].double() @ B.double()).cpu().numpy()
-    got = Cc[rows].cpu().numpy()
-    rel_err = float(np.linalg.norm(got - ref) / np.linalg.norm(ref))
+    # accuracy gate on the timed result: the whole matrix against fp64
+    rel_err = rel_fro_vs_fp64(torch, Cc, A, B)
 
     out = {
         "metric": "fp32 GEMM TFLOP/s (M=N=K=%d) + %% fp32-MFMA peak (1 GPU); MLP train-step ms vs CPU" % S,
@@ -128,98 +149,205 @@ def main() -> int:
         "config": {"workload": "square fp32 GEMM C=A.B, M=N=K=%d, A and B row-major N(0,1), inputs resident in HBM" % S,
                    "device": name.value.decode(), "compute_units": cus.value},
         "roofline": {"bound": "mfma", "achieved": round(achieved, 3), "peak": PEAK_FP32_MFMA_TFLOPS, "unit": "TFLOP/s",
-                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": MEASURED_TRAFFIC_BYTES if S == 8192 else None,
-                     "kernel_ms": round(kernel_ms, 4)},
+                     "frac": round(achieved / PEAK_FP32_MFMA_TFLOPS, 4), "traffic": measured_traffic_bytes() if S == 8192 else None,
+                     "kernel_ms": round(kernel_ms, 4), "effective_mhz": round(mhz.value, 1)},
         "rel_fro_error_vs_fp64": rel_err,
     }
+    del A, B, Cc
+    torch.cuda.empty_cache()
 
     extra = {}
+    worst = rel_err
     if not args.no_extra:
-        extra.update(side_measurements(L, _lib, torch, np))
+        only = [s for s in args.rows.split(",") if s]
+        rows = config_rows(L, _lib, torch, only)
+        extra["rows"] = rows
+        worst = max([worst] + [r["rel_err_vs_fp64"] for r in rows])
+        extra["rows_max_rel_err_vs_fp64"] = worst
+        _lib.check(L.tenmo_hip_clock_probe(50000, C.byref(mhz)))
+        extra["effective_mhz_after_rows"] = round(mhz.value, 1)
     if args.adjacent:
         extra.update(adjacent_operators(L, _lib, torch))
-    if args.attention:
-        extra.update(attention_products(L, _lib, torch))
     if not args.no_cpu:
+        gen.manual_seed(8192)
+        A = torch.randn((S, S), generator=gen, device="cuda", dtype=torch.float32)
+        B = torch.randn((S, S), generator=gen, device="cuda", dtype=torch.float32)
         out["cpu_baseline"] = cpu_gemm_baseline(A, B, S, np)
+        del A, B
         if not args.no_extra:
             extra.update(mlp_step_times(_lib, torch, np))
     if extra:
         out["extra"] = extra
     print(json.dumps(out), flush=True)
-    return 0 if rel_err <= 1e-5 else 1
+    return 0 if worst <= 1e-5 else 1
 
 
-def hip_time(L, _lib, fn, iters, warm=3):
-    for _ in range(warm):
-        fn()
+def rel_fro_vs_fp64(torch, got, A, B):
+    """||got - A.B||_F / ||A.B||_F with the product accumulated in fp64 from the same fp32 operands (views welcome);
+    large results go through in slabs of rows so that the fp64 temporaries stay small."""
+    M = got.shape[-2]
+    slab = max(1, min(M, int(2 ** 27 // max(1, got.shape[-1] * max(1, got.numel() // (got.shape[-1] * M))))))
+    num = den = 0.0
+    for r0 in range(0, M, slab):
+        ref = torch.matmul(A[..., r0:r0 + slab, :].double(), B.double())
+        d = got[..., r0:r0 + slab, :].double() - ref
+        num += float((d * d).sum())
+        den += float((ref * ref).sum())
+    return math.sqrt(num / den) if den > 0 else math.sqrt(num)
+
+
+def hip_time_us(L, _lib, fns, est_us):
+    """Microseconds per launch: the launches `fns` (one per buffer copy, used in rotation) back to back between two
+    HIP events on the library's stream; median of three such groups after a warm-up."""
+    def run(n):
+        for i in range(n):
+            fns[i % len(fns)]()
+    run(max(3, len(fns)))
     _lib.check(L.tenmo_hip_sync())
-    _lib.check(L.tenmo_hip_timer_begin())
-    for _ in range(iters):
-        fn()
-    ms = C.c_float()
-    _lib.check(L.tenmo_hip_timer_end(C.byref(ms)))
-    return ms.value / iters
+    iters = int(min(200, max(10, 4000.0 / max(est_us, 1.0))))
+    iters = (iters + len(fns) - 1) // len(fns) * len(fns)
+    groups = []
+    for _ in range(3):
+        _lib.check(L.tenmo_hip_timer_begin())
+        run(iters)
+        ms = C.c_float()
+        _lib.check(L.tenmo_hip_timer_end(C.byref(ms)))
+        groups.append(ms.value * 1e3 / iters)
+    return sorted(groups)[1]
 
 
-def side_measurements(L, _lib, torch, np):
-    """mv / vm at 16384^2 (HBM-bound): GB/s of algorithmic bytes and fraction of the 8 TB/s peak."""
-    n = 16384
+def config_rows(L, _lib, torch, only):
+    """One row per product of the benchmark configurations (see the module docstring)."""
+    rows = []
     gen = torch.Generator(device="cuda")
-    gen.manual_seed(16384)
-    W = torch.randn((n, n), generator=gen, device="cuda", dtype=torch.float32)
-    x = torch.randn((n,), generator=gen, device="cuda", dtype=torch.float32)
-    out = torch.empty((n,), device="cuda", dtype=torch.float32)
-    mv = lambda: _lib.check(L.tenmo_hip_mv_f32(W.data_ptr(), 0, n, 1, x.data_ptr(), 0, 1, out.data_ptr(), n, n, 0, None, None, None, 0, 0))
-    vm = lambda: _lib.check(L.tenmo_hip_vm_f32(x.data_ptr(), 0, 1, W.data_ptr(), 0, n, 1, out.data_ptr(), n, n, 0, None, None, None, 0, 0))
-    nbytes = (n * n + 2 * n) * 4.0
-    res = {}
-    for nm, fn in (("mv", mv), ("vm", vm)):
-        ms = hip_time(L, _lib, fn, 30)
-        gbps = nbytes / (ms * 1e-3) / 1e9
-        res["%s_16384_us" % nm] = round(ms * 1e3, 2)
-        res["%s_16384_gbps" % nm] = round(gbps, 1)
-        res["%s_16384_frac_hbm_peak" % nm] = round(gbps / PEAK_HBM_GBPS, 4)
-    return res
 
+    def randn(shape, seed, std=1.0):
+        gen.manual_seed(seed)
+        t = torch.randn(shape, generator=gen, device="cuda", dtype=torch.float32)
+        return t * std if std != 1.0 else t
 
-def attention_products(L, _lib, torch):
-    """The broadcast-batched products of attention at Q, K, V = [8, 12, 1024, 64]: S = Q.K^T (K as a transposed view),
-    O = P.V, dV = P^T.dO and Q^T.dS, each 12.88 GFLOP and 453 MB of algorithmic traffic; time, TFLOP/s and the
-    relative Frobenius error of one batch against fp64."""
-    Bn, H, T, D = 8, 12, 1024, 64
-    gen = torch.Generator(device="cuda")
-    gen.manual_seed(64)
-    Q, K, V = (torch.randn((Bn, H, T, D), generator=gen, device="cuda", dtype=torch.float32) for _ in range(3))
-    S = torch.empty((Bn, H, T, T), device="cuda", dtype=torch.float32)
-    O = torch.empty((Bn, H, T, D), device="cuda", dtype=torch.float32)
-    O2 = torch.empty((Bn, H, D, T), device="cuda", dtype=torch.float32)
-    bs, st, pst = (Bn, H), (H * T * D, T * D), (H * T * T, T * T)
+    def view(t):
+        return _lib.make_view(t.data_ptr(), 0, tuple(t.shape), tuple(t.stride()))
 
-    def gemm(A, B, Cc, M, N, Kk, a_rs, a_cs, b_rs, b_cs, ab, bb):
-        _lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, a_rs, a_cs, B.data_ptr(), 0, b_rs, b_cs, Cc.data_ptr(), M, N, Kk,
-                                        2, _lib.i64(bs), _lib.i64(ab), _lib.i64(bb), 0, 0))
+    def wanted(name):
+        return not only or any(s in name for s in only)
 
-    cases = (
-        ("qkt", lambda: gemm(Q, K, S, T, T, D, D, 1, 1, D, st, st), lambda: (S[1, 2], Q[1, 2].double() @ K[1, 2].double().T)),
-        ("pv", lambda: gemm(S, V, O, T, D, T, T, 1, D, 1, pst, st), lambda: (O[1, 2], S[1, 2].double() @ V[1, 2].double())),
-        ("ptdo", lambda: gemm(S, V, O, T, D, T, 1, T, D, 1, pst, st), lambda: (O[1, 2], S[1, 2].double().T @ V[1, 2].double())),
-        ("qtds", lambda: gemm(Q, S, O2, D, T, T, 1, D, T, 1, st, pst), lambda: (O2[1, 2], Q[1, 2].double().T @ S[1, 2].double())),
-    )
-    flop = 96 * 2.0 * T * T * D
-    res = {}
-    for nm, fn, check in cases:
-        ms = hip_time(L, _lib, fn, 20)
-        got, ref = check()
-        res["attn_%s_us" % nm] = round(ms * 1e3, 1)
-        res["attn_%s_tflops" % nm] = round(flop / (ms * 1e-3) / 1e12, 1)
-        res["attn_%s_rel_err" % nm] = float((got.double() - ref).norm() / ref.norm())
-    return res
+    def finish_row(name, cfg, shape, us, flop, nbytes, rel_err, copies):
+        t_mfma, t_hbm = flop / (PEAK_FP32_MFMA_TFLOPS * 1e12) * 1e6, nbytes / (PEAK_HBM_GBPS * 1e9) * 1e6
+        roof = max(t_mfma, t_hbm)
+        rows.append({"name": name, "cfg": cfg, "shape": shape, "us": round(us, 2),
+                     "tflops": round(flop / us / 1e6, 2), "gbps": round(nbytes / us / 1e3, 1),
+                     "bound": "mfma" if t_mfma >= t_hbm else "hbm", "roof_us": round(roof, 2), "frac": round(roof / us, 4),
+                     "rel_err_vs_fp64": rel_err, "buffer_copies": copies})
+
+    def copies_for(nbytes):
+        # enough copies of the buffers that a rotation through them exceeds the memory-side cache twice over
+        return 1 if nbytes >= 2 * MALL_BYTES else int(min(12, math.ceil(2 * MALL_BYTES / nbytes)))
+
+    def gemm_row(name, cfg, make_a, make_b, out_shape):
+        """make_a / make_b: seed -> operand tensor (any torch view; broadcast batch dims have extent 1 or are absent)."""
+        if not wanted(name):
+            return
+        a0, b0 = make_a(0), make_b(0)
+        M, K, N = a0.shape[-2], a0.shape[-1], b0.shape[-1]
+        batch = 1
+        for d in out_shape[:-2]:
+            batch *= d
+        flop = 2.0 * M * N * K * batch
+        nbytes = 4.0 * (a0.numel() + b0.numel() + batch * M * N)
+        n = copies_for(nbytes)
+        As, Bs = [a0] + [make_a(i) for i in range(1, n)], [b0] + [make_b(i) for i in range(1, n)]
+        Cs = [torch.empty(out_shape, device="cuda", dtype=torch.float32) for _ in range(n)]
+        views = [(view(a), view(b)) for a, b in zip(As, Bs)]
+        fns = [(lambda av=av, bv=bv, c=c: _lib.check(L.tenmo_hip_matmul_nd(C.byref(av), C.byref(bv), c.data_ptr(), 0)))
+               for (av, bv), c in zip(views, Cs)]
+        us = hip_time_us(L, _lib, fns, max(flop / 100e6, nbytes / 4e6))
+        err = rel_fro_vs_fp64(torch, Cs[0], As[0], Bs[0])
+        finish_row(name, cfg, "[%s].[%s]" % ("x".join(map(str, a0.shape)), "x".join(map(str, b0.shape))), us, flop, nbytes, err, n)
+        del As, Bs, Cs
+        torch.cuda.empty_cache()
+
+    # ---- config 2: square sweep, A row-major and A as a transposed view (storage [K, M], strides (1, M)) ----
+    for S in (1024, 2048, 4096, 8192):
+        gemm_row("square%d" % S, 2, lambda i, S=S: randn((S, S), 100 + i), lambda i, S=S: randn((S, S), 200 + i), (S, S))
+        gemm_row("square%d_At" % S, 2, lambda i, S=S: randn((S, S), 100 + i).t(), lambda i, S=S: randn((S, S), 200 + i), (S, S))
+
+    # ---- config 3: attention-shaped broadcast-batched products, Q K V dO = [8,12,1024,64], P dS = [8,12,1024,1024] ----
+    bh, T, D = (8, 12), 1024, 64
+    gemm_row("attn_qkt", 3, lambda i: randn(bh + (T, D), 300 + i), lambda i: randn(bh + (T, D), 310 + i).transpose(-1, -2), bh + (T, T))
+    gemm_row("attn_pv", 3, lambda i: torch.softmax(randn(bh + (T, T), 320 + i), -1), lambda i: randn(bh + (T, D), 330 + i), bh + (T, D))
+    gemm_row("attn_dP=dO.Vt", 3, lambda i: randn(bh + (T, D), 340 + i), lambda i: randn(bh + (T, D), 330 + i).transpose(-1, -2), bh + (T, T))
+    gemm_row("attn_dV=Pt.dO", 3, lambda i: torch.softmax(randn(bh + (T, T), 320 + i), -1).transpose(-1, -2), lambda i: randn(bh + (T, D), 340 + i), bh + (T, D))
+    gemm_row("attn_dQ=dS.K", 3, lambda i: randn(bh + (T, T), 350 + i), lambda i: randn(bh + (T, D), 310 + i), bh + (T, D))
+    gemm_row("attn_Qt.dS", 3, lambda i: randn(bh + (T, D), 300 + i).transpose(-1, -2), lambda i: randn(bh + (T, T), 350 + i), bh + (D, T))
+    # README case A[32,512,768] . B[1,768,768] and its backward
+    gemm_row("bcast_fwd", 3, lambda i: randn((32, 512, 768), 360 + i), lambda i: randn((1, 768, 768), 370 + i), (32, 512, 768))
+    gemm_row("bcast_dA=dC.Bt", 3, lambda i: randn((32, 512, 768), 380 + i), lambda i: randn((1, 768, 768), 370 + i).transpose(-1, -2), (32, 512, 768))
+    if wanted("bcast_dB"):
+        # dB = sum over the 32 batches of A_b^T . dC_b through the backward entry (+= into the gradbox of B)
+        nb, M, K, N = 32, 512, 768, 768
+        flop, nbytes = 2.0 * nb * M * K * N, 4.0 * (2 * nb * M * K + K * N)
+        n = copies_for(nbytes)
+        As = [randn((nb, M, K), 360 + i) for i in range(n)]
+        dCs = [randn((nb, M, N), 380 + i) for i in range(n)]
+        Bw = randn((1, K, N), 370)
+        gBs = [torch.zeros((1, K, N), device="cuda") for _ in range(n)]
+        bv = view(Bw)
+        fns = [(lambda av=view(a), dc=dc, g=g: _lib.check(L.tenmo_hip_matmul_backward(C.byref(av), C.byref(bv), dc.data_ptr(), None, g.data_ptr(), 0)))
+               for a, dc, g in zip(As, dCs, gBs)]
+        us = hip_time_us(L, _lib, fns, flop / 100e6)
+        gBs[0].zero_()
+        fns[0]()
+        err = rel_fro_vs_fp64(torch, gBs[0][0], As[0].reshape(-1, K).t(), dCs[0].reshape(-1, N))
+        finish_row("bcast_dB=sum_b(At.dC)", 3, "sum_32 [768x512].[512x768]", us, flop, nbytes, err, n)
+        del As, dCs, gBs
+        torch.cuda.empty_cache()
+
+    # ---- config 4: GPT-2-small linear layers, 8192 tokens: forward, dX = dY.W^T(view), dW = X^T(view).dY ----
+    Tk = 8192
+    for nm, din, dout in (("qkv", 768, 2304), ("proj", 768, 768), ("up", 768, 3072), ("down", 3072, 768), ("lmhead", 768, 50257)):
+        gemm_row("gpt2_%s_fwd" % nm, 4, lambda i, din=din: randn((Tk, din), 400 + i), lambda i, din=din, dout=dout: randn((din, dout), 410 + i, 0.02), (Tk, dout))
+        gemm_row("gpt2_%s_dX" % nm, 4, lambda i, dout=dout: randn((Tk, dout), 420 + i), lambda i, din=din, dout=dout: randn((din, dout), 410 + i, 0.02).t(), (Tk, din))
+        gemm_row("gpt2_%s_dW" % nm, 4, lambda i, din=din: randn((Tk, din), 400 + i).t(), lambda i, dout=dout: randn((Tk, dout), 420 + i), (din, dout))
+
+    # ---- config 5: memory-bound products ----
+    n16 = 16384
+    if wanted("mv") or wanted("vm"):
+        W = randn((n16, n16), 500)
+        x = randn((n16,), 501)
+        o = torch.empty((n16,), device="cuda")
+        nbytes = (n16 * n16 + 2 * n16) * 4.0
+        mv = lambda: _lib.check(L.tenmo_hip_mv_f32(W.data_ptr(), 0, n16, 1, x.data_ptr(), 0, 1, o.data_ptr(), n16, n16, 0, None, None, None, 0, 0))
+        vm = lambda: _lib.check(L.tenmo_hip_vm_f32(x.data_ptr(), 0, 1, W.data_ptr(), 0, n16, 1, o.data_ptr(), n16, n16, 0, None, None, None, 0, 0))
+        for nm, fn, ref in (("mv16384", mv, lambda: W.double() @ x.double()), ("vm16384", vm, lambda: x.double() @ W.double())):
+            if not wanted(nm[:2]):
+                continue
+            us = hip_time_us(L, _lib, [fn], 160.0)
+            r = ref()
+            err = float((o.double() - r).norm() / r.norm())
+            finish_row(nm, 5, "[16384x16384] x [16384]", us, 2.0 * n16 * n16, nbytes, err, 1)
+        del W, x, o
+        torch.cuda.empty_cache()
+    gemm_row("skinny_4x768x50257", 5, lambda i: randn((4, 768), 510 + i), lambda i: randn((768, 50257), 520 + i), (4, 50257))
+    gemm_row("cbow_logits", 5, lambda i: randn((256, 100), 530 + i), lambda i: randn((100, 50000), 540 + i), (256, 50000))
+    gemm_row("cbow_At.dC", 5, lambda i: randn((256, 100), 530 + i).t(), lambda i: randn((256, 50000), 550 + i), (100, 50000))
+    return rows
 
 
 def adjacent_operators(L, _lib, torch):
     """Cross-entropy over GPT-2-sized logits, an SGD step on 2^28 parameters and one convolution layer, forward and
     backward: microseconds per call and fractions of the HBM peak on algorithmic bytes (TFLOP/s for the convolution)."""
+    def hip_time(fn, iters, warm=3):
+        for _ in range(warm):
+            fn()
+        _lib.check(L.tenmo_hip_sync())
+        _lib.check(L.tenmo_hip_timer_begin())
+        for _ in range(iters):
+            fn()
+        ms = C.c_float()
+        _lib.check(L.tenmo_hip_timer_end(C.byref(ms)))
+        return ms.value / iters
+
     res = {}
     M, Cn = 8192, 50257
     x = torch.randn(M, Cn, device="cuda")
@@ -232,22 +360,22 @@ def adjacent_operators(L, _lib, torch):
     fwd = lambda soft: _lib.check(L.tenmo_hip_cross_entropy_forward_f32(x.data_ptr(), t.data_ptr(), 1, M, Cn, -100, 0.0, soft, rows.data_ptr(),
                                                                         tot.data_ptr(), val.data_ptr(), 0))
     by = M * Cn * 4.0
-    ms = hip_time(L, _lib, lambda: fwd(None), 10)
+    ms = hip_time(lambda: fwd(None), 10)
     res["ce_8192x50257_loss_only_us"] = round(ms * 1e3, 1)
     res["ce_8192x50257_loss_only_frac_hbm_peak"] = round(by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 3)
-    ms = hip_time(L, _lib, lambda: fwd(sm.data_ptr()), 10)
+    ms = hip_time(lambda: fwd(sm.data_ptr()), 10)
     res["ce_8192x50257_forward_us"] = round(ms * 1e3, 1)
     res["ce_8192x50257_forward_frac_hbm_peak"] = round(2 * by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 3)
     g = x  # the logits are no longer needed: their storage takes the gradient
-    ms = hip_time(L, _lib, lambda: _lib.check(L.tenmo_hip_cross_entropy_backward_f32(sm.data_ptr(), t.data_ptr(), 1, up.data_ptr(), M, Cn, -100, 0.0, 2, M,
-                                                                                     g.data_ptr(), 0, 0)), 10)
+    ms = hip_time(lambda: _lib.check(L.tenmo_hip_cross_entropy_backward_f32(sm.data_ptr(), t.data_ptr(), 1, up.data_ptr(), M, Cn, -100, 0.0, 2, M,
+                                                                            g.data_ptr(), 0, 0)), 10)
     res["ce_8192x50257_backward_us"] = round(ms * 1e3, 1)
     res["ce_8192x50257_backward_frac_hbm_peak"] = round(2 * by / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 3)
     del x, sm, g
     n = 1 << 28
     p = torch.randn(n, device="cuda")
     gr = torch.randn(n, device="cuda")
-    ms = hip_time(L, _lib, lambda: _lib.check(L.tenmo_hip_sgd_step_f32(p.data_ptr(), gr.data_ptr(), None, n, 0.01, 0.0, 0.0, 0)), 10)
+    ms = hip_time(lambda: _lib.check(L.tenmo_hip_sgd_step_f32(p.data_ptr(), gr.data_ptr(), None, n, 0.01, 0.0, 0.0, 0)), 10)
     res["sgd_2p28_us"] = round(ms * 1e3, 1)
     res["sgd_2p28_frac_hbm_peak"] = round(12.0 * n / (ms * 1e-3) / 1e9 / PEAK_HBM_GBPS, 3)
     del p, gr
@@ -258,13 +386,13 @@ def adjacent_operators(L, _lib, torch):
     ho, wo = h - k + 1, w - k + 1
     out = torch.empty(nb, co, ho, wo, device="cuda")
     flop = 2.0 * nb * co * ho * wo * ci * k * k
-    ms = hip_time(L, _lib, lambda: _lib.check(L.tenmo_hip_conv2d_forward_f32(img.data_ptr(), nb, ci, h, w, ker.data_ptr(), co, k, k, bias.data_ptr(), 1, 1,
-                                                                             out.data_ptr(), 0)), 10)
+    ms = hip_time(lambda: _lib.check(L.tenmo_hip_conv2d_forward_f32(img.data_ptr(), nb, ci, h, w, ker.data_ptr(), co, k, k, bias.data_ptr(), 1, 1,
+                                                                    out.data_ptr(), 0)), 10)
     res["conv_128x64x34x34_k3_to_128_forward_us"] = round(ms * 1e3, 1)
     res["conv_128x64x34x34_k3_to_128_forward_tflops"] = round(flop / (ms * 1e-3) / 1e12, 1)
     gi, gk, gb = torch.empty_like(img), torch.empty_like(ker), torch.empty_like(bias)
-    ms = hip_time(L, _lib, lambda: _lib.check(L.tenmo_hip_conv2d_backward_f32(img.data_ptr(), nb, ci, h, w, ker.data_ptr(), co, k, k, 1, 1, out.data_ptr(),
-                                                                              gi.data_ptr(), gk.data_ptr(), gb.data_ptr(), 0, 0)), 10)
+    ms = hip_time(lambda: _lib.check(L.tenmo_hip_conv2d_backward_f32(img.data_ptr(), nb, ci, h, w, ker.data_ptr(), co, k, k, 1, 1, out.data_ptr(),
+                                                                     gi.data_ptr(), gk.data_ptr(), gb.data_ptr(), 0, 0)), 10)
     res["conv_128x64x34x34_k3_to_128_backward_us"] = round(ms * 1e3, 1)
     res["conv_128x64x34x34_k3_to_128_backward_tflops"] = round(2 * flop / (ms * 1e-3) / 1e12, 1)
     return res

@@ -80,6 +80,10 @@ int tenmo_hip_set_tuning(const char* name, int value);
  * perf_counter_ns around sync=True calls, profile_gpu.mojo:161-258). */
 int tenmo_hip_timer_begin(void);
 int tenmo_hip_timer_end(float* elapsed_ms);
+/* Shader clock under a full matrix-core load, for reporting beside a throughput figure: every CU runs
+ * 4 * rounds fp32 MFMAs per SIMD (64 cycles each) and nothing else, timed with HIP events on the library's stream;
+ * effective_mhz = cycles / time.  Synchronises.  No counterpart in the reference. */
+int tenmo_hip_clock_probe(int32_t rounds, float* effective_mhz);
 
 /* ---- kernel-level entry points ------------------------------------------------------------ */
 

@@ -55,6 +55,7 @@ SIGNATURES = {
     "tenmo_hip_set_tuning": (C.c_int, [C.c_char_p, C.c_int]),
     "tenmo_hip_timer_begin": (C.c_int, []),
     "tenmo_hip_timer_end": (C.c_int, [C.POINTER(C.c_float)]),
+    "tenmo_hip_clock_probe": (C.c_int, [C.c_int32, C.POINTER(C.c_float)]),
     "tenmo_hip_gemm_f32": (C.c_int, [_ptr, C.c_int64, C.c_int64, C.c_int64, _ptr, C.c_int64, C.c_int64, C.c_int64,
                                      _ptr, C.c_int64, C.c_int64, C.c_int64, C.c_int32, _i64p, _i64p, _i64p,
                                      C.c_int32, C.c_int32]),

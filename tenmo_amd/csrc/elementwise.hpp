@@ -8,6 +8,24 @@
 
 namespace tenmo {
 
+// ---- shader-clock probe ---------------------------------------------------------------------------
+// One wavefront per SIMD on every CU runs `n` rounds of four independent v_mfma_f32_32x32x2_f32 and nothing else.
+// An MFMA of this kind occupies the matrix pipe for 16 passes of 4 cycles, so the launch takes 4 * n * 64 shader cycles
+// (plus start-up): cycles / measured time is the clock the chip sustains under a full matrix-core load.
+__global__ __launch_bounds__(256) void clock_probe_kernel(int n, float seed) {
+    f32x16 a0, a1, a2, a3;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) { a0[e] = 0.f; a1[e] = 0.f; a2[e] = 0.f; a3[e] = 0.f; }
+    const float x = seed + (float)threadIdx.x, y = seed * 0.5f;
+    for (int i = 0; i < n; ++i) {
+        a0 = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, a0, 0, 0, 0);
+        a1 = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, a1, 0, 0, 0);
+        a2 = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, a2, 0, 0, 0);
+        a3 = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, a3, 0, 0, 0);
+    }
+    asm volatile("" ::"v"(a0), "v"(a1), "v"(a2), "v"(a3)); // keeps the chains alive without a store
+}
+
 // ---- sum_over_broadcasted_axes (tenmo/sum_mean_reduction.mojo:185-211) fused with the
 // Gradbox "+=" (tenmo/gradbox.mojo:1358-1364): dst[parent shape] += sum over the batch dims that
 // the parent broadcast.  src is dense [batch_shape..., inner]; dst is dense at the parent's shape.

@@ -25,6 +25,7 @@ struct GemvArgs {
     int64_t m_rs, m_cs, v_s;
     int64_t rows, k;       // row kernel: out has `rows` entries per batch, k = reduction length
     int32_t accumulate;
+    int64_t batch0;        // batch index of blockIdx.y == 0 (a grid dimension holds 65535 batches; more go in several launches)
     BatchDesc batch;       // a_str: matrix batch strides, b_str: vector batch strides
 };
 
@@ -46,8 +47,9 @@ __global__ __launch_bounds__(64 * MV_WAVES) void mv_rows_kernel(const GemvArgs g
     const int64_t unit = WPR == 1 ? (int64_t)blockIdx.x * MV_WAVES + wave : (int64_t)blockIdx.x;
     const int64_t row0 = unit * RPW;
     if (row0 >= g.rows) return; // WPR == 4: uniform over the workgroup
+    const int64_t batch = g.batch0 + blockIdx.y;
     int64_t m_off, v_off;
-    batch_offsets(g.batch, blockIdx.y, m_off, v_off);
+    batch_offsets(g.batch, batch, m_off, v_off);
     const float* __restrict vb = g.v + v_off;
     const int64_t k = g.k;
     constexpr int STEP = 64 * WPR * 4;
@@ -108,7 +110,7 @@ __global__ __launch_bounds__(64 * MV_WAVES) void mv_rows_kernel(const GemvArgs g
 #pragma unroll
         for (int j = 0; j < RPW; ++j) acc[j] = fmaf(rowp[j][kx], xe, acc[j]);
     }
-    float* __restrict ob = g.out + (int64_t)blockIdx.y * g.rows + row0;
+    float* __restrict ob = g.out + batch * g.rows + row0;
     if constexpr (WPR == 1) {
 #pragma unroll
         for (int j = 0; j < RPW; ++j) {
@@ -147,6 +149,8 @@ struct ColsArgs {
     int32_t accumulate;
     int32_t k_splits;
     int64_t k_per_split;
+    int64_t batch0;      // batch index of blockIdx.z == 0 (more than 65535 batches go in several launches)
+    int64_t batch_total; // batches of the whole product: the partial sums are laid out [k_splits][batch_total][R][n]
     BatchDesc batch;  // a_str: X batch strides, b_str: Mx batch strides
 };
 
@@ -165,7 +169,7 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
     const int t = threadIdx.x;
     const int64_t col0 = (int64_t)blockIdx.x * COLS_THREADS * 4 + (ALIGNED ? 4 * t : t);
     constexpr int CSTEP = ALIGNED ? 1 : COLS_THREADS; // distance between a lane's 4 columns
-    const int64_t batch = blockIdx.z;
+    const int64_t batch = g.batch0 + blockIdx.z;
     int64_t x_off, m_off;
     batch_offsets(g.batch, batch, x_off, m_off);
     const float* __restrict Xb = g.X + x_off;
@@ -244,7 +248,7 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
     }
     if (!any) return;
     const bool to_partial = g.k_splits > 1;
-    float* __restrict ob = g.out + ((to_partial ? (int64_t)blockIdx.y * gridDim.z : 0) + batch) * g.rows * g.n;
+    float* __restrict ob = g.out + ((to_partial ? (int64_t)blockIdx.y * g.batch_total : 0) + batch) * g.rows * g.n;
     const bool accumulate = g.accumulate && !to_partial;
 #pragma unroll
     for (int r = 0; r < R; ++r) {
@@ -283,7 +287,7 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_shift_kernel(const ColsArgs
     __shared__ float outs[R][COLS_THREADS * 4 + 4];
     const int t = threadIdx.x;
     const int64_t block0 = (int64_t)blockIdx.x * COLS_SHIFT_WIDTH; // first output column of the workgroup
-    const int64_t batch = blockIdx.z;
+    const int64_t batch = g.batch0 + blockIdx.z;
     int64_t x_off, m_off;
     batch_offsets(g.batch, batch, x_off, m_off);
     const float* __restrict Xb = g.X + x_off;
@@ -378,7 +382,7 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_shift_kernel(const ColsArgs
         __syncthreads();
     }
     const bool to_partial = g.k_splits > 1;
-    float* __restrict ob = g.out + ((to_partial ? (int64_t)blockIdx.y * gridDim.z : 0) + batch) * g.rows * g.n;
+    float* __restrict ob = g.out + ((to_partial ? (int64_t)blockIdx.y * g.batch_total : 0) + batch) * g.rows * g.n;
     const bool accumulate = g.accumulate && !to_partial;
     for (int r = 0; r < R; ++r) {
         if (r >= g.rows) break;
@@ -396,13 +400,14 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_shift_kernel(const ColsArgs
 __global__ void mv_generic_kernel(const GemvArgs g) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i >= g.rows) return;
+    const int64_t batch = g.batch0 + blockIdx.y;
     int64_t m_off, v_off;
-    batch_offsets(g.batch, blockIdx.y, m_off, v_off);
+    batch_offsets(g.batch, batch, m_off, v_off);
     const float* Mb = g.Mx + m_off + i * g.m_rs;
     const float* vb = g.v + v_off;
     float acc = 0.f;
     for (int64_t j = 0; j < g.k; ++j) acc = fmaf(Mb[j * g.m_cs], vb[j * g.v_s], acc);
-    float* o = g.out + (int64_t)blockIdx.y * g.rows + i;
+    float* o = g.out + batch * g.rows + i;
     *o = g.accumulate ? *o + acc : acc;
 }
 

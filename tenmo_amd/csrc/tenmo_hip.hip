@@ -67,6 +67,8 @@ struct State {
     float* stage[3] = {nullptr, nullptr, nullptr};
     size_t stage_bytes[3] = {0, 0, 0};
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
+    bool capturing = false;  // a stream capture is open: the scratch cannot grow (no allocation inside a capture)
+    size_t ws_wanted = 0;    // what a kernel selection inside a capture asked of the first scratch buffer
     float* one = nullptr; // device constant 1.0f: a stride-0 vector of ones for column sums
     int32_t* conv_tables = nullptr;  // offset tables [C_in*KH*KW | H_out*W_out] of the last convolution geometry
     size_t conv_tables_len = 0;      // capacity in entries
@@ -94,6 +96,10 @@ int ensure_ready() {
 }
 
 int workspace(size_t bytes, float** out) {
+    if (bytes > S.ws_bytes && S.capturing) { // the caller ends the capture, grows the buffer and captures again
+        S.ws_wanted = std::max(S.ws_wanted, bytes);
+        return fail(TENMO_ERR_HIP, "library scratch of %zu bytes wanted inside a stream capture (have %zu)", bytes, S.ws_bytes);
+    }
     if (bytes > S.ws_bytes) {
         if (S.ws) {
             HIP_TRY(hipStreamSynchronize(S.stream));
@@ -456,9 +462,19 @@ void launch_cols(const ColsArgs& c, dim3 grid, int variant) {
     else if constexpr (R <= 4) hipLaunchKernelGGL((cols_shift_kernel<R>), grid, dim3(COLS_THREADS), 0, S.stream, c);
 }
 
+// largest batch count of one launch (a grid's y and z dimensions hold 65535)
+constexpr int64_t kMaxGridBatches = 65535;
+
+// Scratch for the K-slice partial sums of a column-streaming product: the library's grow-only buffer, or a
+// fixed buffer the caller brings (the allocation-free entry point), which is never grown.
+struct ScratchSource {
+    float* fixed = nullptr;
+    size_t fixed_bytes = 0;
+};
+
 // Runs the column-streaming product described by `c` (c.out is set here): picks the kernel variant,
 // cuts K into slices when the column blocks alone would not fill the chip, and adds the slices.
-int cols_run(ColsArgs c, int64_t batch_count, float* out, int accumulate) {
+int cols_run(ColsArgs c, int64_t batch_count, float* out, int accumulate, const ScratchSource& scratch_src = ScratchSource()) {
     const int variant = cols_aligned(c) ? 0 : cols_shiftable(c) ? 1 : 2; // 16-byte loads / shifted sets / dword loads
     const int64_t width = variant == 1 ? COLS_SHIFT_WIDTH : COLS_THREADS * 4;
     const int64_t col_blocks = (c.n + width - 1) / width;
@@ -472,18 +488,29 @@ int cols_run(ColsArgs c, int64_t batch_count, float* out, int accumulate) {
     splits = (K + per - 1) / per;
     c.k_splits = (int32_t)splits; c.k_per_split = per;
     c.accumulate = accumulate;
+    c.batch_total = batch_count;
     float* target = out;
     if (splits > 1) {
+        const size_t bytes = (size_t)splits * batch_count * R * c.n * sizeof(float);
         float* ws;
-        if (int rc = workspace((size_t)splits * batch_count * R * c.n * sizeof(float), &ws)) return rc;
+        if (scratch_src.fixed) {
+            if (bytes > scratch_src.fixed_bytes)
+                return fail(TENMO_ERR_UNSUPPORTED, "the partial sums of %lld K slices x %lld batches x %lld rows x %lld columns need %zu bytes of scratch; "
+                            "the static buffer of the allocation-free entry point holds %zu", (long long)splits, (long long)batch_count, (long long)R,
+                            (long long)c.n, bytes, scratch_src.fixed_bytes);
+            ws = scratch_src.fixed;
+        } else if (int rc = workspace(bytes, &ws)) return rc;
         target = ws;
     }
     c.out = target;
-    const dim3 grid((unsigned)col_blocks, (unsigned)splits, (unsigned)batch_count);
-    if (R <= 1) launch_cols<1>(c, grid, variant);
-    else if (R <= 2) launch_cols<2>(c, grid, variant);
-    else if (R <= 4) launch_cols<4>(c, grid, variant);
-    else launch_cols<8>(c, grid, variant);
+    for (int64_t b0 = 0; b0 < batch_count; b0 += kMaxGridBatches) {
+        c.batch0 = b0;
+        const dim3 grid((unsigned)col_blocks, (unsigned)splits, (unsigned)std::min(kMaxGridBatches, batch_count - b0));
+        if (R <= 1) launch_cols<1>(c, grid, variant);
+        else if (R <= 2) launch_cols<2>(c, grid, variant);
+        else if (R <= 4) launch_cols<4>(c, grid, variant);
+        else launch_cols<8>(c, grid, variant);
+    }
     if (splits > 1) {
         const int64_t n = batch_count * R * c.n;
         hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
@@ -493,18 +520,30 @@ int cols_run(ColsArgs c, int64_t batch_count, float* out, int accumulate) {
 }
 
 template <int WPR, int RPW, int UNROLL>
-void launch_rows(const GemvArgs& g, int64_t batch_count) {
+void launch_rows(GemvArgs g, int64_t batch_count) {
     const int64_t units = (g.rows + RPW - 1) / RPW;
-    const dim3 grid((unsigned)(WPR == 1 ? (units + MV_WAVES - 1) / MV_WAVES : units), (unsigned)batch_count);
-    if (g.v_s == 1) hipLaunchKernelGGL((mv_rows_kernel<WPR, RPW, UNROLL, true>), grid, dim3(64 * MV_WAVES), 0, S.stream, g);
-    else hipLaunchKernelGGL((mv_rows_kernel<WPR, RPW, UNROLL, false>), grid, dim3(64 * MV_WAVES), 0, S.stream, g);
+    for (int64_t b0 = 0; b0 < batch_count; b0 += kMaxGridBatches) {
+        g.batch0 = b0;
+        const dim3 grid((unsigned)(WPR == 1 ? (units + MV_WAVES - 1) / MV_WAVES : units), (unsigned)std::min(kMaxGridBatches, batch_count - b0));
+        if (g.v_s == 1) hipLaunchKernelGGL((mv_rows_kernel<WPR, RPW, UNROLL, true>), grid, dim3(64 * MV_WAVES), 0, S.stream, g);
+        else hipLaunchKernelGGL((mv_rows_kernel<WPR, RPW, UNROLL, false>), grid, dim3(64 * MV_WAVES), 0, S.stream, g);
+    }
+}
+
+// one thread per output, any strides; grid.x blocks of 256 outputs per batch
+void launch_generic(GemvArgs g, int64_t batch_count) {
+    for (int64_t b0 = 0; b0 < batch_count; b0 += kMaxGridBatches) {
+        g.batch0 = b0;
+        hipLaunchKernelGGL(mv_generic_kernel, dim3((unsigned)((g.rows + 255) / 256), (unsigned)std::min(kMaxGridBatches, batch_count - b0)), dim3(256), 0, S.stream, g);
+    }
 }
 
 // out[b][i] = sum_j Mat[b](i, j) * vec[b](j), i < n_out, j < n_red;  Mat(i,j) = Mx[i*out_s + j*red_s]
 int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* vec, int64_t v_s, float* out,
-                    int64_t n_out, int64_t n_red, const BatchDesc& bd_mat_vec, int64_t batch_count, int accumulate) {
+                    int64_t n_out, int64_t n_red, const BatchDesc& bd_mat_vec, int64_t batch_count, int accumulate,
+                    const ScratchSource& scratch_src = ScratchSource()) {
     if (n_out == 0 || batch_count == 0) return 0;
-    if (batch_count > 65535) return fail(TENMO_ERR_UNSUPPORTED, "more than 65535 batches in mv/vm");
+    if (batch_count > 0x7fffffffLL) return fail(TENMO_ERR_UNSUPPORTED, "more than 2^31 batches in mv/vm");
     if (n_red == 0) {
         if (!accumulate) {
             const int64_t n = batch_count * n_out;
@@ -518,7 +557,7 @@ int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* 
         g.m_rs = out_s; g.m_cs = 1; g.v_s = v_s; g.rows = n_out; g.k = n_red; g.accumulate = accumulate; g.batch = bd_mat_vec;
         if (n_red == 1 && red_s != 1) { // degenerate: a single product per output
             g.m_cs = red_s;
-            hipLaunchKernelGGL(mv_generic_kernel, dim3((unsigned)((n_out + 255) / 256), (unsigned)batch_count), dim3(256), 0, S.stream, g);
+            launch_generic(g, batch_count);
             return 0;
         }
         // long rows: the whole workgroup walks 4 rows (bursts of 32 KiB per row); shorter rows get shorter
@@ -536,7 +575,7 @@ int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* 
             GemvArgs g{};
             g.Mx = Mx; g.v = vec; g.out = out;
             g.m_rs = out_s; g.m_cs = red_s; g.v_s = v_s; g.rows = n_out; g.k = n_red; g.accumulate = accumulate; g.batch = bd_mat_vec;
-            hipLaunchKernelGGL(mv_generic_kernel, dim3(1, (unsigned)batch_count), dim3(256), 0, S.stream, g);
+            launch_generic(g, batch_count);
             return 0;
         }
         ColsArgs c{};
@@ -545,13 +584,13 @@ int matvec_dispatch(const float* Mx, int64_t out_s, int64_t red_s, const float* 
         // in ColsArgs the X operand uses a_str and the matrix b_str: swap relative to (matrix, vector)
         c.batch = bd_mat_vec;
         for (int d = 0; d < MAX_BATCH_RANK; ++d) std::swap(c.batch.a_str[d], c.batch.b_str[d]);
-        if (int rc = cols_run(c, batch_count, out, accumulate)) return rc;
+        if (int rc = cols_run(c, batch_count, out, accumulate, scratch_src)) return rc;
         return 0;
     }
     GemvArgs g{};
     g.Mx = Mx; g.v = vec; g.out = out;
     g.m_rs = out_s; g.m_cs = red_s; g.v_s = v_s; g.rows = n_out; g.k = n_red; g.accumulate = accumulate; g.batch = bd_mat_vec;
-    hipLaunchKernelGGL(mv_generic_kernel, dim3((unsigned)((n_out + 255) / 256), (unsigned)batch_count), dim3(256), 0, S.stream, g);
+    launch_generic(g, batch_count);
     return 0;
 }
 
@@ -592,6 +631,15 @@ int skinny_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, 
     c.batch = bd;
     if (int rc = cols_run(c, batch_count, C, accumulate)) return rc;
     return 0;
+}
+
+// C (+)= A . B: a few rows against a wide row-major B is HBM-bound and streams B once through the column kernel;
+// everything else goes to the matrix cores
+int product_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, int64_t b_rs, int64_t b_cs, float* C,
+                     int64_t M, int64_t N, int64_t K, const BatchDesc& bd, int64_t batch_count, int accumulate, const Epilogue& ep = Epilogue()) {
+    if (M >= 1 && M <= 8 && (b_cs == 1 || N == 1) && N >= 2048 && K > 0 && batch_count > 0 && !ep.any() && !ep.gather_row)
+        return skinny_dispatch(A, a_rs, a_cs, B, b_rs, C, M, N, K, bd, batch_count, accumulate);
+    return gemm_dispatch(A, a_rs, a_cs, B, b_rs, b_cs, C, M, N, K, bd, batch_count, accumulate, ep);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -721,9 +769,7 @@ int matmul_views(const tenmo_view* A, const tenmo_view* B, float* C, int accumul
     const float* Bp = B->data + B->offset;
     const int64_t a_rs = A->strides[A->rank - 2], a_cs = A->strides[A->rank - 1];
     const int64_t b_rs = B->strides[B->rank - 2], b_cs = B->strides[B->rank - 1];
-    if (M <= 8 && (b_cs == 1 || N == 1) && N >= 2048 && K > 0 && !ep.any())
-        return skinny_dispatch(Ap, a_rs, a_cs, Bp, b_rs, C, M, N, K, bd, batch_count, accumulate);
-    return gemm_dispatch(Ap, a_rs, a_cs, Bp, b_rs, b_cs, C, M, N, K, bd, batch_count, accumulate, ep);
+    return product_dispatch(Ap, a_rs, a_cs, Bp, b_rs, b_cs, C, M, N, K, bd, batch_count, accumulate, ep);
 }
 
 // dst (dense, parent's shape) += sum over the batch dims of `full` that the parent broadcast
@@ -916,6 +962,22 @@ int tenmo_hip_timer_end(float* ms) {
     return 0;
 }
 
+int tenmo_hip_clock_probe(int32_t rounds, float* effective_mhz) {
+    if (int rc = ensure_ready()) return rc;
+    if (rounds < 1 || !effective_mhz) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_clock_probe: needs rounds >= 1 and a result pointer");
+    hipLaunchKernelGGL(clock_probe_kernel, dim3((unsigned)S.cus), dim3(256), 0, S.stream, 1000, 1.0f); // brings the clocks up
+    HIP_TRY(hipEventRecord(S.ev0, S.stream));
+    hipLaunchKernelGGL(clock_probe_kernel, dim3((unsigned)S.cus), dim3(256), 0, S.stream, (int)rounds, 1.0f);
+    HIP_TRY(hipEventRecord(S.ev1, S.stream));
+    HIP_TRY(hipEventSynchronize(S.ev1));
+    float ms = 0.f;
+    HIP_TRY(hipEventElapsedTime(&ms, S.ev0, S.ev1));
+    HIP_TRY(hipGetLastError());
+    if (!(ms > 0.f)) return fail(TENMO_ERR_HIP, "tenmo_hip_clock_probe: no elapsed time");
+    *effective_mhz = (float)(4.0 * rounds * 64.0 / (ms * 1e-3) / 1e6);
+    return 0;
+}
+
 int tenmo_hip_gemm_f32(const float* A, int64_t a_off, int64_t a_rs, int64_t a_cs,
                        const float* B, int64_t b_off, int64_t b_rs, int64_t b_cs,
                        float* C, int64_t M, int64_t N, int64_t K,
@@ -929,7 +991,7 @@ int tenmo_hip_gemm_f32(const float* A, int64_t a_off, int64_t a_rs, int64_t a_cs
     BatchDesc bd{};
     int64_t count = 1;
     if (int rc = fill_batch(bd, batch_rank, batch_shape, a_batch_strides, b_batch_strides, &count)) return rc;
-    if (int rc = gemm_dispatch(A + a_off, a_rs, a_cs, B + b_off, b_rs, b_cs, C, M, N, K, bd, count, accumulate)) return rc;
+    if (int rc = product_dispatch(A + a_off, a_rs, a_cs, B + b_off, b_rs, b_cs, C, M, N, K, bd, count, accumulate)) return rc;
     return finish(sync);
 }
 
@@ -1756,13 +1818,23 @@ int tenmo_hip_mlp_step_graph(tenmo_mlp* m, const float* x, const int32_t* y, int
     float* ws;
     if (int rc = workspace(1, &ws)) return rc; // scratch must exist before capture: no allocation may happen inside it
     // the captured kernels hold the scratch pointer: a capture made before the scratch buffer grew is stale
-    if (!m->exec || m->g_batch != B || m->g_lr != lr || m->g_loss != loss_out || m->g_ws != ws) {
+    for (int attempt = 0; !m->exec || m->g_batch != B || m->g_lr != lr || m->g_loss != loss_out || m->g_ws != ws; ++attempt) {
         if (m->exec) { HIP_TRY(hipStreamSynchronize(S.stream)); HIP_TRY(hipGraphExecDestroy(m->exec)); m->exec = nullptr; }
         HIP_TRY(hipStreamBeginCapture(S.stream, hipStreamCaptureModeThreadLocal));
+        S.capturing = true; S.ws_wanted = 0;
         const int rc = mlp_step_enqueue(m, m->x_stage, m->y_stage, B, lr, loss_out);
+        S.capturing = false;
         hipGraph_t graph = nullptr;
         const hipError_t e = hipStreamEndCapture(S.stream, &graph);
-        if (rc) { if (graph) (void)hipGraphDestroy(graph); return rc; }
+        if (rc) {
+            if (graph) (void)hipGraphDestroy(graph);
+            // a kernel selection wanted more scratch than there is: grow it out here, where allocating is allowed, and capture again
+            if (S.ws_wanted > S.ws_bytes && attempt < 4) {
+                if (int rc2 = workspace(S.ws_wanted, &ws)) return rc2;
+                continue;
+            }
+            return rc;
+        }
         if (e != hipSuccess) return fail(TENMO_ERR_HIP, "hipStreamEndCapture failed: %s", hipGetErrorString(e));
         const hipError_t ei = hipGraphInstantiate(&m->exec, graph, nullptr, nullptr, 0);
         (void)hipGraphDestroy(graph);

@@ -12,6 +12,31 @@ def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a gfx950 GPU (run with -m gpu on the GPU machine)")
 
 
+def _gpu_unavailable_reason():
+    """None when the GPU tests can run here: a gfx950 device and the built HIP library."""
+    lib = os.path.join(ROOT, "tenmo_amd", "libtenmo_hip.so")
+    if not os.path.exists(os.environ.get("TENMO_HIP_LIBRARY") or lib):
+        return "libtenmo_hip.so is not built (python -m tenmo_amd.build)"
+    try:
+        import torch
+    except ImportError:
+        return "torch is not importable"
+    if not torch.cuda.is_available():
+        return "no GPU visible to this process"
+    return None
+
+
+def pytest_collection_modifyitems(config, items):
+    gpu_items = [it for it in items if it.get_closest_marker("gpu")]
+    if not gpu_items:
+        return
+    reason = _gpu_unavailable_reason()
+    if reason:
+        skip = pytest.mark.skip(reason="gpu test: " + reason)
+        for it in gpu_items:
+            it.add_marker(skip)
+
+
 @pytest.fixture(scope="session")
 def golden():
     import json

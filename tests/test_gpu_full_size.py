@@ -152,11 +152,33 @@ def test_gpt2_linears(env, name, N):
 
 
 def test_mlp_down_projection(env):
+    """config: the MLP down projection [8192,3072].[3072,768], forward and both gradient products
+    dX = dY.W^T(view) and dW = X^T(view).dY, through the plain entry and through the backward entry (+=)."""
     E = env
-    X, W = randn(E, (8192, 3072), 14), randn(E, (3072, 768), 15, 0.02)
-    Y = E.t.empty(8192, 768, device="cuda")
-    gemm(E, X, (3072, 1), W, (768, 1), Y, 8192, 768, 3072)
-    assert sampled_rows_error(E, Y, X, W, [1, 5000, 8190]) <= RTOL_FRO
+    Tk, D, N = 8192, 3072, 768
+    X, W, dY = randn(E, (Tk, D), 14), randn(E, (D, N), 15, 0.02), randn(E, (Tk, N), 23)
+    Y = E.t.empty(Tk, N, device="cuda")
+    gemm(E, X, (D, 1), W, (N, 1), Y, Tk, N, D)
+    rows = [1, 5000, 8190]
+    assert sampled_rows_error(E, Y, X, W, rows) <= RTOL_FRO
+    idx = E.t.tensor(rows, device="cuda")
+    dX = E.t.empty(Tk, D, device="cuda")
+    gemm(E, dY, (N, 1), W, (1, N), dX, Tk, D, N)                      # [8192,768] . [768,3072] as a transposed view
+    ref_dx = (dY[idx].double() @ W.double().T).cpu().numpy()
+    assert rel_fro(dX[idx].cpu().numpy(), ref_dx) <= RTOL_FRO
+    dW = E.t.empty(D, N, device="cuda")
+    gemm(E, X, (1, D), dY, (N, 1), dW, D, N, Tk)                      # [3072,8192] transposed view . [8192,768]
+    ridx = E.t.tensor([0, 1535, 3071], device="cuda")
+    ref_dw = (X[:, ridx].double().T @ dY.double()).cpu().numpy()
+    assert rel_fro(dW[ridx].cpu().numpy(), ref_dw) <= RTOL_FRO
+    # the backward entry accumulates into the gradboxes: called twice it leaves exactly twice the gradient
+    xv = E.lib.make_view(X.data_ptr(), 0, X.shape, X.stride())
+    wv = E.lib.make_view(W.data_ptr(), 0, W.shape, W.stride())
+    gX, gW = E.t.zeros_like(X), E.t.zeros_like(W)
+    E.lib.check(E.L.tenmo_hip_matmul_backward(C.byref(xv), C.byref(wv), dY.data_ptr(), gX.data_ptr(), gW.data_ptr(), 0))
+    assert rel_fro(gX[idx].cpu().numpy(), ref_dx) <= RTOL_FRO and rel_fro(gW[ridx].cpu().numpy(), ref_dw) <= RTOL_FRO
+    E.lib.check(E.L.tenmo_hip_matmul_backward(C.byref(xv), C.byref(wv), dY.data_ptr(), gX.data_ptr(), gW.data_ptr(), 0))
+    assert rel_fro(gX[idx].cpu().numpy(), 2 * ref_dx) <= RTOL_FRO and rel_fro(gW[ridx].cpu().numpy(), 2 * ref_dw) <= RTOL_FRO
 
 
 def test_memory_bound_cases(env):

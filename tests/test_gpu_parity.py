@@ -1283,6 +1283,95 @@ def test_products_with_more_than_2_31_elements(T):
     assert torch.equal(out.double(), ref), "vm"
 
 
+def test_more_batches_than_a_grid_dimension(T):
+    """mv, vm and a skinny product over more than 65535 batches (a grid's y / z dimension holds 65535): the
+    launches are cut into groups of batches; checked against einsum in fp64."""
+    import torch
+    from tenmo_amd import _lib
+    L = _lib.load()
+    rng = np.random.default_rng(71)
+    nb = 70001
+    # mv, row kernel: M[nb, 3, 8] . v[nb, 8]
+    M = rng.standard_normal((nb, 3, 8), dtype=np.float32)
+    v = rng.standard_normal((nb, 8), dtype=np.float32)
+    Md, vd = torch.from_numpy(M).cuda(), torch.from_numpy(v).cuda()
+    out = torch.empty((nb, 3), device="cuda")
+    _lib.check(L.tenmo_hip_mv_f32(Md.data_ptr(), 0, 8, 1, vd.data_ptr(), 0, 1, out.data_ptr(), 3, 8, 1, _lib.i64([nb]), _lib.i64([24]), _lib.i64([8]), 0, 1))
+    assert rel_fro(out.cpu().numpy(), np.einsum("bmk,bk->bm", M.astype(np.float64), v.astype(np.float64))) <= RTOL_FRO
+    # vm, column kernel: v[nb, 3] . M[nb, 3, 8]
+    v3 = rng.standard_normal((nb, 3), dtype=np.float32)
+    v3d = torch.from_numpy(v3).cuda()
+    out = torch.empty((nb, 8), device="cuda")
+    _lib.check(L.tenmo_hip_vm_f32(v3d.data_ptr(), 0, 1, Md.data_ptr(), 0, 8, 1, out.data_ptr(), 3, 8, 1, _lib.i64([nb]), _lib.i64([3]), _lib.i64([24]), 0, 1))
+    assert rel_fro(out.cpu().numpy(), np.einsum("bk,bkn->bn", v3.astype(np.float64), M.astype(np.float64))) <= RTOL_FRO
+    # generic strides (both non-unit): one thread per output
+    out = torch.empty((nb, 2), device="cuda")
+    _lib.check(L.tenmo_hip_mv_f32(Md.data_ptr(), 0, 8, 2, vd.data_ptr(), 0, 2, out.data_ptr(), 2, 4, 1, _lib.i64([nb]), _lib.i64([24]), _lib.i64([8]), 0, 1))
+    assert rel_fro(out.cpu().numpy(), np.einsum("bmk,bk->bm", M[:, :2, ::2].astype(np.float64), v[:, ::2].astype(np.float64))) <= RTOL_FRO
+    # skinny product [2, 4] . [4, 2048] per batch through the view-level entry
+    nb2 = 66000
+    A = rng.standard_normal((nb2, 2, 4), dtype=np.float32)
+    B = rng.standard_normal((4, 2048), dtype=np.float32)
+    got = T.Tensor.from_numpy(A).matmul(T.Tensor.from_numpy(B), track_grad=False).to_numpy()
+    assert rel_fro(got, ref_matmul64(A, B)) <= RTOL_FRO
+
+
+def test_kernel_level_entry_routes_skinny_products(T):
+    """tenmo_hip_gemm_f32 and tenmo_hip_matmul_nd choose the same kernel for a few rows against a wide
+    row-major matrix (the column-streaming one): identical results."""
+    import torch
+    from tenmo_amd import _lib
+    L = _lib.load()
+    rng = np.random.default_rng(73)
+    a = rng.standard_normal((4, 768), dtype=np.float32)
+    b = rng.standard_normal((768, 50257), dtype=np.float32)
+    via_views = T.Tensor.from_numpy(a).matmul(T.Tensor.from_numpy(b), track_grad=False).to_numpy()
+    Ad, Bd = torch.from_numpy(a).cuda(), torch.from_numpy(b).cuda()
+    out = torch.empty((4, 50257), device="cuda")
+    _lib.check(L.tenmo_hip_gemm_f32(Ad.data_ptr(), 0, 768, 1, Bd.data_ptr(), 0, 50257, 1, out.data_ptr(), 4, 50257, 768, 0, None, None, None, 0, 1))
+    assert np.array_equal(out.cpu().numpy(), via_views)
+    assert rel_fro(via_views, ref_matmul64(a, b)) <= RTOL_FRO
+
+
+def test_clock_probe(T):
+    from tenmo_amd import _lib
+    L = _lib.load()
+    mhz = C.c_float()
+    _lib.check(L.tenmo_hip_clock_probe(20000, C.byref(mhz)))
+    assert 500.0 < mhz.value < 2600.0, mhz.value   # MI355X: 2400 MHz peak engine clock
+    assert L.tenmo_hip_clock_probe(0, C.byref(mhz)) == -3
+
+
+def test_zz_graph_capture_grows_scratch(T, oracle):
+    """A captured training step whose kernel selection wants more library scratch than exists when the capture starts:
+    the capture is abandoned, the scratch grown outside it and the step captured again — same losses as the eager step."""
+    from tenmo_amd import _lib, rng as R
+    from tenmo_amd.net import MLP
+    L = _lib.load()
+    _lib.check(L.tenmo_hip_shutdown())   # the scratch is grow-only: start from none
+    _lib._initialised = False
+    _lib.init(0)
+    dims, seed, lr, batch = [2048, 1024, 10], 5, 0.01, 1024
+    Ws, bs = R.xavier_mlp(dims, seed)
+    eager, graph = MLP(dims, Ws, bs, batch), MLP(dims, Ws, bs, batch)
+    # stream-K with the 256x128 tile keeps 2 partial tiles per workgroup: 2 * 512 * 256 * 128 * 4 B = 128 MiB of scratch
+    _lib.check(L.tenmo_hip_set_tuning(b"gemm_tile", 0))
+    _lib.check(L.tenmo_hip_set_tuning(b"gemm_streamk", 2))
+    try:
+        rng = np.random.default_rng(seed)
+        x = rng.random((batch, dims[0]), dtype=np.float32)
+        y = rng.integers(0, 10, batch).astype(np.int32)
+        lg = graph.step(x, y, lr, graph=True)      # the first library call after the re-initialisation
+        le = eager.step(x, y, lr)
+        assert lg == le
+        assert graph.step(x, y, lr, graph=True) == eager.step(x, y, lr)
+    finally:
+        _lib.check(L.tenmo_hip_set_tuning(b"gemm_tile", -1))
+        _lib.check(L.tenmo_hip_set_tuning(b"gemm_streamk", -1))
+    for l in range(2):
+        np.testing.assert_array_equal(eager.params(l)[0], graph.params(l)[0])
+
+
 def test_zz_shutdown_and_reinit(T):
     """tenmo_hip_shutdown releases the library's stream and scratch; after tenmo_hip_init everything works again and
     gives the same results (split-K workspace, column-kernel partial sums and the convolution tables are re-grown)."""
