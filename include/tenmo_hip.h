@@ -134,6 +134,22 @@ int tenmo_hip_vm_f32(const float* v, int64_t v_off, int64_t v_s,
                      const int64_t* v_batch_strides, const int64_t* m_batch_strides,
                      int32_t accumulate, int32_t sync);
 
+/* tenmo_hip_vm_f32 for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference.  Same arguments, same kernels and
+ * bit-identical results; the only difference is where the partial sums of the K slices live: a static device
+ * array of TENMO_VM_NOALLOC_SCRATCH_BYTES that every GPU the library runs on holds until the process ends, instead
+ * of the library's grow-only scratch.  The call allocates and frees nothing.  A product whose partial sums
+ * (K slices x batches x n floats; the slice count follows the "cols_wg_per_cu" knob) exceed the array is refused with
+ * TENMO_ERR_UNSUPPORTED and a message giving both sizes; with the default knob every shape fits.  Every call on a
+ * GPU shares that GPU's array: calls that overlap in time on one GPU (two streams, two threads) race. */
+#define TENMO_VM_NOALLOC_SCRATCH_BYTES (8u << 20)
+int tenmo_hip_vm_f32_noalloc(const float* v, int64_t v_off, int64_t v_s,
+                             const float* Mx, int64_t m_off, int64_t m_rs, int64_t m_cs,
+                             float* out, int64_t k, int64_t n,
+                             int32_t batch_rank, const int64_t* batch_shape,
+                             const int64_t* v_batch_strides, const int64_t* m_batch_strides,
+                             int32_t accumulate, int32_t sync);
+
 /* out[c] (+)= sum over r < rows of G[g_off + r*g_rs + c], c < cols: the bias gradient of a Linear
  * layer, i.e. the upstream gradient summed over its broadcast (row) axis — what
  * sum_over_broadcasted_axes does for the bias operand of Adder (tenmo/broadcast.mojo:66-88,

@@ -66,6 +66,8 @@ SIGNATURES = {
                                    C.c_int64, C.c_int64, C.c_int32, _i64p, _i64p, _i64p, C.c_int32, C.c_int32]),
     "tenmo_hip_vm_f32": (C.c_int, [_ptr, C.c_int64, C.c_int64, _ptr, C.c_int64, C.c_int64, C.c_int64, _ptr,
                                    C.c_int64, C.c_int64, C.c_int32, _i64p, _i64p, _i64p, C.c_int32, C.c_int32]),
+    "tenmo_hip_vm_f32_noalloc": (C.c_int, [_ptr, C.c_int64, C.c_int64, _ptr, C.c_int64, C.c_int64, C.c_int64, _ptr,
+                                           C.c_int64, C.c_int64, C.c_int32, _i64p, _i64p, _i64p, C.c_int32, C.c_int32]),
     "tenmo_hip_column_sum_f32": (C.c_int, [_ptr, C.c_int64, C.c_int64, C.c_int64, C.c_int64, _ptr, C.c_int32, C.c_int32]),
     "tenmo_hip_dot_f32": (C.c_int, [_ptr, C.c_int64, C.c_int64, _ptr, C.c_int64, C.c_int64, C.c_int64, _ptr, C.c_int32]),
     "tenmo_hip_classify_matmul": (C.c_int, [C.c_int32, _i64p, C.c_int32, _i64p]),

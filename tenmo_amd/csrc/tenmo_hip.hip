@@ -30,7 +30,16 @@
 
 using namespace tenmo;
 
+// Device memory of the allocation-free entry point (tenmo_hip_vm_f32_noalloc): the partial sums of its K slices.
+// One copy per GPU, at its own address there, held until the process ends.  Host code never uses this name as an
+// address: tenmo_hip_init asks each device for the array's address once and keeps it in `g_scratch_ptr`.
+constexpr size_t TENMO_STATIC_SCRATCH_BYTES = TENMO_VM_NOALLOC_SCRATCH_BYTES;
+static __device__ __align__(256) float scratch[TENMO_STATIC_SCRATCH_BYTES / sizeof(float)];
+
 namespace {
+
+constexpr int kMaxDevices = 64;
+float* g_scratch_ptr[kMaxDevices] = {nullptr}; // device id -> address of `scratch` on that device (survives shutdown / re-init)
 
 thread_local std::string t_err;
 
@@ -886,6 +895,12 @@ int tenmo_hip_init(int device_id) {
     S.stream = S.own_stream;
     HIP_TRY(hipEventCreate(&S.ev0));
     HIP_TRY(hipEventCreate(&S.ev1));
+    // address of the static scratch array on THIS device (each GPU holds its own copy); asked for once per device
+    if (device_id < kMaxDevices && !g_scratch_ptr[device_id]) {
+        float* p = nullptr;
+        HIP_TRY(hipGetSymbolAddress((void**)&p, HIP_SYMBOL(scratch)));
+        g_scratch_ptr[device_id] = p;
+    }
     HIP_TRY(hipMalloc(&S.one, sizeof(float)));
     const float one = 1.0f;
     HIP_TRY(hipMemcpy(S.one, &one, sizeof one, hipMemcpyHostToDevice));
@@ -1048,6 +1063,32 @@ int tenmo_hip_vm_f32(const float* v, int64_t v_off, int64_t v_s,
     if ((!Mx || !v) && n * k * count > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_vm_f32: null operand");
     // out[j] = sum_i Mx(i, j) v(i): outputs walk the matrix columns, the reduction walks its rows
     if (int rc = matvec_dispatch(Mx + m_off, m_cs, m_rs, v + v_off, v_s, out, n, k, bd, count, accumulate)) return rc;
+    return finish(sync);
+}
+
+// tenmo_hip_vm_f32 for callers that cannot allocate: the K-slice partial sums go to the static device array
+// `scratch` (through the address this device reported at init) instead of the grow-only library buffer.  No
+// hipMalloc / hipFree on this path; every partial sum the slice reduction reads is written by the launch before it,
+// so nothing has to be cleared between calls.
+int tenmo_hip_vm_f32_noalloc(const float* v, int64_t v_off, int64_t v_s,
+                             const float* Mx, int64_t m_off, int64_t m_rs, int64_t m_cs,
+                             float* out, int64_t k, int64_t n,
+                             int32_t batch_rank, const int64_t* batch_shape,
+                             const int64_t* v_batch_strides, const int64_t* m_batch_strides,
+                             int32_t accumulate, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    if (n < 0 || k < 0) return fail(TENMO_ERR_INVALID_SHAPE, "tenmo_hip_vm_f32_noalloc: negative dimension");
+    if (S.device < 0 || S.device >= kMaxDevices || !g_scratch_ptr[S.device])
+        return fail(TENMO_ERR_NOT_INITIALIZED, "tenmo_hip_vm_f32_noalloc: no static scratch address for device %d", S.device);
+    BatchDesc bd{};
+    int64_t count = 1;
+    if (int rc = fill_batch(bd, batch_rank, batch_shape, m_batch_strides, v_batch_strides, &count)) return rc;
+    if (int rc = need(out, n * count > 0, "tenmo_hip_vm_f32_noalloc", "result pointer")) return rc;
+    if ((!Mx || !v) && n * k * count > 0) return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_vm_f32_noalloc: null operand");
+    ScratchSource src;
+    src.fixed = g_scratch_ptr[S.device];
+    src.fixed_bytes = TENMO_STATIC_SCRATCH_BYTES;
+    if (int rc = matvec_dispatch(Mx + m_off, m_cs, m_rs, v + v_off, v_s, out, n, k, bd, count, accumulate, src)) return rc;
     return finish(sync);
 }
 
