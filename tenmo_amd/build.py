@@ -18,7 +18,8 @@ from concurrent.futures import ThreadPoolExecutor
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(HERE)
 CSRC = os.path.join(HERE, "csrc")
-LIB = os.path.join(HERE, "libtenmo_hip.so")
+# TENMO_HIP_BUILD_OUT: another output path (a variant library to compare against; load it with TENMO_HIP_LIBRARY)
+LIB = os.environ.get("TENMO_HIP_BUILD_OUT") or os.path.join(HERE, "libtenmo_hip.so")
 
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
@@ -31,7 +32,7 @@ FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-result",
     "-I", os.path.join(ROOT, "include"),
-]
+] + os.environ.get("TENMO_HIP_BUILD_FLAGS", "").split()  # extra compiler flags, e.g. -D overrides of kernel constants
 
 # (rows, cols, part) units of the GEMM: part 0 = one workgroup per tile, 1 = the stream-K kernels
 TILES = [(256, 128, 0), (256, 128, 1), (128, 128, 0), (128, 128, 1), (64, 64, 0), (64, 64, 1), (128, 64, 0), (128, 64, 1), (64, 128, 0)]
