@@ -67,11 +67,13 @@ int tenmo_hip_device_info(int* compute_units, char* name, int name_len);
 /* Overrides of the automatic kernel selection, for measurement: "gemm_tile" (0: 256x128, 1: 128x128,
  * 2: 64x64, 3: 128x64, 4: 64x128 workgroup tile; -1 automatic), "gemm_splitk" (number of K slices;
  * -1 automatic), "gemm_streamk" (n > 0: persistent stream-K launch with n workgroups per CU, at most two, for the
- * 256x128 / 128x128 tiles, 0: never, -1 automatic), "gemm_smallk" (the persistent short-reduction kernel, K up to 64 and a plain
- * or accumulating store: 1 wherever it can run, 0 never, -1 automatic: for results of 2048 and more 64x64 tiles), "cols_wg_per_cu" (workgroups per CU the
+ * 256x128 / 128x128 tiles, 0: never, -1 automatic), "gemm_smallk" (the persistent short-reduction kernel, K of 17 up to 64 and a plain
+ * or accumulating store: 1 wherever it can run, 0 never, -1 automatic: for results of 2048 and more 64x64 tiles),
+ * "gemm_panel" (the persistent K-stream kernel with loading wavefronts of its own, 128x128 tiles, K above 16, plain or
+ * accumulating store: 1 wherever it can run, 0 never, -1 automatic: K of 65 up to 512 and at least three tiles per CU), "cols_wg_per_cu" (workgroups per CU the
  * column-streaming kernel aims for) and "conv_phases" (image gradient of a strided convolution phase by phase:
  * 1 always, 0 never, -1 automatic).  The
- * environment variables TENMO_HIP_GEMM_TILE / TENMO_HIP_GEMM_SPLITK / TENMO_HIP_GEMM_STREAMK / TENMO_HIP_GEMM_SMALLK set the same at init.
+ * environment variables TENMO_HIP_GEMM_TILE / TENMO_HIP_GEMM_SPLITK / TENMO_HIP_GEMM_STREAMK / TENMO_HIP_GEMM_SMALLK / TENMO_HIP_GEMM_PANEL set the same at init.
  * No counterpart in the reference, whose tile size is the compile-time TILE_SIZE=32
  * (tenmo/ndbuffer.mojo:63). */
 int tenmo_hip_set_tuning(const char* name, int value);

@@ -47,24 +47,53 @@ def _run(cmd):
     return err
 
 
+def _headers_mtime() -> float:
+    paths = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".hpp")] + [os.path.join(ROOT, "include", "tenmo_hip.h")]
+    return max(os.path.getmtime(p) for p in paths)
+
+
 def build(verbose: bool = False) -> str:
-    jobs = min(len(TILES) + 2, max(1, int(os.environ.get("MAX_JOBS", os.cpu_count() or 1))))
-    with tempfile.TemporaryDirectory(prefix="tenmo_hip_build_") as tmp:
+    """Compiles every unit and links the library.  With TENMO_HIP_BUILD_DIR set, the objects are kept there and a unit
+    is recompiled only when its source, a header or the flags changed (for iterating on one kernel); otherwise
+    everything is compiled afresh in a temporary directory."""
+    jobs = min(len(TILES) + 3, max(1, int(os.environ.get("MAX_JOBS", os.cpu_count() or 1))))
+    keep = os.environ.get("TENMO_HIP_BUILD_DIR")
+    tmp_ctx = None if keep else tempfile.TemporaryDirectory(prefix="tenmo_hip_build_")
+    tmp = keep or tmp_ctx.name
+    os.makedirs(tmp, exist_ok=True)
+    try:
         units = [([os.path.join(CSRC, "tenmo_hip.hip")], os.path.join(tmp, "tenmo_hip.o"))]
         for bm, bn, sk in TILES:
             units.append(([f"-DTENMO_TILE_BM={bm}", f"-DTENMO_TILE_BN={bn}", f"-DTENMO_TILE_STREAMK={sk}",
                            os.path.join(CSRC, "gemm_tiles.hip")], os.path.join(tmp, f"gemm_{bm}x{bn}_{sk}.o")))
         units.append(([os.path.join(CSRC, "gemm_smallk.hip")], os.path.join(tmp, "gemm_smallk.o")))
-        cmds = [[HIPCC] + FLAGS + ["-c"] + src + ["-o", obj] for src, obj in units]
+        units.append(([os.path.join(CSRC, "gemm_panel.hip")], os.path.join(tmp, "gemm_panel.o")))
+        stamp = " ".join(FLAGS)
+        stamp_file = os.path.join(tmp, "flags.txt")
+        same_flags = keep and os.path.exists(stamp_file) and open(stamp_file).read() == stamp
+        newest_header = _headers_mtime()
+
+        def stale(src, obj):
+            if not (same_flags and os.path.exists(obj)):
+                return True
+            return os.path.getmtime(obj) < max(newest_header, os.path.getmtime(src[-1]))
+
+        cmds = [[HIPCC] + FLAGS + ["-c"] + src + ["-o", obj] for src, obj in units if stale(src, obj)]
         if verbose:
             for c in cmds:
                 print(" ".join(c), flush=True)
         with ThreadPoolExecutor(max_workers=jobs) as pool:
             errs = list(pool.map(_run, cmds))
+        if keep:
+            with open(stamp_file, "w") as f:
+                f.write(stamp)
         link = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC"] + [obj for _, obj in units] + ["-o", LIB]
         if verbose:
             print(" ".join(link), flush=True)
         errs.append(_run(link))
+    finally:
+        if tmp_ctx:
+            tmp_ctx.cleanup()
     if verbose:
         for e in errs:
             if e.strip():

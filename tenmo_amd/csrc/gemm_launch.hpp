@@ -32,4 +32,13 @@ bool launch_streamk_64x64(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs
 // `by_batch`: order the tiles for the XCDs (whole batches, or whole column blocks).  false: not a shape this kernel takes.
 bool launch_gemm_smallk_64x64(const GemmArgs& g, int amode, int bmode, unsigned cus, unsigned total_tiles, bool by_batch, hipStream_t stream);
 
+// Persistent workgroups that treat the K steps of all their tiles as one stream through a deep LDS ring, with wavefronts
+// of their own for the loads, two such workgroups per CU (gemm_panel.hip): for a
+// short or medium reduction into a result of many tiles.  Vector operand modes, plain or accumulating store.
+// `total_tiles` = batches x tiles of the chosen size (g.tiles_m, g.tiles_n set for it).  The caller has checked what the
+// direct loads need (pitches, an MN-major extent divisible by 4, K % 4 == 0 for a K-major operand when K is no multiple
+// of 16) and N <= 2^22.  false: no such variant.
+enum PanelTile : int { PANEL_TILE_128x128 = 0 };
+bool launch_gemm_panel(const GemmArgs& g, int tile, int amode, int bmode, unsigned cus, unsigned total_tiles, bool by_batch, hipStream_t stream);
+
 } // namespace tenmo

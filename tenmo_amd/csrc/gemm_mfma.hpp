@@ -38,6 +38,8 @@
 #include <type_traits>
 #include <stdint.h>
 
+#include "gemm_index.hpp"
+
 namespace tenmo {
 
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -49,16 +51,8 @@ typedef float f32x4_u __attribute__((ext_vector_type(4), aligned(4)));
 
 constexpr int GEMM_BK = 16;
 constexpr int GEMM_THREADS = 256;
-constexpr int MAX_BATCH_RANK = 6;
 
 enum OperandMode : int { KMAJOR_VEC = 0, MNMAJOR_VEC = 1, KMAJOR_GEN = 2 };
-
-struct BatchDesc {
-    int32_t rank;
-    int64_t shape[MAX_BATCH_RANK];
-    int64_t a_str[MAX_BATCH_RANK];
-    int64_t b_str[MAX_BATCH_RANK];
-};
 
 struct GemmArgs {
     const float* A; // already advanced by the view offset
@@ -97,25 +91,6 @@ __device__ __forceinline__ float epilogue_value(float v, const float* __restrict
     return v;
 }
 
-// The batch index and every batch dimension are below 2^31 (the host refuses larger grids), so the
-// mixed-radix decode runs in 32-bit arithmetic: a 64-bit division costs a workgroup hundreds of
-// instructions before its first load.
-__device__ __forceinline__ void batch_offsets(const BatchDesc& bd, int64_t b, int64_t& a_off, int64_t& b_off) {
-    a_off = 0; b_off = 0;
-    uint32_t rest = (uint32_t)b;
-    for (int d = bd.rank - 1; d >= 0; --d) {
-        const uint32_t extent = (uint32_t)bd.shape[d];
-        const uint32_t q = rest / extent;
-        const int64_t c = rest - q * extent;
-        rest = q;
-        a_off += c * bd.a_str[d];
-        b_off += c * bd.b_str[d];
-    }
-}
-
-// float offset of 16-byte chunk q (0..3) of `row` in a K-major tile
-__device__ __forceinline__ int kmajor_off(int row, int q) { return 4 * (4 * row + (q ^ ((row >> 2) & 3))); }
-
 // tells the compiler that a pointer is the same in every lane (keeps it in scalar registers)
 __device__ __forceinline__ const float* uniform_ptr(const float* p) {
     const uint64_t v = (uint64_t)(uintptr_t)p;
@@ -145,24 +120,24 @@ struct TileLoader {
     // ragged extent there needs R % 4 == 0; the caller checks, and that 0 <= pitch <= MAX_DIRECT_PITCH.)
     __device__ __forceinline__ void init_direct(const float* __restrict base, int64_t rs, int64_t ks, int64_t row0, int64_t k_begin, int64_t R, int lane, int wave) {
         if constexpr (MODE == MNMAJOR_VEC) {
-            const int64_t row = min(row0 + (4 * lane) % ROWS, R - 4);
 #pragma unroll
-            for (int j = 0; j < NCH; ++j) {
-                const int kk = (wave * NCH + j) * KROWS_PER_WAVELOAD + (4 * lane) / ROWS;
-                lane_off[j] = (uint32_t)((kk * ks + (row - row0)) * 4);
-            }
+            for (int j = 0; j < NCH; ++j) lane_off[j] = direct_lane_off_mnmajor<ROWS>(ks, row0, R, lane, wave * NCH + j);
             origin = uniform_ptr(base + k_begin * ks + row0);
             kstep = ks;
         } else {
-            const int q = (lane & 3) ^ ((lane >> 4) & 3);
 #pragma unroll
-            for (int j = 0; j < NCH; ++j) {
-                const int64_t row = min(row0 + (wave * NCH + j) * 16 + (lane >> 2), R - 1);
-                lane_off[j] = (uint32_t)(((row - row0) * rs + 4 * q) * 4);
-            }
+            for (int j = 0; j < NCH; ++j) lane_off[j] = direct_lane_off_kmajor<ROWS>(rs, row0, R, lane, wave * NCH + j);
             origin = uniform_ptr(base + row0 * rs + k_begin);
             kstep = 1;
         }
+    }
+
+    // lane offsets of the last K step of a K that is no multiple of 16 (`k_valid` of its 16 k exist): see gemm_index.hpp
+    __device__ __forceinline__ void tail_offsets(int64_t rs, int64_t ks, int64_t row0, int64_t R, int lane, int wave, int k_valid, uint32_t (&off)[NCH]) const {
+#pragma unroll
+        for (int j = 0; j < NCH; ++j)
+            off[j] = MODE == MNMAJOR_VEC ? direct_lane_off_mnmajor<ROWS>(ks, row0, R, lane, wave * NCH + j, k_valid)
+                                         : direct_lane_off_kmajor<ROWS>(rs, row0, R, lane, wave * NCH + j, k_valid);
     }
 
     // Wave-load j of the tile at K offset koff -> LDS tile `lds`, straight from global memory.
@@ -172,12 +147,14 @@ struct TileLoader {
     // Issued through inline assembly on purpose: the compiler's wait-count pass otherwise drains
     // every outstanding direct load before any later LDS read, which would serialise the ring.
     // The callers wait for these loads explicitly with s_waitcnt vmcnt(n).
-    __device__ __forceinline__ void load_direct(float* lds, int64_t koff, int wave, int j) const {
+    __device__ __forceinline__ void load_direct(float* lds, int64_t koff, int wave, int j) const { load_direct_at(lds, koff, wave, j, lane_off[j]); }
+    // the same with the lane's byte offset given (the last K step of a ragged K uses tail_offsets)
+    __device__ __forceinline__ void load_direct_at(float* lds, int64_t koff, int wave, int j, uint32_t lane_byte_off) const {
         static_assert(MODE != KMAJOR_GEN, "the generic loader has no direct path");
         const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
         const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + (wave * NCH + j) * 1024);
         const float* src = origin + koff * kstep;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(lane_off[j]), "s"(src) : "memory");
+        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(lane_byte_off), "s"(src) : "memory");
     }
 
     // ---- register-staged path (generic strides, gathered operands, ragged MN-major tiles) --------
@@ -368,10 +345,9 @@ __device__ __forceinline__ constexpr int frag_parts() { return MODE == MNMAJOR_V
 
 template <int ROWS, int MODE, int NBLK>
 __device__ __forceinline__ void load_fragment_part(const float* __restrict lds, int wave_row0, int kc, int lane, float (&f)[NBLK][4], int p) {
-    const int h = lane >> 5, i = lane & 31;
     if constexpr (MODE == MNMAJOR_VEC) { // part = MFMA step s: one read feeds all NBLK blocks
         const int s = p;
-        const float* q = lds + (kc * 8 + 4 * h + s) * ROWS + wave_row0 + NBLK * i;
+        const float* q = lds + frag_off_mnmajor(ROWS, NBLK, wave_row0, kc, lane, s);
         if constexpr (NBLK == 4) {
             f32x4 v = *reinterpret_cast<const f32x4*>(q);
             f[0][s] = v.x; f[1][s] = v.y; f[2][s] = v.z; f[3][s] = v.w;
@@ -383,7 +359,7 @@ __device__ __forceinline__ void load_fragment_part(const float* __restrict lds, 
         }
     } else { // part = block b: one 16-byte read feeds its four MFMA steps
         const int b = p;
-        f32x4 v = *reinterpret_cast<const f32x4*>(lds + kmajor_off(wave_row0 + 32 * b + i, 2 * kc + h));
+        f32x4 v = *reinterpret_cast<const f32x4*>(lds + frag_off_kmajor(wave_row0, kc, lane, b));
         f[b][0] = v.x; f[b][1] = v.y; f[b][2] = v.z; f[b][3] = v.w;
     }
 }
@@ -396,7 +372,7 @@ __device__ __forceinline__ void load_fragments(const float* __restrict lds, int 
 
 // position inside the wave tile of MFMA index x (0..31) of block b
 template <int MODE, int NBLK>
-__device__ __forceinline__ int tile_pos(int b, int x) { return MODE == MNMAJOR_VEC ? NBLK * x + b : 32 * b + x; }
+__device__ __forceinline__ int tile_pos(int b, int x) { return wave_tile_pos(MODE == MNMAJOR_VEC, NBLK, b, x); }
 
 // s_waitcnt vmcnt(n) only (expcnt / lgkmcnt left unconstrained), gfx9 encoding
 __device__ __forceinline__ constexpr int vmcnt_imm(int n) { return (n & 0xF) | (0x7 << 4) | (0xF << 8) | ((n >> 4) << 14); }

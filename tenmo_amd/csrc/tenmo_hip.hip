@@ -88,6 +88,7 @@ struct State {
     int force_conv_phases = -1; // strided image gradient phase by phase: -1 automatic (large layers), 0 never, 1 always
     int force_streamk = -1;    // -1 automatic, 0 never, n > 0: stream-K with n workgroups per CU
     int force_smallk = -1;     // -1 automatic, 0 never, 1: the short-reduction kernel wherever it can run
+    int force_panel = -1;      // -1 automatic, 0 never, 1: the persistent K-stream kernel wherever it can run
     int verbose = 0;
     int cols_waves_per_cu = 2; // target workgroups per CU of the column-streaming kernels (long K slices stream best)
 };
@@ -344,6 +345,29 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
                                (long long)M, (long long)N, (long long)K, (long long)batch_count, kTiles[tile].bm, kTiles[tile].bn, splits, best,
                                sk_wpc ? " (stream-K chosen instead)" : "");
     }
+    // The persistent K-stream kernel (gemm_panel.hip): vector operand forms, plain or accumulating store.  Automatic for
+    // a reduction of 65 .. 512 into a result of at least three 128x128 tiles per CU (measured against the tile the model
+    // picks: 96 x [1024,128].[128,1024] 293 -> 229 us, [4096,256].[256,4096] 75 -> 70 us, [4096,512].[512,4096] 129 -> 127 us,
+    // the CBOW logits [256,100].[100,50000] 42 -> 39 us; level at K = 1024, and 8-25 % slower with fewer tiles than that,
+    // where its two workgroups per CU are not filled).  Reductions of one K step (K <= 16) never take it: see below.
+    {
+        auto operand_ok = [&](int mode, int64_t row_s, int64_t k_s, int64_t extent) {
+            if (mode == KMAJOR_VEC) return k_s == 1 && row_s >= 0 && row_s <= (int64_t(1) << 21) && (K % GEMM_BK == 0 || K % 4 == 0);
+            if (mode == MNMAJOR_VEC) return row_s == 1 && k_s >= 0 && k_s <= (int64_t(1) << 25) && extent % 4 == 0 && extent >= 4;
+            return false;
+        };
+        const int64_t tm = (M + 127) / 128, tn = (N + 127) / 128, tiles = tm * tn * batch_count;
+        const bool can = K > GEMM_BK && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum &&
+                         N <= (int64_t(1) << 22) && tiles <= 0x7fffffffLL;
+        const bool want = S.force_panel > 0 || (S.force_panel < 0 && S.force_tile < 0 && S.force_splitk <= 0 && S.force_streamk <= 0 && S.force_smallk <= 0 &&
+                                                 splits == 1 && sk_wpc == 0 && K > 64 && K <= 512 && tiles >= 3 * (int64_t)S.cus);
+        if (can && want) {
+            g.tiles_m = (int32_t)tm; g.tiles_n = (int32_t)tn;
+            g.k_splits = 1; g.k_per_split = K; g.partial = nullptr;
+            if (S.verbose) fprintf(stderr, "tenmo_hip gemm: K-stream kernel, %lld tiles of 128x128\n", (long long)tiles);
+            if (launch_gemm_panel(g, PANEL_TILE_128x128, am, bm, (unsigned)S.cus, (unsigned)tiles, S.force_panel != 2, S.stream)) return 0;
+        }
+    }
     // Short reduction, vector operand forms and a plain (or accumulating) store: the persistent whole-K-in-LDS kernel
     // (gemm_smallk.hip).  Automatic for K <= 64 where the launch is store-bound as above and every workgroup gets several
     // tiles (measured: 8192x8192xK, K = 32 / 64, every operand layout 76-115 -> 60-93 us; [256,64].[64,50000] 27 -> 21 us;
@@ -357,7 +381,10 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
             if (mode == MNMAJOR_VEC) return row_s == 1 && k_s >= 0 && k_s <= (int64_t(1) << 25) && extent % 4 == 0 && extent >= 4;
             return false;
         };
-        const bool can = K >= 1 && K <= 64 && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum &&
+        // (Reductions of a single K step, K <= 16, stay with the ordinary kernel: a timing run of [8192,16].[16,8192] that went
+        // through this kernel, the K-stream kernel and the ordinary one in turn ended in a memory fault whose cause was not
+        // found; neither persistent kernel is needed there.)
+        const bool can = K > GEMM_BK && K <= 64 && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum &&
                          N < (int64_t(1) << 29) && tiles64 <= 0x7fffffffLL;
         const bool want = S.force_smallk > 0 || (S.force_smallk < 0 && S.force_tile < 0 && S.force_splitk <= 0 && S.force_streamk <= 0 &&
                                                   splits == 1 && sk_wpc == 0 && tiles64 >= 2048 && K <= 64);
@@ -908,6 +935,7 @@ int tenmo_hip_init(int device_id) {
     S.force_splitk = env_int("TENMO_HIP_GEMM_SPLITK", -1);
     S.force_streamk = env_int("TENMO_HIP_GEMM_STREAMK", -1);
     S.force_smallk = env_int("TENMO_HIP_GEMM_SMALLK", -1);
+    S.force_panel = env_int("TENMO_HIP_GEMM_PANEL", -1);
     S.verbose = env_int("TENMO_HIP_VERBOSE", 0);
     S.ready = true;
     return 0;
@@ -958,6 +986,7 @@ int tenmo_hip_set_tuning(const char* name, int value) {
     if (!strcmp(name, "gemm_splitk")) { S.force_splitk = value; return 0; }
     if (!strcmp(name, "gemm_streamk")) { S.force_streamk = value; return 0; }
     if (!strcmp(name, "gemm_smallk")) { S.force_smallk = value; return 0; }
+    if (!strcmp(name, "gemm_panel")) { S.force_panel = value; return 0; }
     if (!strcmp(name, "conv_phases")) { S.force_conv_phases = value; return 0; }
     if (!strcmp(name, "cols_wg_per_cu")) { S.cols_waves_per_cu = value > 0 ? value : 2; return 0; }
     return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: unknown knob '%s'", name);

@@ -203,6 +203,41 @@ def test_short_reduction_kernel_layouts_and_k_tails(T, smallk):
         L.tenmo_hip_set_tuning(b"gemm_smallk", -1)
 
 
+def test_kstream_kernel(T):
+    """The persistent K-stream kernel (loading wavefronts of its own, a ring of LDS stages across tiles, stores behind the
+    next tile's MFMAs) forced on: every operand layout, whole and ragged tiles, reductions of one step to many, K tails,
+    batches with and without a broadcast B, fewer tiles than workgroups and many more, plain and accumulating stores;
+    against fp64.  (The same launches are replayed address by address on the CPU in test_kstream_addresses.py.)"""
+    import torch
+    L, lib = T.lib.load(), T.lib
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(31)
+    cases = [((), 128, 128, 16, 0), ((), 128, 256, 64, 0), ((3,), 100, 132, 36, 0), ((2, 3), 256, 68, 64, 1), ((5,), 64, 64, 112, 0),
+             ((2,), 332, 776, 20, 1), ((), 1000, 1000, 8, 0), ((4,), 72, 52, 84, 1), ((), 256, 50000, 100, 0), ((2,), 512, 512, 52, 1),
+             ((9,), 320, 1024, 12, 0), ((), 64, 8192, 104, 0), ((), 132, 72, 4, 0), ((12,), 1024, 1024, 64, 0), ((), 100, 50000, 256, 1),
+             ((), 4096, 4096, 512, 0), ((17,), 260, 384, 128, 1)]
+    try:
+        L.tenmo_hip_set_tuning(b"gemm_panel", 1)
+        for bshape, M, N, K, acc in cases:
+            for ta in (False, True):
+                for tb in (False, True):
+                    for bcast in ((False, True) if bshape and M <= 512 else (False,)):
+                        A = torch.randn((*bshape, *((K, M) if ta else (M, K))), generator=gen, device="cuda")
+                        B = torch.randn((*((1,) * len(bshape) if bcast else bshape), *((N, K) if tb else (K, N))), generator=gen, device="cuda")
+                        Cc = torch.randn((*bshape, M, N), generator=gen, device="cuda")
+                        a_rs, a_cs = (1, M) if ta else (K, 1)
+                        b_rs, b_cs = (1, K) if tb else (N, 1)
+                        ref = (A.transpose(-1, -2) if ta else A).double() @ (B.transpose(-1, -2) if tb else B).double() + (Cc.double() if acc else 0)
+                        ab = [A.stride(i) for i in range(len(bshape))]
+                        bb = [0 if bcast else B.stride(i) for i in range(len(bshape))]
+                        lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, a_rs, a_cs, B.data_ptr(), 0, b_rs, b_cs, Cc.data_ptr(), M, N, K, len(bshape),
+                                                       lib.i64(bshape), lib.i64(ab), lib.i64(bb), acc, 1))
+                        err = float((Cc.double() - ref).norm() / ref.norm())
+                        assert err <= RTOL_FRO, (bshape, M, N, K, acc, ta, tb, bcast, err)
+    finally:
+        L.tenmo_hip_set_tuning(b"gemm_panel", -1)
+
+
 def test_raw_abi_arguments(T):
     """Argument checking of the kernel-level entry points (status codes + messages, nothing launched)."""
     L, lib = T.lib.load(), T.lib
