@@ -23,7 +23,7 @@ __global__ __launch_bounds__(256) void clock_probe_kernel(int n, float seed) {
         a2 = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, a2, 0, 0, 0);
         a3 = __builtin_amdgcn_mfma_f32_32x32x2f32(x, y, a3, 0, 0, 0);
     }
-    asm volatile("" ::"v"(a0), "v"(a1), "v"(a2), "v"(a3)); // keeps the chains alive without a store
+    keep_alive(a0, a1, a2, a3);
 }
 
 // ---- sum_over_broadcasted_axes (tenmo/sum_mean_reduction.mojo:185-211) fused with the

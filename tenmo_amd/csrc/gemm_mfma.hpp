@@ -39,6 +39,7 @@
 #include <stdint.h>
 
 #include "gemm_index.hpp"
+#include "gfx950_asm.hpp"
 
 namespace tenmo {
 
@@ -140,21 +141,14 @@ struct TileLoader {
                                          : direct_lane_off_kmajor<ROWS>(rs, row0, R, lane, wave * NCH + j, k_valid);
     }
 
-    // Wave-load j of the tile at K offset koff -> LDS tile `lds`, straight from global memory.
-    // Lane L writes bytes [16L, 16L+16) of that load's 1 KiB LDS block (M0 holds the block's LDS
-    // address).  Scalar base + 32-bit lane offset addressing keeps vector ALU work out of the MFMA
-    // stream: 64-bit per-lane address arithmetic between MFMAs was measured to cost 2 % at 8192^3.
-    // Issued through inline assembly on purpose: the compiler's wait-count pass otherwise drains
-    // every outstanding direct load before any later LDS read, which would serialise the ring.
-    // The callers wait for these loads explicitly with s_waitcnt vmcnt(n).
+    // Wave-load j of the tile at K offset koff -> LDS tile `lds`, straight from global memory (direct_load_16B,
+    // gfx950_asm.hpp: lane L writes bytes [16L, 16L+16) of that load's 1 KiB LDS block).  The callers wait for these
+    // loads explicitly with s_waitcnt vmcnt(n).
     __device__ __forceinline__ void load_direct(float* lds, int64_t koff, int wave, int j) const { load_direct_at(lds, koff, wave, j, lane_off[j]); }
     // the same with the lane's byte offset given (the last K step of a ragged K uses tail_offsets)
     __device__ __forceinline__ void load_direct_at(float* lds, int64_t koff, int wave, int j, uint32_t lane_byte_off) const {
         static_assert(MODE != KMAJOR_GEN, "the generic loader has no direct path");
-        const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
-        const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + (wave * NCH + j) * 1024);
-        const float* src = origin + koff * kstep;
-        asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(lane_byte_off), "s"(src) : "memory");
+        direct_load_16B(lds, (uint32_t)((wave * NCH + j) * 1024), lane_byte_off, origin + koff * kstep);
     }
 
     // ---- register-staged path (generic strides, gathered operands, ragged MN-major tiles) --------

@@ -26,29 +26,15 @@ namespace tenmo {
 
 constexpr int SMALLK_THREADS = 512; // four computing wavefronts and four loading ones
 
-// AMODE / BMODE: KMAJOR_VEC or MNMAJOR_VEC (the LDS layouts and loaders of gemm_mfma.hpp).  NK = K steps of 16 that
-// cover K; `col_major`: tiles are numbered column block by column block (few tile-rows: see the launcher).
 // TileLoader::load_direct (one 16-row / 4-k part `part` of the tile at K offset koff) for the lanes with `ok` only:
-// the others neither read memory nor write LDS.  The execution mask is narrowed inside the assembly block, because
-// under a divergent branch the compiler no longer keeps the block's scalar operands in scalar registers.
+// the others neither read memory nor write LDS.
 template <class Loader>
 __device__ __forceinline__ void load_direct_where(const Loader& l, float* lds, int64_t koff, int part, bool ok) {
-    const uint32_t lds0 = (uint32_t)(uintptr_t)(__attribute__((address_space(3))) void*)lds;
-    const uint32_t dst = __builtin_amdgcn_readfirstlane(lds0 + part * 1024);
-    const float* src = l.origin + koff * l.kstep;
-    const uint32_t pred = ok ? 1u : 0u;
-    uint64_t saved_exec;
-    asm volatile("s_mov_b32 m0, %1\n\t"
-                 "s_mov_b64 %0, exec\n\t"
-                 "v_cmp_ne_u32_e32 vcc, 0, %4\n\t"
-                 "s_and_b64 exec, exec, vcc\n\t"
-                 "global_load_lds_dwordx4 %2, %3\n\t"
-                 "s_mov_b64 exec, %0"
-                 : "=&s"(saved_exec)
-                 : "s"(dst), "v"(l.lane_off[0]), "s"(src), "v"(pred)
-                 : "memory", "vcc");
+    direct_load_16B_where(lds, (uint32_t)(part * 1024), l.lane_off[0], l.origin + koff * l.kstep, ok);
 }
 
+// AMODE / BMODE: KMAJOR_VEC or MNMAJOR_VEC (the LDS layouts and loaders of gemm_mfma.hpp).  NK = K steps of 16 that
+// cover K; `col_major`: tiles are numbered column block by column block (few tile-rows: see the launcher).
 template <int AMODE, int BMODE, int NK, int WGS_PER_CU, bool ACC>
 __global__ __launch_bounds__(SMALLK_THREADS, WGS_PER_CU) void gemm_smallk_kernel(const GemmArgs g, const uint32_t total_tiles, const uint32_t xcds, const uint32_t chunk,
                                                                                  const int col_major) {

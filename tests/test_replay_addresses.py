@@ -1,0 +1,139 @@
+"""Every GEMM kernel of the library, run on the CPU under AddressSanitizer before it ever meets a GPU.
+
+tests/replay/ holds a CPU stand-in for the HIP runtime against which the kernel sources of tenmo_amd/csrc compile
+unchanged (only the three gfx950 assembly snippets of gfx950_asm.hpp are swapped for models): a launch runs every
+workgroup, every thread a fibre, wavefront-wide operations and barriers where the source has them.  Here the whole
+library plus a small driver (tests/replay/replay_gemm_main.cpp) is built with -fsanitize=address and
+tenmo_hip_gemm_f32 is called on operands that are heap blocks of exactly the operands' sizes: a load or store of any
+kernel one byte outside an operand ends the run with the sanitizer's report, a workgroup whose wavefronts disagree
+about their barriers ends it as a deadlock, and the result is compared with a float64 product.  Each group runs in both
+models of the direct global->LDS loads: landing at issue ("early": a ring stage refilled too soon shows) and landing at
+the s_waitcnt that covers them ("late": a wait that is too lenient shows).  No GPU involved.
+"""
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "tests", "replay"))
+import build as replay_build  # noqa: E402
+
+pytestmark = pytest.mark.skipif(not replay_build.available(), reason="no host clang++ at " + replay_build.CXX)
+
+LAYOUTS = [("n", "n"), ("n", "t"), ("t", "n"), ("t", "t")]
+
+
+@pytest.fixture(scope="module")
+def exe():
+    return replay_build.build_gemm_asan()
+
+
+def case(M, N, K, la="n", lb="n", batch=0, b_shared=0, acc=0, **knobs):
+    return ",".join([str(M), str(N), str(K), la, lb, str(batch), str(b_shared), str(acc)] + [f"{k}={v}" for k, v in knobs.items()])
+
+
+def run(exe, cases, cus=256, modes=("early", "late"), timeout=600):
+    env = dict(os.environ, REPLAY_CUS=str(cus), ASAN_OPTIONS="detect_leaks=0:detect_stack_use_after_return=0")
+    for mode in modes:
+        res = subprocess.run([exe, mode] + cases, capture_output=True, text=True, env=env, timeout=timeout)
+        tail = (res.stdout[-3000:] + "\n" + res.stderr[-6000:]).strip()
+        assert res.returncode == 0, f"mode {mode}, {cus} CUs:\n{tail}"
+        assert res.stdout.count("relative error") == len(cases), tail
+
+
+def test_the_checks_bite():
+    """tests/replay/replay_selftest.cpp: toy kernels that are wrong on purpose, each in one way, and what becomes of them."""
+    exe = replay_build.build_selftest()
+    env = dict(os.environ, ASAN_OPTIONS="detect_leaks=0:detect_stack_use_after_return=0")
+    outcome = {}
+    for what in ("ok", "overread", "overwrite", "direct_overread", "divergent_collective", "lenient_wait"):
+        res = subprocess.run([exe, what], capture_output=True, text=True, env=env, timeout=120)
+        outcome[what] = (res.returncode, res.stdout + res.stderr)
+    assert outcome["ok"][0] == 0 and "ok" in outcome["ok"][1]
+    for what in ("overread", "overwrite"):   # a plain load / store one element past a device allocation
+        assert outcome[what][0] != 0 and "heap-buffer-overflow" in outcome[what][1], outcome[what][1][-2000:]
+    assert outcome["direct_overread"][0] != 0 and "lies outside every device allocation" in outcome["direct_overread"][1]
+    assert outcome["divergent_collective"][0] != 0 and "deadlock" in outcome["divergent_collective"][1]
+    assert outcome["lenient_wait"][0] == 3 and "stale data" in outcome["lenient_wait"][1]   # a wait that leaves a needed load in flight
+
+
+@pytest.mark.parametrize("tile", [0, 1, 2, 3, 4])
+def test_one_workgroup_per_tile_kernels(exe, tile):
+    """gemm_mfma_kernel of every workgroup tile: whole and ragged tiles, K of one step, K tails (the register-staged loop
+    behind the direct ring), every layout, batches with a shared B, accumulate, and both strides non-unit (the
+    element-wise loader)."""
+    cases = []
+    for la, lb in LAYOUTS:
+        for (M, N, K) in [(64, 64, 16), (130, 70, 33), (257, 129, 100), (300, 520, 48), (128, 256, 7)]:
+            cases.append(case(M, N, K, la, lb, gemm_tile=tile))
+        cases.append(case(132, 260, 84, la, lb, batch=3, b_shared=1, acc=1, gemm_tile=tile))
+        cases.append(case(131, 77, 50, la, lb, batch=2, acc=0, gemm_tile=tile))  # extents that are no multiple of 4: an MN-major ragged tile leaves the direct path
+    cases += [case(100, 90, 40, "g", "n", gemm_tile=tile), case(100, 90, 40, "n", "g", gemm_tile=tile), case(65, 130, 24, "g", "g", batch=2, acc=1, gemm_tile=tile)]
+    run(exe, cases)
+
+
+def test_k_slices_and_stream_k(exe):
+    cases = []
+    for la, lb in LAYOUTS:
+        cases.append(case(200, 100, 400, la, lb, gemm_splitk=3))
+        cases.append(case(130, 70, 1000, la, lb, batch=2, acc=1, gemm_splitk=8))
+        for tile in (0, 1, 2, 3):
+            cases.append(case(520, 300, 256, la, lb, gemm_streamk=1, gemm_tile=tile))
+            cases.append(case(260, 392, 132, la, lb, batch=3, acc=1, gemm_streamk=2, gemm_tile=tile))
+    run(exe, cases, cus=4)   # few CUs: every workgroup of a stream-K grid takes whole tiles and a shared piece
+    run(exe, [case(1024, 768, 512), case(1000, 1000, 300, "n", "t")], cus=16, modes=("late",))  # what the automatic choice picks
+
+
+def test_short_reduction_kernel(exe):
+    """gemm_smallk_kernel forced on: K of 17..64 (K <= 16 goes to the ordinary kernel), every layout, K tails, ragged tiles,
+    batches, a shared B, accumulate; on 2 CUs every workgroup walks many tiles, on 256 most tiles have a workgroup each."""
+    cases = []
+    for la, lb in LAYOUTS:
+        for (M, N, K) in [(128, 192, 64), (100, 132, 36), (1000, 1000, 48), (64, 64, 20), (332, 776, 32)]:
+            cases.append(case(M, N, K, la, lb, gemm_smallk=1))
+        cases.append(case(256, 68, 64, la, lb, batch=6, acc=1, gemm_smallk=1))
+        cases.append(case(320, 192, 32, la, lb, batch=9, b_shared=1, gemm_smallk=1))
+    cases.append(case(257, 65, 64, "n", "t", batch=6, acc=1, gemm_smallk=1))   # a K-major operand may have any row count
+    cases.append(case(8, 8192, 64, "n", "n", gemm_smallk=1))                  # few tile-rows, many tile-columns: column blocks per XCD
+    run(exe, cases, cus=2)
+    run(exe, cases[:8] + cases[-3:], cus=256, modes=("late",))
+    run(exe, [case(64, 64, 16, gemm_smallk=1), case(300, 200, 12, "n", "t", gemm_smallk=1)], cus=4)  # K <= 16: not this kernel, still right
+
+
+def test_k_stream_kernel(exe):
+    """gemm_panel_kernel forced on: reductions of two steps to many, K tails, every layout, ragged tiles, batches, a shared
+    B, accumulate (atomic adds); few CUs (long walks, the ring runs across many tile boundaries) and the real 256."""
+    cases = []
+    for la, lb in LAYOUTS:
+        for (M, N, K) in [(128, 128, 32), (300, 520, 100), (132, 260, 20), (1000, 136, 24), (256, 384, 112), (128, 256, 36), (512, 512, 256)]:
+            cases.append(case(M, N, K, la, lb, gemm_panel=1))
+        cases.append(case(256, 384, 64, la, lb, batch=16, gemm_panel=1))
+        cases.append(case(132, 260, 48, la, lb, batch=9, b_shared=1, acc=1, gemm_panel=1))
+    cases.append(case(129, 131, 48, "n", "t", gemm_panel=1))
+    cases.append(case(256, 128 * 70, 32, "n", "n", gemm_panel=1))
+    run(exe, cases, cus=2)
+    run(exe, cases[:9] + cases[-2:], cus=256, modes=("late",))
+    run(exe, [case(128, 128, 16, gemm_panel=1), case(300, 260, 8, "t", "n", gemm_panel=1)], cus=4)  # K <= 16: not this kernel, still right
+
+
+def test_automatic_choice_on_benchmark_shapes(exe):
+    """What the dispatch picks by itself for the shapes the benchmarks run, at their real sizes (attention: 8 of the 96
+    batches; the square products reduced to 1024)."""
+    cases = [case(1024, 1024, 64, "n", "t", batch=8),        # Q.K^T: the short-reduction kernel
+             case(1024, 64, 1024, "n", "n", batch=8),        # P.V
+             case(1024, 1024, 128, "n", "t", batch=8),       # K = 128, many tiles: the K-stream kernel
+             case(256, 50000, 100, "n", "n"),                # CBOW logits
+             case(100, 50000, 256, "t", "n"),                # CBOW A^T.dC
+             case(8, 4096, 1024, "n", "n"),                  # skinny: the column-streaming kernels
+             case(1024, 1024, 1024)]
+    run(exe, cases, modes=("late",), timeout=1200)
+
+
+def test_one_step_reduction_into_a_large_result(exe):
+    """[8192,16].[16,8192] with B a transposed view, at full size and on the real 256 CUs: the launch after which a GPU run
+    once ended in a memory fault (what ran then: this shape through the short-reduction kernel, the K-stream kernel and
+    the ordinary one in turn; replayed here with the two persistent kernels still admitted for K <= 16, all three were
+    clean).  With K <= 16 the persistent kernels are no longer taken, so this replays the ordinary 64x64 kernel."""
+    run(exe, [case(8192, 8192, 16, "n", "t")], modes=("early",), timeout=1200)
