@@ -254,6 +254,10 @@ void complete_loads(int leave) {
 }
 
 void check_global(const void* p, size_t bytes, bool write, const char* what) {
+    // REPLAY_STRICT=0: operands come from an allocator this runtime does not see (a test that passes its own arrays);
+    // the direct loads are then as unchecked as the plain ones
+    static const bool strict = [] { const char* e = getenv("REPLAY_STRICT"); return !(e && e[0] == '0'); }();
+    if (!strict) return;
     const uintptr_t a = (uintptr_t)p;
     bool ok = false;
     size_t count;

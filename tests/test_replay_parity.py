@@ -1,0 +1,54 @@
+"""The GPU parity tests, run on the CPU against the replay build of the library.
+
+tests/test_gpu_parity.py and tests/test_zz_no_alloc.py drive every entry point of the C ABI through the host mirror and
+compare with the oracle and with float64.  Here the same test functions run in a child pytest process in which the
+library is the CPU replay (tests/replay: the kernel sources compiled for the host, launches executed thread by thread)
+and torch's "cuda" allocations are redirected to host memory (tests/replay/torch_on_host.py).  What this proves without
+a GPU: the host side (dispatch, views, batching, workspace handling, error paths) and the kernels' arithmetic and
+synchronisation as written in the source.  What it cannot: anything about the code the GPU compiler generates or timing.
+The tests left out are the ones whose shapes would take minutes at CPU speed (TENMO_REPLAY_FULL=1 runs those too, about
+a quarter of an hour; the kernels they cover are replayed on smaller shapes in tests/test_replay_addresses.py).
+"""
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "tests", "replay"))
+import build as replay_build  # noqa: E402
+
+pytestmark = pytest.mark.skipif(not replay_build.available(), reason="no host clang++ at " + replay_build.CXX)
+
+# too large for any CPU replay (more than 2^31 elements), or about the GPU itself
+LEFT_OUT = ["test_products_with_more_than_2_31_elements", "test_clock_probe"]
+# minutes each at CPU speed
+SLOW = ["test_stream_k", "test_kstream_kernel", "test_more_batches_than_a_grid_dimension", "test_conv2d_stream_k", "test_blocked_tile_order"]
+
+
+def run_child(files, extra=()):
+    lib = replay_build.build_library()
+    env = dict(os.environ, TENMO_HIP_LIBRARY=lib, REPLAY_STRICT="0", PYTHONPATH=os.path.join(ROOT, "tests", "replay") + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    left_out = LEFT_OUT + ([] if os.environ.get("TENMO_REPLAY_FULL") == "1" else SLOW)
+    deselect = " and ".join("not " + name for name in left_out)
+    cmd = [sys.executable, "-m", "pytest", "-p", "torch_on_host", "-m", "gpu", "-x", "-q", "-k", deselect, "-p", "no:cacheprovider"] + list(extra) + files
+    try:
+        import xdist  # noqa: F401
+
+        cmd += ["-n", "4"]
+    except ImportError:
+        pass
+    res = subprocess.run(cmd, cwd=ROOT, env=env, capture_output=True, text=True, timeout=3000)
+    tail = (res.stdout[-6000:] + "\n" + res.stderr[-3000:]).strip()
+    assert res.returncode == 0, tail
+    assert " passed" in res.stdout and "skipped" not in res.stdout.splitlines()[-1], tail
+    return res.stdout
+
+
+def test_gpu_parity_suite_on_the_replay():
+    run_child([os.path.join("tests", "test_gpu_parity.py")])
+
+
+def test_allocation_free_entry_point_on_the_replay():
+    run_child([os.path.join("tests", "test_zz_no_alloc.py")])
