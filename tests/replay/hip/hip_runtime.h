@@ -216,11 +216,12 @@ struct hipDeviceProp_t {
     size_t totalGlobalMem;
 };
 
+// (C linkage, as in the real runtime: a plain C program can call them)
+extern "C" {
 hipError_t hipGetDeviceCount(int* n);
 hipError_t hipSetDevice(int d);
 hipError_t hipGetDeviceProperties(hipDeviceProp_t* p, int d);
 hipError_t hipMalloc(void** p, size_t bytes);
-template <class T> inline hipError_t hipMalloc(T** p, size_t bytes) { return hipMalloc(reinterpret_cast<void**>(p), bytes); }
 hipError_t hipFree(void* p);
 hipError_t hipMemcpy(void* dst, const void* src, size_t bytes, hipMemcpyKind kind);
 hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKind kind, hipStream_t s);
@@ -244,6 +245,8 @@ hipError_t hipGraphInstantiate(hipGraphExec_t* exec, hipGraph_t g, void*, void*,
 hipError_t hipGraphDestroy(hipGraph_t g);
 hipError_t hipGraphExecDestroy(hipGraphExec_t e);
 hipError_t hipGraphLaunch(hipGraphExec_t e, hipStream_t s);
+} // extern "C"
+template <class T> inline hipError_t hipMalloc(T** p, size_t bytes) { return hipMalloc(reinterpret_cast<void**>(p), bytes); }
 
 namespace replay {
 void enqueue(hipStream_t s, const char* name, dim3 grid, dim3 block, std::function<void()> body);
