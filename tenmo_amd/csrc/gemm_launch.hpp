@@ -18,6 +18,12 @@ bool launch_gemm_64x128(const GemmArgs& g, dim3 grid, int amode, int bmode, hipS
 bool launch_gemm_pair_64x64(const GemmArgs& g0, const GemmArgs& g1, unsigned count0, unsigned count1, int amode0, int bmode0, int amode1, int bmode1,
                             hipStream_t stream);
 
+// C[kept batch] (+)= the sum over the reduced batch dimensions `red` of A . B (gemm_reduce_kernel): `wgs` = kept batches x
+// tiles of the chosen size (g.tiles_m, g.tiles_n set for it; g.batch, g.batch_count = the kept dimensions).  Vector
+// operand modes only; false: no variant for these modes.
+bool launch_gemm_reduce_128x128(const GemmArgs& g, const BatchReduce& red, unsigned wgs, int amode, int bmode, hipStream_t stream);
+bool launch_gemm_reduce_64x64(const GemmArgs& g, const BatchReduce& red, unsigned wgs, int amode, int bmode, hipStream_t stream);
+
 // Stream-K: `wgs` persistent workgroups, then the fix-up over `tiles` tiles in `fix_parts` parts
 // each (0: no tile is shared, no fix-up).  Vector operand modes only.
 bool launch_streamk_256x128(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);

@@ -449,7 +449,8 @@ struct TileDest {
 // workgroup.  The three LDS stages are the caller's; on return every wavefront has left them.
 template <int BM, int BN, int AMODE, int BMODE>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, float* stage1, float* stage2,
-                                          int64_t batch, int64_t tile_m, int64_t tile_n, int64_t k_begin, int64_t k_end, const TileDest dst) {
+                                          int64_t batch, int64_t tile_m, int64_t tile_n, int64_t k_begin, int64_t k_end, const TileDest dst,
+                                          const int64_t a_extra = 0, const int64_t b_extra = 0) { // (element offsets on top of the batch's)
     constexpr int TM = BM / 2, TN = BN / 2;     // wave tile (2x2 waves)
     constexpr int MB = TM / 32, NB = TN / 32;   // 32x32 MFMA blocks per wave tile
     constexpr int A_FLOATS = BM * GEMM_BK;
@@ -461,8 +462,8 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
 
     int64_t a_boff, b_boff;
     batch_offsets(g.batch, batch, a_boff, b_boff);
-    const float* __restrict Ab = g.A + a_boff;
-    const float* __restrict Bb = g.B + b_boff;
+    const float* __restrict Ab = g.A + a_boff + a_extra;
+    const float* __restrict Bb = g.B + b_boff + b_extra;
 
     // operand strides in (row, k) form
     const int64_t a_row_s = g.a_rs, a_k_s = g.a_cs;   // A(m,k)
@@ -893,6 +894,41 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
     __shared__ __attribute__((aligned(1024))) float stage2[DIRECT ? STAGE_FLOATS : 4];
     gemm_workgroup<BM, BN, AMODE, BMODE>(g, stage0, stage1, stage2, blockIdx.x, blockIdx.y);
+}
+
+// Batch dimensions that a product is SUMMED over (the gradient of a parent that was broadcast along them,
+// tenmo/matmul.mojo:115-135 with sum_over_broadcasted_axes).  `dims` holds the reduced dimensions only.
+struct BatchReduce {
+    BatchDesc dims;
+    int64_t count; // product of dims.shape
+};
+
+// C[kept batch] (+)= sum over the reduced batch dimensions of A[kept, reduced] . B[kept, reduced]: one workgroup per tile of
+// a kept batch (g.batch and g.batch_count describe the kept dimensions only; one K slice, no fused epilogue).  The
+// workgroup runs the tile once per index of the reduced dimensions, each round adding onto what the round before stored
+// (the same lanes touch the same elements, which stay in the L2): the gradient of a broadcast parent without a batched
+// intermediate, without a reduction pass, and summed in a fixed order.
+template <int BM, int BN, int AMODE, int BMODE>
+__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_reduce_kernel(const GemmArgs g, const BatchReduce red) {
+    constexpr int STAGE_FLOATS = (BM + BN) * GEMM_BK;
+    __shared__ __attribute__((aligned(1024))) float stage0[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage2[STAGE_FLOATS];
+    const uint32_t tiles = (uint32_t)g.tiles_m * (uint32_t)g.tiles_n;
+    const uint32_t batch32 = blockIdx.x / tiles;
+    int64_t tile_m, tile_n;
+    tile_coords(g, blockIdx.x - batch32 * tiles, tile_m, tile_n);
+    const int64_t batch = batch32;
+    TileDest dst;
+    dst.ld = g.N; dst.row0 = 0; dst.col0 = 0;
+    dst.base = g.C + batch * g.M * g.N;
+    dst.fused = false;
+    for (int64_t r = 0; r < red.count; ++r) {
+        int64_t a_roff, b_roff;
+        batch_offsets(red.dims, r, a_roff, b_roff);
+        dst.accumulate = r > 0 || g.accumulate != 0;
+        gemm_tile<BM, BN, AMODE, BMODE>(g, stage0, stage1, stage2, batch, tile_m, tile_n, 0, g.K, dst, a_roff, b_roff);
+    }
 }
 
 // Two independent products in one launch (both with one K slice and vector operand forms): workgroups below `first_count`

@@ -26,6 +26,19 @@ bool TENMO_NAME(launch_gemm_, TENMO_TILE_BM, TENMO_TILE_BN)(const GemmArgs& g, d
 #undef TENMO_CASE
     return false;
 }
+#if (TENMO_TILE_BM == 64 && TENMO_TILE_BN == 64) || (TENMO_TILE_BM == 128 && TENMO_TILE_BN == 128)
+bool TENMO_NAME(launch_gemm_reduce_, TENMO_TILE_BM, TENMO_TILE_BN)(const GemmArgs& g, const BatchReduce& red, unsigned wgs, int amode, int bmode, hipStream_t stream) {
+    constexpr int BM = TENMO_TILE_BM, BN = TENMO_TILE_BN;
+#define TENMO_CASE(A_, B_)                                                                                               \
+    if (amode == A_ && bmode == B_) {                                                                                    \
+        hipLaunchKernelGGL((gemm_reduce_kernel<BM, BN, A_, B_>), dim3(wgs), dim3(GEMM_THREADS), 0, stream, g, red);     \
+        return true;                                                                                                     \
+    }
+    TENMO_CASE(KMAJOR_VEC, KMAJOR_VEC) TENMO_CASE(KMAJOR_VEC, MNMAJOR_VEC) TENMO_CASE(MNMAJOR_VEC, KMAJOR_VEC) TENMO_CASE(MNMAJOR_VEC, MNMAJOR_VEC)
+#undef TENMO_CASE
+    return false;
+}
+#endif
 #if TENMO_TILE_BM == 64 && TENMO_TILE_BN == 64
 bool launch_gemm_pair_64x64(const GemmArgs& g0, const GemmArgs& g1, unsigned count0, unsigned count1, int amode0, int bmode0, int amode1, int bmode1,
                             hipStream_t stream) {

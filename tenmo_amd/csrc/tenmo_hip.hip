@@ -89,6 +89,7 @@ struct State {
     int force_streamk = -1;    // -1 automatic, 0 never, n > 0: stream-K with n workgroups per CU
     int force_smallk = -1;     // -1 automatic, 0 never, 1: the short-reduction kernel wherever it can run
     int force_panel = -1;      // -1 automatic, 0 never, 1: the persistent K-stream kernel wherever it can run
+    int fold_reduce = -1;      // the gradient of a broadcast parent summed inside the GEMM launch: -1 automatic, 0 never, 1 wherever it can
     int verbose = 0;
     int cols_waves_per_cu = 2; // target workgroups per CU of the column-streaming kernels (long K slices stream best)
 };
@@ -867,6 +868,56 @@ bool same_batch(const Geometry& g, const tenmo_view* parent, int trailing) {
     return true;
 }
 
+// grad (dense, at `parent`'s shape) += the product X . Y summed over the batch dims of the result that `parent` broadcast:
+// the sum runs inside the GEMM launch (gemm_reduce_kernel), so no batched gradient is written and no reduction pass
+// follows.  X, Y: the two factors as views whose batch dims broadcast to g's.  Returns 1 when it ran, 0 when the shape is
+// not one the reducing launch takes (generic strides, or a result of so few tiles that spreading the batches over the
+// chip and adding them afterwards is the better plan), a negative status on error.
+int folded_gradient(const tenmo_view* X, const tenmo_view* Y, const Geometry& g, const tenmo_view* parent, float* grad) {
+    if (S.fold_reduce == 0) return 0;
+    const int64_t M = X->shape[X->rank - 2], K = X->shape[X->rank - 1], N = Y->shape[Y->rank - 1];
+    const int64_t x_rs = X->strides[X->rank - 2], x_cs = X->strides[X->rank - 1], y_rs = Y->strides[Y->rank - 2], y_cs = Y->strides[Y->rank - 1];
+    const int am = operand_mode(x_rs, x_cs, M, K), bm = operand_mode(y_cs, y_rs, N, K);
+    if (am == KMAJOR_GEN || bm == KMAJOR_GEN || M == 0 || N == 0) return 0;
+    int64_t xs[MAX_BATCH_RANK] = {0}, ys[MAX_BATCH_RANK] = {0};
+    batch_strides_of(X, X->rank - 2, g.batch_rank, xs);
+    batch_strides_of(Y, Y->rank - 2, g.batch_rank, ys);
+    GemmArgs a{};
+    BatchReduce red{};
+    for (int d = 0; d < MAX_BATCH_RANK; ++d) { a.batch.shape[d] = 1; red.dims.shape[d] = 1; }
+    const int own = parent->rank - 2;
+    int64_t kept_count = 1;
+    red.count = 1;
+    for (int d = 0; d < g.batch_rank; ++d) {
+        const int od = d - (g.batch_rank - own);
+        const bool kept = od >= 0 && parent->shape[od] > 1;
+        BatchDesc& bd = kept ? a.batch : red.dims;
+        bd.shape[bd.rank] = g.oshape[d];
+        bd.a_str[bd.rank] = xs[d];
+        bd.b_str[bd.rank] = ys[d];
+        ++bd.rank;
+        (kept ? kept_count : red.count) *= g.oshape[d];
+    }
+    if (red.count <= 1) return 0;
+    const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128) * kept_count, tiles64 = ((M + 63) / 64) * ((N + 63) / 64) * kept_count;
+    const bool big = tiles128 >= (int64_t)S.cus;
+    if (S.fold_reduce < 0 && !big && tiles64 < (int64_t)S.cus / 2) return 0;
+    if (tiles64 > 0x7fffffffLL) return 0;
+    a.A = X->data + X->offset; a.B = Y->data + Y->offset; a.C = grad;
+    a.a_rs = x_rs; a.a_cs = x_cs; a.b_rs = y_rs; a.b_cs = y_cs;
+    a.M = M; a.N = N; a.K = K;
+    a.accumulate = 1;
+    a.batch_count = kept_count;
+    a.k_splits = 1; a.k_per_split = K;
+    const int t = big ? 128 : 64;
+    a.tiles_m = (int32_t)((M + t - 1) / t);
+    a.tiles_n = (int32_t)((N + t - 1) / t);
+    if (S.verbose) fprintf(stderr, "tenmo_hip gradient of a broadcast parent: %lld batches summed inside %lld tiles of %dx%d\n", (long long)red.count,
+                           (long long)(big ? tiles128 : tiles64), t, t);
+    const bool ok = big ? launch_gemm_reduce_128x128(a, red, (unsigned)tiles128, am, bm, S.stream) : launch_gemm_reduce_64x64(a, red, (unsigned)tiles64, am, bm, S.stream);
+    return ok ? 1 : 0;
+}
+
 // ---- cross-entropy forward: pick the kernel that reads a row once --------------------------------
 template <typename IdxT, bool VEC>
 void launch_ce_forward_t(const CeForwardArgs& a) {
@@ -987,6 +1038,7 @@ int tenmo_hip_set_tuning(const char* name, int value) {
     if (!strcmp(name, "gemm_streamk")) { S.force_streamk = value; return 0; }
     if (!strcmp(name, "gemm_smallk")) { S.force_smallk = value; return 0; }
     if (!strcmp(name, "gemm_panel")) { S.force_panel = value; return 0; }
+    if (!strcmp(name, "fold_reduce")) { S.fold_reduce = value; return 0; }
     if (!strcmp(name, "conv_phases")) { S.force_conv_phases = value; return 0; }
     if (!strcmp(name, "cols_wg_per_cu")) { S.cols_waves_per_cu = value > 0 ? value : 2; return 0; }
     return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: unknown knob '%s'", name);
@@ -1520,6 +1572,8 @@ int tenmo_hip_matmul_backward(const tenmo_view* A, const tenmo_view* B, const fl
         const tenmo_view Bt = transposed_last2(B);
         if (same_batch(g, A, 2)) {
             if (int rc = matmul_views(&dCv, &Bt, grad_A, 1, "tenmo_hip_matmul_backward")) return rc;
+        } else if (const int folded = folded_gradient(&dCv, &Bt, g, A, grad_A)) {
+            if (folded < 0) return folded;
         } else {
             Geometry gg;
             if (int rc = resolve(TENMO_OP_MM, &dCv, &Bt, &gg, "tenmo_hip_matmul_backward")) return rc;
@@ -1544,6 +1598,8 @@ int tenmo_hip_matmul_backward(const tenmo_view* A, const tenmo_view* B, const fl
                                        K, N, g.batch_count * M, none, 1, 1)) return rc;
         } else if (same_batch(g, B, 2)) {
             if (int rc = matmul_views(&At, &dCv, grad_B, 1, "tenmo_hip_matmul_backward")) return rc;
+        } else if (const int folded = folded_gradient(&At, &dCv, g, B, grad_B)) {
+            if (folded < 0) return folded;
         } else {
             Geometry gg;
             if (int rc = resolve(TENMO_OP_MM, &At, &dCv, &gg, "tenmo_hip_matmul_backward")) return rc;

@@ -131,6 +131,19 @@ def test_automatic_choice_on_benchmark_shapes(exe):
     run(exe, cases, modes=("late",), timeout=1200)
 
 
+def test_gradients_of_broadcast_parents(exe):
+    """tenmo_hip_matmul_backward with a parent that was broadcast over the batch: the sum over batches inside the GEMM
+    launch (gemm_reduce_kernel, forced on), and the batched gradient reduced afterwards (forced off)."""
+    cases = []
+    for la, lb in LAYOUTS:
+        for fold in (1, 0):
+            cases.append(f"bwd:70,41,33,{la},{lb},0,5,fold_reduce={fold}")     # A shared by 5 batches
+            cases.append(f"bwd:132,260,48,{la},{lb},4,1,fold_reduce={fold}")   # B shared (its partner's rows stack: one folded GEMM either way)
+            cases.append(f"bwd:300,200,100,{la},{lb},1,3,fold_reduce={fold}")
+    run(exe, cases, cus=8)
+    run(exe, ["bwd:256,1024,512,n,n,0,4,fold_reduce=1", "bwd:512,256,1024,n,n,1,6"], cus=256, modes=("late",))
+
+
 def test_one_step_reduction_into_a_large_result(exe):
     """[8192,16].[16,8192] with B a transposed view, at full size and on the real 256 CUs: the launch after which a GPU run
     once ended in a memory fault (what ran then: this shape through the short-reduction kernel, the K-stream kernel and
