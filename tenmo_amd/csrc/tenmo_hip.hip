@@ -1666,6 +1666,14 @@ int tenmo_hip_mv_backward(const tenmo_view* Mx, const tenmo_view* v, const float
         Geometry gg = g;
         gg.oshape[g.batch_rank] = k; gg.orank = g.batch_rank + 1;
         const bool direct = same_batch(g, v, 1);
+        if (!direct && S.fold_reduce != 0 && all_broadcast(v, 1) && rows_fold(Mx, g)) {
+            // v is shared by every batch and the matrices stack at a constant row pitch: the sum over batches of
+            // M_b^T . dy_b is ONE product dy[batch*m] . M[batch*m, k], added straight into the gradbox
+            BatchDesc none{};
+            for (int d = 0; d < MAX_BATCH_RANK; ++d) none.shape[d] = 1;
+            if (int rc = matvec_dispatch(Mx->data + Mx->offset, Mx->strides[Mx->rank - 1], Mx->strides[Mx->rank - 2], dy, 1, grad_v, k, g.batch_count * m, none, 1, 1)) return rc;
+            return finish(sync);
+        }
         float* target = grad_v;
         float* full = nullptr;
         if (!direct) {

@@ -682,7 +682,9 @@ def test_mv_vm_forward_all_layouts(T, oracle):
 
 def test_mv_vm_backward_against_oracle(T, oracle):
     rng = np.random.default_rng(43)
-    for ms, vs in [((6, 5), (5,)), ((3, 6, 5), (5,)), ((6, 5), (4, 5)), ((2, 3, 6, 5), (3, 5)), ((1, 6, 5), (4, 5))]:
+    # (a vector shared by every batch of stacked matrices: its gradient is one product with the batch folded into the reduction)
+    for ms, vs in [((6, 5), (5,)), ((3, 6, 5), (5,)), ((6, 5), (4, 5)), ((2, 3, 6, 5), (3, 5)), ((1, 6, 5), (4, 5)), ((4, 70, 33), (33,)),
+                   ((2, 3, 40, 1030), (1030,))]:
         Mn = rng.standard_normal(ms, dtype=np.float32)
         vn = rng.standard_normal(vs, dtype=np.float32)
         Mt, vt = T.Tensor.from_numpy(Mn, True), T.Tensor.from_numpy(vn, True)
