@@ -8,6 +8,11 @@
 //     storage of twice the width of which every second element is used: no unit stride, the element-wise loader)
 //     batch: number of matrices (0: no batch dimension); b_shared: 1 = every batch uses the same B
 //     a case may carry check=0: do not compute the float64 product (large shapes: the addresses are the point)
+//   CASE = mv:m,k,layout,batch,pad,accumulate   out[m] = Mx[m,k] . v[k]; layout n (rows of k, pitch k + pad) or t (a transposed view of [k][m + pad])
+//   CASE = vm:k,n,layout,batch,pad,accumulate[,entry=noalloc]   out[n] = v[k] . Mx[k,n]; the matrix shared by every batch when batch < 0
+//   CASE = ce:M,C,target_is_int64,label_smoothing_percent    cross-entropy forward (all outputs) and backward (mean), addresses only
+//   CASE = conv:N,C_in,H_pad,W_pad,C_out,KH,KW,stride,dilation    convolution forward and backward (all three gradients), addresses only
+//   CASE = misc:n      dot, column sum ([n/64+1, 64.. ] shapes derived from n), SGD with and without momentum, addresses only
 //   CASE = bwd:M,N,K,a_layout,b_layout,a_batch,b_batch[,knob=value...]   tenmo_hip_matmul_backward of A[a_batch, M, K] . B[b_batch, K, N]
 //     (a batch of 0: no batch dimension; 1: one that broadcasts): both gradients against float64, accumulated onto a start value
 #include <cmath>
@@ -113,6 +118,146 @@ static int run_case(const std::string& spec) {
     return bad;
 }
 
+__attribute__((no_sanitize("address"))) static double gradient_error(const float* got, const std::vector<double>& want) {
+    double num = 0.0, den = 0.0;
+    for (size_t i = 0; i < want.size(); ++i) { const double d = (double)got[i] - want[i]; num += d * d; den += want[i] * want[i]; }
+    return std::sqrt(num / (den > 0 ? den : 1.0));
+}
+
+// mv / vm on exactly-sized blocks; the vector has one element per k and no padding
+static int run_vector_case(const std::string& spec, bool is_mv) {
+    std::vector<std::string> f;
+    size_t pos = 3;
+    while (pos <= spec.size()) {
+        const size_t c = spec.find(',', pos);
+        f.push_back(spec.substr(pos, c == std::string::npos ? std::string::npos : c - pos));
+        if (c == std::string::npos) break;
+        pos = c + 1;
+    }
+    if (f.size() < 6) { fprintf(stderr, "bad case %s\n", spec.c_str()); return 2; }
+    const int64_t d0 = atoll(f[0].c_str()), d1 = atoll(f[1].c_str());   // mv: m, k   vm: k, n
+    const bool t = f[2] == "t";
+    int64_t batch = atoll(f[3].c_str());
+    const int64_t pad = atoll(f[4].c_str());
+    const int accumulate = atoi(f[5].c_str());
+    bool noalloc = false;
+    for (size_t i = 6; i < f.size(); ++i) if (f[i] == "entry=noalloc") noalloc = true;
+    const bool shared_matrix = batch < 0;
+    if (batch < 0) batch = -batch;
+    const int64_t nb = batch > 0 ? batch : 1, nmat = shared_matrix ? 1 : nb;
+    const int64_t rows = is_mv ? d0 : d0, cols = d1;       // logical matrix [rows][cols]: mv [m][k], vm [k][n]
+    const int64_t pitch = (t ? rows : cols) + pad, lines = t ? cols : rows;
+    const int64_t mat_elems = lines * pitch - pad;        // the last line carries no padding: the block ends with the matrix
+    const int64_t rs = t ? 1 : pitch, cs = t ? pitch : 1;
+    const int64_t vec_len = is_mv ? cols : rows, out_len = is_mv ? rows : cols;
+    const size_t m_n = (size_t)(nmat * lines * pitch - pad), v_n = (size_t)(nb * vec_len), o_n = (size_t)(nb * out_len);
+    float* Mx = (float*)malloc(m_n * 4); float* v = (float*)malloc(v_n * 4); float* out = (float*)malloc(o_n * 4);
+    for (size_t i = 0; i < m_n; ++i) Mx[i] = next_float();
+    for (size_t i = 0; i < v_n; ++i) v[i] = next_float();
+    for (size_t i = 0; i < o_n; ++i) out[i] = next_float();
+    std::vector<double> want(o_n);
+    for (int64_t b = 0; b < nb; ++b) {
+        const float* Mb = Mx + (shared_matrix ? 0 : b * lines * pitch);
+        for (int64_t o = 0; o < out_len; ++o) {
+            double s2 = accumulate ? (double)out[b * out_len + o] : 0.0;
+            for (int64_t r = 0; r < vec_len; ++r)
+                s2 += (is_mv ? (double)Mb[o * rs + r * cs] : (double)Mb[r * rs + o * cs]) * (double)v[b * vec_len + r];
+            want[(size_t)(b * out_len + o)] = s2;
+        }
+    }
+    (void)mat_elems;
+    replay_register(Mx, m_n * 4); replay_register(v, v_n * 4); replay_register(out, o_n * 4);
+    const int64_t bshape[1] = {nb}, mstr[1] = {shared_matrix ? 0 : lines * pitch}, vstr[1] = {vec_len};
+    int rc;
+    if (is_mv) rc = tenmo_hip_mv_f32(Mx, 0, rs, cs, v, 0, 1, out, rows, cols, batch > 0 ? 1 : 0, bshape, mstr, vstr, accumulate, 1);
+    else if (noalloc) rc = tenmo_hip_vm_f32_noalloc(v, 0, 1, Mx, 0, rs, cs, out, rows, cols, batch > 0 ? 1 : 0, bshape, vstr, mstr, accumulate, 1);
+    else rc = tenmo_hip_vm_f32(v, 0, 1, Mx, 0, rs, cs, out, rows, cols, batch > 0 ? 1 : 0, bshape, vstr, mstr, accumulate, 1);
+    int bad = 0;
+    double err = -1;
+    if (rc != 0) { fprintf(stderr, "%s: error %d: %s\n", spec.c_str(), rc, tenmo_hip_last_error()); bad = 1; }
+    else { err = gradient_error(out, want); if (!(err <= 2e-6)) bad = 1; }
+    printf("%s: rc %d, relative error %.3g%s\n", spec.c_str(), rc, err, bad ? "  <-- FAILED" : "");
+    fflush(stdout);
+    replay_register(Mx, 0); replay_register(v, 0); replay_register(out, 0);
+    free(Mx); free(v); free(out);
+    return bad;
+}
+
+static std::vector<int64_t> numbers_of(const std::string& spec, size_t from) {
+    std::vector<int64_t> out;
+    size_t pos = from;
+    while (pos <= spec.size()) {
+        const size_t c = spec.find(',', pos);
+        out.push_back(atoll(spec.substr(pos, c == std::string::npos ? std::string::npos : c - pos).c_str()));
+        if (c == std::string::npos) break;
+        pos = c + 1;
+    }
+    return out;
+}
+
+static float* exact_block(size_t n, bool fill = true) {
+    float* p = (float*)malloc(n ? n * 4 : 1);
+    for (size_t i = 0; i < n && fill; ++i) p[i] = next_float();
+    replay_register(p, n ? n * 4 : 1);
+    return p;
+}
+static void drop_block(void* p) { replay_register(p, 0); free(p); }
+
+// entry points whose numbers the parity tests check: here only that every access stays inside exactly-sized operands
+static int run_address_only_case(const std::string& spec) {
+    int rc = 0;
+    if (spec.compare(0, 3, "ce:") == 0) {
+        const std::vector<int64_t> a = numbers_of(spec, 3);
+        if (a.size() < 4) return 2;
+        const int64_t M = a[0], C = a[1];
+        const bool i64 = a[2] != 0;
+        const float ls = (float)a[3] / 100.f;
+        float* logits = exact_block((size_t)(M * C));
+        void* target = malloc((size_t)M * (i64 ? 8 : 4));
+        replay_register(target, (size_t)M * (i64 ? 8 : 4));
+        for (int64_t m = 0; m < M; ++m) {
+            const int64_t t = (m % 7 == 3) ? -100 : (m * 31) % C;
+            if (i64) ((int64_t*)target)[m] = t; else ((int32_t*)target)[m] = (int32_t)t;
+        }
+        float* softmax = exact_block((size_t)(M * C), false); float* per = exact_block((size_t)M, false); float* sum = exact_block(1, false);
+        int32_t* valid = (int32_t*)exact_block(1, false); float* up = exact_block(1); float* grad = exact_block((size_t)(M * C));
+        rc = tenmo_hip_cross_entropy_forward_f32(logits, target, i64, M, C, -100, ls, softmax, per, sum, valid, 1);
+        if (rc == 0) rc = tenmo_hip_cross_entropy_forward_f32(logits, target, i64, M, C, -100, ls, nullptr, per, sum, valid, 1);
+        if (rc == 0) rc = tenmo_hip_cross_entropy_backward_f32(softmax, target, i64, up, M, C, -100, ls, 2, valid[0], grad, 0, 1);
+        if (rc == 0) rc = tenmo_hip_cross_entropy_backward_f32(softmax, target, i64, up, M, C, -100, ls, 1, valid[0], grad, 1, 1);
+        drop_block(logits); drop_block(target); drop_block(softmax); drop_block(per); drop_block(sum); drop_block(valid); drop_block(up); drop_block(grad);
+    } else if (spec.compare(0, 5, "conv:") == 0) {
+        const std::vector<int64_t> a = numbers_of(spec, 5);
+        if (a.size() < 9) return 2;
+        const int64_t N = a[0], Ci = a[1], H = a[2], W = a[3], Co = a[4], KH = a[5], KW = a[6], st = a[7], dil = a[8];
+        const int64_t Ho = (H - (KH + (KH - 1) * (dil - 1))) / st + 1, Wo = (W - (KW + (KW - 1) * (dil - 1))) / st + 1;
+        float* img = exact_block((size_t)(N * Ci * H * W)); float* ker = exact_block((size_t)(Co * Ci * KH * KW)); float* bias = exact_block((size_t)Co);
+        float* out = exact_block((size_t)(N * Co * Ho * Wo), false); float* gout = exact_block((size_t)(N * Co * Ho * Wo));
+        float* gimg = exact_block((size_t)(N * Ci * H * W)); float* gker = exact_block((size_t)(Co * Ci * KH * KW)); float* gbias = exact_block((size_t)Co);
+        rc = tenmo_hip_conv2d_forward_f32(img, N, Ci, H, W, ker, Co, KH, KW, bias, st, dil, out, 1);
+        if (rc == 0) rc = tenmo_hip_conv2d_backward_f32(img, N, Ci, H, W, ker, Co, KH, KW, st, dil, gout, gimg, gker, gbias, 0, 1);
+        if (rc == 0) rc = tenmo_hip_conv2d_backward_f32(img, N, Ci, H, W, ker, Co, KH, KW, st, dil, gout, gimg, gker, gbias, 1, 1);
+        drop_block(img); drop_block(ker); drop_block(bias); drop_block(out); drop_block(gout); drop_block(gimg); drop_block(gker); drop_block(gbias);
+    } else {
+        const std::vector<int64_t> a = numbers_of(spec, 5);
+        if (a.empty()) return 2;
+        const int64_t n = a[0];
+        float* x = exact_block((size_t)n); float* y = exact_block((size_t)n); float* d = exact_block(1, false);
+        rc = tenmo_hip_dot_f32(x, 0, 1, y, 0, 1, n, d, 1);
+        float* vel = exact_block((size_t)n);
+        if (rc == 0) rc = tenmo_hip_sgd_step_f32(x, y, nullptr, n, 0.01f, 0.f, 0.f, 1);
+        if (rc == 0) rc = tenmo_hip_sgd_step_f32(x, y, vel, n, 0.01f, 0.9f, 1e-4f, 1);
+        const int64_t rows = n / 64 + 1, cols = 64 + n % 61;
+        float* G = exact_block((size_t)(rows * cols)); float* cs = exact_block((size_t)cols);
+        if (rc == 0) rc = tenmo_hip_column_sum_f32(G, 0, cols, rows, cols, cs, 1, 1);
+        drop_block(x); drop_block(y); drop_block(d); drop_block(vel); drop_block(G); drop_block(cs);
+    }
+    if (rc != 0) fprintf(stderr, "%s: error %d: %s\n", spec.c_str(), rc, tenmo_hip_last_error());
+    printf("%s: rc %d, relative error n/a\n", spec.c_str(), rc);
+    fflush(stdout);
+    return rc != 0;
+}
+
 static tenmo_view view_of(const float* p, int64_t batch, int64_t rows, int64_t cols, bool transposed) {
     tenmo_view v;
     memset(&v, 0, sizeof(v));
@@ -123,12 +268,6 @@ static tenmo_view view_of(const float* p, int64_t batch, int64_t rows, int64_t c
     v.shape[r] = cols; v.strides[r] = transposed ? rows : 1; ++r;
     v.rank = r;
     return v;
-}
-
-__attribute__((no_sanitize("address"))) static double gradient_error(const float* got, const std::vector<double>& want) {
-    double num = 0.0, den = 0.0;
-    for (size_t i = 0; i < want.size(); ++i) { const double d = (double)got[i] - want[i]; num += d * d; den += want[i] * want[i]; }
-    return std::sqrt(num / (den > 0 ? den : 1.0));
 }
 
 static int run_backward_case(const std::string& spec) {
@@ -199,7 +338,11 @@ int main(int argc, char** argv) {
     for (int i = 1; i < argc; ++i) {
         if (!strcmp(argv[i], "late")) { replay_set_late_loads(1); continue; }
         if (!strcmp(argv[i], "early")) { replay_set_late_loads(0); continue; }
-        bad |= strncmp(argv[i], "bwd:", 4) == 0 ? run_backward_case(argv[i]) : run_case(argv[i]);
+        if (strncmp(argv[i], "bwd:", 4) == 0) bad |= run_backward_case(argv[i]);
+        else if (strncmp(argv[i], "ce:", 3) == 0 || strncmp(argv[i], "conv:", 5) == 0 || strncmp(argv[i], "misc:", 5) == 0) bad |= run_address_only_case(argv[i]);
+        else if (strncmp(argv[i], "mv:", 3) == 0) bad |= run_vector_case(argv[i], true);
+        else if (strncmp(argv[i], "vm:", 3) == 0) bad |= run_vector_case(argv[i], false);
+        else bad |= run_case(argv[i]);
     }
     tenmo_hip_shutdown();
     return bad;

@@ -144,6 +144,38 @@ def test_gradients_of_broadcast_parents(exe):
     run(exe, ["bwd:256,1024,512,n,n,0,4,fold_reduce=1", "bwd:512,256,1024,n,n,1,6"], cus=256, modes=("late",))
 
 
+def test_matrix_vector_kernels(exe):
+    """mv and vm (tenmo_amd/csrc/gemv.hpp: the row kernel, the column kernels with aligned, shifted and element loads, their K
+    slices and the slice reduction, the allocation-free entry) on matrices that END with their last element: row pitches that
+    are and are not multiples of four floats, row counts and widths around the kernels' vector and unroll widths, batches, a
+    matrix shared by the batches, accumulate."""
+    cases = []
+    for m, k in [(1, 1), (7, 5), (64, 1024), (515, 1030), (130, 4097), (1000, 33), (33, 6000)]:
+        for layout in ("n", "t"):
+            for pad in (0, 1, 4):
+                cases.append(f"mv:{m},{k},{layout},0,{pad},0")
+    cases += ["mv:70,300,n,3,0,1", "mv:70,300,t,3,2,1", "mv:65,257,n,-4,0,0", "mv:2048,768,n,0,0,0"]
+    for k, n in [(1, 1), (5, 7), (1024, 64), (1030, 515), (300, 4099), (33, 1000), (2000, 50257 // 8)]:
+        for layout in ("n", "t"):
+            for pad in (0, 1, 4):
+                cases.append(f"vm:{k},{n},{layout},0,{pad},0")
+    cases += ["vm:300,70,n,3,0,1", "vm:300,1027,n,3,1,1", "vm:257,65,t,-4,0,0", "vm:4096,1500,n,0,0,1,entry=noalloc", "vm:700,260,n,2,0,1,entry=noalloc",
+              "vm:768,4096,n,0,0,0", "vm:100,50000,n,0,0,0"]
+    run(exe, cases, cus=16, modes=("early",))
+    run(exe, cases[::5], cus=256, modes=("early",))
+
+
+def test_adjacent_operators(exe):
+    """Cross-entropy (forward with and without the softmax written, backward mean / sum), the convolution (forward and the
+    three gradients: gathered operands, dilated and strided phases), dot, SGD and the column sum on exactly-sized operands:
+    addresses only (their numbers are the parity tests' business)."""
+    cases = ["ce:1,1,0,0", "ce:7,10,0,0", "ce:64,10,1,10", "ce:33,1000,0,0", "ce:5,50257,1,10", "ce:300,4099,0,0", "ce:2,100003,0,5",
+             "conv:1,1,5,5,1,3,3,1,1", "conv:2,3,12,11,8,3,3,1,1", "conv:2,4,15,14,6,3,2,2,1", "conv:1,5,17,17,7,3,3,1,2", "conv:3,16,10,10,32,3,3,1,1",
+             "conv:2,3,9,9,4,1,1,1,1", "conv:1,8,20,20,16,5,5,3,1",
+             "misc:1", "misc:63", "misc:1000", "misc:300001"]
+    run(exe, cases, cus=16, modes=("early",))
+
+
 def test_one_step_reduction_into_a_large_result(exe):
     """[8192,16].[16,8192] with B a transposed view, at full size and on the real 256 CUs: the launch after which a GPU run
     once ended in a memory fault (what ran then: this shape through the short-reduction kernel, the K-stream kernel and
