@@ -63,6 +63,8 @@ def main() -> int:
     ap.add_argument("--size", type=int, default=8192, help="M=N=K of the square GEMM (default: the headline size)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-extra", action="store_true", help="skip the per-configuration rows and the MLP-step measurement")
+    ap.add_argument("--mlp-fused-tail", action="store_true",
+                    help="also time the MLP step with its last two layers, loss, backward and update fused into one launch (mlp_fused_tail knob)")
     ap.add_argument("--rows", default="", help="comma-separated substrings: only the rows whose name contains one of them")
     ap.add_argument("--adjacent", action="store_true",
                     help="also time the adjacent operators (cross-entropy, SGD step, convolution) into `extra`; off by default")
@@ -175,7 +177,7 @@ def main() -> int:
         out["cpu_baseline"] = cpu_gemm_baseline(A, B, S, np)
         del A, B
         if not args.no_extra:
-            extra.update(mlp_step_times(_lib, torch, np))
+            extra.update(mlp_step_times(_lib, torch, np, args.mlp_fused_tail))
     if extra:
         out["extra"] = extra
     print(json.dumps(out), flush=True)
@@ -437,9 +439,11 @@ def _timed(fn):
     return time.perf_counter() - t0
 
 
-def mlp_step_times(_lib, torch, np):
+def mlp_step_times(_lib, torch, np, fused_tail=False):
     """MNIST-shaped MLP 784->128->32->10, batch 64, SGD lr 0.01: ms per training step on the GPU (inputs
-    already on the device) and on the CPU restatement, and the largest per-step loss difference."""
+    already on the device) and on the CPU restatement, and the largest per-step loss difference.  With
+    `fused_tail` the same 20 steps once more with the last two layers, the loss, their backward and their
+    update as one launch."""
     from oracle import oracle as O
     from tenmo_amd import rng as R
     from tenmo_amd.net import MLP
@@ -469,11 +473,23 @@ def mlp_step_times(_lib, torch, np):
         gpu.step_device(xd, yd, lr, sync=False, graph=True)
     _lib.check(L.tenmo_hip_sync())
     graph_ms = (time.perf_counter() - t0) * 1e3 / 20
+    fused = {}
+    if fused_tail:
+        L.tenmo_hip_set_tuning(b"mlp_fused_tail", 1)
+        try:
+            first = float(gpu.step_device(*dev[0], lr, sync=True).item())
+            t0 = time.perf_counter()
+            for xd, yd in dev[10:]:
+                gpu.step_device(xd, yd, lr, sync=False)
+            _lib.check(L.tenmo_hip_sync())
+            fused = {"mlp_step_ms_gpu_fused_tail": round((time.perf_counter() - t0) * 1e3 / 20, 4), "mlp_fused_tail_first_loss": first}
+        finally:
+            L.tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
     t0 = time.perf_counter()
     for x, y in batches[10:]:
         cpu.step(x, y, lr)
     cpu_ms = (time.perf_counter() - t0) * 1e3 / 20
-    return {"mlp_step_ms_gpu": round(gpu_ms, 4), "mlp_step_ms_gpu_graph": round(graph_ms, 4), "mlp_step_ms_cpu": round(cpu_ms, 4), "mlp_cpu_cores": O.num_physical_cores(),
+    return {**fused, "mlp_step_ms_gpu": round(gpu_ms, 4), "mlp_step_ms_gpu_graph": round(graph_ms, 4), "mlp_step_ms_cpu": round(cpu_ms, 4), "mlp_cpu_cores": O.num_physical_cores(),
             "mlp_max_abs_loss_diff_first10": worst}
 
 

@@ -218,6 +218,150 @@ __global__ void cross_entropy_kernel(const float* __restrict logits, const int32
     }
 }
 
+// ---- the small end of an MLP training step in ONE launch ------------------------------------------------------------
+// For a network whose last two Linear layers are small (the MNIST example's 128 -> 32 -> 10 at batch 64,
+// examples/mnist.mojo:150-162): both layers forward (bias, ReLU between them), the class-index cross-entropy (mean) with
+// its gradient, both layers backward (weight and bias gradients, ReLU masks), the gradient handed to the layer below with
+// that layer's ReLU mask and bias gradient, and the SGD update of both layers — by one workgroup with every operand in
+// LDS.  Run op by op these are eight dependent launches of a few microseconds each, which is what such a step costs; the
+// reference names the same cause for its GPU time (docs/from-bytes-to-gradients.md:454).
+constexpr int MLP_TAIL_THREADS = 256;
+constexpr int MLP_TAIL_MAX_B = 64, MLP_TAIL_MAX_D0 = 128, MLP_TAIL_MAX_D1 = 64, MLP_TAIL_MAX_C = 32;
+struct MlpTailArgs {
+    const float* h0;      // [B, D0] output of the layer below (after its ReLU)
+    const int32_t* y;     // [B]
+    float *W1, *b1;       // [D0, D1], [D1]: updated in place
+    float *W2, *b2;       // [D1, C], [C]
+    float *dW1, *db1, *dW2, *db2;
+    float *h1, *logits;   // [B, D1], [B, C]: the two layers' outputs, kept as the op-by-op path keeps them
+    float* g0;            // [B, D0]: gradient for the layer below, already multiplied by its ReLU gradient (h0 > 0)
+    float* db0;           // [D0]: that layer's bias gradient (column sums of g0)
+    float* row_loss;      // [B]
+    float* loss_out;      // [1]
+    float lr;
+    int32_t B, D0, D1, C;
+};
+
+// C[M][N] = A[M][K] . B[K][N] on LDS operands with arbitrary element strides; every thread of the workgroup takes blocks of 2
+// rows x 4 columns (the columns a quarter of the width apart, so that neighbouring lanes read neighbouring columns); rows and
+// columns beyond the extents are clamped for the loads and skipped by `emit(m, n, value)`.
+template <class Emit>
+__device__ __forceinline__ void lds_product(int M, int N, int K, const float* A, int a_rs, int a_cs, const float* B, int b_rs, int b_cs, Emit&& emit) {
+    const int nq = (N + 3) / 4, mh = (M + 1) / 2;
+    for (int blk = threadIdx.x; blk < mh * nq; blk += MLP_TAIL_THREADS) {
+        const int m0 = (blk / nq) * 2, q = blk % nq;
+        const int m1 = min(m0 + 1, M - 1);
+        int n[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) n[j] = min(q + j * nq, N - 1);
+        float acc[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+        for (int k = 0; k < K; ++k) {
+            const float a0 = A[m0 * a_rs + k * a_cs], a1 = A[m1 * a_rs + k * a_cs];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const float b = B[k * b_rs + n[j] * b_cs];
+                acc[0][j] += a0 * b;
+                acc[1][j] += a1 * b;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            if (q + j * nq >= N) continue;
+            emit(m0, n[j], acc[0][j]);
+            if (m0 + 1 < M) emit(m0 + 1, n[j], acc[1][j]);
+        }
+    }
+}
+
+__global__ __launch_bounds__(MLP_TAIL_THREADS) void mlp_tail_kernel(const MlpTailArgs a) {
+    // odd pitches: a column walk never stays on one LDS bank
+    constexpr int P0 = MLP_TAIL_MAX_D0 + 1, P1 = MLP_TAIL_MAX_D1 + 1, PC = MLP_TAIL_MAX_C + 1;
+    __shared__ float h0[MLP_TAIL_MAX_B * P0];   // [B][D0]; becomes g0 at the end
+    __shared__ float w1[MLP_TAIL_MAX_D0 * P1];  // [D0][D1]
+    __shared__ float h1[MLP_TAIL_MAX_B * P1];   // [B][D1]
+    __shared__ float g1[MLP_TAIL_MAX_B * P1];   // [B][D1]
+    __shared__ float w2[MLP_TAIL_MAX_D1 * PC];  // [D1][C]
+    __shared__ float z[MLP_TAIL_MAX_B * PC];    // [B][C]: logits, then their gradient
+    __shared__ float bias1[MLP_TAIL_MAX_D1], bias2[MLP_TAIL_MAX_C];
+    const int B = a.B, D0 = a.D0, D1 = a.D1, C = a.C, t = threadIdx.x;
+    for (int i = t; i < B * D0; i += MLP_TAIL_THREADS) h0[(i / D0) * P0 + i % D0] = a.h0[i];
+    for (int i = t; i < D0 * D1; i += MLP_TAIL_THREADS) w1[(i / D1) * P1 + i % D1] = a.W1[i];
+    for (int i = t; i < D1 * C; i += MLP_TAIL_THREADS) w2[(i / C) * PC + i % C] = a.W2[i];
+    for (int i = t; i < D1; i += MLP_TAIL_THREADS) bias1[i] = a.b1[i];
+    for (int i = t; i < C; i += MLP_TAIL_THREADS) bias2[i] = a.b2[i];
+    __syncthreads();
+    // forward: h1 = relu(h0 . W1 + b1), logits = h1 . W2 + b2      (tenmo/net.mojo:193-201, tenmo/relu.mojo:99-118)
+    lds_product(B, D1, D0, h0, P0, 1, w1, P1, 1, [&](int m, int n, float v) {
+        v += bias1[n];
+        v = v > 0.f ? v : 0.f;
+        h1[m * P1 + n] = v;
+        a.h1[m * D1 + n] = v;
+    });
+    __syncthreads();
+    lds_product(B, C, D1, h1, P1, 1, w2, PC, 1, [&](int m, int n, float v) {
+        v += bias2[n];
+        z[m * PC + n] = v;
+        a.logits[m * C + n] = v;
+    });
+    __syncthreads();
+    // cross-entropy, mean over the batch, and its gradient (tenmo/crossentropy.mojo:285-432, :775-793): one thread per row
+    if (t < B) {
+        float* x = z + t * PC;
+        float mx = -3.402823466e+38f;
+        for (int c = 0; c < C; ++c) mx = fmaxf(mx, x[c]);
+        float sum_exp = 0.f;
+        for (int c = 0; c < C; ++c) sum_exp += expf(x[c] - mx);
+        const float lse = logf(fmaxf(sum_exp, 1e-7f));
+        const int32_t label = a.y[t];
+        a.row_loss[t] = (label >= 0 && label < C) ? -(x[label] - mx - lse) : __builtin_nanf("");
+        const float inv = 1.f / sum_exp, scale = 1.f / (float)B;
+        for (int c = 0; c < C; ++c) x[c] = (expf(x[c] - mx) * inv - (c == label ? 1.f : 0.f)) * scale;
+    }
+    __syncthreads();
+    if (t == 0) { // the reference's scalar loop order
+        float s = 0.f;
+        for (int r = 0; r < B; ++r) s += a.row_loss[r];
+        *a.loss_out = s / (float)B;
+    }
+    if (t < C) { // db2 = column sums of the logits' gradient, rows ascending (tenmo/broadcast.mojo:81-87)
+        float s = 0.f;
+        for (int r = 0; r < B; ++r) s += z[r * PC + t];
+        a.db2[t] = s;
+        a.b2[t] = bias2[t] - a.lr * s;
+    }
+    // dW2 = h1^T . dz, g1 = (dz . W2^T) masked by h1 > 0      (tenmo/matmul.mojo:36-48, tenmo/relu.mojo:120-123)
+    lds_product(D1, C, B, h1, 1, P1, z, PC, 1, [&](int m, int n, float v) {
+        a.dW2[m * C + n] = v;
+        a.W2[m * C + n] = w2[m * PC + n] - a.lr * v;
+    });
+    lds_product(B, D1, C, z, PC, 1, w2, 1, PC, [&](int m, int n, float v) { g1[m * P1 + n] = h1[m * P1 + n] > 0.f ? v : 0.f; });
+    __syncthreads();
+    if (t < D1) {
+        float s = 0.f;
+        for (int r = 0; r < B; ++r) s += g1[r * P1 + t];
+        a.db1[t] = s;
+        a.b1[t] = bias1[t] - a.lr * s;
+    }
+    // dW1 = h0^T . g1 (with the update of W1 in global memory; the LDS copy keeps the old weights for g0)
+    lds_product(D0, D1, B, h0, 1, P0, g1, P1, 1, [&](int m, int n, float v) {
+        a.dW1[m * D1 + n] = v;
+        a.W1[m * D1 + n] = w1[m * P1 + n] - a.lr * v;
+    });
+    __syncthreads(); // h0 is overwritten below
+    // g0 = (g1 . W1^T) masked by h0 > 0, in place of h0
+    lds_product(B, D0, D1, g1, P1, 1, w1, 1, P1, [&](int m, int n, float v) {
+        v = h0[m * P0 + n] > 0.f ? v : 0.f;
+        h0[m * P0 + n] = v;
+        a.g0[m * D0 + n] = v;
+    });
+    __syncthreads();
+    if (t < D0) {
+        float s = 0.f;
+        for (int r = 0; r < B; ++r) s += h0[r * P0 + t];
+        a.db0[t] = s;
+    }
+}
+
 // loss = (sum of row losses in row order) / rows — the order of the reference's scalar loop
 __global__ void ordered_mean_kernel(const float* __restrict row_loss, int64_t rows, float* __restrict out) {
     if (blockIdx.x == 0 && threadIdx.x == 0) {

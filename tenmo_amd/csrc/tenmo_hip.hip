@@ -89,6 +89,7 @@ struct State {
     int force_streamk = -1;    // -1 automatic, 0 never, n > 0: stream-K with n workgroups per CU
     int force_smallk = -1;     // -1 automatic, 0 never, 1: the short-reduction kernel wherever it can run
     int force_panel = -1;      // -1 automatic, 0 never, 1: the persistent K-stream kernel wherever it can run
+    int mlp_fused_tail = 0;    // the last two layers of an MLP step, loss, their backward and update in one launch: 1 when the shapes fit, 0 never
     int fold_reduce = -1;      // the gradient of a broadcast parent summed inside the GEMM launch: -1 automatic, 0 never, 1 wherever it can
     int verbose = 0;
     int cols_waves_per_cu = 2; // target workgroups per CU of the column-streaming kernels (long K slices stream best)
@@ -1039,6 +1040,7 @@ int tenmo_hip_set_tuning(const char* name, int value) {
     if (!strcmp(name, "gemm_smallk")) { S.force_smallk = value; return 0; }
     if (!strcmp(name, "gemm_panel")) { S.force_panel = value; return 0; }
     if (!strcmp(name, "fold_reduce")) { S.fold_reduce = value; return 0; }
+    if (!strcmp(name, "mlp_fused_tail")) { S.mlp_fused_tail = value; return 0; }
     if (!strcmp(name, "conv_phases")) { S.force_conv_phases = value; return 0; }
     if (!strcmp(name, "cols_wg_per_cu")) { S.cols_waves_per_cu = value > 0 ? value : 2; return 0; }
     return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: unknown knob '%s'", name);
@@ -1850,11 +1852,13 @@ void tenmo_hip_mlp_destroy(tenmo_mlp* m) {
     delete m;
 }
 
-static int mlp_forward(tenmo_mlp* m, const float* x, int64_t B) {
+// the first `layers` layers (all of them by default)
+static int mlp_forward(tenmo_mlp* m, const float* x, int64_t B, int layers = -1) {
+    if (layers < 0) layers = m->L;
     BatchDesc bd{};
     for (int d = 0; d < MAX_BATCH_RANK; ++d) bd.shape[d] = 1;
     const float* in = x;
-    for (int l = 0; l < m->L; ++l) {
+    for (int l = 0; l < layers; ++l) {
         const int64_t I = m->dims[l], O = m->dims[l + 1];
         Epilogue ep; // bias add and ReLU happen in the GEMM store
         ep.bias = m->b[l]; ep.relu = l + 1 < m->L ? 1 : 0;
@@ -1875,11 +1879,29 @@ int tenmo_hip_mlp_forward(tenmo_mlp* m, const float* x, int64_t B, float* logits
 
 // enqueues every kernel of one training step on the library stream
 static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int64_t B, float lr, float* loss_out) {
-    if (int rc = mlp_forward(m, x, B)) return rc;
     const int L = m->L;
     const int64_t C = m->dims[L];
+    // The last two layers, the loss, their backward and their update as one launch (mlp_tail_kernel) when they fit one
+    // workgroup's LDS; the layers below run as usual on either side of it.
+    const bool fused_tail = S.mlp_fused_tail > 0 && L >= 3 && B <= MLP_TAIL_MAX_B && m->dims[L - 2] <= MLP_TAIL_MAX_D0 &&
+                            m->dims[L - 1] <= MLP_TAIL_MAX_D1 && C <= MLP_TAIL_MAX_C;
+    const int top = fused_tail ? L - 2 : L; // layers [0, top) run op by op
+    if (int rc = mlp_forward(m, x, B, top)) return rc;
+    if (fused_tail) {
+        MlpTailArgs t{};
+        t.h0 = m->act[L - 3]; t.y = y;
+        t.W1 = m->W[L - 2]; t.b1 = m->b[L - 2]; t.W2 = m->W[L - 1]; t.b2 = m->b[L - 1];
+        t.dW1 = m->dW[L - 2]; t.db1 = m->db[L - 2]; t.dW2 = m->dW[L - 1]; t.db2 = m->db[L - 1];
+        t.h1 = m->act[L - 2]; t.logits = m->act[L - 1];
+        t.g0 = m->grad[L - 3]; t.db0 = m->db[L - 3];
+        t.row_loss = m->row_loss; t.loss_out = loss_out; t.lr = lr;
+        t.B = (int32_t)B; t.D0 = (int32_t)m->dims[L - 2]; t.D1 = (int32_t)m->dims[L - 1]; t.C = (int32_t)C;
+        hipLaunchKernelGGL(mlp_tail_kernel, dim3(1), dim3(MLP_TAIL_THREADS), 0, S.stream, t);
+    }
     const bool one_block = B <= 256; // loss, its gradient, the mean and the last bias gradient in one launch
-    if (one_block) {
+    if (fused_tail) {
+        // done by the tail launch
+    } else if (one_block) {
         hipLaunchKernelGGL(cross_entropy_kernel, dim3(1), dim3((unsigned)((B + 63) / 64 * 64)), 0, S.stream, m->act[L - 1], y, B, C, m->grad[L - 1], m->row_loss, loss_out, m->db[L - 1]);
     } else {
         hipLaunchKernelGGL(cross_entropy_kernel, dim3((unsigned)((B + 63) / 64)), dim3(64), 0, S.stream, m->act[L - 1], y, B, C, m->grad[L - 1], m->row_loss, (float*)nullptr, (float*)nullptr);
@@ -1887,12 +1909,14 @@ static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int6
     }
     BatchDesc bd{};
     for (int d = 0; d < MAX_BATCH_RANK; ++d) bd.shape[d] = 1;
-    for (int l = L - 1; l >= 0; --l) {
+    for (int l = top - 1; l >= 0; --l) {
         const int64_t I = m->dims[l], O = m->dims[l + 1];
         const float* in = l == 0 ? x : m->act[l - 1];
         const float* gl = m->grad[l];
         const bool from_gemm = B <= 128; // hidden layers: summed in the store of the GEMM that produced this gradient (below)
-        if (one_block && l == L - 1) {
+        if (fused_tail && l == top - 1) {
+            // done by the tail launch
+        } else if (one_block && l == L - 1) {
             // done by the cross-entropy launch
         } else if (from_gemm && l < L - 1) {
             // done by the dX product of layer l+1
@@ -1918,11 +1942,11 @@ static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int6
                 if (int rc = gemm_dispatch(gl, O, 1, m->W[l], 1, O, m->grad[l - 1], B, I, O, bd, 1, 0, ep)) return rc;
         }
     }
-    // every parameter tensor in one launch
-    for (int l0 = 0; l0 < L; l0 += SGD_MAX_TENSORS / 2) {
+    // every parameter tensor (below the fused tail, which updates its own) in one launch
+    for (int l0 = 0; l0 < top; l0 += SGD_MAX_TENSORS / 2) {
         SgdArgs sa{};
         int64_t largest = 0;
-        for (int l = l0; l < L && sa.count + 2 <= SGD_MAX_TENSORS; ++l) {
+        for (int l = l0; l < top && sa.count + 2 <= SGD_MAX_TENSORS; ++l) {
             const int64_t wn = m->dims[l] * m->dims[l + 1], bn = m->dims[l + 1];
             sa.p[sa.count] = m->W[l]; sa.g[sa.count] = m->dW[l]; sa.n[sa.count] = wn; ++sa.count;
             sa.p[sa.count] = m->b[l]; sa.g[sa.count] = m->db[l]; sa.n[sa.count] = bn; ++sa.count;

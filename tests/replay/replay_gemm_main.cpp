@@ -12,6 +12,7 @@
 //   CASE = vm:k,n,layout,batch,pad,accumulate[,entry=noalloc]   out[n] = v[k] . Mx[k,n]; the matrix shared by every batch when batch < 0
 //   CASE = ce:M,C,target_is_int64,label_smoothing_percent    cross-entropy forward (all outputs) and backward (mean), addresses only
 //   CASE = conv:N,C_in,H_pad,W_pad,C_out,KH,KW,stride,dilation    convolution forward and backward (all three gradients), addresses only
+//   CASE = mlp:batch,d0,d1,d2,d3,fused    two training steps of a 3-layer MLP (tenmo_hip_mlp_step), addresses only
 //   CASE = misc:n      dot, column sum ([n/64+1, 64.. ] shapes derived from n), SGD with and without momentum, addresses only
 //   CASE = bwd:M,N,K,a_layout,b_layout,a_batch,b_batch[,knob=value...]   tenmo_hip_matmul_backward of A[a_batch, M, K] . B[b_batch, K, N]
 //     (a batch of 0: no batch dimension; 1: one that broadcasts): both gradients against float64, accumulated onto a start value
@@ -238,6 +239,31 @@ static int run_address_only_case(const std::string& spec) {
         if (rc == 0) rc = tenmo_hip_conv2d_backward_f32(img, N, Ci, H, W, ker, Co, KH, KW, st, dil, gout, gimg, gker, gbias, 0, 1);
         if (rc == 0) rc = tenmo_hip_conv2d_backward_f32(img, N, Ci, H, W, ker, Co, KH, KW, st, dil, gout, gimg, gker, gbias, 1, 1);
         drop_block(img); drop_block(ker); drop_block(bias); drop_block(out); drop_block(gout); drop_block(gimg); drop_block(gker); drop_block(gbias);
+    } else if (spec.compare(0, 4, "mlp:") == 0) {
+        const std::vector<int64_t> a = numbers_of(spec, 4);
+        if (a.size() < 6) return 2;
+        const int64_t B = a[0], dims[4] = {a[1], a[2], a[3], a[4]};
+        std::vector<std::vector<float>> W(3), bvec(3);
+        const float* Wp[3];
+        const float* bp[3];
+        for (int l = 0; l < 3; ++l) {
+            W[l].resize((size_t)(dims[l] * dims[l + 1])); bvec[l].resize((size_t)dims[l + 1]);
+            for (float& w : W[l]) w = 0.1f * next_float();
+            for (float& w : bvec[l]) w = 0.1f * next_float();
+            Wp[l] = W[l].data(); bp[l] = bvec[l].data();
+        }
+        tenmo_mlp* m = tenmo_hip_mlp_create(3, dims, Wp, bp, B);
+        float* x = exact_block((size_t)(B * dims[0]));
+        int32_t* y = (int32_t*)exact_block((size_t)B, false);
+        for (int64_t i = 0; i < B; ++i) y[i] = (int32_t)((i * 7) % dims[3]);
+        float* loss = exact_block(1, false);
+        tenmo_hip_set_tuning("mlp_fused_tail", (int)a[5]);
+        rc = m ? 0 : -1;
+        for (int step = 0; step < 2 && rc == 0; ++step) rc = tenmo_hip_mlp_step(m, x, y, B, 0.05f, loss, 1);
+        tenmo_hip_set_tuning("mlp_fused_tail", 0);
+        if (rc == 0 && !(loss[0] == loss[0])) rc = -100; // NaN
+        tenmo_hip_mlp_destroy(m);
+        drop_block(x); drop_block(y); drop_block(loss);
     } else {
         const std::vector<int64_t> a = numbers_of(spec, 5);
         if (a.empty()) return 2;
@@ -339,7 +365,8 @@ int main(int argc, char** argv) {
         if (!strcmp(argv[i], "late")) { replay_set_late_loads(1); continue; }
         if (!strcmp(argv[i], "early")) { replay_set_late_loads(0); continue; }
         if (strncmp(argv[i], "bwd:", 4) == 0) bad |= run_backward_case(argv[i]);
-        else if (strncmp(argv[i], "ce:", 3) == 0 || strncmp(argv[i], "conv:", 5) == 0 || strncmp(argv[i], "misc:", 5) == 0) bad |= run_address_only_case(argv[i]);
+        else if (strncmp(argv[i], "ce:", 3) == 0 || strncmp(argv[i], "conv:", 5) == 0 || strncmp(argv[i], "misc:", 5) == 0 || strncmp(argv[i], "mlp:", 4) == 0)
+            bad |= run_address_only_case(argv[i]);
         else if (strncmp(argv[i], "mv:", 3) == 0) bad |= run_vector_case(argv[i], true);
         else if (strncmp(argv[i], "vm:", 3) == 0) bad |= run_vector_case(argv[i], false);
         else bad |= run_case(argv[i]);

@@ -324,7 +324,10 @@ void run_on_pool(const std::function<void()>& job) {
 }
 } // namespace
 
+std::atomic<long> g_launches{0};
+
 void launch(const char* name, dim3 grid, dim3 block, std::function<void()> body) {
+    ++g_launches;
     const int64_t total = (int64_t)grid.x * grid.y * grid.z;
     if ((int64_t)block.x * block.y * block.z > MAX_LANES || total <= 0) fail("launch of %s: bad grid or block", name);
     std::atomic<int64_t> next{0};
@@ -454,4 +457,5 @@ void replay_register(const void* p, size_t bytes) {
     else replay::g_allocs.erase((uintptr_t)p);
 }
 void replay_set_late_loads(int on) { replay::late_loads = on; }
+long replay_launch_count() { return replay::g_launches.load(); } // kernel launches executed so far
 }

@@ -819,12 +819,22 @@ def test_sgd_vectors(T, golden):
         np.testing.assert_allclose(w.to_numpy(), s["expect"], rtol=1e-6)
 
 
-def test_mlp_loss_curve_tracks_cpu(T, oracle):
+@pytest.mark.parametrize("fused_tail", [0, 1])
+def test_mlp_loss_curve_tracks_cpu(T, oracle, fused_tail):
     """MNIST-shaped MLP 784->128->32->10, batch 64, Xavier, SGD lr=0.01: the per-step loss of the
-    GPU run stays within 1e-4 of the CPU restatement for every step."""
+    GPU run stays within 1e-4 of the CPU restatement for every step.  Op by op, and with the last two layers, the loss,
+    their backward and their update as one launch (the other shapes below fit that launch or fall back to op by op)."""
     from tenmo_amd import rng as R
     from tenmo_amd.net import MLP
 
+    T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", fused_tail)
+    try:
+        _mlp_loss_curve(T, oracle, R, MLP)
+    finally:
+        T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
+
+
+def _mlp_loss_curve(T, oracle, R, MLP):
     dims, seed, lr = [784, 128, 32, 10], 2024, 0.01
     Ws, bs = R.xavier_mlp(dims, seed)
     gpu, cpu = MLP(dims, Ws, bs, 64), oracle.MLP(dims, Ws, bs, 64)

@@ -172,7 +172,10 @@ def test_adjacent_operators(exe):
     cases = ["ce:1,1,0,0", "ce:7,10,0,0", "ce:64,10,1,10", "ce:33,1000,0,0", "ce:5,50257,1,10", "ce:300,4099,0,0", "ce:2,100003,0,5",
              "conv:1,1,5,5,1,3,3,1,1", "conv:2,3,12,11,8,3,3,1,1", "conv:2,4,15,14,6,3,2,2,1", "conv:1,5,17,17,7,3,3,1,2", "conv:3,16,10,10,32,3,3,1,1",
              "conv:2,3,9,9,4,1,1,1,1", "conv:1,8,20,20,16,5,5,3,1",
-             "misc:1", "misc:63", "misc:1000", "misc:300001"]
+             "misc:1", "misc:63", "misc:1000", "misc:300001",
+             # the MLP training step op by op and with its last two layers fused into one launch: the MNIST shape, the largest
+             # widths the fused launch takes, ragged ones, and a batch of one
+             "mlp:64,784,128,32,10,0", "mlp:64,784,128,32,10,1", "mlp:64,300,128,64,32,1", "mlp:37,50,77,33,7,1", "mlp:1,9,5,3,2,1"]
     run(exe, cases, cus=16, modes=("early",))
 
 
