@@ -54,40 +54,49 @@ def test_allocation_free_entry_point_on_the_replay():
     run_child([os.path.join("tests", "test_zz_no_alloc.py")])
 
 
+MLP_LAUNCH_COUNT_SCRIPT = r"""
+import ctypes as C, json, sys
+import numpy as np
+lib = C.CDLL(sys.argv[1])
+lib.replay_launch_count.restype = C.c_long
+lib.tenmo_hip_mlp_create.restype = C.c_void_p
+assert lib.tenmo_hip_init(0) == 0
+dims = [784, 128, 32, 10]
+rng = np.random.default_rng(3)
+Ws = [(rng.standard_normal((dims[i], dims[i + 1])) * 0.05).astype(np.float32) for i in range(3)]
+bs = [np.zeros(dims[i + 1], np.float32) for i in range(3)]
+x = rng.standard_normal((64, 784)).astype(np.float32)
+y = rng.integers(0, 10, 64).astype(np.int32)
+loss = np.zeros(1, np.float32)
+for arr in (x, y, loss):
+    lib.replay_register(C.c_void_p(arr.ctypes.data), C.c_size_t(arr.nbytes))
+fp = C.POINTER(C.c_float)
+results = {}
+for fused in (0, 1):
+    W_ptrs = (fp * 3)(*[w.ctypes.data_as(fp) for w in Ws])
+    b_ptrs = (fp * 3)(*[b.ctypes.data_as(fp) for b in bs])
+    m = lib.tenmo_hip_mlp_create(3, (C.c_int64 * 4)(*dims), W_ptrs, b_ptrs, C.c_int64(64))
+    assert m
+    lib.tenmo_hip_set_tuning(b"mlp_fused_tail", fused)
+    before = lib.replay_launch_count()
+    rc = lib.tenmo_hip_mlp_step(C.c_void_p(m), x.ctypes.data_as(fp), y.ctypes.data_as(C.POINTER(C.c_int32)), C.c_int64(64), C.c_float(0.01),
+                                loss.ctypes.data_as(fp), 1)
+    assert rc == 0
+    results[fused] = (lib.replay_launch_count() - before, float(loss[0]))
+    lib.tenmo_hip_mlp_destroy(C.c_void_p(m))
+print(json.dumps(results))
+"""
+
+
 def test_mlp_step_launch_count():
     """The MNIST-shaped training step (784 -> 128 -> 32 -> 10, batch 64) through the C ABI on the replay, counting kernel
     launches: op by op, and with the last two layers, the loss, their backward and their update fused into one launch
     (layer-1 forward as K slices and their reduction, the fused tail, layer-1 weight gradient, the update of layer 1: five against
-    nine); same loss either way."""
-    import ctypes as C
+    nine); same loss either way.  (In a child process: the replay ends the process when a kernel misbehaves.)"""
+    import json
 
-    import numpy as np
-
-    lib = C.CDLL(replay_build.build_library())
-    lib.replay_launch_count.restype = C.c_long
-    lib.tenmo_hip_mlp_create.restype = C.c_void_p
-    assert lib.tenmo_hip_init(0) == 0
-    dims = [784, 128, 32, 10]
-    rng = np.random.default_rng(3)
-    Ws = [(rng.standard_normal((dims[i], dims[i + 1])) * 0.05).astype(np.float32) for i in range(3)]
-    bs = [np.zeros(dims[i + 1], np.float32) for i in range(3)]
-    x = rng.standard_normal((64, 784)).astype(np.float32)
-    y = rng.integers(0, 10, 64).astype(np.int32)
-    loss = np.zeros(1, np.float32)
-    fp = C.POINTER(C.c_float)
-    results = {}
-    for fused in (0, 1):
-        W_ptrs = (fp * 3)(*[w.ctypes.data_as(fp) for w in Ws])
-        b_ptrs = (fp * 3)(*[b.ctypes.data_as(fp) for b in bs])
-        m = lib.tenmo_hip_mlp_create(3, (C.c_int64 * 4)(*dims), W_ptrs, b_ptrs, C.c_int64(64))
-        assert m
-        lib.tenmo_hip_set_tuning(b"mlp_fused_tail", fused)
-        before = lib.replay_launch_count()
-        rc = lib.tenmo_hip_mlp_step(C.c_void_p(m), x.ctypes.data_as(fp), y.ctypes.data_as(C.POINTER(C.c_int32)), C.c_int64(64), C.c_float(0.01),
-                                    loss.ctypes.data_as(fp), 1)
-        assert rc == 0
-        results[fused] = (lib.replay_launch_count() - before, float(loss[0]))
-        lib.tenmo_hip_mlp_destroy(C.c_void_p(m))
-    lib.tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
+    res = subprocess.run([sys.executable, "-c", MLP_LAUNCH_COUNT_SCRIPT, replay_build.build_library()], capture_output=True, text=True, timeout=600)
+    assert res.returncode == 0, res.stdout + res.stderr
+    results = {int(k): v for k, v in json.loads(res.stdout.strip().splitlines()[-1]).items()}
     assert results[1][0] <= 5 < results[0][0], results
     assert abs(results[0][1] - results[1][1]) <= 1e-5, results
