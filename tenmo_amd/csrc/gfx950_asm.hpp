@@ -16,6 +16,8 @@ __device__ __forceinline__ uint32_t lds_address(const float* lds) { return (uint
 // same in every lane: it lives in scalar registers) to bytes [16L, 16L+16) of the 1 KiB LDS block that starts
 // `block_byte_off` bytes into the LDS object `lds` (M0 holds the block's LDS address).  Scalar base + 32-bit lane offset addressing keeps vector ALU work out of the MFMA
 // stream: 64-bit per-lane address arithmetic between MFMAs was measured to cost 2 % at 8192^3.
+// (M0 is a register the compiler reserves: it sets it itself right before each of its own uses and keeps nothing in it
+// across other code, so writing it here needs no declaration — and the compiler rejects one.)
 // Issued through inline assembly on purpose: the compiler's wait-count pass otherwise drains every outstanding direct
 // load before any later LDS read, which would serialise a ring of stages.  The callers wait for these loads explicitly
 // with s_waitcnt vmcnt(n).
@@ -26,7 +28,9 @@ __device__ __forceinline__ void direct_load_16B(float* lds, uint32_t block_byte_
 
 // The same for the lanes with `ok` only: the others neither read memory nor write LDS.  The execution mask is narrowed
 // inside the assembly block, because under a divergent branch the compiler no longer keeps the block's scalar operands
-// in scalar registers.
+// in scalar registers.  Everything the block overwrites is declared: s_and_b64 sets SCC, and a block that does not say so
+// lets the compiler keep a carry in SCC across it — it then scheduled the s_addc_u32 of a 64-bit address behind this
+// block, the high half came out one too large (4 GiB off) and the next load faulted.
 __device__ __forceinline__ void direct_load_16B_where(float* lds, uint32_t block_byte_off, uint32_t lane_byte_off, const float* src, bool ok) {
     const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(lds) + block_byte_off);
     const uint32_t pred = ok ? 1u : 0u;
@@ -39,7 +43,7 @@ __device__ __forceinline__ void direct_load_16B_where(float* lds, uint32_t block
                  "s_mov_b64 exec, %0"
                  : "=&s"(saved_exec)
                  : "s"(dst), "v"(lane_byte_off), "s"(src), "v"(pred)
-                 : "memory", "vcc");
+                 : "memory", "vcc", "scc");
 }
 
 // keeps four accumulator chains alive without a store

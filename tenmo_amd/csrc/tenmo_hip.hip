@@ -383,9 +383,9 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
             if (mode == MNMAJOR_VEC) return row_s == 1 && k_s >= 0 && k_s <= (int64_t(1) << 25) && extent % 4 == 0 && extent >= 4;
             return false;
         };
-        // (Reductions of a single K step, K <= 16, stay with the ordinary kernel: a timing run of [8192,16].[16,8192] that went
-        // through this kernel, the K-stream kernel and the ordinary one in turn ended in a memory fault whose cause was not
-        // found; neither persistent kernel is needed there.)
+        // (Reductions of a single K step, K <= 16, stay with the ordinary kernel for now: a timing run of [8192,16].[16,8192]
+        // through this kernel faulted — an undeclared SCC clobber of the masked direct load, since fixed (gfx950_asm.hpp) — and
+        // the one-step instantiations come back once the fix has been confirmed on a GPU.)
         const bool can = K > GEMM_BK && K <= 64 && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum &&
                          N < (int64_t(1) << 29) && tiles64 <= 0x7fffffffLL;
         const bool want = S.force_smallk > 0 || (S.force_smallk < 0 && S.force_tile < 0 && S.force_splitk <= 0 && S.force_streamk <= 0 &&

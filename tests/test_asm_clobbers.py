@@ -1,0 +1,123 @@
+"""Inline assembly and the register allocator: what an asm block overwrites, it must declare.
+
+The direct global->LDS load for a subset of lanes (tenmo_amd/csrc/gfx950_asm.hpp) narrows the execution mask with
+s_and_b64, which also sets SCC.  While the block did not declare "scc", the compiler was free to keep a carry in SCC across
+it, and in some instantiations of the short-reduction kernel it did: s_add_u32 before the block, s_addc_u32 behind it, the
+high half of a 64-bit load address one too large — a load 4 GiB away from its operand and a GPU memory fault in exactly the
+instantiations that had this schedule (never in the others, never on the CPU).  Two checks:
+  * every asm statement of the kernel sources that contains an instruction writing SCC or VCC lists that register;
+  * the generated gfx950 ISA of gemm_smallk.hip (the one unit that uses such a block) has no instruction reading SCC behind
+    an asm block that overwrites it before something else sets it again.
+"""
+import os
+import re
+import subprocess
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+CSRC = os.path.join(ROOT, "tenmo_amd", "csrc")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+# scalar instructions that set SCC (gfx9: the SOP2 / SOP1 / SOPC arithmetic, logic, shift and compare groups)
+SCC_WRITERS = re.compile(r"\b(s_add_[ui]32|s_sub_[ui]32|s_addc_u32|s_subb_u32|s_cmp_\w+|s_and_b\d+|s_or_b\d+|s_xor_b\d+|s_andn2_b\d+|s_orn2_b\d+|"
+                         r"s_nand_b\d+|s_nor_b\d+|s_xnor_b\d+|s_lshl_b\d+|s_lshr_b\d+|s_ashr_i\d+|s_bfe_\w+|s_abs_i32|s_min_[ui]32|s_max_[ui]32|s_not_b\d+|"
+                         r"s_wqm_b\d+|s_quadmask_b\d+|s_bitcmp\d_b\d+|s_absdiff_i32|s_\w+_saveexec_b64|s_lshl[1-4]_add_u32)\b")
+SCC_READERS = re.compile(r"^\s*(s_addc_u32|s_subb_u32|s_cselect_b32|s_cselect_b64|s_cbranch_scc0|s_cbranch_scc1|s_cmov_b32|s_cmov_b64)\b")
+VCC_WRITERS = re.compile(r"\bv_cmp\w*_e32\b|\bvcc\s*,")
+
+
+def asm_statements(text):
+    """(template string, clobber string) of every asm statement with a non-empty template."""
+    out = []
+    for m in re.finditer(r"asm\s+volatile\s*\(", text):
+        depth, i = 1, m.end()
+        while depth:
+            depth += {"(": 1, ")": -1}.get(text[i], 0)
+            i += 1
+        body = text[m.end():i - 1]
+        strings = "".join(re.findall(r'"((?:[^"\\]|\\.)*)"', body.split(":")[0]))
+        clobbers = body.split(":")[3] if body.count(":") >= 3 else ""
+        if strings.strip():
+            out.append((strings, clobbers))
+    return out
+
+
+def test_asm_statements_declare_what_they_overwrite():
+    seen = 0
+    for name in sorted(os.listdir(CSRC)):
+        for template, clobbers in asm_statements(open(os.path.join(CSRC, name)).read()):
+            seen += 1
+            if SCC_WRITERS.search(template):
+                assert '"scc"' in clobbers, (name, template)
+            if VCC_WRITERS.search(template):
+                assert '"vcc"' in clobbers, (name, template)
+            if "exec" in template:  # the execution mask is saved and restored inside the block
+                assert re.search(r"s_mov_b64 %\d, exec", template) and re.search(r"s_mov_b64 exec, %\d", template), (name, template)
+    assert seen >= 2
+
+
+def scan_isa(text):
+    """SCC readers scheduled behind an asm block that overwrites SCC, before anything else sets it."""
+    hits, kernel = [], None
+    lines = text.split("\n")
+    i = 0
+    while i < len(lines):
+        m = re.match(r"^(_Z\S+):", lines[i])
+        if m:
+            kernel = m.group(1)
+        if "ASMSTART" in lines[i]:
+            j = i + 1
+            overwrites = False
+            while "ASMEND" not in lines[j]:
+                overwrites = overwrites or bool(SCC_WRITERS.search(lines[j]))
+                j += 1
+            if overwrites:
+                k = j + 1
+                while k < len(lines):
+                    t = lines[k]
+                    if "ASMSTART" in t or t.strip().startswith(".LBB") or "s_endpgm" in t:
+                        break
+                    if SCC_READERS.match(t):
+                        hits.append((kernel, k + 1, t.strip()))
+                        break
+                    if SCC_WRITERS.search(t):
+                        break
+                    k += 1
+            i = j
+        i += 1
+    return hits
+
+
+def test_the_scan_finds_the_schedule_that_faulted():
+    """The scanner on the sequence the compiler produced while the clobber was missing (K-major operands, one K step)."""
+    bad = """_ZN5tenmo18gemm_smallk_kernelILi0ELi0ELi1ELi4ELb0EEEvNS_8GemmArgsEjjji:
+	s_add_u32 s2, s17, s2
+	v_readfirstlane_b32 s17, v10
+	;;#ASMSTART
+	s_mov_b32 m0, s17
+	s_mov_b64 s[34:35], exec
+	v_cmp_ne_u32_e32 vcc, 0, v7
+	s_and_b64 exec, exec, vcc
+	global_load_lds_dwordx4 v11, s[30:31]
+	s_mov_b64 exec, s[34:35]
+	;;#ASMEND
+	v_add_lshl_u32 v12, v4, v12, 2
+	s_addc_u32 s3, s20, s3
+	s_endpgm
+"""
+    assert [h[2] for h in scan_isa(bad)] == ["s_addc_u32 s3, s20, s3"]
+    good = bad.replace("\ts_addc_u32 s3, s20, s3\n", "").replace("\tv_readfirstlane_b32 s17, v10\n", "\ts_addc_u32 s3, s20, s3\n\tv_readfirstlane_b32 s17, v10\n")
+    assert scan_isa(good) == []
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")
+def test_generated_isa_keeps_nothing_in_scc_across_the_masked_load(tmp_path):
+    out = str(tmp_path / "gemm_smallk.s")
+    cmd = [HIPCC, "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+           "-Wno-unused-result", "-I", os.path.join(ROOT, "include"), "--cuda-device-only", "-S", os.path.join(CSRC, "gemm_smallk.hip"), "-o", out]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    assert res.returncode == 0, res.stderr[-3000:]
+    text = open(out).read()
+    assert text.count("global_load_lds_dwordx4") > 100 and "s_and_b64 exec, exec, vcc" in text  # the blocks are there
+    assert scan_isa(text) == []

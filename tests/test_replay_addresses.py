@@ -181,7 +181,7 @@ def test_adjacent_operators(exe):
 
 def test_one_step_reduction_into_a_large_result(exe):
     """[8192,16].[16,8192] with B a transposed view, at full size and on the real 256 CUs: the launch after which a GPU run
-    once ended in a memory fault (what ran then: this shape through the short-reduction kernel, the K-stream kernel and
-    the ordinary one in turn; replayed here with the two persistent kernels still admitted for K <= 16, all three were
-    clean).  With K <= 16 the persistent kernels are no longer taken, so this replays the ordinary 64x64 kernel."""
+    once ended in a memory fault.  The source was right (this replay was clean for all three kernels that ran then); the
+    cause was an undeclared SCC clobber in an inline-assembly block, which only the generated ISA shows
+    (tests/test_asm_clobbers.py).  K <= 16 currently takes the ordinary 64x64 kernel, which is what this replays."""
     run(exe, [case(8192, 8192, 16, "n", "t")], modes=("early",), timeout=1200)
