@@ -23,7 +23,10 @@ __device__ __forceinline__ uint32_t lds_address(const float* lds) { return (uint
 // with s_waitcnt vmcnt(n).
 __device__ __forceinline__ void direct_load_16B(float* lds, uint32_t block_byte_off, uint32_t lane_byte_off, const float* src) {
     const uint32_t dst = __builtin_amdgcn_readfirstlane(lds_address(lds) + block_byte_off);
-    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(lane_byte_off), "s"(src) : "memory");
+    // s_nop 3: the scalar base may have come out of a v_readfirstlane right before this block, and a vector-memory
+    // instruction must not read a scalar register within 5 wait states of a vector instruction writing it — the compiler
+    // pads its own loads for that, but it does not look inside an asm block (the same padding covers M0: 1 wait state).
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 3\n\tglobal_load_lds_dwordx4 %1, %2" : : "s"(dst), "v"(lane_byte_off), "s"(src) : "memory");
 }
 
 // The same for the lanes with `ok` only: the others neither read memory nor write LDS.  The execution mask is narrowed
@@ -36,6 +39,7 @@ __device__ __forceinline__ void direct_load_16B_where(float* lds, uint32_t block
     const uint32_t pred = ok ? 1u : 0u;
     uint64_t saved_exec;
     asm volatile("s_mov_b32 m0, %1\n\t"
+                 "s_nop 1\n\t" // with the three instructions below: 5 wait states between code before the block and the load
                  "s_mov_b64 %0, exec\n\t"
                  "v_cmp_ne_u32_e32 vcc, 0, %4\n\t"
                  "s_and_b64 exec, exec, vcc\n\t"

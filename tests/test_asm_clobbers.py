@@ -5,7 +5,10 @@ s_and_b64, which also sets SCC.  While the block did not declare "scc", the comp
 it, and in some instantiations of the short-reduction kernel it did: s_add_u32 before the block, s_addc_u32 behind it, the
 high half of a 64-bit load address one too large — a load 4 GiB away from its operand and a GPU memory fault in exactly the
 instantiations that had this schedule (never in the others, never on the CPU).  Two checks:
-  * every asm statement of the kernel sources that contains an instruction writing SCC or VCC lists that register;
+  * every asm statement of the kernel sources that contains an instruction writing SCC or VCC lists that register, and one
+    that contains a vector-memory load keeps 5 wait states between its first instruction and that load (the load's scalar
+    base may have been written by a vector instruction just before the block: the compiler pads its own loads for that
+    documented hazard of the chip but does not look inside a block);
   * the generated gfx950 ISA of gemm_smallk.hip (the one unit that uses such a block) has no instruction reading SCC behind
     an asm block that overwrites it before something else sets it again.
 """
@@ -35,11 +38,28 @@ def asm_statements(text):
         while depth:
             depth += {"(": 1, ")": -1}.get(text[i], 0)
             i += 1
-        body = text[m.end():i - 1]
-        strings = "".join(re.findall(r'"((?:[^"\\]|\\.)*)"', body.split(":")[0]))
-        clobbers = body.split(":")[3] if body.count(":") >= 3 else ""
-        if strings.strip():
-            out.append((strings, clobbers))
+        body = re.sub(r"//[^\n]*", "", text[m.end():i - 1])  # comments between the template's lines
+        # the sections of the statement: split at the colons that are outside string literals
+        sections, current, in_string, k = [], "", False, 0
+        while k < len(body):
+            c = body[k]
+            if c == "\\" and in_string:
+                current += body[k:k + 2]
+                k += 2
+                continue
+            if c == '"':
+                in_string = not in_string
+            if c == ":" and not in_string:
+                sections.append(current)
+                current = ""
+            else:
+                current += c
+            k += 1
+        sections.append(current)
+        template = "".join(re.findall(r'"((?:[^"\\]|\\.)*)"', sections[0])).replace("\\n", "\n").replace("\\t", "\t")
+        clobbers = sections[3] if len(sections) > 3 else ""
+        if template.strip():
+            out.append((template, clobbers))
     return out
 
 
@@ -52,6 +72,15 @@ def test_asm_statements_declare_what_they_overwrite():
                 assert '"scc"' in clobbers, (name, template)
             if VCC_WRITERS.search(template):
                 assert '"vcc"' in clobbers, (name, template)
+            if "global_load" in template:
+                wait_states = 0
+                for instr in template.split("\n"):
+                    instr = instr.strip()
+                    if instr.startswith("global_load"):
+                        break
+                    nop = re.match(r"s_nop\s+(\d+)", instr)
+                    wait_states += int(nop.group(1)) + 1 if nop else (1 if instr else 0)
+                assert wait_states >= 5, (name, template, wait_states)
             if "exec" in template:  # the execution mask is saved and restored inside the block
                 assert re.search(r"s_mov_b64 %\d, exec", template) and re.search(r"s_mov_b64 exec, %\d", template), (name, template)
     assert seen >= 2
