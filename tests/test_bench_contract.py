@@ -1,0 +1,53 @@
+"""bench.py's one JSON line, checked without a GPU: the benchmark driver runs end to end against the CPU replay of the
+library at a small size (tests/replay: the numbers mean nothing there, the code path and the fields do)."""
+import json
+import os
+import subprocess
+import sys
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "tests", "replay"))
+import build as replay_build  # noqa: E402
+
+pytestmark = pytest.mark.skipif(not replay_build.available(), reason="no host clang++ at " + replay_build.CXX)
+
+RUNNER = """
+import runpy, sys
+import torch_on_host  # torch's cuda allocations on the host (tests/replay)
+sys.argv = ["bench.py"] + sys.argv[1:]
+runpy.run_path("bench.py", run_name="__main__")
+"""
+
+
+def run_bench(*flags):
+    env = dict(os.environ, TENMO_HIP_LIBRARY=replay_build.build_library(), REPLAY_STRICT="0",
+               PYTHONPATH=os.path.join(ROOT, "tests", "replay") + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    return subprocess.run([sys.executable, "-c", RUNNER] + list(flags), cwd=ROOT, env=env, capture_output=True, text=True, timeout=900)
+
+
+def test_one_json_line_with_every_field():
+    res = run_bench("--size", "256", "--steps", "2", "--warmup", "1", "--rows", "no-such-row", "--mlp-fused-tail", "--clock-probe-rounds", "4")
+    lines = [l for l in res.stdout.splitlines() if l.strip()]
+    assert res.returncode == 0 and len(lines) == 1, res.stdout[-2000:] + res.stderr[-2000:]
+    out = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step", "higher_is_better", "scaling", "vs_baseline", "dtype",
+                "data", "config", "roofline", "cpu_baseline"):
+        assert key in out, key
+    assert out["n_gpus"] == 1 and out["steps"] == 2 and out["warmup"] == 1 and out["dtype"] == "f32" and out["vs_baseline"] is None
+    assert out["unit"] == "TFLOP/s" and out["higher_is_better"] is True and "workload" in out["config"] and "model" not in out["config"]
+    roof = out["roofline"]
+    assert roof["bound"] == "mfma" and roof["unit"] == "TFLOP/s" and roof["peak"] == 157.3 and abs(roof["frac"] - roof["achieved"] / roof["peak"]) < 1e-3
+    assert "traffic" in roof and "effective_mhz" in roof
+    cpu = out["cpu_baseline"]
+    assert cpu["kind"] == "port" and cpu["unit"] == "TFLOP/s" and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
+    extra = out["extra"]
+    assert extra["rows"] == [] and "mlp_step_ms_gpu" in extra and "mlp_step_ms_gpu_fused_tail" in extra and "mlp_step_ms_cpu" in extra
+    assert extra["mlp_max_abs_loss_diff_first10"] <= 1e-4
+    assert not [k for k in extra if k.endswith("_error")], extra
+
+
+def test_more_than_one_gpu_is_refused():
+    res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
+    assert res.returncode != 0 and "ONE GPU" in (res.stdout + res.stderr)
