@@ -1,5 +1,5 @@
-"""bench.py's one JSON line, checked without a GPU: the benchmark driver runs end to end against the CPU replay of the
-library at a small size (tests/replay: the numbers mean nothing there, the code path and the fields do)."""
+"""bench.py's one JSON line and __graft_entry__.smoke(), checked without a GPU: both run end to end against the CPU replay
+of the library (tests/replay: the timings mean nothing there, the code path, the fields and the parity checks do)."""
 import json
 import os
 import subprocess
@@ -51,3 +51,11 @@ def test_one_json_line_with_every_field():
 def test_more_than_one_gpu_is_refused():
     res = subprocess.run([sys.executable, os.path.join(ROOT, "bench.py"), "--gpus", "2"], capture_output=True, text=True, timeout=120)
     assert res.returncode != 0 and "ONE GPU" in (res.stdout + res.stderr)
+
+
+def test_smoke_entry_runs_on_the_replay():
+    env = dict(os.environ, TENMO_HIP_LIBRARY=replay_build.build_library(), REPLAY_STRICT="0",
+               PYTHONPATH=os.path.join(ROOT, "tests", "replay") + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    res = subprocess.run([sys.executable, "-c", "import torch_on_host, __graft_entry__ as g; g.smoke()"], cwd=ROOT, env=env, capture_output=True, text=True,
+                         timeout=900)
+    assert res.returncode == 0 and "smoke ok" in res.stdout, res.stdout[-2000:] + res.stderr[-2000:]
