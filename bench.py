@@ -66,6 +66,8 @@ def main() -> int:
     ap.add_argument("--clock-probe-rounds", type=int, default=50000, help="length of the shader-clock probe (rounds of four MFMAs per wavefront)")
     ap.add_argument("--mlp-fused-tail", action="store_true",
                     help="also time the MLP step with its last two layers, loss, backward and update fused into one launch (mlp_fused_tail knob)")
+    ap.add_argument("--tune", default="", help="comma-separated name=value overrides of the kernel selection (tenmo_hip_set_tuning) for the rows, "
+                    "e.g. gemm_panel=1,gemm_smallk=0: the same committed rows under another kernel choice")
     ap.add_argument("--rows", default="", help="comma-separated substrings: only the rows whose name contains one of them")
     ap.add_argument("--adjacent", action="store_true",
                     help="also time the adjacent operators (cross-entropy, SGD step, convolution) into `extra`; off by default")
@@ -176,7 +178,14 @@ def main() -> int:
 
     if not args.no_extra:
         only = [s for s in args.rows.split(",") if s]
+        tuned = [kv.split("=", 1) for kv in args.tune.split(",") if "=" in kv]
+        for name_, value_ in tuned:
+            _lib.check(L.tenmo_hip_set_tuning(name_.encode(), int(value_)))
+        if tuned:
+            extra["tune"] = {n: int(v) for n, v in tuned}
         rows = attempt("rows", lambda: config_rows(L, _lib, torch, only))
+        for name_, _ in tuned:
+            L.tenmo_hip_set_tuning(name_.encode(), -1 if name_ != "mlp_fused_tail" else 0)
         if rows is not None:
             extra["rows"] = rows
             worst = max([worst] + [r["rel_err_vs_fp64"] for r in rows])
