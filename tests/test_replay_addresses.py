@@ -179,6 +179,44 @@ def test_adjacent_operators(exe):
     run(exe, cases, cus=16, modes=("early",))
 
 
+def test_randomized_products(exe):
+    """Seeded random shapes (small extents, the tile widths and their neighbours, anything up to 400), layouts including
+    generic strides, batches with and without a shared B, accumulate, and kernel choices (every tile, K slices, stream-K, the
+    short-reduction and the K-stream kernel forced on): whatever the dispatch makes of them must stay in bounds and be right.
+    (TENMO_REPLAY_FUZZ=<n> runs n cases instead of 150.)"""
+    import random
+
+    rnd = random.Random(20240611)
+
+    def extent(limit):
+        r = rnd.random()
+        if r < 0.15:
+            return rnd.choice([1, 2, 3, 4, 5, 7, 8])
+        if r < 0.5:
+            return rnd.choice([16, 31, 32, 33, 63, 64, 65, 100, 127, 128, 129, 130, 132, 255, 256, 257, 260])
+        return rnd.randint(1, limit)
+
+    cases = []
+    for _ in range(int(os.environ.get("TENMO_REPLAY_FUZZ", "150"))):
+        batch = rnd.choice([0, 0, 0, 1, 2, 3, 5, 9])
+        knobs = {}
+        r = rnd.random()
+        if r < 0.2:
+            knobs["gemm_tile"] = rnd.randint(0, 4)
+        elif r < 0.3:
+            knobs["gemm_splitk"] = rnd.choice([2, 3, 5, 8])
+        elif r < 0.45:
+            knobs["gemm_streamk"], knobs["gemm_tile"] = rnd.choice([1, 2]), rnd.randint(0, 3)
+        elif r < 0.6:
+            knobs["gemm_smallk"] = 1
+        elif r < 0.75:
+            knobs["gemm_panel"] = 1
+        cases.append(case(extent(400), extent(400), extent(300), rnd.choice("nntg"), rnd.choice("nntg"), batch,
+                          rnd.choice([0, 0, 1]) if batch else 0, rnd.choice([0, 0, 1]), **knobs))
+    for start in range(0, len(cases), 75):
+        run(exe, cases[start:start + 75], cus=3)
+
+
 def test_one_step_reduction_into_a_large_result(exe):
     """[8192,16].[16,8192] with B a transposed view, at full size and on the real 256 CUs: the launch after which a GPU run
     once ended in a memory fault.  The source was right (this replay was clean for all three kernels that ran then); the
