@@ -176,7 +176,7 @@ static int run_vector_case(const std::string& spec, bool is_mv) {
     int bad = 0;
     double err = -1;
     if (rc != 0) { fprintf(stderr, "%s: error %d: %s\n", spec.c_str(), rc, tenmo_hip_last_error()); bad = 1; }
-    else { err = gradient_error(out, want); if (!(err <= 2e-6)) bad = 1; }
+    else { err = gradient_error(out, want); if (!(err <= 1e-5)) bad = 1; } // (one output can be a sum with cancellation: the stated tolerance, not a tighter one)
     printf("%s: rc %d, relative error %.3g%s\n", spec.c_str(), rc, err, bad ? "  <-- FAILED" : "");
     fflush(stdout);
     replay_register(Mx, 0); replay_register(v, 0); replay_register(out, 0);
