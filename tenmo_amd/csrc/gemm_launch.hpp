@@ -44,7 +44,7 @@ bool launch_gemm_smallk_64x64(const GemmArgs& g, int amode, int bmode, unsigned 
 // `total_tiles` = batches x tiles of the chosen size (g.tiles_m, g.tiles_n set for it).  The caller has checked what the
 // direct loads need (pitches, an MN-major extent divisible by 4, K % 4 == 0 for a K-major operand when K is no multiple
 // of 16) and N <= 2^22.  false: no such variant.
-enum PanelTile : int { PANEL_TILE_128x128 = 0 };
+enum PanelTile : int { PANEL_TILE_128x128 = 0, PANEL_TILE_64x64 = 1 }; // (64x64: a ring of eight stages, for long reductions over few tiles)
 bool launch_gemm_panel(const GemmArgs& g, int tile, int amode, int bmode, unsigned cus, unsigned total_tiles, bool by_batch, hipStream_t stream);
 
 } // namespace tenmo

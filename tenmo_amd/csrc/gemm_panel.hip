@@ -120,7 +120,8 @@ __global__ __launch_bounds__(PANEL_THREADS, 2 * PANEL_WGS_PER_CU) void gemm_pane
     constexpr int PA = frag_parts<AMODE, MB>(), PB = frag_parts<BMODE, NB>(); // LDS reads per 8-wide k chunk
     constexpr int NMFMA = 4 * MB * NB;                                        // MFMAs per chunk
     constexpr int NSLOT = MB * 16;                                            // store slots of a tile: (block row i, accumulator element e)
-    static_assert(PA + PB <= NMFMA, "one operand fetch per MFMA at most");
+    constexpr int PER_MFMA = (PA + PB + NMFMA - 1) / NMFMA;                   // operand fetches placed behind one MFMA: 1, or 2 for the 64x64 tile
+    static_assert(PER_MFMA <= 2, "at most two operand fetches behind an MFMA");
 
     f32x16 acc[MB][NB];
     float fa[2][MB][4], fb[2][NB][4]; // operand registers of the two k chunks of a step
@@ -220,12 +221,20 @@ __global__ __launch_bounds__(PANEL_THREADS, 2 * PANEL_WGS_PER_CU) void gemm_pane
                 const int klimit = ragged_k && last_step ? pa.k_tail : GEMM_BK;
                 if (klimit < GEMM_BK) mask_tail(0, klimit);
                 // chunk 0; behind its MFMAs the operand fetch of chunk 1
-                mfma_chunk(0, [&](int n) { if (n < PA + PB) fetch_part(st, 1, n); });
+                mfma_chunk(0, [&](int n) {
+#pragma unroll
+                    for (int q = 0; q < PER_MFMA; ++q)
+                        if (n * PER_MFMA + q < PA + PB) fetch_part(st, 1, n * PER_MFMA + q);
+                });
                 if (klimit > 8) {
                     if (klimit < GEMM_BK) mask_tail(1, klimit);
                     // chunk 1; behind its MFMAs the operand fetch of the next step's chunk 0 (harmless when there is no
                     // next step: the registers are not used)
-                    mfma_chunk(1, [&](int n) { if (n < PA + PB) fetch_part(st_next, 0, n); });
+                    mfma_chunk(1, [&](int n) {
+#pragma unroll
+                        for (int q = 0; q < PER_MFMA; ++q)
+                            if (n * PER_MFMA + q < PA + PB) fetch_part(st_next, 0, n * PER_MFMA + q);
+                    });
                 } else {
 #pragma unroll
                     for (int p = 0; p < PA + PB; ++p) fetch_part(st_next, 0, p);
@@ -282,9 +291,11 @@ bool launch_panel_modes(const GemmArgs& g, int amode, int bmode, const PanelLaun
 } // namespace
 
 bool launch_gemm_panel(const GemmArgs& g, int tile, int amode, int bmode, unsigned cus, unsigned total_tiles, bool by_batch, hipStream_t stream) {
-    if (g.K < 1 || total_tiles == 0 || tile != PANEL_TILE_128x128) return false;
+    if (g.K < 1 || total_tiles == 0) return false;
     const PanelLaunch l{cus, total_tiles, by_batch, stream};
-    return launch_panel_modes<128, 128>(g, amode, bmode, l);
+    if (tile == PANEL_TILE_128x128) return launch_panel_modes<128, 128>(g, amode, bmode, l);
+    if (tile == PANEL_TILE_64x64) return launch_panel_modes<64, 64>(g, amode, bmode, l);
+    return false;
 }
 
 } // namespace tenmo

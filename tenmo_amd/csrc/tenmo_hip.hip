@@ -88,7 +88,7 @@ struct State {
     int force_conv_phases = -1; // strided image gradient phase by phase: -1 automatic (large layers), 0 never, 1 always
     int force_streamk = -1;    // -1 automatic, 0 never, n > 0: stream-K with n workgroups per CU
     int force_smallk = -1;     // -1 automatic, 0 never, 1: the short-reduction kernel wherever it can run
-    int force_panel = -1;      // -1 automatic, 0 never, 1: the persistent K-stream kernel wherever it can run
+    int force_panel = -1;      // -1 automatic, 0 never, 1: the persistent K-stream kernel wherever it can run (2: without XCD grouping, 3: 64x64 tiles)
     int mlp_fused_tail = 0;    // the last two layers of an MLP step, loss, their backward and update in one launch: 1 when the shapes fit, 0 never
     int fold_reduce = -1;      // the gradient of a broadcast parent summed inside the GEMM launch: -1 automatic, 0 never, 1 wherever it can
     int verbose = 0;
@@ -358,7 +358,8 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
             if (mode == MNMAJOR_VEC) return row_s == 1 && k_s >= 0 && k_s <= (int64_t(1) << 25) && extent % 4 == 0 && extent >= 4;
             return false;
         };
-        const int64_t tm = (M + 127) / 128, tn = (N + 127) / 128, tiles = tm * tn * batch_count;
+        const int pt = S.force_panel == 3 ? 64 : 128; // (3: its 64x64-tile variant, a ring of eight stages, forced: for long reductions over few tiles)
+        const int64_t tm = (M + pt - 1) / pt, tn = (N + pt - 1) / pt, tiles = tm * tn * batch_count;
         const bool can = K > GEMM_BK && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum &&
                          N <= (int64_t(1) << 22) && tiles <= 0x7fffffffLL;
         const bool want = S.force_panel > 0 || (S.force_panel < 0 && S.force_tile < 0 && S.force_splitk <= 0 && S.force_streamk <= 0 && S.force_smallk <= 0 &&
@@ -366,8 +367,8 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         if (can && want) {
             g.tiles_m = (int32_t)tm; g.tiles_n = (int32_t)tn;
             g.k_splits = 1; g.k_per_split = K; g.partial = nullptr;
-            if (S.verbose) fprintf(stderr, "tenmo_hip gemm: K-stream kernel, %lld tiles of 128x128\n", (long long)tiles);
-            if (launch_gemm_panel(g, PANEL_TILE_128x128, am, bm, (unsigned)S.cus, (unsigned)tiles, S.force_panel != 2, S.stream)) return 0;
+            if (S.verbose) fprintf(stderr, "tenmo_hip gemm: K-stream kernel, %lld tiles of %dx%d\n", (long long)tiles, pt, pt);
+            if (launch_gemm_panel(g, pt == 64 ? PANEL_TILE_64x64 : PANEL_TILE_128x128, am, bm, (unsigned)S.cus, (unsigned)tiles, S.force_panel != 2, S.stream)) return 0;
         }
     }
     // Short reduction, vector operand forms and a plain (or accumulating) store: the persistent whole-K-in-LDS kernel

@@ -204,6 +204,10 @@ def test_short_reduction_kernel_layouts_and_k_tails(T, smallk):
 
 
 def test_kstream_kernel(T):
+    _kstream_cases(T, 1)
+
+
+def _kstream_cases(T, knob):
     """The persistent K-stream kernel (loading wavefronts of its own, a ring of LDS stages across tiles, stores behind the
     next tile's MFMAs) forced on: every operand layout, whole and ragged tiles, reductions of one step to many, K tails,
     batches with and without a broadcast B, fewer tiles than workgroups and many more, plain and accumulating stores;
@@ -217,7 +221,7 @@ def test_kstream_kernel(T):
              ((9,), 320, 1024, 12, 0), ((), 64, 8192, 104, 0), ((), 132, 72, 4, 0), ((12,), 1024, 1024, 64, 0), ((), 100, 50000, 256, 1),
              ((), 4096, 4096, 512, 0), ((17,), 260, 384, 128, 1)]
     try:
-        L.tenmo_hip_set_tuning(b"gemm_panel", 1)
+        L.tenmo_hip_set_tuning(b"gemm_panel", knob)
         for bshape, M, N, K, acc in cases:
             for ta in (False, True):
                 for tb in (False, True):
@@ -1431,6 +1435,12 @@ def test_backward_of_broadcast_parents(T, oracle, fold):
         assert rel_fro(W.grad(), gW) <= 2 * RTOL_FRO and rel_fro(A.grad(), gA) <= 2 * RTOL_FRO
     finally:
         L.tenmo_hip_set_tuning(b"fold_reduce", -1)
+
+
+def test_kstream_kernel_with_64x64_tiles(T):
+    """The same cases through the kernel's 64x64-tile variant (a ring of eight stages; two operand fetches behind an MFMA
+    where an operand is MN-major)."""
+    _kstream_cases(T, 3)
 
 
 def test_mlp_loss_curve_with_the_fused_tail(T, oracle):

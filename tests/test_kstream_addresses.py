@@ -126,6 +126,15 @@ def test_benchmark_shapes(emu):
     run(emu, problem(4096, 4096, 256, "k", "k"))
     run(emu, problem(1024, 1024, 128, "k", "mn", batch=(8,), cus=64, wpc=1))
 
+@pytest.mark.parametrize("la,lb", LAYOUTS)
+def test_64x64_tiles_with_a_ring_of_eight(emu, la, lb):
+    for (M, N, K) in [(64, 64, 32), (300, 520, 100), (132, 260, 20), (1000, 136, 24), (1024, 1024, 1024), (64, 192, 36)]:
+        for cus in (1, 3, 256):
+            run(emu, problem(M, N, K, la, lb, tile=(64, 64), np_=8, cus=cus))
+    run(emu, problem(256, 384, 64, la, lb, batch=(16,), tile=(64, 64), np_=8, cus=8))
+    run(emu, problem(132, 260, 48, la, lb, batch=(9,), b_shared=True, tile=(64, 64), np_=8, cus=16))  # (an MN-major extent must be a multiple of 4)
+
+
 def test_one_workgroup_per_cu(emu):
     run(emu, problem(300, 520, 100, "k", "mn", cus=8, wpc=1))
     run(emu, problem(256, 384, 64, "mn", "k", batch=(16,), cus=8, wpc=1))

@@ -116,6 +116,15 @@ def test_k_stream_kernel(exe):
     run(exe, cases, cus=2)
     run(exe, cases[:9] + cases[-2:], cus=256, modes=("late",))
     run(exe, [case(128, 128, 16, gemm_panel=1), case(300, 260, 8, "t", "n", gemm_panel=1)], cus=4)  # K <= 16: not this kernel, still right
+    # the 64x64-tile variant (a ring of eight stages, two operand fetches behind an MFMA for MN-major operands)
+    small = []
+    for la, lb in LAYOUTS:
+        for (M, N, K) in [(64, 64, 32), (300, 520, 100), (132, 260, 20), (256, 384, 112), (512, 512, 256), (1024, 64, 1024)]:
+            small.append(case(M, N, K, la, lb, gemm_panel=3))
+        small.append(case(256, 384, 64, la, lb, batch=16, gemm_panel=3))
+        small.append(case(132, 260, 48, la, lb, batch=9, b_shared=1, acc=1, gemm_panel=3))
+    run(exe, small, cus=2)
+    run(exe, small[:8] + [case(1024, 1024, 1024, gemm_panel=3)], cus=256, modes=("late",))
 
 
 def test_automatic_choice_on_benchmark_shapes(exe):
