@@ -68,6 +68,8 @@ def main() -> int:
                     help="also time the MLP step with its last two layers, loss, backward and update fused into one launch (mlp_fused_tail knob)")
     ap.add_argument("--tune", default="", help="comma-separated name=value overrides of the kernel selection (tenmo_hip_set_tuning) for the rows, "
                     "e.g. gemm_panel=1,gemm_smallk=0: the same committed rows under another kernel choice")
+    ap.add_argument("--sweep", default="", help="semicolon-separated lists in the form of --tune: the chosen rows (--rows) are timed once more "
+                    "under each list, in this process, and reported under extra.sweep")
     ap.add_argument("--rows", default="", help="comma-separated substrings: only the rows whose name contains one of them")
     ap.add_argument("--adjacent", action="store_true",
                     help="also time the adjacent operators (cross-entropy, SGD step, convolution) into `extra`; off by default")
@@ -178,18 +180,32 @@ def main() -> int:
 
     if not args.no_extra:
         only = [s for s in args.rows.split(",") if s]
-        tuned = [kv.split("=", 1) for kv in args.tune.split(",") if "=" in kv]
-        for name_, value_ in tuned:
-            _lib.check(L.tenmo_hip_set_tuning(name_.encode(), int(value_)))
-        if tuned:
-            extra["tune"] = {n: int(v) for n, v in tuned}
-        rows = attempt("rows", lambda: config_rows(L, _lib, torch, only))
-        for name_, _ in tuned:
-            L.tenmo_hip_set_tuning(name_.encode(), -1 if name_ != "mlp_fused_tail" else 0)
-        if rows is not None:
+
+        def rows_under(tune_list):
+            """The rows timed with the kernel selection overridden by `tune_list` ("name=value,...", may be empty)."""
+            tuned = [kv.split("=", 1) for kv in tune_list.split(",") if "=" in kv]
+            for name_, value_ in tuned:
+                _lib.check(L.tenmo_hip_set_tuning(name_.strip().encode(), int(value_)))
+            try:
+                return {n.strip(): int(v) for n, v in tuned}, config_rows(L, _lib, torch, only)
+            finally:
+                for name_, _ in tuned:
+                    L.tenmo_hip_set_tuning(name_.strip().encode(), -1 if name_.strip() != "mlp_fused_tail" else 0)
+
+        got = attempt("rows", lambda: rows_under(args.tune))
+        if got is not None:
+            if got[0]:
+                extra["tune"] = got[0]
+            rows = got[1]
             extra["rows"] = rows
             worst = max([worst] + [r["rel_err_vs_fp64"] for r in rows])
             extra["rows_max_rel_err_vs_fp64"] = worst
+        for i, tune_list in enumerate(t for t in args.sweep.split(";") if t.strip()):
+            got = attempt("sweep%d" % i, lambda: rows_under(tune_list))
+            if got is not None:
+                extra.setdefault("sweep", []).append({"tune": got[0], "rows": [
+                    {k: r[k] for k in ("name", "us", "frac", "rel_err_vs_fp64")} for r in got[1]]})
+                worst = max([worst] + [r["rel_err_vs_fp64"] for r in got[1]])
 
         def clock_after_rows():
             _lib.check(L.tenmo_hip_clock_probe(args.clock_probe_rounds, C.byref(mhz)))
@@ -266,7 +282,10 @@ def config_rows(L, _lib, torch, only):
         return _lib.make_view(t.data_ptr(), 0, tuple(t.shape), tuple(t.stride()))
 
     def wanted(name):
-        return not only or any(s in name for s in only)
+        if only and not any(s in name for s in only):
+            return False
+        print("bench row: " + name, file=sys.stderr, flush=True)  # a run that dies names the row it died in
+        return True
 
     def finish_row(name, cfg, shape, us, flop, nbytes, rel_err, copies):
         t_mfma, t_hbm = flop / (PEAK_FP32_MFMA_TFLOPS * 1e12) * 1e6, nbytes / (PEAK_HBM_GBPS * 1e9) * 1e6

@@ -28,7 +28,8 @@ def run_bench(*flags):
 
 
 def test_one_json_line_with_every_field():
-    res = run_bench("--size", "256", "--steps", "2", "--warmup", "1", "--rows", "no-such-row", "--mlp-fused-tail", "--clock-probe-rounds", "4")
+    res = run_bench("--size", "256", "--steps", "2", "--warmup", "1", "--rows", "no-such-row", "--mlp-fused-tail", "--clock-probe-rounds", "4",
+                    "--sweep", "gemm_panel=0;gemm_panel=1,gemm_smallk=0")
     lines = [l for l in res.stdout.splitlines() if l.strip()]
     assert res.returncode == 0 and len(lines) == 1, res.stdout[-2000:] + res.stderr[-2000:]
     out = json.loads(lines[0])
@@ -45,6 +46,7 @@ def test_one_json_line_with_every_field():
     extra = out["extra"]
     assert extra["rows"] == [] and "mlp_step_ms_gpu" in extra and "mlp_step_ms_gpu_fused_tail" in extra and "mlp_step_ms_cpu" in extra
     assert extra["mlp_max_abs_loss_diff_first10"] <= 1e-4
+    assert extra["sweep"] == [{"tune": {"gemm_panel": 0}, "rows": []}, {"tune": {"gemm_panel": 1, "gemm_smallk": 0}, "rows": []}]
     assert not [k for k in extra if k.endswith("_error")], extra
 
 
