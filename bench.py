@@ -65,7 +65,8 @@ def main() -> int:
     ap.add_argument("--no-extra", action="store_true", help="skip the per-configuration rows and the MLP-step measurement")
     ap.add_argument("--clock-probe-rounds", type=int, default=50000, help="length of the shader-clock probe (rounds of four MFMAs per wavefront)")
     ap.add_argument("--mlp-fused-tail", action="store_true",
-                    help="also time the MLP step with its last two layers, loss, backward and update fused into one launch (mlp_fused_tail knob)")
+                    help="also time the MLP step with its last two layers, loss, backward and update fused into one launch, and with the first layer's "
+                    "gradient and update fused as well (mlp_fused_tail knob 1 and 2)")
     ap.add_argument("--tune", default="", help="comma-separated name=value overrides of the kernel selection (tenmo_hip_set_tuning) for the rows, "
                     "e.g. gemm_panel=1,gemm_smallk=0: the same committed rows under another kernel choice")
     ap.add_argument("--sweep", default="", help="semicolon-separated lists in the form of --tune: the chosen rows (--rows) are timed once more "
@@ -528,16 +529,19 @@ def mlp_step_times(_lib, torch, np, fused_tail=False):
     graph_ms = (time.perf_counter() - t0) * 1e3 / 20
     fused = {}
     if fused_tail:
-        L.tenmo_hip_set_tuning(b"mlp_fused_tail", 1)
-        try:
-            first = float(gpu.step_device(*dev[0], lr, sync=True).item())
-            t0 = time.perf_counter()
-            for xd, yd in dev[10:]:
-                gpu.step_device(xd, yd, lr, sync=False)
-            _lib.check(L.tenmo_hip_sync())
-            fused = {"mlp_step_ms_gpu_fused_tail": round((time.perf_counter() - t0) * 1e3 / 20, 4), "mlp_fused_tail_first_loss": first}
-        finally:
-            L.tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
+        # 1: the last two layers, loss, backward and update in one launch; 2: also the first layer's gradient with its update
+        for level, key in ((1, "mlp_step_ms_gpu_fused_tail"), (2, "mlp_step_ms_gpu_fused_tail_and_first")):
+            L.tenmo_hip_set_tuning(b"mlp_fused_tail", level)
+            try:
+                first = float(gpu.step_device(*dev[0], lr, sync=True).item())
+                t0 = time.perf_counter()
+                for xd, yd in dev[10:]:
+                    gpu.step_device(xd, yd, lr, sync=False)
+                _lib.check(L.tenmo_hip_sync())
+                fused[key] = round((time.perf_counter() - t0) * 1e3 / 20, 4)
+                fused[key.replace("mlp_step_ms_gpu", "mlp") + "_first_loss"] = first
+            finally:
+                L.tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
     t0 = time.perf_counter()
     for x, y in batches[10:]:
         cpu.step(x, y, lr)

@@ -362,6 +362,41 @@ __global__ __launch_bounds__(MLP_TAIL_THREADS) void mlp_tail_kernel(const MlpTai
     }
 }
 
+// The weight gradient of the network's first layer and that layer's SGD update in one launch, for the small batches of
+// the launch above: dW = x^T . g (tenmo/matmul.mojo:46-48), W -= lr * dW, b -= lr * db (tenmo/optim.mojo:93-120).  A
+// workgroup takes MLP_FIRST_ROWS input features (rows of W) and all O <= MLP_TAIL_MAX_D0 outputs: the gradient g [B, O] and
+// the workgroup's columns of x lie in LDS, every thread sums one 2 x 4 block over the batch in ascending order.
+constexpr int MLP_FIRST_ROWS = 16;
+struct MlpFirstArgs {
+    const float* x;   // [B, I] network input
+    const float* g;   // [B, O] gradient of the layer's output (its ReLU gradient applied)
+    const float* db;  // [O] column sums of g
+    float *W, *b;     // [I, O], [O]: updated in place
+    float* dW;        // [I, O]
+    float lr;
+    int32_t B, I, O;
+};
+__global__ __launch_bounds__(MLP_TAIL_THREADS) void mlp_first_layer_kernel(const MlpFirstArgs a) {
+    constexpr int PX = MLP_TAIL_MAX_B + 1; // x strip held feature-major with an odd pitch
+    __shared__ float gs[MLP_TAIL_MAX_B * MLP_TAIL_MAX_D0]; // [B][O], pitch O
+    __shared__ float xs[MLP_FIRST_ROWS * PX];              // [row][B]
+    const int B = a.B, I = a.I, O = a.O, t = threadIdx.x;
+    const int k0 = blockIdx.x * MLP_FIRST_ROWS, rows = min(MLP_FIRST_ROWS, I - k0);
+    for (int i = t; i < B * O; i += MLP_TAIL_THREADS) gs[i] = a.g[i];
+    for (int i = t; i < B * MLP_FIRST_ROWS; i += MLP_TAIL_THREADS) {
+        const int bb = i / MLP_FIRST_ROWS, r = i % MLP_FIRST_ROWS;
+        xs[r * PX + bb] = r < rows ? a.x[(int64_t)bb * I + k0 + r] : 0.f;
+    }
+    __syncthreads();
+    lds_product(rows, O, B, xs, PX, 1, gs, O, 1, [&](int m, int n, float v) {
+        const int64_t at = (int64_t)(k0 + m) * O + n;
+        a.dW[at] = v;
+        a.W[at] = a.W[at] - a.lr * v;
+    });
+    if (blockIdx.x == 0)
+        for (int i = t; i < O; i += MLP_TAIL_THREADS) a.b[i] = a.b[i] - a.lr * a.db[i];
+}
+
 // loss = (sum of row losses in row order) / rows — the order of the reference's scalar loop
 __global__ void ordered_mean_kernel(const float* __restrict row_loss, int64_t rows, float* __restrict out) {
     if (blockIdx.x == 0 && threadIdx.x == 0) {

@@ -89,7 +89,7 @@ struct State {
     int force_streamk = -1;    // -1 automatic, 0 never, n > 0: stream-K with n workgroups per CU
     int force_smallk = -1;     // -1 automatic, 0 never, 1: the short-reduction kernel wherever it can run
     int force_panel = -1;      // -1 automatic, 0 never, 1: the persistent K-stream kernel wherever it can run (2: without XCD grouping, 3: 64x64 tiles)
-    int mlp_fused_tail = 0;    // the last two layers of an MLP step, loss, their backward and update in one launch: 1 when the shapes fit, 0 never
+    int mlp_fused_tail = 0;    // MLP step: 1 the last two layers, loss, their backward and update in one launch when the shapes fit; 2 also the first layer's weight gradient and update in one; 0 neither
     int fold_reduce = -1;      // the gradient of a broadcast parent summed inside the GEMM launch: -1 automatic, 0 never, 1 wherever it can
     int verbose = 0;
     int cols_waves_per_cu = 2; // target workgroups per CU of the column-streaming kernels (long K slices stream best)
@@ -1910,11 +1910,15 @@ static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int6
     }
     BatchDesc bd{};
     for (int d = 0; d < MAX_BATCH_RANK; ++d) bd.shape[d] = 1;
+    bool first_done = false; // layer 0 updated by its own fused launch
     for (int l = top - 1; l >= 0; --l) {
         const int64_t I = m->dims[l], O = m->dims[l + 1];
         const float* in = l == 0 ? x : m->act[l - 1];
         const float* gl = m->grad[l];
         const bool from_gemm = B <= 128; // hidden layers: summed in the store of the GEMM that produced this gradient (below)
+        // the first layer's weight gradient and update as one launch beside the fused tail (the two together leave
+        // the step with the first layer's forward, the tail and this)
+        const bool first_fused = S.mlp_fused_tail >= 2 && l == 0 && B <= MLP_TAIL_MAX_B && O <= MLP_TAIL_MAX_D0 && I <= 0x7fffffffLL / MLP_TAIL_MAX_D0;
         if (fused_tail && l == top - 1) {
             // done by the tail launch
         } else if (one_block && l == L - 1) {
@@ -1934,6 +1938,14 @@ static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int6
             if (from_gemm) ep.colsum = m->db[l - 1]; // bias gradient of layer l-1 = column sums of its (masked) gradient
         }
         // both consume the same upstream gradient and are independent: one launch for the two when they are small
+        if (first_fused) {
+            MlpFirstArgs f{};
+            f.x = in; f.g = gl; f.db = m->db[0]; f.W = m->W[0]; f.b = m->b[0]; f.dW = m->dW[0];
+            f.lr = lr; f.B = (int32_t)B; f.I = (int32_t)I; f.O = (int32_t)O;
+            hipLaunchKernelGGL(mlp_first_layer_kernel, dim3((unsigned)((I + MLP_FIRST_ROWS - 1) / MLP_FIRST_ROWS)), dim3(MLP_TAIL_THREADS), 0, S.stream, f);
+            first_done = true;
+            continue;
+        }
         int paired = 1;
         if (l > 0) paired = gemm_pair_dispatch(in, 1, I, gl, O, 1, m->dW[l], I, O, B, gl, O, 1, m->W[l], 1, O, m->grad[l - 1], B, I, O, ep);
         if (paired < 0) return paired;
@@ -1944,7 +1956,7 @@ static int mlp_step_enqueue(tenmo_mlp* m, const float* x, const int32_t* y, int6
         }
     }
     // every parameter tensor (below the fused tail, which updates its own) in one launch
-    for (int l0 = 0; l0 < top; l0 += SGD_MAX_TENSORS / 2) {
+    for (int l0 = first_done ? 1 : 0; l0 < top; l0 += SGD_MAX_TENSORS / 2) {
         SgdArgs sa{};
         int64_t largest = 0;
         for (int l = l0; l < top && sa.count + 2 <= SGD_MAX_TENSORS; ++l) {

@@ -330,6 +330,10 @@ void launch(const char* name, dim3 grid, dim3 block, std::function<void()> body)
     ++g_launches;
     const int64_t total = (int64_t)grid.x * grid.y * grid.z;
     if ((int64_t)block.x * block.y * block.z > MAX_LANES || total <= 0) fail("launch of %s: bad grid or block", name);
+    // what the HIP runtime refuses: more than 65535 workgroups along y or z, 2^32 or more threads along one dimension
+    if (grid.y > 65535u || grid.z > 65535u || (uint64_t)grid.x * block.x > 0xffffffffull || (uint64_t)grid.y * block.y > 0xffffffffull ||
+        (uint64_t)grid.z * block.z > 0xffffffffull)
+        fail("launch of %s: grid (%u,%u,%u) x block (%u,%u,%u) is beyond what a HIP launch takes", name, grid.x, grid.y, grid.z, block.x, block.y, block.z);
     std::atomic<int64_t> next{0};
     run_on_pool([&]() {
         for (;;) {

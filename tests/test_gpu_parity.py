@@ -1449,11 +1449,12 @@ def test_mlp_loss_curve_with_the_fused_tail(T, oracle):
     from tenmo_amd import rng as R
     from tenmo_amd.net import MLP
 
-    T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 1)
-    try:
-        _mlp_loss_curve(T, oracle, R, MLP)
-    finally:
-        T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
+    for level in (1, 2):  # 2: the first layer's weight gradient and its update as one launch as well
+        T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", level)
+        try:
+            _mlp_loss_curve(T, oracle, R, MLP)
+        finally:
+            T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
 
 
 def test_zz_graph_capture_grows_scratch(T, oracle):

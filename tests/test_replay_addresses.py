@@ -184,7 +184,8 @@ def test_adjacent_operators(exe):
              "misc:1", "misc:63", "misc:1000", "misc:300001",
              # the MLP training step op by op and with its last two layers fused into one launch: the MNIST shape, the largest
              # widths the fused launch takes, ragged ones, and a batch of one
-             "mlp:64,784,128,32,10,0", "mlp:64,784,128,32,10,1", "mlp:64,300,128,64,32,1", "mlp:37,50,77,33,7,1", "mlp:1,9,5,3,2,1"]
+             "mlp:64,784,128,32,10,0", "mlp:64,784,128,32,10,1", "mlp:64,300,128,64,32,1", "mlp:37,50,77,33,7,1", "mlp:1,9,5,3,2,1",
+             "mlp:64,784,128,32,10,2", "mlp:37,50,77,33,7,2", "mlp:1,9,5,3,2,2", "mlp:64,17,128,64,32,2", "mlp:5,33,1,1,1,2"]
     run(exe, cases, cus=16, modes=("early",))
 
 
