@@ -76,7 +76,9 @@ int tenmo_hip_device_info(int* compute_units, char* name, int name_len);
  * of materialised and reduced: 1 wherever it can run, 0 never, -1 automatic), "mlp_fused_tail" (tenmo_hip_mlp_step: the last
  * two layers, the loss, their backward and their update as one launch when they fit one workgroup — batch <= 64, widths
  * <= 128 / 64 / 32: 1 on, 2 the same and the first layer's weight gradient with its update as one launch, 0 off, the default), "cols_wg_per_cu" (workgroups per CU the
- * column-streaming kernel aims for) and "conv_phases" (image gradient of a strided convolution phase by phase:
+ * column-streaming kernel aims for), "cols_join" (vm, mv of a transposed view and skinny products whose reduction is cut
+ * into K slices: 1 the slices are added by the last workgroup of the streaming launch — same bits, one launch less —, 0 by a
+ * second launch, the default) and "conv_phases" (image gradient of a strided convolution phase by phase:
  * 1 always, 0 never, -1 automatic).  The
  * environment variables TENMO_HIP_GEMM_TILE / TENMO_HIP_GEMM_SPLITK / TENMO_HIP_GEMM_STREAMK / TENMO_HIP_GEMM_SMALLK / TENMO_HIP_GEMM_PANEL set the same at init.
  * No counterpart in the reference, whose tile size is the compile-time TILE_SIZE=32

@@ -152,17 +152,76 @@ struct ColsArgs {
     int64_t batch0;      // batch index of blockIdx.z == 0 (more than 65535 batches go in several launches)
     int64_t batch_total; // batches of the whole product: the partial sums are laid out [k_splits][batch_total][R][n]
     BatchDesc batch;  // a_str: X batch strides, b_str: Mx batch strides
+    // K slices added inside the launch (the JOIN instantiations): the dense result [batch][R][n], and one arrival counter per
+    // column block and batch of the launch, all zero between launches
+    float* joined;
+    uint32_t* arrivals;
 };
 
 constexpr int COLS_THREADS = 256;
 constexpr int COLS_STAGE_FLOATS = 2048; // R x (2048 / R) left-operand values are staged in LDS per refill
 constexpr int COLS_KSLICE_MIN = 32; // granularity of the K slices handed to workgroups
 
+// The K slices of one column block added by the workgroup that finishes last, inside the streaming launch: every
+// workgroup stores its partial sums, makes them visible to the device (fence) and counts itself in on the block's
+// counter; the one that sees all others' arrivals reads the k_splits partial sums of the block back — slices in ascending
+// order, on top of the old value when accumulating: the order of splitk_reduce_kernel, so the result is the same to the bit
+// and independent of scheduling — and puts the counter back to zero for the next launch.  Nobody waits for anybody.
+// Columns [first, first + width) of every row; 32 loads in flight per thread.
+__device__ __forceinline__ void cols_join_slices(const ColsArgs& g, int64_t batch, int64_t first, int width) {
+    __shared__ uint32_t last_to_arrive;
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t* counter = g.arrivals + (int64_t)blockIdx.z * gridDim.x + blockIdx.x;
+        const bool last = atomicAdd(counter, 1u) == (uint32_t)g.k_splits - 1u;
+        if (last) *counter = 0u;
+        last_to_arrive = last ? 1u : 0u;
+    }
+    __syncthreads();
+    if (!last_to_arrive) return;
+    __threadfence(); // nothing below may be served from before the other workgroups' arrival
+    const int64_t plane = (int64_t)g.rows * g.n, slice_stride = g.batch_total * plane;
+    const float* part = g.out + batch * plane;
+    float* dst = g.joined + batch * plane;
+    const int64_t live = min((int64_t)width, g.n - first); // columns of this block inside the row
+    const int items = (int)(g.rows * live);
+    constexpr int IU = 4, SU = 8;
+    for (int i0 = threadIdx.x; i0 < items; i0 += IU * COLS_THREADS) {
+        int64_t at[IU];
+        float sum[IU];
+#pragma unroll
+        for (int u = 0; u < IU; ++u) {
+            const int i = min(i0 + u * COLS_THREADS, items - 1); // surplus threads repeat the last item and do not store
+            at[u] = (int64_t)(i / (int)live) * g.n + first + i % (int)live;
+            sum[u] = g.accumulate ? dst[at[u]] : 0.f;
+        }
+        int p = 0;
+        for (; p + SU <= g.k_splits; p += SU) {
+            float v[IU][SU];
+#pragma unroll
+            for (int u = 0; u < IU; ++u)
+#pragma unroll
+                for (int q = 0; q < SU; ++q) v[u][q] = part[(p + q) * slice_stride + at[u]];
+#pragma unroll
+            for (int u = 0; u < IU; ++u)
+#pragma unroll
+                for (int q = 0; q < SU; ++q) sum[u] += v[u][q];
+        }
+        for (; p < g.k_splits; ++p)
+#pragma unroll
+            for (int u = 0; u < IU; ++u) sum[u] += part[p * slice_stride + at[u]];
+#pragma unroll
+        for (int u = 0; u < IU; ++u)
+            if (i0 + u * COLS_THREADS < items) dst[at[u]] = sum[u];
+    }
+}
+
 // ALIGNED: every row of the matrix starts on a 16-byte boundary -> a lane owns 4 consecutive columns
 // and moves them with one 16-byte load.  Otherwise (row pitch not a multiple of 4 floats, e.g.
 // N = 50257) 16-byte loads would straddle and run at half rate, so a lane owns 4 columns 256 apart
 // and uses dword loads, each still one contiguous 256-byte burst per wavefront.
-template <int R, bool ALIGNED>
+template <int R, bool ALIGNED, bool JOIN = false> // JOIN: k_splits > 1 and the slices are added inside the launch (cols_join_slices)
 __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
     constexpr int COLS_KCHUNK = COLS_STAGE_FLOATS / R; // k rows per LDS refill
     __shared__ float xs[R][COLS_KCHUNK];
@@ -246,25 +305,30 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
         if (wave_full) { stream(p, first, len, load_full); stream(p, 0, first, load_full); }
         else if (any) { stream(p, first, len, load_clamped); stream(p, 0, first, load_clamped); }
     }
-    if (!any) return;
-    const bool to_partial = g.k_splits > 1;
-    float* __restrict ob = g.out + ((to_partial ? (int64_t)blockIdx.y * g.batch_total : 0) + batch) * g.rows * g.n;
-    const bool accumulate = g.accumulate && !to_partial;
+    if constexpr (!JOIN) {
+        if (!any) return;
+    }
+    if (!JOIN || any) {
+        const bool to_partial = g.k_splits > 1;
+        float* __restrict ob = g.out + ((to_partial ? (int64_t)blockIdx.y * g.batch_total : 0) + batch) * g.rows * g.n;
+        const bool accumulate = g.accumulate && !to_partial;
 #pragma unroll
-    for (int r = 0; r < R; ++r) {
-        if (r >= g.rows) break;
-        float* o = ob + (int64_t)r * g.n + col0;
-        if (ALIGNED && full) {
-            f32x4 v = acc[r];
-            if (accumulate) v += *reinterpret_cast<const f32x4_u*>(o);
-            *reinterpret_cast<f32x4_u*>(o) = v;
-        } else {
-            const float a[4] = {acc[r].x, acc[r].y, acc[r].z, acc[r].w};
+        for (int r = 0; r < R; ++r) {
+            if (r >= g.rows) break;
+            float* o = ob + (int64_t)r * g.n + col0;
+            if (ALIGNED && full) {
+                f32x4 v = acc[r];
+                if (accumulate) v += *reinterpret_cast<const f32x4_u*>(o);
+                *reinterpret_cast<f32x4_u*>(o) = v;
+            } else {
+                const float a[4] = {acc[r].x, acc[r].y, acc[r].z, acc[r].w};
 #pragma unroll
-            for (int e = 0; e < 4; ++e)
-                if (col0 + e * CSTEP < g.n) o[e * CSTEP] = accumulate ? o[e * CSTEP] + a[e] : a[e];
+                for (int e = 0; e < 4; ++e)
+                    if (col0 + e * CSTEP < g.n) o[e * CSTEP] = accumulate ? o[e * CSTEP] + a[e] : a[e];
+            }
         }
     }
+    if constexpr (JOIN) cols_join_slices(g, batch, (int64_t)blockIdx.x * COLS_THREADS * 4, COLS_THREADS * 4);
 }
 
 // ---- columns kernel for rows that do not start on 16-byte boundaries ---------------------------
@@ -280,7 +344,7 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_kernel(const ColsArgs g) {
 // row's first elements, which are discarded.
 constexpr int COLS_SHIFT_WIDTH = COLS_THREADS * 4 - 4;
 
-template <int R>
+template <int R, bool JOIN = false>
 __global__ __launch_bounds__(COLS_THREADS) void cols_shift_kernel(const ColsArgs g) {
     constexpr int COLS_KCHUNK = COLS_STAGE_FLOATS / R; // k rows per LDS refill
     __shared__ float xs[R][COLS_KCHUNK];
@@ -394,6 +458,7 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_shift_kernel(const ColsArgs
             }
         }
     }
+    if constexpr (JOIN) cols_join_slices(g, batch, block0, COLS_SHIFT_WIDTH);
 }
 
 // ---- generic kernel: any strides, one thread per output (correct, not fast) -------------------

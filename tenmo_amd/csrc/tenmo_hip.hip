@@ -71,6 +71,7 @@ struct State {
     size_t ws_bytes = 0;
     // second scratch, for results that must outlive a kernel which itself uses `ws`
     float* ws2 = nullptr;
+    uint32_t* arrivals = nullptr; // zeroed counters of the in-launch K-slice reduction of the column kernels
     size_t ws2_bytes = 0;
     // staging buffers of the host-pointer CBLAS entry point
     float* stage[3] = {nullptr, nullptr, nullptr};
@@ -92,6 +93,7 @@ struct State {
     int mlp_fused_tail = 0;    // MLP step: 1 the last two layers, loss, their backward and update in one launch when the shapes fit; 2 also the first layer's weight gradient and update in one; 0 neither
     int fold_reduce = -1;      // the gradient of a broadcast parent summed inside the GEMM launch: -1 automatic, 0 never, 1 wherever it can
     int verbose = 0;
+    int cols_join = 0;         // column kernels: 1 the K slices are added by the last workgroup of the streaming launch, 0 by a second launch
     int cols_waves_per_cu = 2; // target workgroups per CU of the column-streaming kernels (long K slices stream best)
 };
 State S;
@@ -495,7 +497,13 @@ bool cols_shiftable(const ColsArgs& c) {
 }
 
 template <int R>
-void launch_cols(const ColsArgs& c, dim3 grid, int variant) {
+void launch_cols(const ColsArgs& c, dim3 grid, int variant, bool join) {
+    if (join) { // the K slices are added by the last workgroup of each column block
+        if (variant == 0) hipLaunchKernelGGL((cols_kernel<R, true, true>), grid, dim3(COLS_THREADS), 0, S.stream, c);
+        else if (variant == 2) hipLaunchKernelGGL((cols_kernel<R, false, true>), grid, dim3(COLS_THREADS), 0, S.stream, c);
+        else if constexpr (R <= 4) hipLaunchKernelGGL((cols_shift_kernel<R, true>), grid, dim3(COLS_THREADS), 0, S.stream, c);
+        return;
+    }
     if (variant == 0) hipLaunchKernelGGL((cols_kernel<R, true>), grid, dim3(COLS_THREADS), 0, S.stream, c);
     else if (variant == 2) hipLaunchKernelGGL((cols_kernel<R, false>), grid, dim3(COLS_THREADS), 0, S.stream, c);
     else if constexpr (R <= 4) hipLaunchKernelGGL((cols_shift_kernel<R>), grid, dim3(COLS_THREADS), 0, S.stream, c);
@@ -503,6 +511,8 @@ void launch_cols(const ColsArgs& c, dim3 grid, int variant) {
 
 // largest batch count of one launch (a grid's y and z dimensions hold 65535)
 constexpr int64_t kMaxGridBatches = 65535;
+// arrival counters of the in-launch K-slice reduction (one per column block and batch of a launch)
+constexpr int64_t kArrivalCounters = 1 << 16;
 
 // Scratch for the K-slice partial sums of a column-streaming product: the library's grow-only buffer, or a
 // fixed buffer the caller brings (the allocation-free entry point), which is never grown.
@@ -542,15 +552,21 @@ int cols_run(ColsArgs c, int64_t batch_count, float* out, int accumulate, const 
         target = ws;
     }
     c.out = target;
+    // One launch instead of two: the last workgroup of a column block adds the block's K slices (cols_join knob).  The
+    // arrival counters are the library's, zero between launches; products with more column blocks x batches than there
+    // are counters keep the separate reduction.
+    const bool join = splits > 1 && S.cols_join > 0 && S.arrivals && col_blocks * std::min(kMaxGridBatches, batch_count) <= kArrivalCounters;
+    c.joined = out;
+    c.arrivals = S.arrivals;
     for (int64_t b0 = 0; b0 < batch_count; b0 += kMaxGridBatches) {
         c.batch0 = b0;
         const dim3 grid((unsigned)col_blocks, (unsigned)splits, (unsigned)std::min(kMaxGridBatches, batch_count - b0));
-        if (R <= 1) launch_cols<1>(c, grid, variant);
-        else if (R <= 2) launch_cols<2>(c, grid, variant);
-        else if (R <= 4) launch_cols<4>(c, grid, variant);
-        else launch_cols<8>(c, grid, variant);
+        if (R <= 1) launch_cols<1>(c, grid, variant, join);
+        else if (R <= 2) launch_cols<2>(c, grid, variant, join);
+        else if (R <= 4) launch_cols<4>(c, grid, variant, join);
+        else launch_cols<8>(c, grid, variant, join);
     }
-    if (splits > 1) {
+    if (splits > 1 && !join) {
         const int64_t n = batch_count * R * c.n;
         hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
                            target, out, n, (int)splits, accumulate, (const float*)nullptr, (const float*)nullptr, 0, (int64_t)1);
@@ -984,6 +1000,8 @@ int tenmo_hip_init(int device_id) {
     HIP_TRY(hipMalloc(&S.one, sizeof(float)));
     const float one = 1.0f;
     HIP_TRY(hipMemcpy(S.one, &one, sizeof one, hipMemcpyHostToDevice));
+    HIP_TRY(hipMalloc(&S.arrivals, kArrivalCounters * sizeof(uint32_t)));
+    HIP_TRY(hipMemset(S.arrivals, 0, kArrivalCounters * sizeof(uint32_t)));
     S.force_tile = env_int("TENMO_HIP_GEMM_TILE", -1);
     S.force_splitk = env_int("TENMO_HIP_GEMM_SPLITK", -1);
     S.force_streamk = env_int("TENMO_HIP_GEMM_STREAMK", -1);
@@ -1002,6 +1020,7 @@ int tenmo_hip_shutdown(void) {
     if (S.ws) (void)hipFree(S.ws);
     if (S.ws2) (void)hipFree(S.ws2);
     if (S.one) (void)hipFree(S.one);
+    if (S.arrivals) (void)hipFree(S.arrivals);
     if (S.conv_tables) (void)hipFree(S.conv_tables);
     for (int i = 0; i < 3; ++i) if (S.stage[i]) (void)hipFree(S.stage[i]);
     (void)hipEventDestroy(S.ev0);
@@ -1043,6 +1062,7 @@ int tenmo_hip_set_tuning(const char* name, int value) {
     if (!strcmp(name, "fold_reduce")) { S.fold_reduce = value; return 0; }
     if (!strcmp(name, "mlp_fused_tail")) { S.mlp_fused_tail = value; return 0; }
     if (!strcmp(name, "conv_phases")) { S.force_conv_phases = value; return 0; }
+    if (!strcmp(name, "cols_join")) { S.cols_join = value > 0 ? 1 : 0; return 0; }
     if (!strcmp(name, "cols_wg_per_cu")) { S.cols_waves_per_cu = value > 0 ? value : 2; return 0; }
     return fail(TENMO_ERR_INVALID_ARGUMENT, "tenmo_hip_set_tuning: unknown knob '%s'", name);
 }

@@ -170,6 +170,8 @@ inline float unsafeAtomicAdd(float* p, float v) {
     return old;
 }
 inline float atomicAdd(float* p, float v) { return unsafeAtomicAdd(p, v); }
+inline unsigned atomicAdd(unsigned* p, unsigned v) { return __atomic_fetch_add(p, v, __ATOMIC_RELAXED); } // the fences around it order it
+inline void __threadfence() { __atomic_thread_fence(__ATOMIC_SEQ_CST); }
 
 // HIP's device-side min / max for mixed integer types
 template <class A, class B, class = std::enable_if_t<std::is_arithmetic<A>::value && std::is_arithmetic<B>::value>>
@@ -227,6 +229,7 @@ hipError_t hipMemcpy(void* dst, const void* src, size_t bytes, hipMemcpyKind kin
 hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKind kind, hipStream_t s);
 hipError_t hipMemcpy2DAsync(void* dst, size_t dpitch, const void* src, size_t spitch, size_t width, size_t height, hipMemcpyKind kind, hipStream_t s);
 hipError_t hipMemsetAsync(void* dst, int value, size_t bytes, hipStream_t s);
+hipError_t hipMemset(void* dst, int value, size_t bytes);
 hipError_t hipStreamCreate(hipStream_t* s);
 hipError_t hipStreamDestroy(hipStream_t s);
 hipError_t hipStreamSynchronize(hipStream_t s);

@@ -28,6 +28,7 @@
 
 extern "C" void replay_register(const void* p, size_t bytes);
 extern "C" void replay_set_late_loads(int on);
+extern "C" long replay_launch_count();
 
 static uint32_t g_rng = 12345;
 static float next_float() {
@@ -141,8 +142,11 @@ static int run_vector_case(const std::string& spec, bool is_mv) {
     int64_t batch = atoll(f[3].c_str());
     const int64_t pad = atoll(f[4].c_str());
     const int accumulate = atoi(f[5].c_str());
-    bool noalloc = false;
-    for (size_t i = 6; i < f.size(); ++i) if (f[i] == "entry=noalloc") noalloc = true;
+    bool noalloc = false, join = false;
+    for (size_t i = 6; i < f.size(); ++i) {
+        if (f[i] == "entry=noalloc") noalloc = true;
+        if (f[i] == "join=1") join = true; // K slices added inside the streaming launch; must equal the two-launch result bit for bit
+    }
     const bool shared_matrix = batch < 0;
     if (batch < 0) batch = -batch;
     const int64_t nb = batch > 0 ? batch : 1, nmat = shared_matrix ? 1 : nb;
@@ -169,15 +173,35 @@ static int run_vector_case(const std::string& spec, bool is_mv) {
     (void)mat_elems;
     replay_register(Mx, m_n * 4); replay_register(v, v_n * 4); replay_register(out, o_n * 4);
     const int64_t bshape[1] = {nb}, mstr[1] = {shared_matrix ? 0 : lines * pitch}, vstr[1] = {vec_len};
-    int rc;
-    if (is_mv) rc = tenmo_hip_mv_f32(Mx, 0, rs, cs, v, 0, 1, out, rows, cols, batch > 0 ? 1 : 0, bshape, mstr, vstr, accumulate, 1);
-    else if (noalloc) rc = tenmo_hip_vm_f32_noalloc(v, 0, 1, Mx, 0, rs, cs, out, rows, cols, batch > 0 ? 1 : 0, bshape, vstr, mstr, accumulate, 1);
-    else rc = tenmo_hip_vm_f32(v, 0, 1, Mx, 0, rs, cs, out, rows, cols, batch > 0 ? 1 : 0, bshape, vstr, mstr, accumulate, 1);
+    auto product = [&](float* dst) {
+        if (is_mv) return tenmo_hip_mv_f32(Mx, 0, rs, cs, v, 0, 1, dst, rows, cols, batch > 0 ? 1 : 0, bshape, mstr, vstr, accumulate, 1);
+        if (noalloc) return tenmo_hip_vm_f32_noalloc(v, 0, 1, Mx, 0, rs, cs, dst, rows, cols, batch > 0 ? 1 : 0, bshape, vstr, mstr, accumulate, 1);
+        return tenmo_hip_vm_f32(v, 0, 1, Mx, 0, rs, cs, dst, rows, cols, batch > 0 ? 1 : 0, bshape, vstr, mstr, accumulate, 1);
+    };
+    std::vector<float> two_launches;
+    long launches_apart = 0;
+    int rc = 0;
+    if (join) { // first the separate reduction into a copy of the same initial contents
+        two_launches.assign(out, out + o_n);
+        replay_register(two_launches.data(), o_n * 4);
+        const long before = replay_launch_count();
+        rc = product(two_launches.data());
+        launches_apart = replay_launch_count() - before;
+        replay_register(two_launches.data(), 0);
+        tenmo_hip_set_tuning("cols_join", 1);
+    }
+    const long before = replay_launch_count();
+    if (rc == 0) rc = product(out);
+    const long launches = replay_launch_count() - before;
+    if (join) tenmo_hip_set_tuning("cols_join", 0);
     int bad = 0;
     double err = -1;
     if (rc != 0) { fprintf(stderr, "%s: error %d: %s\n", spec.c_str(), rc, tenmo_hip_last_error()); bad = 1; }
     else { err = gradient_error(out, want); if (!(err <= 1e-5)) bad = 1; } // (one output can be a sum with cancellation: the stated tolerance, not a tighter one)
-    printf("%s: rc %d, relative error %.3g%s\n", spec.c_str(), rc, err, bad ? "  <-- FAILED" : "");
+    if (join && rc == 0 && memcmp(out, two_launches.data(), o_n * 4) != 0) { fprintf(stderr, "%s: joined slices differ from the two-launch result\n", spec.c_str()); bad = 1; }
+    // a product cut into K slices takes one launch less when they are joined inside the streaming launch
+    if (join && rc == 0 && launches_apart > 1 && launches != launches_apart - 1) { fprintf(stderr, "%s: %ld launches joined, %ld apart\n", spec.c_str(), launches, launches_apart); bad = 1; }
+    printf("%s: rc %d, relative error %.3g, %ld launch%s%s\n", spec.c_str(), rc, err, launches, launches == 1 ? "" : "es", bad ? "  <-- FAILED" : "");
     fflush(stdout);
     replay_register(Mx, 0); replay_register(v, 0); replay_register(out, 0);
     free(Mx); free(v); free(out);

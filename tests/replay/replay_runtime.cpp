@@ -407,6 +407,7 @@ hipError_t hipMemcpy2DAsync(void* dst, size_t dpitch, const void* src, size_t sp
     for (size_t r = 0; r < height; ++r) std::memmove((char*)dst + r * dpitch, (const char*)src + r * spitch, width);
     return hipSuccess;
 }
+hipError_t hipMemset(void* dst, int value, size_t bytes) { std::memset(dst, value, bytes); return hipSuccess; }
 hipError_t hipMemsetAsync(void* dst, int value, size_t bytes, hipStream_t s) {
     replayStream* st = stream_of(s);
     if (st->capturing) { st->graph->nodes.push_back(LaunchRecord{"memset", dim3(0), dim3(0), [=]() { std::memset(dst, value, bytes); }}); return hipSuccess; }

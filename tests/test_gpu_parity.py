@@ -1457,6 +1457,64 @@ def test_mlp_loss_curve_with_the_fused_tail(T, oracle):
             T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
 
 
+def test_column_kernels_join_slices_in_the_launch(T):
+    """vm, mv on a transposed view, skinny and batched skinny products with the K slices added by the last workgroup of
+    the streaming launch (cols_join) instead of a second launch: the same bits as the two-launch result — the slices are
+    added in the same order — call after call (the arrival counters must be back at zero), with `+=`, and through the
+    allocation-free entry."""
+    import ctypes as C
+    from tenmo_amd import _lib
+    L = _lib.load()
+    rng = np.random.default_rng(67)
+
+    def both(fn):
+        apart = fn()
+        L.tenmo_hip_set_tuning(b"cols_join", 1)
+        try:
+            joined, again = fn(), fn()
+        finally:
+            L.tenmo_hip_set_tuning(b"cols_join", 0)
+        assert np.array_equal(apart, joined) and np.array_equal(apart, again)
+        return joined
+
+    for (m, k, n) in [(1, 4096, 4096), (4, 768, 50257), (3, 2000, 3001), (8, 1024, 2048), (1, 16384, 1024), (2, 515, 1030), (1, 100, 50000)]:
+        a = rng.standard_normal((m, k), dtype=np.float32)
+        b = rng.standard_normal((k, n), dtype=np.float32)
+        A, B = T.Tensor.from_numpy(a), T.Tensor.from_numpy(b)
+        got = both(lambda: A.matmul(B, track_grad=False).to_numpy())
+        assert rel_fro(got, ref_matmul64(a, b)) <= RTOL_FRO, (m, k, n)
+        if m == 1:
+            v = T.Tensor.from_numpy(a[0])
+            got = both(lambda: v.matmul(B, track_grad=False).to_numpy())                      # vector x matrix
+            assert rel_fro(got, ref_matmul64(a, b)[0]) <= RTOL_FRO, ("vm", k, n)
+            Bt = T.Tensor.from_numpy(b).transpose()                                           # [n, k] view: mv through the column kernel
+            got = both(lambda: Bt.matmul(v, track_grad=False).to_numpy())
+            assert rel_fro(got, ref_matmul64(a, b)[0]) <= RTOL_FRO, ("mv of a transposed view", k, n)
+    # batches of a right operand with an odd pitch
+    a = rng.standard_normal((2, 768), dtype=np.float32)
+    b = rng.standard_normal((4, 768, 2503), dtype=np.float32)
+    A, B = T.Tensor.from_numpy(a), T.Tensor.from_numpy(b)
+    assert rel_fro(both(lambda: A.matmul(B, track_grad=False).to_numpy()), ref_matmul64(a, b)) <= RTOL_FRO
+    # += and the allocation-free entry
+    a = rng.standard_normal((1, 3000), dtype=np.float32)
+    b = rng.standard_normal((3000, 5000), dtype=np.float32)
+    c0 = rng.standard_normal((1, 5000), dtype=np.float32)
+    A, B = T.Tensor.from_numpy(a), T.Tensor.from_numpy(b)
+
+    def accumulate(entry):
+        out = T.Tensor.from_numpy(c0.copy())
+        if entry == "gemm":
+            _lib.check(L.tenmo_hip_gemm_f32(A.buffer.data_ptr(), 0, 3000, 1, B.buffer.data_ptr(), 0, 5000, 1, out.buffer.data_ptr(),
+                                            1, 5000, 3000, 0, None, None, None, 1, 1))
+        else:
+            _lib.check(L.tenmo_hip_vm_f32_noalloc(A.buffer.data_ptr(), 0, 1, B.buffer.data_ptr(), 0, 5000, 1, out.buffer.data_ptr(),
+                                                  3000, 5000, 0, None, None, None, 1, 1))
+        return out.to_numpy()
+
+    for entry in ("gemm", "noalloc"):
+        assert rel_fro(both(lambda: accumulate(entry)), c0.astype(np.float64) + ref_matmul64(a, b)) <= RTOL_FRO, entry
+
+
 def test_zz_graph_capture_grows_scratch(T, oracle):
     """A captured training step whose kernel selection wants more library scratch than exists when the capture starts:
     the capture is abandoned, the scratch grown outside it and the step captured again — same losses as the eager step."""

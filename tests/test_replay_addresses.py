@@ -170,8 +170,14 @@ def test_matrix_vector_kernels(exe):
                 cases.append(f"vm:{k},{n},{layout},0,{pad},0")
     cases += ["vm:300,70,n,3,0,1", "vm:300,1027,n,3,1,1", "vm:257,65,t,-4,0,0", "vm:4096,1500,n,0,0,1,entry=noalloc", "vm:700,260,n,2,0,1,entry=noalloc",
               "vm:768,4096,n,0,0,0", "vm:100,50000,n,0,0,0"]
-    run(exe, cases, cus=16, modes=("early",))
-    run(exe, cases[::5], cus=256, modes=("early",))
+    # the K slices added by the last workgroup of the streaming launch (join=1: the driver also requires the bits of the
+    # two-launch result and one launch less), on few and on many modelled CUs (other slice counts)
+    joined = ["vm:1024,64,n,0,0,0,join=1", "vm:1030,515,n,0,1,0,join=1", "vm:1030,515,n,0,0,1,join=1", "vm:300,4099,n,0,0,0,join=1",
+              "vm:2000,6282,n,0,0,1,join=1", "vm:2000,6282,n,3,1,0,join=1", "vm:257,65,n,-4,0,0,join=1", "mv:515,1030,t,0,1,0,join=1",
+              "mv:64,1024,t,2,0,1,join=1", "vm:4096,1500,n,0,0,1,entry=noalloc,join=1", "vm:100,50000,n,0,0,0,join=1", "vm:5000,9,n,0,0,0,join=1",
+              "4,6282,768,n,n,0,0,1,cols_join=1", "8,1000,300,n,n,3,0,0,cols_join=1", "2,4099,515,n,n,0,0,0,cols_join=1"]
+    run(exe, cases + joined, cus=16, modes=("early",))
+    run(exe, cases[::5] + joined, cus=256, modes=("early",))
 
 
 def test_adjacent_operators(exe):
