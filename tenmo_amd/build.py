@@ -68,6 +68,7 @@ def build(verbose: bool = False) -> str:
                            os.path.join(CSRC, "gemm_tiles.hip")], os.path.join(tmp, f"gemm_{bm}x{bn}_{sk}.o")))
         units.append(([os.path.join(CSRC, "gemm_smallk.hip")], os.path.join(tmp, "gemm_smallk.o")))
         units.append(([os.path.join(CSRC, "gemm_panel.hip")], os.path.join(tmp, "gemm_panel.o")))
+        units.append(([os.path.join(CSRC, "gemm_resident.hip")], os.path.join(tmp, "gemm_resident.o")))
         stamp = " ".join(FLAGS)
         stamp_file = os.path.join(tmp, "flags.txt")
         same_flags = keep and os.path.exists(stamp_file) and open(stamp_file).read() == stamp

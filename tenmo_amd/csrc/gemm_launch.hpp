@@ -47,4 +47,11 @@ bool launch_gemm_smallk_64x64(const GemmArgs& g, int amode, int bmode, unsigned 
 enum PanelTile : int { PANEL_TILE_128x128 = 0, PANEL_TILE_64x64 = 1 }; // (64x64: a ring of eight stages, for long reductions over few tiles)
 bool launch_gemm_panel(const GemmArgs& g, int tile, int amode, int bmode, unsigned cus, unsigned total_tiles, bool by_batch, hipStream_t stream);
 
+// A small left operand against a very wide right one (one matrix, K up to 256, B with unit stride along N, plain store):
+// persistent workgroups that keep their tile row of A in LDS and stream B alone (gemm_resident.hip).  `bm`: 128 (one
+// workgroup per CU) or 64 (two) rows per tile, 64 columns; g.tiles_m, g.tiles_n set for that tile; the number of tile
+// rows must not exceed the workgroups of an XCD.  The caller has checked what the direct loads need, as for the K-stream
+// kernel.  false: not a shape this kernel takes.
+bool launch_gemm_resident(const GemmArgs& g, int bm, int amode, int bmode, unsigned cus, hipStream_t stream);
+
 } // namespace tenmo

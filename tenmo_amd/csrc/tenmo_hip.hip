@@ -89,6 +89,7 @@ struct State {
     int force_conv_phases = -1; // strided image gradient phase by phase: -1 automatic (large layers), 0 never, 1 always
     int force_streamk = -1;    // -1 automatic, 0 never, n > 0: stream-K with n workgroups per CU
     int force_smallk = -1;     // -1 automatic, 0 never, 1: the short-reduction kernel wherever it can run
+    int force_resident = 0;    // the resident-A kernel for a few tile rows against a very wide B: 1 with 128x64 tiles, 2 with 64x64, 0 never
     int force_panel = -1;      // -1 automatic, 0 never, 1: the persistent K-stream kernel wherever it can run (2: without XCD grouping, 3: 64x64 tiles)
     int mlp_fused_tail = 0;    // MLP step: 1 the last two layers, loss, their backward and update in one launch when the shapes fit; 2 also the first layer's weight gradient and update in one; 0 neither
     int fold_reduce = -1;      // the gradient of a broadcast parent summed inside the GEMM launch: -1 automatic, 0 never, 1 wherever it can
@@ -348,6 +349,23 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         if (S.verbose) fprintf(stderr, "tenmo_hip gemm M=%lld N=%lld K=%lld batch=%lld -> tile %dx%d, %d K slice(s), est %.1f us%s\n",
                                (long long)M, (long long)N, (long long)K, (long long)batch_count, kTiles[tile].bm, kTiles[tile].bn, splits, best,
                                sk_wpc ? " (stream-K chosen instead)" : "");
+    }
+    // A few tile rows against a very wide B (gemm_resident.hip): the tile row of A stays in LDS, B alone is streamed.
+    // Only on request (gemm_resident knob: 1 tiles of 128x64, 2 of 64x64) until it has been measured.
+    if (S.force_resident > 0) {
+        const int rbm = S.force_resident == 2 ? 64 : 128;
+        const int64_t tm = (M + rbm - 1) / rbm, tn = (N + 63) / 64;
+        const bool a_ok = am == KMAJOR_VEC ? (a_cs == 1 && a_rs >= 0 && a_rs <= (int64_t(1) << 21) && K % 4 == 0)
+                                           : (am == MNMAJOR_VEC && a_rs == 1 && a_cs >= 0 && a_cs <= (int64_t(1) << 25) && M % 4 == 0 && M >= 4);
+        const bool b_ok = bm == MNMAJOR_VEC && b_cs == 1 && b_rs >= 0 && b_rs <= (int64_t(1) << 25) && N % 4 == 0 && N >= 4;
+        const bool can = batch_count == 1 && !accumulate && K > GEMM_BK && K <= 256 && a_ok && b_ok && !ep.any() && !ep.gather_row && !ep.colsum &&
+                         N <= (int64_t(1) << 22) && tm <= (int64_t)S.cus * (rbm == 64 ? 2 : 1) / 8; // (worth it with several column blocks per workgroup: for the policy that will choose it once it has been measured)
+        if (can) {
+            g.tiles_m = (int32_t)tm; g.tiles_n = (int32_t)tn;
+            g.k_splits = 1; g.k_per_split = K; g.partial = nullptr;
+            if (S.verbose) fprintf(stderr, "tenmo_hip gemm: resident-A kernel, %lld x %lld tiles of %dx64\n", (long long)tm, (long long)tn, rbm);
+            if (launch_gemm_resident(g, rbm, am, bm, (unsigned)S.cus, S.stream)) return 0;
+        }
     }
     // The persistent K-stream kernel (gemm_panel.hip): vector operand forms, plain or accumulating store.  Automatic for
     // a reduction of 65 .. 512 into a result of at least three 128x128 tiles per CU (measured against the tile the model
@@ -1059,6 +1077,7 @@ int tenmo_hip_set_tuning(const char* name, int value) {
     if (!strcmp(name, "gemm_streamk")) { S.force_streamk = value; return 0; }
     if (!strcmp(name, "gemm_smallk")) { S.force_smallk = value; return 0; }
     if (!strcmp(name, "gemm_panel")) { S.force_panel = value; return 0; }
+    if (!strcmp(name, "gemm_resident")) { S.force_resident = value > 0 ? value : 0; return 0; }
     if (!strcmp(name, "fold_reduce")) { S.fold_reduce = value; return 0; }
     if (!strcmp(name, "mlp_fused_tail")) { S.mlp_fused_tail = value; return 0; }
     if (!strcmp(name, "conv_phases")) { S.force_conv_phases = value; return 0; }

@@ -41,7 +41,8 @@ def _units(extra_sources):
     units = [(["-c", os.path.join(HERE, "replay_runtime.cpp")], "runtime.o"),
              (["-c", os.path.join(CSRC, "tenmo_hip.hip")], "host.o"),
              (["-c", os.path.join(CSRC, "gemm_smallk.hip")], "smallk.o"),
-             (["-c", os.path.join(CSRC, "gemm_panel.hip")], "panel.o")]
+             (["-c", os.path.join(CSRC, "gemm_panel.hip")], "panel.o"),
+             (["-c", os.path.join(CSRC, "gemm_resident.hip")], "resident.o")]
     for bm, bn, sk in TILES:
         units.append(([f"-DTENMO_TILE_BM={bm}", f"-DTENMO_TILE_BN={bn}", f"-DTENMO_TILE_STREAMK={sk}", "-c", os.path.join(CSRC, "gemm_tiles.hip")],
                       f"tile_{bm}x{bn}_{sk}.o"))

@@ -29,6 +29,7 @@
 extern "C" void replay_register(const void* p, size_t bytes);
 extern "C" void replay_set_late_loads(int on);
 extern "C" long replay_launch_count();
+extern "C" const char* replay_last_kernel();
 
 static uint32_t g_rng = 12345;
 static float next_float() {
@@ -78,6 +79,7 @@ static int run_case(const std::string& spec) {
     const bool b_shared = atoi(f[6].c_str()) != 0;
     const int accumulate = atoi(f[7].c_str());
     bool check = true;
+    std::string ran;
     std::vector<std::pair<std::string, int>> knobs;
     for (size_t i = 8; i < f.size(); ++i) {
         const size_t eq = f[i].find('=');
@@ -85,6 +87,7 @@ static int run_case(const std::string& spec) {
         const std::string name = f[i].substr(0, eq);
         const int value = atoi(f[i].c_str() + eq + 1);
         if (name == "check") check = value != 0;
+        else if (name == "ran") ran = f[i].substr(eq + 1); // the kernel that must have served the product (a part of its name)
         else knobs.push_back({name, value});
     }
     const int64_t nb = batch > 0 ? batch : 1, nbb = b_shared ? 1 : nb;
@@ -108,6 +111,10 @@ static int run_case(const std::string& spec) {
     for (auto& kv : knobs) tenmo_hip_set_tuning(kv.first.c_str(), -1);
     int bad = 0;
     if (rc != 0) { fprintf(stderr, "%s: error %d: %s\n", spec.c_str(), rc, tenmo_hip_last_error()); bad = 1; }
+    if (rc == 0 && !ran.empty() && !strstr(replay_last_kernel(), ran.c_str())) {
+        fprintf(stderr, "%s: served by %s\n", spec.c_str(), replay_last_kernel());
+        bad = 1;
+    }
     double err = -1.0;
     if (rc == 0 && check) {
         err = reference_error(A, B, Cm, accumulate ? C0.data() : nullptr, nb, b_shared, M, N, K, a_mat, b_mat, a_rs, a_cs, b_rs, b_cs);

@@ -325,9 +325,11 @@ void run_on_pool(const std::function<void()>& job) {
 } // namespace
 
 std::atomic<long> g_launches{0};
+std::string g_last_kernel; // (launches are serialized)
 
 void launch(const char* name, dim3 grid, dim3 block, std::function<void()> body) {
     ++g_launches;
+    g_last_kernel = name;
     const int64_t total = (int64_t)grid.x * grid.y * grid.z;
     if ((int64_t)block.x * block.y * block.z > MAX_LANES || total <= 0) fail("launch of %s: bad grid or block", name);
     // what the HIP runtime refuses: more than 65535 workgroups along y or z, 2^32 or more threads along one dimension
@@ -463,4 +465,5 @@ void replay_register(const void* p, size_t bytes) {
 }
 void replay_set_late_loads(int on) { replay::late_loads = on; }
 long replay_launch_count() { return replay::g_launches.load(); } // kernel launches executed so far
+const char* replay_last_kernel() { return replay::g_last_kernel.c_str(); } // the kernel expression of the last launch, as the source spells it
 }

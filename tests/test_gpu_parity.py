@@ -1457,6 +1457,40 @@ def test_mlp_loss_curve_with_the_fused_tail(T, oracle):
             T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
 
 
+def test_resident_left_operand_kernel(T):
+    """The kernel that keeps its tile row of A in LDS for all of K and streams B alone (gemm_resident knob: tiles of 128x64
+    and of 64x64), forced on: the CBOW logits and their gradient at full size, K tails, a row-major and a transposed-view A,
+    ragged last tile rows and column blocks, several tile rows, a result of fewer tiles than workgroups; and, with the knob
+    still on, what the kernel does not take (falls through to the others).  Against fp64; the element behind the result
+    stays untouched.  (The same launches run address by address on the CPU in test_replay_addresses.py.)"""
+    import torch
+    L, lib = T.lib.load(), T.lib
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(37)
+    cases = [(256, 50000, 100), (100, 50000, 256), (128, 2052, 32), (64, 4096, 20), (36, 3000, 112), (200, 2500, 132), (1024, 6400, 48),
+             (256, 128, 100), (256, 3200, 248), (128, 3200, 272), (128, 3202, 64)]
+    try:
+        for knob in (1, 2):
+            L.tenmo_hip_set_tuning(b"gemm_resident", knob)
+            for M, N, K in cases:
+                for ta in (False, True):
+                    for tb, acc in ((False, 0), (True, 0), (False, 1)) if (M, N, K) == (128, 2052, 32) else ((False, 0),):
+                        A = torch.randn(((K, M) if ta else (M, K)), generator=gen, device="cuda")
+                        B = torch.randn(((N, K) if tb else (K, N)), generator=gen, device="cuda")
+                        out = torch.randn((M * N + 1,), generator=gen, device="cuda")
+                        guard = float(out[-1])
+                        a_rs, a_cs = (1, M) if ta else (K, 1)
+                        b_rs, b_cs = (1, K) if tb else (N, 1)
+                        ref = (A.t() if ta else A).double() @ (B.t() if tb else B).double() + (out[:-1].view(M, N).double() if acc else 0)
+                        lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, a_rs, a_cs, B.data_ptr(), 0, b_rs, b_cs, out.data_ptr(), M, N, K, 0,
+                                                       None, None, None, acc, 1))
+                        err = float((out[:-1].view(M, N).double() - ref).norm() / ref.norm())
+                        assert err <= RTOL_FRO, (knob, M, N, K, ta, tb, acc, err)
+                        assert float(out[-1]) == guard, (knob, M, N, K, ta, tb, acc)
+    finally:
+        L.tenmo_hip_set_tuning(b"gemm_resident", 0)
+
+
 def test_column_kernels_join_slices_in_the_launch(T):
     """vm, mv on a transposed view, skinny and batched skinny products with the K slices added by the last workgroup of
     the streaming launch (cols_join) instead of a second launch: the same bits as the two-launch result — the slices are

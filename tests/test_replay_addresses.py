@@ -127,6 +127,28 @@ def test_k_stream_kernel(exe):
     run(exe, small[:8] + [case(1024, 1024, 1024, gemm_panel=3)], cus=256, modes=("late",))
 
 
+def test_resident_left_operand_kernel(exe):
+    """gemm_resident_kernel forced on (both tile heights): a few tile rows of A held in LDS for all of K against a wide B
+    with unit stride along N — K of two steps up to 256 and K tails, a row-major and a transposed-view A, ragged last tile
+    rows and column blocks, more tile rows than one, walks of many column blocks per workgroup (few CUs) and the real 256;
+    `ran=` makes the driver check that this kernel, not another one, served the case.  What it does not take (a transposed
+    B, batches, accumulate, K beyond 256, a K-major A with K % 4 != 0) falls through to the other kernels and is still right."""
+    cases = []
+    for knob in (1, 2):
+        for la in ("n", "t"):
+            for (M, N, K) in [(256, 3200, 100), (100, 3204, 256), (128, 2052, 32), (64, 4096, 20), (36, 3000, 112), (200, 2500, 132), (256, 2048, 250 if la == "t" else 248)]:
+                cases.append(case(M, N, K, la, "n", gemm_resident=knob, ran="gemm_resident_kernel"))
+    run(exe, cases, cus=16)
+    # the chip's real width: 32 or 64 workgroups per XCD, up to 32 tile rows, column blocks left over at the end of the walks
+    wide = [case(256, 50000, 100, "n", "n", gemm_resident=1, ran="gemm_resident_kernel"), case(100, 50000, 256, "t", "n", gemm_resident=2, ran="gemm_resident_kernel"),
+            case(1024, 6400, 48, "n", "n", gemm_resident=1, ran="gemm_resident_kernel"), case(2048, 3300, 36, "t", "n", gemm_resident=2, ran="gemm_resident_kernel")]
+    run(exe, wide, cus=256, modes=("late",))
+    others = [case(256, 3200, 100, "n", "t", gemm_resident=1), case(256, 3200, 100, "n", "n", batch=2, gemm_resident=1), case(256, 3200, 100, "n", "n", acc=1, gemm_resident=1),
+              case(128, 3200, 272, "n", "n", gemm_resident=1), case(128, 3200, 250, "n", "n", gemm_resident=2), case(128, 3202, 64, "n", "n", gemm_resident=1),
+              case(256, 128, 100, "n", "n", gemm_resident=1)]
+    run(exe, others, cus=16, modes=("early",))
+
+
 def test_automatic_choice_on_benchmark_shapes(exe):
     """What the dispatch picks by itself for the shapes the benchmarks run, at their real sizes (attention: 8 of the 96
     batches; the square products reduced to 1024)."""
