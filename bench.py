@@ -529,8 +529,8 @@ def mlp_step_times(_lib, torch, np, fused_tail=False):
     graph_ms = (time.perf_counter() - t0) * 1e3 / 20
     fused = {}
     if fused_tail:
-        # 1: the last two layers, loss, backward and update in one launch; 2: also the first layer's gradient with its update
-        for level, key in ((1, "mlp_step_ms_gpu_fused_tail"), (2, "mlp_step_ms_gpu_fused_tail_and_first")):
+        # 1: the last two layers, loss, backward and update in one launch; 2: also the first layer's gradient with its update; 3: also its forward
+        for level, key in ((1, "mlp_step_ms_gpu_fused_tail"), (2, "mlp_step_ms_gpu_fused_tail_and_first"), (3, "mlp_step_ms_gpu_three_launches")):
             L.tenmo_hip_set_tuning(b"mlp_fused_tail", level)
             try:
                 first = float(gpu.step_device(*dev[0], lr, sync=True).item())

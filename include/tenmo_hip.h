@@ -77,7 +77,7 @@ int tenmo_hip_device_info(int* compute_units, char* name, int name_len);
  * "fold_reduce" (the gradient of a parent that was broadcast over batch dimensions summed inside the GEMM launch instead
  * of materialised and reduced: 1 wherever it can run, 0 never, -1 automatic), "mlp_fused_tail" (tenmo_hip_mlp_step: the last
  * two layers, the loss, their backward and their update as one launch when they fit one workgroup — batch <= 64, widths
- * <= 128 / 64 / 32: 1 on, 2 the same and the first layer's weight gradient with its update as one launch, 0 off, the default), "cols_wg_per_cu" (workgroups per CU the
+ * <= 128 / 64 / 32: 1 on, 2 the same and the first layer's weight gradient with its update as one launch, 3 the same and the first layer's forward as one launch, 0 off, the default), "cols_wg_per_cu" (workgroups per CU the
  * column-streaming kernel aims for), "cols_join" (vm, mv of a transposed view and skinny products whose reduction is cut
  * into K slices: 1 the slices are added by the last workgroup of the streaming launch — same bits, one launch less —, 0 by a
  * second launch, the default) and "conv_phases" (image gradient of a strided convolution phase by phase:

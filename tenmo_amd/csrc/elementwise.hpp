@@ -397,6 +397,71 @@ __global__ __launch_bounds__(MLP_TAIL_THREADS) void mlp_first_layer_kernel(const
         for (int i = t; i < O; i += MLP_TAIL_THREADS) a.b[i] = a.b[i] - a.lr * a.db[i];
 }
 
+// The first layer's forward for a small batch in ONE launch: h = relu(x . W + b) (tenmo/net.mojo:193-201) for a batch of a
+// few dozen rows against a long input (784).  The ordinary path cuts such a product into K slices over many workgroups and
+// adds them in a second launch; here a workgroup of 16 wavefronts owns one 32x32 block of h and cuts K among its OWN
+// wavefronts — wavefront w takes the 8-wide k chunks w, w + 16, ... with operands straight from global memory (x: one
+// 16-byte read per lane and chunk, W: four dword reads of 128 contiguous bytes per half wavefront) — and the 16 partial
+// blocks are added through LDS in wavefront order, so the result does not depend on scheduling.
+constexpr int MLP_FWD_THREADS = 1024, MLP_FWD_WAVES = MLP_FWD_THREADS / 64;
+struct MlpFwdArgs {
+    const float* x;  // [B, I]
+    const float* W;  // [I, O]
+    const float* b;  // [O]
+    float* h;        // [B, O]
+    int32_t B, I, O, relu;
+};
+__global__ __launch_bounds__(MLP_FWD_THREADS) void mlp_first_forward_kernel(const MlpFwdArgs a) {
+    __shared__ float part[MLP_FWD_WAVES][16 * 64];
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6, half = lane >> 5, i = lane & 31;
+    const int I = a.I, O = a.O;
+    const int row = min((int)blockIdx.y * 32 + i, a.B - 1), col = min((int)blockIdx.x * 32 + i, O - 1); // clamped: loaded, never stored
+    const float* __restrict xr = a.x + (int64_t)row * I;
+    const float* __restrict wc = a.W + col;
+    f32x16 acc;
+#pragma unroll
+    for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+    const int chunks = (I + 7) / 8;
+    constexpr int U = 4; // chunks in flight per wavefront
+    for (int c0 = wave; c0 < chunks; c0 += U * MLP_FWD_WAVES) {
+        float fa[U][4], fb[U][4];
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            const int k = 8 * (c0 + u * MLP_FWD_WAVES) + 4 * half; // this lane's four k of the chunk (MFMA steps 0..3)
+            if (k + 3 < I) {
+                const f32x4 v = *reinterpret_cast<const f32x4_u*>(xr + k);
+                fa[u][0] = v.x; fa[u][1] = v.y; fa[u][2] = v.z; fa[u][3] = v.w;
+#pragma unroll
+                for (int s = 0; s < 4; ++s) fb[u][s] = wc[(int64_t)(k + s) * O];
+            } else {
+#pragma unroll
+                for (int s = 0; s < 4; ++s) {
+                    const bool ok = k + s < I;
+                    fa[u][s] = ok ? xr[k + s] : 0.f;
+                    fb[u][s] = ok ? wc[(int64_t)(k + s) * O] : 0.f;
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int s = 0; s < 4; ++s) acc = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[u][s], fb[u][s], acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int e = 0; e < 16; ++e) part[wave][e * 64 + lane] = acc[e];
+    __syncthreads();
+    // thread t adds element (e, l) = (t / 64, t % 64) of the 16 partial blocks: block row 8(e>>2) + 4(l>>5) + (e&3), column l & 31
+    float sum = 0.f;
+#pragma unroll
+    for (int w = 0; w < MLP_FWD_WAVES; ++w) sum += part[w][t];
+    const int e = t >> 6;
+    const int r = (int)blockIdx.y * 32 + 8 * (e >> 2) + 4 * half + (e & 3), c = (int)blockIdx.x * 32 + i;
+    if (r < a.B && c < O) {
+        sum += a.b[c];
+        a.h[(int64_t)r * O + c] = a.relu && !(sum > 0.f) ? 0.f : sum;
+    }
+}
+
 // loss = (sum of row losses in row order) / rows — the order of the reference's scalar loop
 __global__ void ordered_mean_kernel(const float* __restrict row_loss, int64_t rows, float* __restrict out) {
     if (blockIdx.x == 0 && threadIdx.x == 0) {

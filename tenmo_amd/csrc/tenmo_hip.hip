@@ -91,7 +91,7 @@ struct State {
     int force_smallk = -1;     // -1 automatic, 0 never, 1: the short-reduction kernel wherever it can run
     int force_resident = 0;    // the resident-A kernel for a few tile rows against a very wide B: 1 with 128x64 tiles, 2 with 64x64, 0 never
     int force_panel = -1;      // -1 automatic, 0 never, 1: the persistent K-stream kernel wherever it can run (2: without XCD grouping, 3: 64x64 tiles)
-    int mlp_fused_tail = 0;    // MLP step: 1 the last two layers, loss, their backward and update in one launch when the shapes fit; 2 also the first layer's weight gradient and update in one; 0 neither
+    int mlp_fused_tail = 0;    // MLP step: 1 the last two layers, loss, their backward and update in one launch when the shapes fit; 2 also the first layer's weight gradient and update in one; 3 also the first layer's forward in one; 0 neither
     int fold_reduce = -1;      // the gradient of a broadcast parent summed inside the GEMM launch: -1 automatic, 0 never, 1 wherever it can
     int verbose = 0;
     int cols_join = 0;         // column kernels: 1 the K slices are added by the last workgroup of the streaming launch, 0 by a second launch
@@ -1902,6 +1902,16 @@ static int mlp_forward(tenmo_mlp* m, const float* x, int64_t B, int layers = -1)
         const int64_t I = m->dims[l], O = m->dims[l + 1];
         Epilogue ep; // bias add and ReLU happen in the GEMM store
         ep.bias = m->b[l]; ep.relu = l + 1 < m->L ? 1 : 0;
+        // a small batch against a long input: one launch whose workgroups cut K among their own wavefronts, instead of K
+        // slices over many workgroups and a launch that adds them (mlp_fused_tail knob, level 3)
+        if (S.mlp_fused_tail >= 3 && l == 0 && B <= 128 && O <= 256 && I >= 256 && I <= (1 << 20)) {
+            MlpFwdArgs f{};
+            f.x = in; f.W = m->W[0]; f.b = m->b[0]; f.h = m->act[0];
+            f.B = (int32_t)B; f.I = (int32_t)I; f.O = (int32_t)O; f.relu = ep.relu;
+            hipLaunchKernelGGL(mlp_first_forward_kernel, dim3((unsigned)((O + 31) / 32), (unsigned)((B + 31) / 32)), dim3(MLP_FWD_THREADS), 0, S.stream, f);
+            in = m->act[l];
+            continue;
+        }
         if (int rc = gemm_dispatch(in, I, 1, m->W[l], O, 1, m->act[l], B, O, I, bd, 1, 0, ep)) return rc;
         in = m->act[l];
     }

@@ -1449,12 +1449,32 @@ def test_mlp_loss_curve_with_the_fused_tail(T, oracle):
     from tenmo_amd import rng as R
     from tenmo_amd.net import MLP
 
-    for level in (1, 2):  # 2: the first layer's weight gradient and its update as one launch as well
+    for level in (1, 2, 3):  # 2: the first layer's weight gradient and its update as one launch as well; 3: its forward too
         T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", level)
         try:
             _mlp_loss_curve(T, oracle, R, MLP)
         finally:
             T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
+    # every fused launch on ragged shapes: inputs that end inside an 8-wide k chunk in each way, widths that are no
+    # multiples of the 32x32 blocks, batches that do not fill them
+    rs = np.random.default_rng(71)
+    T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 3)
+    try:
+        for batch, dims in ((37, [257, 77, 33, 7]), (64, [1001, 128, 64, 32]), (1, [262, 5, 3, 2]), (100, [518, 130, 40, 9]), (33, [259, 97, 4])):
+            Ws, bs = R.xavier_mlp(dims, 11)
+            gpu, cpu = MLP(dims, Ws, bs, batch), oracle.MLP(dims, Ws, bs, batch)
+            for step in range(3):
+                x = rs.standard_normal((batch, dims[0])).astype(np.float32)
+                y = rs.integers(0, dims[-1], batch).astype(np.int32)
+                assert abs(gpu.step(x, y, 0.05) - cpu.step(x, y, 0.05)) <= 1e-4, (batch, dims, step)
+            for l in range(len(dims) - 1):
+                (Wg, bg), (Wc, bc) = gpu.params(l), cpu.params(l)
+                assert rel_fro(Wg, Wc) <= 1e-5 and np.abs(bg - bc).max() <= 1e-5, (batch, dims, l)
+                (dWg, dbg), (dWc, dbc) = gpu.grads(l), cpu.grads(l)
+                assert rel_fro(dWg, dWc) <= 1e-4 and rel_fro(dbg, dbc) <= 1e-4, (batch, dims, l)
+            assert rel_fro(gpu.forward(x), cpu.forward(x)) <= 1e-5, (batch, dims)
+    finally:
+        T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
 
 
 def test_resident_left_operand_kernel(T):

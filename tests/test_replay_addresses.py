@@ -213,7 +213,9 @@ def test_adjacent_operators(exe):
              # the MLP training step op by op and with its last two layers fused into one launch: the MNIST shape, the largest
              # widths the fused launch takes, ragged ones, and a batch of one
              "mlp:64,784,128,32,10,0", "mlp:64,784,128,32,10,1", "mlp:64,300,128,64,32,1", "mlp:37,50,77,33,7,1", "mlp:1,9,5,3,2,1",
-             "mlp:64,784,128,32,10,2", "mlp:37,50,77,33,7,2", "mlp:1,9,5,3,2,2", "mlp:64,17,128,64,32,2", "mlp:5,33,1,1,1,2"]
+             "mlp:64,784,128,32,10,2", "mlp:37,50,77,33,7,2", "mlp:1,9,5,3,2,2", "mlp:64,17,128,64,32,2", "mlp:5,33,1,1,1,2",
+             # ... and the first layer's forward as one launch (inputs of 256 and more; K tails of every kind, ragged blocks)
+             "mlp:64,784,128,32,10,3", "mlp:37,257,77,33,7,3", "mlp:1,1001,5,3,2,3", "mlp:64,300,128,64,32,3", "mlp:100,518,130,40,9,3"]
     run(exe, cases, cus=16, modes=("early",))
 
 

@@ -72,7 +72,7 @@ for arr in (x, y, loss):
     lib.replay_register(C.c_void_p(arr.ctypes.data), C.c_size_t(arr.nbytes))
 fp = C.POINTER(C.c_float)
 results = {}
-for fused in (0, 1, 2):
+for fused in (0, 1, 2, 3):
     W_ptrs = (fp * 3)(*[w.ctypes.data_as(fp) for w in Ws])
     b_ptrs = (fp * 3)(*[b.ctypes.data_as(fp) for b in bs])
     m = lib.tenmo_hip_mlp_create(3, (C.c_int64 * 4)(*dims), W_ptrs, b_ptrs, C.c_int64(64))
@@ -92,12 +92,13 @@ def test_mlp_step_launch_count():
     """The MNIST-shaped training step (784 -> 128 -> 32 -> 10, batch 64) through the C ABI on the replay, counting kernel
     launches: op by op (nine); with the last two layers, the loss, their backward and their update fused into one launch
     (first-layer forward as K slices and their reduction, the fused tail, first-layer weight gradient, its update: five);
-    and with that gradient and update in one launch as well (four); same loss every way.  (In a child process: the replay
+    with that gradient and update in one launch as well (four); and with the first-layer forward as one launch that cuts K
+    inside its workgroups (three); same loss every way.  (In a child process: the replay
     ends the process when a kernel misbehaves.)"""
     import json
 
     res = subprocess.run([sys.executable, "-c", MLP_LAUNCH_COUNT_SCRIPT, replay_build.build_library()], capture_output=True, text=True, timeout=600)
     assert res.returncode == 0, res.stdout + res.stderr
     results = {int(k): v for k, v in json.loads(res.stdout.strip().splitlines()[-1]).items()}
-    assert results[2][0] <= 4 < results[1][0] <= 5 < results[0][0], results
-    assert abs(results[0][1] - results[1][1]) <= 1e-5 and abs(results[0][1] - results[2][1]) <= 1e-5, results
+    assert results[3][0] <= 3 < results[2][0] <= 4 < results[1][0] <= 5 < results[0][0], results
+    assert max(abs(results[0][1] - results[k][1]) for k in (1, 2, 3)) <= 1e-5, results
