@@ -273,6 +273,58 @@ __device__ __forceinline__ void lds_product(int M, int N, int K, const float* A,
     }
 }
 
+// The same product on the matrix cores: the 32x32 blocks of C are dealt to the workgroup's four wavefronts (v_mfma_f32_32x32x2,
+// operands read from LDS one element per lane and MFMA: 2 LDS reads per 2048 multiply-adds, where the vector form above
+// needs 1536 and is bound by the LDS).  With fewer blocks than wavefronts K is cut among 4 / blocks wavefronts per block and
+// the partial blocks are added through `scratch` (MLP_TAIL_THREADS * 16 floats) in a fixed order.  Every thread of the
+// workgroup must call it (it synchronises when it cuts K).
+template <class Emit>
+__device__ __forceinline__ void lds_product_mfma(int M, int N, int K, const float* A, int a_rs, int a_cs, const float* B, int b_rs, int b_cs, float* scratch,
+                                                 Emit&& emit) {
+    constexpr int WAVES = MLP_TAIL_THREADS / 64;
+    const int t = threadIdx.x, wave = t >> 6, lane = t & 63, half = lane >> 5, i = lane & 31;
+    const int bn = (N + 31) / 32, nblk = ((M + 31) / 32) * bn;
+    const int ks = nblk >= WAVES ? 1 : WAVES / nblk;          // wavefronts per block
+    const int kpart = ((K + ks - 1) / ks + 1) & ~1;           // k per part, even (an MFMA takes two)
+    for (int u = wave; u < nblk * ks; u += WAVES) {
+        const int blk = u / ks, part = u - blk * ks;
+        const int m0 = (blk / bn) * 32, n0 = (blk % bn) * 32;
+        const int kb = part * kpart, ke = min(K, kb + kpart);
+        const int m = min(m0 + i, M - 1), n = min(n0 + i, N - 1); // clamped: computed, never emitted
+        f32x16 acc;
+#pragma unroll
+        for (int e = 0; e < 16; ++e) acc[e] = 0.f;
+        for (int k = kb; k < ke; k += 2) {
+            const int kk = k + half;
+            const bool ok = kk < ke;
+            const float av = ok ? A[m * a_rs + kk * a_cs] : 0.f;
+            const float bv = ok ? B[kk * b_rs + n * b_cs] : 0.f;
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(av, bv, acc, 0, 0, 0);
+        }
+        if (ks == 1) {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) {
+                const int r = m0 + 8 * (e >> 2) + 4 * half + (e & 3), c = n0 + i;
+                if (r < M && c < N) emit(r, c, acc[e]);
+            }
+        } else {
+#pragma unroll
+            for (int e = 0; e < 16; ++e) scratch[u * 1024 + e * 64 + lane] = acc[e]; // (u < WAVES here)
+        }
+    }
+    if (ks > 1) {
+        __syncthreads();
+        for (int idx = t; idx < nblk * 1024; idx += MLP_TAIL_THREADS) {
+            const int blk = idx >> 10, el = idx & 1023, e = el >> 6, l = el & 63;
+            float sum = 0.f;
+            for (int part = 0; part < ks; ++part) sum += scratch[(blk * ks + part) * 1024 + el];
+            const int r = (blk / bn) * 32 + 8 * (e >> 2) + 4 * (l >> 5) + (e & 3), c = (blk % bn) * 32 + (l & 31);
+            if (r < M && c < N) emit(r, c, sum);
+        }
+        __syncthreads(); // the scratch is free again
+    }
+}
+
 __global__ __launch_bounds__(MLP_TAIL_THREADS) void mlp_tail_kernel(const MlpTailArgs a) {
     // odd pitches: a column walk never stays on one LDS bank
     constexpr int P0 = MLP_TAIL_MAX_D0 + 1, P1 = MLP_TAIL_MAX_D1 + 1, PC = MLP_TAIL_MAX_C + 1;
@@ -283,6 +335,7 @@ __global__ __launch_bounds__(MLP_TAIL_THREADS) void mlp_tail_kernel(const MlpTai
     __shared__ float w2[MLP_TAIL_MAX_D1 * PC];  // [D1][C]
     __shared__ float z[MLP_TAIL_MAX_B * PC];    // [B][C]: logits, then their gradient
     __shared__ float bias1[MLP_TAIL_MAX_D1], bias2[MLP_TAIL_MAX_C];
+    __shared__ float scratch[MLP_TAIL_THREADS * 16]; // partial blocks of the products that cut K among the wavefronts
     const int B = a.B, D0 = a.D0, D1 = a.D1, C = a.C, t = threadIdx.x;
     for (int i = t; i < B * D0; i += MLP_TAIL_THREADS) h0[(i / D0) * P0 + i % D0] = a.h0[i];
     for (int i = t; i < D0 * D1; i += MLP_TAIL_THREADS) w1[(i / D1) * P1 + i % D1] = a.W1[i];
@@ -291,14 +344,14 @@ __global__ __launch_bounds__(MLP_TAIL_THREADS) void mlp_tail_kernel(const MlpTai
     for (int i = t; i < C; i += MLP_TAIL_THREADS) bias2[i] = a.b2[i];
     __syncthreads();
     // forward: h1 = relu(h0 . W1 + b1), logits = h1 . W2 + b2      (tenmo/net.mojo:193-201, tenmo/relu.mojo:99-118)
-    lds_product(B, D1, D0, h0, P0, 1, w1, P1, 1, [&](int m, int n, float v) {
+    lds_product_mfma(B, D1, D0, h0, P0, 1, w1, P1, 1, scratch, [&](int m, int n, float v) {
         v += bias1[n];
         v = v > 0.f ? v : 0.f;
         h1[m * P1 + n] = v;
         a.h1[m * D1 + n] = v;
     });
     __syncthreads();
-    lds_product(B, C, D1, h1, P1, 1, w2, PC, 1, [&](int m, int n, float v) {
+    lds_product_mfma(B, C, D1, h1, P1, 1, w2, PC, 1, scratch, [&](int m, int n, float v) {
         v += bias2[n];
         z[m * PC + n] = v;
         a.logits[m * C + n] = v;
@@ -330,11 +383,11 @@ __global__ __launch_bounds__(MLP_TAIL_THREADS) void mlp_tail_kernel(const MlpTai
         a.b2[t] = bias2[t] - a.lr * s;
     }
     // dW2 = h1^T . dz, g1 = (dz . W2^T) masked by h1 > 0      (tenmo/matmul.mojo:36-48, tenmo/relu.mojo:120-123)
-    lds_product(D1, C, B, h1, 1, P1, z, PC, 1, [&](int m, int n, float v) {
+    lds_product_mfma(D1, C, B, h1, 1, P1, z, PC, 1, scratch, [&](int m, int n, float v) {
         a.dW2[m * C + n] = v;
         a.W2[m * C + n] = w2[m * PC + n] - a.lr * v;
     });
-    lds_product(B, D1, C, z, PC, 1, w2, 1, PC, [&](int m, int n, float v) { g1[m * P1 + n] = h1[m * P1 + n] > 0.f ? v : 0.f; });
+    lds_product_mfma(B, D1, C, z, PC, 1, w2, 1, PC, scratch, [&](int m, int n, float v) { g1[m * P1 + n] = h1[m * P1 + n] > 0.f ? v : 0.f; });
     __syncthreads();
     if (t < D1) {
         float s = 0.f;
@@ -343,13 +396,13 @@ __global__ __launch_bounds__(MLP_TAIL_THREADS) void mlp_tail_kernel(const MlpTai
         a.b1[t] = bias1[t] - a.lr * s;
     }
     // dW1 = h0^T . g1 (with the update of W1 in global memory; the LDS copy keeps the old weights for g0)
-    lds_product(D0, D1, B, h0, 1, P0, g1, P1, 1, [&](int m, int n, float v) {
+    lds_product_mfma(D0, D1, B, h0, 1, P0, g1, P1, 1, scratch, [&](int m, int n, float v) {
         a.dW1[m * D1 + n] = v;
         a.W1[m * D1 + n] = w1[m * P1 + n] - a.lr * v;
     });
     __syncthreads(); // h0 is overwritten below
     // g0 = (g1 . W1^T) masked by h0 > 0, in place of h0
-    lds_product(B, D0, D1, g1, P1, 1, w1, 1, P1, [&](int m, int n, float v) {
+    lds_product_mfma(B, D0, D1, g1, P1, 1, w1, 1, P1, scratch, [&](int m, int n, float v) {
         v = h0[m * P0 + n] > 0.f ? v : 0.f;
         h0[m * P0 + n] = v;
         a.g0[m * D0 + n] = v;
