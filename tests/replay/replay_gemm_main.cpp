@@ -87,7 +87,10 @@ static int run_case(const std::string& spec) {
         const std::string name = f[i].substr(0, eq);
         const int value = atoi(f[i].c_str() + eq + 1);
         if (name == "check") check = value != 0;
-        else if (name == "ran") ran = f[i].substr(eq + 1); // the kernel that must have served the product (a part of its name)
+        else if (name == "ran") { // the kernel that must have served the product (a part of its launch expression; ';' stands for ',')
+            ran = f[i].substr(eq + 1);
+            for (char& c : ran) if (c == ';') c = ',';
+        }
         else knobs.push_back({name, value});
     }
     const int64_t nb = batch > 0 ? batch : 1, nbb = b_shared ? 1 : nb;

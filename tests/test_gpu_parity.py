@@ -1443,6 +1443,13 @@ def test_kstream_kernel_with_64x64_tiles(T):
     _kstream_cases(T, 3)
 
 
+def test_kstream_kernel_with_paired_k_steps(T):
+    """The same cases with the loading wavefronts issuing two K steps at a time (128x128 and 64x64 tiles; the cases with
+    a transposed-view A or an accumulating store take the unpaired kernel)."""
+    _kstream_cases(T, 4)
+    _kstream_cases(T, 5)
+
+
 def test_mlp_loss_curve_with_the_fused_tail(T, oracle):
     """The same curves with the last two layers, the loss, their backward and their update as one launch (mlp_fused_tail:
     the MNIST shape fits that launch, the other shapes of the curve test fall back to op by op)."""

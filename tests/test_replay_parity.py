@@ -24,7 +24,7 @@ pytestmark = pytest.mark.skipif(not replay_build.available(), reason="no host cl
 # too large for any CPU replay (more than 2^31 elements), or about the GPU itself
 LEFT_OUT = ["test_products_with_more_than_2_31_elements", "test_clock_probe"]
 # minutes each at CPU speed
-SLOW = ["test_stream_k", "test_kstream_kernel", "test_more_batches_than_a_grid_dimension", "test_conv2d_stream_k", "test_blocked_tile_order"]  # (test_kstream_kernel: both of them)
+SLOW = ["test_stream_k", "test_kstream_kernel", "test_more_batches_than_a_grid_dimension", "test_conv2d_stream_k", "test_blocked_tile_order"]  # (test_kstream_kernel: every test whose name starts so)
 
 
 def run_child(files, extra=()):
