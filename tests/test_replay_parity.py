@@ -29,7 +29,8 @@ SLOW = ["test_stream_k", "test_kstream_kernel", "test_more_batches_than_a_grid_d
 
 def run_child(files, extra=()):
     lib = replay_build.build_library()
-    env = dict(os.environ, TENMO_HIP_LIBRARY=lib, REPLAY_STRICT="0", PYTHONPATH=os.path.join(ROOT, "tests", "replay") + os.pathsep + os.environ.get("PYTHONPATH", ""))
+    small = {} if os.environ.get("TENMO_REPLAY_FULL") == "1" else {"TENMO_TEST_SMALL": "1"}  # a few tests shrink their largest cases at CPU speed
+    env = dict(os.environ, **small, TENMO_HIP_LIBRARY=lib, REPLAY_STRICT="0", PYTHONPATH=os.path.join(ROOT, "tests", "replay") + os.pathsep + os.environ.get("PYTHONPATH", ""))
     left_out = LEFT_OUT + ([] if os.environ.get("TENMO_REPLAY_FULL") == "1" else SLOW)
     deselect = " and ".join("not " + name for name in left_out)
     cmd = [sys.executable, "-m", "pytest", "-p", "torch_on_host", "-m", "gpu", "-x", "-q", "-k", deselect, "-p", "no:cacheprovider"] + list(extra) + files
