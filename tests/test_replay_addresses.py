@@ -236,7 +236,7 @@ def test_adjacent_operators(exe):
 def test_randomized_products(exe):
     """Seeded random shapes (small extents, the tile widths and their neighbours, anything up to 400), layouts including
     generic strides, batches with and without a shared B, accumulate, and kernel choices (every tile, K slices, stream-K, the
-    short-reduction and the K-stream kernel forced on): whatever the dispatch makes of them must stay in bounds and be right.
+    short-reduction and the K-stream kernel in its variants forced on): whatever the dispatch makes of them must stay in bounds and be right.
     (TENMO_REPLAY_FUZZ=<n> runs n cases instead of 150.)"""
     import random
 
@@ -264,7 +264,7 @@ def test_randomized_products(exe):
         elif r < 0.6:
             knobs["gemm_smallk"] = 1
         elif r < 0.75:
-            knobs["gemm_panel"] = 1
+            knobs["gemm_panel"] = rnd.choice([1, 1, 3, 4, 5])
         cases.append(case(extent(400), extent(400), extent(300), rnd.choice("nntg"), rnd.choice("nntg"), batch,
                           rnd.choice([0, 0, 1]) if batch else 0, rnd.choice([0, 0, 1]), **knobs))
     for start in range(0, len(cases), 75):
