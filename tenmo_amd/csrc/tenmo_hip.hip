@@ -1857,6 +1857,7 @@ struct tenmo_mlp {
     float g_lr = 0.f;
     float* g_loss = nullptr;
     float* g_ws = nullptr;      // library scratch pointer the captured kernels hold
+    int g_fused = 0;            // mlp_fused_tail level the capture was made at
 };
 
 static unsigned grid_for(int64_t n) { return (unsigned)std::max<int64_t>(1, std::min<int64_t>((n + 255) / 256, 4096)); }
@@ -2042,7 +2043,7 @@ int tenmo_hip_mlp_step_graph(tenmo_mlp* m, const float* x, const int32_t* y, int
     float* ws;
     if (int rc = workspace(1, &ws)) return rc; // scratch must exist before capture: no allocation may happen inside it
     // the captured kernels hold the scratch pointer: a capture made before the scratch buffer grew is stale
-    for (int attempt = 0; !m->exec || m->g_batch != B || m->g_lr != lr || m->g_loss != loss_out || m->g_ws != ws; ++attempt) {
+    for (int attempt = 0; !m->exec || m->g_batch != B || m->g_lr != lr || m->g_loss != loss_out || m->g_ws != ws || m->g_fused != S.mlp_fused_tail; ++attempt) {
         if (m->exec) { HIP_TRY(hipStreamSynchronize(S.stream)); HIP_TRY(hipGraphExecDestroy(m->exec)); m->exec = nullptr; }
         HIP_TRY(hipStreamBeginCapture(S.stream, hipStreamCaptureModeThreadLocal));
         S.capturing = true; S.ws_wanted = 0;
@@ -2063,7 +2064,7 @@ int tenmo_hip_mlp_step_graph(tenmo_mlp* m, const float* x, const int32_t* y, int
         const hipError_t ei = hipGraphInstantiate(&m->exec, graph, nullptr, nullptr, 0);
         (void)hipGraphDestroy(graph);
         if (ei != hipSuccess) { m->exec = nullptr; return fail(TENMO_ERR_HIP, "hipGraphInstantiate failed: %s", hipGetErrorString(ei)); }
-        m->g_batch = B; m->g_lr = lr; m->g_loss = loss_out; m->g_ws = ws;
+        m->g_batch = B; m->g_lr = lr; m->g_loss = loss_out; m->g_ws = ws; m->g_fused = S.mlp_fused_tail;
     }
     HIP_TRY(hipGraphLaunch(m->exec, S.stream));
     return finish(sync);

@@ -1482,6 +1482,16 @@ def test_mlp_loss_curve_with_the_fused_tail(T, oracle):
                 (dWg, dbg), (dWc, dbc) = gpu.grads(l), cpu.grads(l)
                 assert rel_fro(dWg, dWc) <= 1e-4 and rel_fro(dbg, dbc) <= 1e-4, (batch, dims, l)
             assert rel_fro(gpu.forward(x), cpu.forward(x)) <= 1e-5, (batch, dims)
+        # the captured step holds the fused launches too, and a change of the knob captures anew
+        dims = [784, 128, 32, 10]
+        Ws, bs = R.xavier_mlp(dims, 13)
+        eager, graph = MLP(dims, Ws, bs, 64), MLP(dims, Ws, bs, 64)
+        for step in range(6):
+            if step == 3:
+                T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
+            x, y = R.mnist_like_batch(64, 13, step)
+            assert eager.step(x, y, 0.01) == graph.step(x, y, 0.01, graph=True), step
+        np.testing.assert_array_equal(eager.params(0)[0], graph.params(0)[0])
     finally:
         T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
 
