@@ -393,7 +393,7 @@ __global__ __launch_bounds__(CE_THREADS) void ce_softmax_flat_kernel(const float
         col += st.pass_cols; row += st.pass_rows;
         if (col >= C) { col -= C; ++row; }
     }
-    if (blockIdx.x == 0 && threadIdx.x < (int)(total & 3)) { // the last total % 4 elements lie in the last row
+    if (blockIdx.x == 0 && threadIdx.x < (unsigned)(total & 3)) { // the last total % 4 elements lie in the last row
         const int64_t e = (total & ~(int64_t)3) + threadIdx.x;
         softmax[e] = __expf(logits[e] - stats[M - 1].max) * stats[M - 1].inv_sum;
     }
@@ -575,7 +575,7 @@ __global__ __launch_bounds__(CE_THREADS) void ce_backward_flat_kernel(const CeBa
         col += st.pass_cols; row += st.pass_rows;
         if (col >= a.C) { col -= a.C; ++row; }
     }
-    if (blockIdx.x == 0 && threadIdx.x < (int)(total & 3)) { // the last total % 4 elements lie in the last row
+    if (blockIdx.x == 0 && threadIdx.x < (unsigned)(total & 3)) { // the last total % 4 elements lie in the last row
         const int64_t e = (total & ~(int64_t)3) + threadIdx.x, rl = a.M - 1;
         const float v = value(a.softmax[e], e - rl * a.C, (int64_t)target[rl], a.reduction == 0 ? a.upstream[rl] : scale_all);
         a.grad[e] = a.accumulate ? a.grad[e] + v : v;
