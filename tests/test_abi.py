@@ -128,3 +128,32 @@ def test_conv_padding_parse_matches_reference_shapes(golden):
         w_out = (image.shape[3] + left + right - dkw) // kw["stride"] + 1
         want = case.get("expect_shape") or list(__import__("numpy").array(case["expect"]).shape)
         assert [image.shape[0], kernel.shape[0], h_out, w_out] == want, case["name"]
+
+
+def test_mojo_glue_matches_the_header():
+    """integration/mojo/hiphandle.mojo cannot be compiled here; what can be checked is that every symbol it looks up is
+    declared in include/tenmo_hip.h and that the function type it is looked up with has as many parameters as the C
+    prototype (a maintainer's first build would otherwise fail, or worse, call with a shifted argument list)."""
+    header = re.sub(r"/\*.*?\*/", "", open(os.path.join(ROOT, "include", "tenmo_hip.h")).read(), flags=re.S)
+    glue = open(os.path.join(ROOT, "integration", "mojo", "hiphandle.mojo")).read()
+
+    def top_level_commas(args):
+        depth = count = 0
+        for ch in args:
+            depth += ch in "([" 
+            depth -= ch in ")]"
+            count += ch == "," and depth == 0
+        return count
+
+    def arity(args):
+        args = args.strip()
+        return 0 if args in ("", "void") else top_level_commas(args) + 1
+
+    c_arity = {m.group(1): arity(m.group(2)) for m in re.finditer(r"\b(tenmo_hip_[a-z0-9_]+|cblas_sgemm)\s*\(([^;{]*?)\)\s*;", header, re.S)}
+    types = {m.group(1): arity(m.group(2)) for m in re.finditer(r"comptime\s+(\w+_FN)\s*=\s*def\((.*?)\)\s*thin", glue, re.S)}
+    lookups = re.findall(r"get_function\[(\w+)\]\(\"(\w+)\"\)", glue)
+    assert len(lookups) >= 15 and len(types) >= 15
+    for fn_type, symbol in lookups:
+        assert symbol in c_arity, f"{symbol}: looked up by the Mojo glue, not declared in the header"
+        assert fn_type in types, fn_type
+        assert types[fn_type] == c_arity[symbol], f"{symbol}: {c_arity[symbol]} parameters in C, {types[fn_type]} in {fn_type}"
