@@ -411,9 +411,12 @@ __global__ __launch_bounds__(COLS_THREADS) void cols_shift_kernel(const ColsArgs
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int u = 0; u < U; ++u) {
-                if (kk + u >= vlen) m[u] = f32x4{0.f, 0.f, 0.f, 0.f};
+                // (skipped, not multiplied by zero: xs[.][vlen] is the vector's real last value when the matrix's last row is
+                // done apart below, and 0 x inf would put a NaN where the reference has an infinity)
+                if (kk + u < vlen) {
 #pragma unroll
-                for (int r = 0; r < R; ++r) acc[u & 3][r] += m[u] * xs[r][kk + u];
+                    for (int r = 0; r < R; ++r) acc[u & 3][r] += m[u] * xs[r][kk + u];
+                }
             }
         }
         if (vlen < len) { // the matrix's last row: element by element, bounds-checked

@@ -1530,6 +1530,57 @@ def test_resident_left_operand_kernel(T):
         L.tenmo_hip_set_tuning(b"gemm_resident", 0)
 
 
+def test_non_finite_values_propagate_as_in_ieee(T):
+    """An infinity or a NaN in an operand must come out where, and as what, the reference's plain loops put it: in the
+    rows / columns it touches, as +inf, -inf or NaN — never a NaN from a padding lane's 0 x inf.  Poisoned positions are the
+    ones tails and clamps handle specially (first and last k, last row, last column) in every product kernel: the GEMM
+    tiles with K tails, K slices, stream-K, the short-reduction, K-stream and resident-A kernels, mv / vm / skinny products on
+    aligned and odd row pitches."""
+    import ctypes as C
+    import torch
+    L, lib = T.lib.load(), T.lib
+    rng = np.random.default_rng(83)
+
+    def classes(x):
+        return np.where(np.isnan(x), 2, np.where(np.isposinf(x), 1, np.where(np.isneginf(x), -1, 0)))
+
+    def product(a, b, ta, tb):
+        M, K = a.shape
+        N = b.shape[1]
+        A = torch.from_numpy(np.ascontiguousarray(a.T if ta else a)).cuda()
+        B = torch.from_numpy(np.ascontiguousarray(b.T if tb else b)).cuda()
+        out = torch.zeros((M, N), device="cuda")
+        a_rs, a_cs = (1, M) if ta else (K, 1)
+        b_rs, b_cs = (1, K) if tb else (N, 1)
+        lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, a_rs, a_cs, B.data_ptr(), 0, b_rs, b_cs, out.data_ptr(), M, N, K, 0, None, None, None, 0, 1))
+        return out.cpu().numpy()
+
+    cases = [(70, 90, 37, (), False, False), (70, 92, 37, (), True, True), (130, 260, 100, (("gemm_panel", 1),), False, False),
+             (130, 260, 52, (("gemm_smallk", 1),), False, True), (130, 260, 100, (("gemm_panel", 5),), False, True),
+             (256, 3200, 100, (("gemm_resident", 1),), False, False), (100, 3200, 250, (("gemm_resident", 2),), True, False),
+             (200, 200, 333, (("gemm_splitk", 3),), False, False), (300, 500, 333, (("gemm_streamk", 1), ("gemm_tile", 1)), False, False),
+             (4, 3000, 77, (), False, False), (1, 2049, 515, (), False, False), (3, 2051, 1030, (("cols_join", 1),), False, False),
+             (8, 4099, 200, (), False, False), (70, 1, 300, (), False, True), (515, 1, 1030, (), True, False), (33, 1, 6000, (), True, False)]
+    for M, N, K, knobs, ta, tb in cases:
+        poisons = [("a", (M // 2, K - 1), np.inf), ("a", (0, 0), -np.inf), ("b", (K - 1, N // 2), np.inf), ("b", (0, N - 1), np.nan), ("a", (M - 1, K // 2), np.inf)]
+        for which, at, value in poisons:
+            a = rng.standard_normal((M, K)).astype(np.float32)
+            b = rng.standard_normal((K, N)).astype(np.float32)
+            (a if which == "a" else b)[at] = value
+            for name, v in knobs:
+                L.tenmo_hip_set_tuning(name.encode(), v)
+            try:
+                got = product(a, b, ta, tb)
+            finally:
+                for name, _ in knobs:
+                    L.tenmo_hip_set_tuning(name.encode(), -1)
+            with np.errstate(all="ignore"):
+                ref = a.astype(np.float64) @ b.astype(np.float64)
+            assert np.array_equal(classes(got), classes(ref)), (M, N, K, knobs, ta, tb, which, at, value)
+            finite = np.isfinite(ref)
+            assert np.allclose(got[finite], ref[finite], rtol=1e-4, atol=1e-4), (M, N, K, knobs, which, at)
+
+
 def test_column_kernels_join_slices_in_the_launch(T):
     """vm, mv on a transposed view, skinny and batched skinny products with the K slices added by the last workgroup of
     the streaming launch (cols_join) instead of a second launch: the same bits as the two-launch result — the slices are
