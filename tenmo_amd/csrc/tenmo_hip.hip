@@ -410,11 +410,12 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         };
         // (Reductions of a single K step, K <= 16, stay with the ordinary kernel for now: a timing run of [8192,16].[16,8192]
         // through this kernel faulted — an undeclared SCC clobber of the masked direct load, since fixed (gfx950_asm.hpp) — and
-        // the one-step instantiations come back once the fix has been confirmed on a GPU.)
+        // the one-step instantiations come back once the fix has been confirmed on a GPU.  Until then the automatic choice
+        // is also limited to K % 16 == 0, which never takes the masked load; a ragged K reaches it only through the knob.)
         const bool can = K > GEMM_BK && K <= 64 && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum &&
                          N < (int64_t(1) << 29) && tiles64 <= 0x7fffffffLL;
         const bool want = S.force_smallk > 0 || (S.force_smallk < 0 && S.force_tile < 0 && S.force_splitk <= 0 && S.force_streamk <= 0 &&
-                                                  splits == 1 && sk_wpc == 0 && tiles64 >= 2048 && K <= 64);
+                                                  splits == 1 && sk_wpc == 0 && tiles64 >= 2048 && K <= 64 && K % GEMM_BK == 0);
         if (can && want) {
             g.tiles_m = (int32_t)tm; g.tiles_n = (int32_t)tn;
             g.k_splits = 1; g.k_per_split = K; g.partial = nullptr;

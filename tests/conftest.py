@@ -30,6 +30,13 @@ def pytest_collection_modifyitems(config, items):
     gpu_items = [it for it in items if it.get_closest_marker("gpu")]
     if not gpu_items:
         return
+    # The GPU tests are parity evidence for the HIP library of this tree and nothing else: another library put in its
+    # place through TENMO_HIP_LIBRARY is accepted only together with the host stand-in for torch's device (the CPU
+    # replay of the kernels, tests/replay), which says what it is.
+    override = os.environ.get("TENMO_HIP_LIBRARY")
+    in_tree = os.path.join(ROOT, "tenmo_amd", "libtenmo_hip.so")
+    if override and os.path.realpath(override) != os.path.realpath(in_tree) and not config.pluginmanager.has_plugin("torch_on_host"):
+        raise pytest.UsageError("TENMO_HIP_LIBRARY=%s: the gpu tests run on %s only" % (override, in_tree))
     reason = _gpu_unavailable_reason()
     if reason:
         skip = pytest.mark.skip(reason="gpu test: " + reason)

@@ -45,7 +45,7 @@ def test_one_json_line_with_every_field():
     assert cpu["kind"] == "port" and cpu["unit"] == "TFLOP/s" and cpu["cores"] >= 1 and cpu["value"] > 0 and cpu["sample"]
     extra = out["extra"]
     assert extra["rows"] == [] and "mlp_step_ms_gpu" in extra and "mlp_step_ms_gpu_fused_tail" in extra and "mlp_step_ms_gpu_fused_tail_and_first" in extra and "mlp_step_ms_cpu" in extra
-    assert extra["mlp_max_abs_loss_diff_first10"] <= 1e-4
+    assert extra["mlp_max_abs_loss_diff"] <= 1e-4 and extra["mlp_parity_steps"] >= 20 and out["gates"]["mlp_loss_ok"] and out["gates"]["rel_err_ok"]
     assert extra["sweep"] == [{"tune": {"gemm_panel": 0}, "rows": []}, {"tune": {"gemm_panel": 1, "gemm_smallk": 0}, "rows": []}]
     assert not [k for k in extra if k.endswith("_error")], extra
 

@@ -25,9 +25,34 @@ def build_gpu_driver() -> str:
     os.makedirs(OUT, exist_ok=True)
     exe = os.path.join(OUT, "c_abi_driver")
     lib_dir = os.path.join(ROOT, "tenmo_amd")
+    # the run path is relative to the program ($ORIGIN = tests/_build), so the prebuilt program finds the library
+    # wherever the tree is copied to
     subprocess.run(["gcc"] + CFLAGS + [SRC, "-L", lib_dir, "-ltenmo_hip", "-L", "/opt/rocm/lib", "-lamdhip64", "-lm",
-                                       "-Wl,-rpath," + lib_dir, "-Wl,-rpath,/opt/rocm/lib", "-o", exe], check=True, capture_output=True, text=True)
+                                       "-Wl,-rpath,$ORIGIN/../../tenmo_amd", "-Wl,-rpath,/opt/rocm/lib", "-o", exe],
+                   check=True, capture_output=True, text=True)
     return exe
+
+
+def test_prebuilt_driver_finds_the_library_in_a_relocated_tree(tmp_path):
+    """The program is built in one place and run in a copy of the tree somewhere else: its run path must not name
+    the place it was built in."""
+    import shutil
+
+    lib = os.path.join(ROOT, "tenmo_amd", "libtenmo_hip.so")
+    if not os.path.exists(lib):
+        pytest.skip("libtenmo_hip.so is not built")
+    exe = build_gpu_driver()
+    dyn = subprocess.run(["readelf", "-d", exe], capture_output=True, text=True).stdout
+    assert ROOT not in dyn and "$ORIGIN/../../tenmo_amd" in dyn, dyn
+    tree = tmp_path / "elsewhere" / "repo"
+    os.makedirs(tree / "tests" / "_build")
+    os.makedirs(tree / "tenmo_amd")
+    shutil.copy(exe, tree / "tests" / "_build" / "c_abi_driver")
+    shutil.copy(lib, tree / "tenmo_amd" / "libtenmo_hip.so")
+    env = {k: v for k, v in os.environ.items() if k != "LD_LIBRARY_PATH"}
+    out = subprocess.run(["ldd", str(tree / "tests" / "_build" / "c_abi_driver")], capture_output=True, text=True, env=env).stdout
+    line = [ln for ln in out.splitlines() if "libtenmo_hip.so" in ln]
+    assert line and str(tree / "tenmo_amd" / "libtenmo_hip.so") in os.path.normpath(line[0].split("=>")[1].split("(")[0].strip()), out
 
 
 def test_header_is_c11_and_every_symbol_is_referenced(tmp_path):
@@ -58,5 +83,8 @@ def test_driver_runs_on_the_gpu():
     exe = os.path.join(OUT, "c_abi_driver")
     if not os.path.exists(exe):
         exe = build_gpu_driver()
-    run = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    # belt and braces: the library of THIS tree first on the loader's path as well
+    env = dict(os.environ)
+    env["LD_LIBRARY_PATH"] = os.path.join(ROOT, "tenmo_amd") + os.pathsep + env.get("LD_LIBRARY_PATH", "")
+    run = subprocess.run([exe], capture_output=True, text=True, timeout=300, env=env)
     assert run.returncode == 0 and "c_abi_driver: ok" in run.stdout, run.stdout + run.stderr
