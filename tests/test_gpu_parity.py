@@ -172,39 +172,6 @@ def test_short_reduction_kernel(T, smallk):
         L.tenmo_hip_set_tuning(b"gemm_smallk", -1)
 
 
-@pytest.mark.parametrize("smallk", [1, 0])
-def test_short_reduction_kernel_layouts_and_k_tails(T, smallk):
-    """The same kernel over every operand layout (row-major and transposed views of A and of B) and reductions that
-    are no multiple of 16 (zero-filled K tail; a K-major operand then needs K % 4 == 0, other K fall back to the
-    ordinary kernel), whole and ragged tiles, batches, accumulation; against fp64."""
-    import torch
-    L, lib = T.lib.load(), T.lib
-    gen = torch.Generator(device="cuda")
-    gen.manual_seed(29)
-    cases = [((), 64, 64, 16, 0), ((), 128, 192, 100, 0), ((3,), 100, 132, 36, 0), ((2, 3), 256, 68, 64, 1), ((5,), 64, 64, 112, 0),
-             ((2,), 332, 776, 20, 1), ((), 1000, 1000, 7, 0), ((4,), 72, 52, 84, 0), ((), 256, 5000, 100, 0), ((2,), 512, 512, 50, 1),
-             ((9,), 320, 1024, 12, 0), ((), 64, 8192, 104, 0), ((), 130, 70, 33, 0)]
-    try:
-        L.tenmo_hip_set_tuning(b"gemm_smallk", smallk)
-        for bshape, M, N, K, acc in cases:
-            for ta in (False, True):
-                for tb in (False, True):
-                    A = torch.randn((*bshape, *((K, M) if ta else (M, K))), generator=gen, device="cuda")
-                    B = torch.randn((*bshape, *((N, K) if tb else (K, N))), generator=gen, device="cuda")
-                    Cc = torch.randn((*bshape, M, N), generator=gen, device="cuda")
-                    a_rs, a_cs = (1, M) if ta else (K, 1)
-                    b_rs, b_cs = (1, K) if tb else (N, 1)
-                    ref = (A.transpose(-1, -2) if ta else A).double() @ (B.transpose(-1, -2) if tb else B).double() + (Cc.double() if acc else 0)
-                    ab = [A.stride(i) for i in range(len(bshape))]
-                    bb = [B.stride(i) for i in range(len(bshape))]
-                    lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, a_rs, a_cs, B.data_ptr(), 0, b_rs, b_cs, Cc.data_ptr(), M, N, K, len(bshape),
-                                                   lib.i64(bshape), lib.i64(ab), lib.i64(bb), acc, 1))
-                    err = float((Cc.double() - ref).norm() / ref.norm())
-                    assert err <= RTOL_FRO, (smallk, bshape, M, N, K, acc, ta, tb, err)
-    finally:
-        L.tenmo_hip_set_tuning(b"gemm_smallk", -1)
-
-
 def test_kstream_kernel(T):
     _kstream_cases(T, 1)
 
@@ -1392,144 +1359,6 @@ def test_clock_probe(T):
 # ---- written after the last GPU run: checked on the CPU replay only so far (kept late in the file so that a surprise here
 # hides as little as possible of the rest under pytest -x) ----
 
-@pytest.mark.parametrize("fold", [1, 0, -1])
-def test_backward_of_broadcast_parents(T, oracle, fold):
-    """Gradients of parents that were broadcast over batch dimensions (tenmo/matmul.mojo:115-135: the batched product, then
-    sum_over_broadcasted_axes): a shared A, a shared B whose partner's rows do not stack, partially broadcast batches on both
-    sides, transposed views, tiles that are whole and ragged.  With the sum folded into the GEMM launch (1), with the
-    batched gradient materialised and reduced (0) and with the automatic choice; against the oracle, twice (the second
-    backward accumulates)."""
-    L = T.lib.load()
-    rng = np.random.default_rng(83 + fold)
-    cases = [((70, 33), (5, 33, 41), False, False),          # A shared by 5 batches
-             ((2, 1, 66, 20), (1, 3, 20, 130), False, False),  # each side broadcast along one batch dim
-             ((3, 1, 40, 24), (4, 24, 36), False, False),      # A: one dim kept, one reduced; B: reduced over the leading dim
-             ((130, 64), (2, 3, 64, 70), True, False),         # A a transposed view
-             ((4, 50, 32), (32, 260), False, True),            # B a transposed view, shared
-             ((1, 300, 16), (6, 16, 200), False, False)]
-    try:
-        L.tenmo_hip_set_tuning(b"fold_reduce", fold)
-        for sa, sb, ta, tb in cases:
-            a = rng.standard_normal(sa[:-2] + (sa[-1], sa[-2]) if ta else sa, dtype=np.float32)
-            b = rng.standard_normal(sb[:-2] + (sb[-1], sb[-2]) if tb else sb, dtype=np.float32)
-            A, B = T.Tensor.from_numpy(a, True), T.Tensor.from_numpy(b, True)
-            Av, Bv = (A.transpose(-1, -2) if ta else A), (B.transpose(-1, -2) if tb else B)
-            al, bl = (np.swapaxes(a, -1, -2) if ta else a), (np.swapaxes(b, -1, -2) if tb else b)
-            out = Av.matmul(Bv)
-            seed = rng.standard_normal(out.shape(), dtype=np.float32)
-            out.backward(T.Tensor.from_numpy(seed), retain_graph=True)
-            gA, gB = oracle.matmul_backward(al, bl, seed)
-            assert rel_fro(Av.grad(), gA) <= 2 * RTOL_FRO, (fold, sa, sb)
-            assert rel_fro(Bv.grad(), gB) <= 2 * RTOL_FRO, (fold, sa, sb)
-            out.backward(T.Tensor.from_numpy(seed))
-            assert rel_fro(Av.grad(), 2 * gA) <= 2 * RTOL_FRO, (fold, sa, sb)
-            assert rel_fro(Bv.grad(), 2 * gB) <= 2 * RTOL_FRO, (fold, sa, sb)
-        # a batch-strided A (its matrices do not stack at a constant row pitch) against a shared B: dB through the fold
-        big = rng.standard_normal((6, 24, 20), dtype=np.float32)
-        w = rng.standard_normal((20, 68), dtype=np.float32)
-        sub = big[::2]
-        A = as_strided_tensor(T, sub, requires_grad=True)
-        W = T.Tensor.from_numpy(w, True)
-        out = A.matmul(W)
-        seed = rng.standard_normal(out.shape(), dtype=np.float32)
-        out.backward(T.Tensor.from_numpy(seed))
-        gA, gW = oracle.matmul_backward(sub, w, seed)
-        assert rel_fro(W.grad(), gW) <= 2 * RTOL_FRO and rel_fro(A.grad(), gA) <= 2 * RTOL_FRO
-    finally:
-        L.tenmo_hip_set_tuning(b"fold_reduce", -1)
-
-
-def test_kstream_kernel_with_64x64_tiles(T):
-    """The same cases through the kernel's 64x64-tile variant (a ring of eight stages; two operand fetches behind an MFMA
-    where an operand is MN-major)."""
-    _kstream_cases(T, 3)
-
-
-def test_kstream_kernel_with_paired_k_steps(T):
-    """The same cases with the loading wavefronts issuing two K steps at a time (128x128 and 64x64 tiles; the cases with
-    a transposed-view A or an accumulating store take the unpaired kernel)."""
-    _kstream_cases(T, 4)
-    _kstream_cases(T, 5)
-
-
-def test_mlp_loss_curve_with_the_fused_tail(T, oracle):
-    """The same curves with the last two layers, the loss, their backward and their update as one launch (mlp_fused_tail:
-    the MNIST shape fits that launch, the other shapes of the curve test fall back to op by op)."""
-    from tenmo_amd import rng as R
-    from tenmo_amd.net import MLP
-
-    for level in (1, 2, 3):  # 2: the first layer's weight gradient and its update as one launch as well; 3: its forward too
-        T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", level)
-        try:
-            _mlp_loss_curve(T, oracle, R, MLP)
-        finally:
-            T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
-    # every fused launch on ragged shapes: inputs that end inside an 8-wide k chunk in each way, widths that are no
-    # multiples of the 32x32 blocks, batches that do not fill them
-    rs = np.random.default_rng(71)
-    T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 3)
-    try:
-        for batch, dims in ((37, [257, 77, 33, 7]), (64, [1001, 128, 64, 32]), (1, [262, 5, 3, 2]), (100, [518, 130, 40, 9]), (33, [259, 97, 4])):
-            Ws, bs = R.xavier_mlp(dims, 11)
-            gpu, cpu = MLP(dims, Ws, bs, batch), oracle.MLP(dims, Ws, bs, batch)
-            for step in range(3):
-                x = rs.standard_normal((batch, dims[0])).astype(np.float32)
-                y = rs.integers(0, dims[-1], batch).astype(np.int32)
-                assert abs(gpu.step(x, y, 0.05) - cpu.step(x, y, 0.05)) <= 1e-4, (batch, dims, step)
-            for l in range(len(dims) - 1):
-                (Wg, bg), (Wc, bc) = gpu.params(l), cpu.params(l)
-                assert rel_fro(Wg, Wc) <= 1e-5 and np.abs(bg - bc).max() <= 1e-5, (batch, dims, l)
-                (dWg, dbg), (dWc, dbc) = gpu.grads(l), cpu.grads(l)
-                assert rel_fro(dWg, dWc) <= 1e-4 and rel_fro(dbg, dbc) <= 1e-4, (batch, dims, l)
-            assert rel_fro(gpu.forward(x), cpu.forward(x)) <= 1e-5, (batch, dims)
-        # the captured step holds the fused launches too, and a change of the knob captures anew
-        dims = [784, 128, 32, 10]
-        Ws, bs = R.xavier_mlp(dims, 13)
-        eager, graph = MLP(dims, Ws, bs, 64), MLP(dims, Ws, bs, 64)
-        for step in range(6):
-            if step == 3:
-                T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
-            x, y = R.mnist_like_batch(64, 13, step)
-            assert eager.step(x, y, 0.01) == graph.step(x, y, 0.01, graph=True), step
-        np.testing.assert_array_equal(eager.params(0)[0], graph.params(0)[0])
-    finally:
-        T.lib.load().tenmo_hip_set_tuning(b"mlp_fused_tail", 0)
-
-
-def test_resident_left_operand_kernel(T):
-    """The kernel that keeps its tile row of A in LDS for all of K and streams B alone (gemm_resident knob: tiles of 128x64
-    and of 64x64), forced on: the CBOW logits and their gradient at full size, K tails, a row-major and a transposed-view A,
-    ragged last tile rows and column blocks, several tile rows, a result of fewer tiles than workgroups; and, with the knob
-    still on, what the kernel does not take (falls through to the others).  Against fp64; the element behind the result
-    stays untouched.  (The same launches run address by address on the CPU in test_replay_addresses.py.)"""
-    import torch
-    L, lib = T.lib.load(), T.lib
-    gen = torch.Generator(device="cuda")
-    gen.manual_seed(37)
-    cases = [(256, 50000, 100), (100, 50000, 256), (128, 2052, 32), (64, 4096, 20), (36, 3000, 112), (200, 2500, 132), (1024, 6400, 48),
-             (256, 128, 100), (256, 3200, 248), (128, 3200, 272), (128, 3202, 64)]
-    try:
-        for knob in (1, 2):
-            L.tenmo_hip_set_tuning(b"gemm_resident", knob)
-            for M, N, K in cases:
-                for ta in (False, True):
-                    for tb, acc in ((False, 0), (True, 0), (False, 1)) if (M, N, K) == (128, 2052, 32) else ((False, 0),):
-                        A = torch.randn(((K, M) if ta else (M, K)), generator=gen, device="cuda")
-                        B = torch.randn(((N, K) if tb else (K, N)), generator=gen, device="cuda")
-                        out = torch.randn((M * N + 1,), generator=gen, device="cuda")
-                        guard = float(out[-1])
-                        a_rs, a_cs = (1, M) if ta else (K, 1)
-                        b_rs, b_cs = (1, K) if tb else (N, 1)
-                        ref = (A.t() if ta else A).double() @ (B.t() if tb else B).double() + (out[:-1].view(M, N).double() if acc else 0)
-                        lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, a_rs, a_cs, B.data_ptr(), 0, b_rs, b_cs, out.data_ptr(), M, N, K, 0,
-                                                       None, None, None, acc, 1))
-                        err = float((out[:-1].view(M, N).double() - ref).norm() / ref.norm())
-                        assert err <= RTOL_FRO, (knob, M, N, K, ta, tb, acc, err)
-                        assert float(out[-1]) == guard, (knob, M, N, K, ta, tb, acc)
-    finally:
-        L.tenmo_hip_set_tuning(b"gemm_resident", 0)
-
-
 def test_non_finite_values_propagate_as_in_ieee(T):
     """An infinity or a NaN in an operand must come out where, and as what, the reference's plain loops put it: in the
     rows / columns it touches, as +inf, -inf or NaN — never a NaN from a padding lane's 0 x inf.  Poisoned positions are the
@@ -1741,64 +1570,6 @@ def test_non_finite_values_in_a_convolution(T, oracle):
                     # padding zero is NaN here, where the reference never forms that product.  Border positions only.
                     differ &= ~np.isnan(g)
                 assert not differ.any(), "%s gradient, case %r" % (what, case)
-
-
-def test_column_kernels_join_slices_in_the_launch(T):
-    """vm, mv on a transposed view, skinny and batched skinny products with the K slices added by the last workgroup of
-    the streaming launch (cols_join) instead of a second launch: the same bits as the two-launch result — the slices are
-    added in the same order — call after call (the arrival counters must be back at zero), with `+=`, and through the
-    allocation-free entry."""
-    import ctypes as C
-    from tenmo_amd import _lib
-    L = _lib.load()
-    rng = np.random.default_rng(67)
-
-    def both(fn):
-        apart = fn()
-        L.tenmo_hip_set_tuning(b"cols_join", 1)
-        try:
-            joined, again = fn(), fn()
-        finally:
-            L.tenmo_hip_set_tuning(b"cols_join", 0)
-        assert np.array_equal(apart, joined) and np.array_equal(apart, again)
-        return joined
-
-    for (m, k, n) in [(1, 4096, 4096), (4, 768, 50257), (3, 2000, 3001), (8, 1024, 2048), (1, 16384, 1024), (2, 515, 1030), (1, 100, 50000)]:
-        a = rng.standard_normal((m, k), dtype=np.float32)
-        b = rng.standard_normal((k, n), dtype=np.float32)
-        A, B = T.Tensor.from_numpy(a), T.Tensor.from_numpy(b)
-        got = both(lambda: A.matmul(B, track_grad=False).to_numpy())
-        assert rel_fro(got, ref_matmul64(a, b)) <= RTOL_FRO, (m, k, n)
-        if m == 1:
-            v = T.Tensor.from_numpy(a[0])
-            got = both(lambda: v.matmul(B, track_grad=False).to_numpy())                      # vector x matrix
-            assert rel_fro(got, ref_matmul64(a, b)[0]) <= RTOL_FRO, ("vm", k, n)
-            Bt = T.Tensor.from_numpy(b).transpose()                                           # [n, k] view: mv through the column kernel
-            got = both(lambda: Bt.matmul(v, track_grad=False).to_numpy())
-            assert rel_fro(got, ref_matmul64(a, b)[0]) <= RTOL_FRO, ("mv of a transposed view", k, n)
-    # batches of a right operand with an odd pitch
-    a = rng.standard_normal((2, 768), dtype=np.float32)
-    b = rng.standard_normal((4, 768, 2503), dtype=np.float32)
-    A, B = T.Tensor.from_numpy(a), T.Tensor.from_numpy(b)
-    assert rel_fro(both(lambda: A.matmul(B, track_grad=False).to_numpy()), ref_matmul64(a, b)) <= RTOL_FRO
-    # += and the allocation-free entry
-    a = rng.standard_normal((1, 3000), dtype=np.float32)
-    b = rng.standard_normal((3000, 5000), dtype=np.float32)
-    c0 = rng.standard_normal((1, 5000), dtype=np.float32)
-    A, B = T.Tensor.from_numpy(a), T.Tensor.from_numpy(b)
-
-    def accumulate(entry):
-        out = T.Tensor.from_numpy(c0.copy())
-        if entry == "gemm":
-            _lib.check(L.tenmo_hip_gemm_f32(A.buffer.data_ptr(), 0, 3000, 1, B.buffer.data_ptr(), 0, 5000, 1, out.buffer.data_ptr(),
-                                            1, 5000, 3000, 0, None, None, None, 1, 1))
-        else:
-            _lib.check(L.tenmo_hip_vm_f32_noalloc(A.buffer.data_ptr(), 0, 1, B.buffer.data_ptr(), 0, 5000, 1, out.buffer.data_ptr(),
-                                                  3000, 5000, 0, None, None, None, 1, 1))
-        return out.to_numpy()
-
-    for entry in ("gemm", "noalloc"):
-        assert rel_fro(both(lambda: accumulate(entry)), c0.astype(np.float64) + ref_matmul64(a, b)) <= RTOL_FRO, entry
 
 
 def test_zz_graph_capture_grows_scratch(T, oracle):

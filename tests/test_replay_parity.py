@@ -1,6 +1,6 @@
 """The GPU parity tests, run on the CPU against the replay build of the library.
 
-tests/test_gpu_parity.py and tests/test_zz_no_alloc.py drive every entry point of the C ABI through the host mirror and
+tests/test_gpu_parity.py, tests/test_zzz_gpu_first_run.py and tests/test_zz_no_alloc.py drive every entry point of the C ABI through the host mirror and
 compare with the oracle and with float64.  Here the same test functions run in a child pytest process in which the
 library is the CPU replay (tests/replay: the kernel sources compiled for the host, launches executed thread by thread)
 and torch's "cuda" allocations are redirected to host memory (tests/replay/torch_on_host.py).  What this proves without
@@ -49,6 +49,10 @@ def run_child(files, extra=()):
 
 def test_gpu_parity_suite_on_the_replay():
     run_child([os.path.join("tests", "test_gpu_parity.py")])
+
+
+def test_kernels_awaiting_their_first_gpu_run_on_the_replay():
+    run_child([os.path.join("tests", "test_zzz_gpu_first_run.py")])
 
 
 def test_allocation_free_entry_point_on_the_replay():
