@@ -374,6 +374,33 @@ def config_rows(L, _lib, torch, only):
         gemm_row("gpt2_%s_dX" % nm, 4, lambda i, dout=dout: randn((Tk, dout), 420 + i), lambda i, din=din, dout=dout: randn((din, dout), 410 + i, 0.02).t(), (Tk, din))
         gemm_row("gpt2_%s_dW" % nm, 4, lambda i, din=din: randn((Tk, din), 400 + i).t(), lambda i, dout=dout: randn((Tk, dout), 420 + i), (din, dout))
 
+    if wanted("gpt2_up_linear_backward"):
+        # the whole backward of the MLP-up Linear layer in one call: dX += dY.W^T, dW += X^T.dY, db += column sums of dY
+        # (the bias gradient comes out of the dW launch: dY is streamed twice, not three times)
+        din, dout = 768, 3072
+        flop = 2 * 2.0 * Tk * din * dout
+        nbytes = 4.0 * (2 * Tk * din + 2 * din * dout + Tk * dout + dout)
+        n = copies_for(nbytes)
+        Xs = [randn((Tk, din), 400 + i) for i in range(n)]
+        dYs = [randn((Tk, dout), 420 + i) for i in range(n)]
+        Wt = randn((din, dout), 410, 0.02)
+        gXs = [torch.zeros((Tk, din), device="cuda") for _ in range(n)]
+        gWs = [torch.zeros((din, dout), device="cuda") for _ in range(n)]
+        gbs = [torch.zeros((dout,), device="cuda") for _ in range(n)]
+        wv = view(Wt)
+        fns = [(lambda xv=view(x), dy=dy, gx=gx, gw=gw, gb=gb: _lib.check(L.tenmo_hip_linear_backward(C.byref(xv), C.byref(wv), dy.data_ptr(), gx.data_ptr(),
+                                                                                                      gw.data_ptr(), gb.data_ptr(), 0)))
+               for x, dy, gx, gw, gb in zip(Xs, dYs, gXs, gWs, gbs)]
+        us = hip_time_us(L, _lib, fns, flop / 100e6)
+        for t in (gXs[0], gWs[0], gbs[0]):
+            t.zero_()
+        fns[0]()
+        errs = [rel_fro_vs_fp64(torch, gXs[0], dYs[0], Wt.t()), rel_fro_vs_fp64(torch, gWs[0], Xs[0].t(), dYs[0]),
+                float((gbs[0].double() - dYs[0].double().sum(0)).norm() / dYs[0].double().sum(0).norm())]
+        finish_row("gpt2_up_linear_backward(dX,dW,db)", 4, "[8192x3072].[3072x768] + [768x8192].[8192x3072] + colsum", us, flop, nbytes, max(errs), n)
+        del Xs, dYs, gXs, gWs, gbs
+        torch.cuda.empty_cache()
+
     # ---- config 5: memory-bound products ----
     n16 = 16384
     if wanted("mv") or wanted("vm"):

@@ -208,6 +208,16 @@ int tenmo_hip_vector_matmul_nd(const tenmo_view* v, const tenmo_view* Mx, float*
  * tenmo/ancestry.mojo:72-105).  Pass NULL for a parent that does not require grad (:34, :45). */
 int tenmo_hip_matmul_backward(const tenmo_view* A, const tenmo_view* B, const float* dC,
                               float* grad_A, float* grad_B, int32_t sync);
+/* Backward of Linear.forward — tenmo/net.mojo:193-201 is Matmul.forward followed by Adder.forward (bias broadcast over
+ * the rows), so its backward is Adder's (tenmo/addition.mojo:73-112: the upstream gradient passes through to the product
+ * and, summed over the broadcast axes, to the bias — sum_over_broadcasted_axes, tenmo/broadcast.mojo:66-88) followed by
+ * tenmo_hip_matmul_backward.  dY: dense upstream gradient at the shape of X.W.  For each non-NULL pointer:
+ * grad_X += dY . W^T(view), grad_W += X^T(view) . dY (summed over X's batch axes), grad_bias[c] += sum of dY over every
+ * axis but the last.  dY is streamed twice, not three times: the launch that computes grad_W reads dY as its right operand
+ * and adds up those fragments on the way (a dense row-major X and dY, one weight matrix; any other form, or grad_W == NULL,
+ * takes one extra streaming pass over dY as tenmo_hip_column_sum_f32 does). */
+int tenmo_hip_linear_backward(const tenmo_view* X, const tenmo_view* W, const float* dY,
+                              float* grad_X, float* grad_W, float* grad_bias, int32_t sync);
 /* MatrixVectorMulNdBackward — tenmo/matrixvector.mojo:19-201 (CPU-only in the reference):
  * grad_M += outer(dy, v), grad_v += M^T . dy, both dense at the parents' shapes. */
 int tenmo_hip_mv_backward(const tenmo_view* Mx, const tenmo_view* v, const float* dy,

@@ -77,6 +77,7 @@ SIGNATURES = {
     "tenmo_hip_matrix_vector_nd": (C.c_int, [_vp, _vp, _ptr, C.c_int32]),
     "tenmo_hip_vector_matmul_nd": (C.c_int, [_vp, _vp, _ptr, C.c_int32]),
     "tenmo_hip_matmul_backward": (C.c_int, [_vp, _vp, _ptr, _ptr, _ptr, C.c_int32]),
+    "tenmo_hip_linear_backward": (C.c_int, [_vp, _vp, _ptr, _ptr, _ptr, _ptr, C.c_int32]),
     "tenmo_hip_mv_backward": (C.c_int, [_vp, _vp, _ptr, _ptr, _ptr, C.c_int32]),
     "tenmo_hip_vm_backward": (C.c_int, [_vp, _vp, _ptr, _ptr, _ptr, C.c_int32]),
     "tenmo_hip_cross_entropy_forward_f32": (C.c_int, [_ptr, _ptr, C.c_int32, C.c_int64, C.c_int64, C.c_int64, C.c_float,

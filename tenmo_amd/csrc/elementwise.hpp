@@ -613,10 +613,18 @@ __global__ void sgd_step_kernel(float* __restrict p, const float* __restrict g, 
 
 // Sums the k_splits partial results into C (plain or accumulating), slices in a fixed order, then
 // applies the fused epilogue.  One thread per output; eight slice loads in flight per thread.
+// (extra_*: a second, small set of slices added the same way onto extra_out — the column sums of B that a launch with
+// GemmArgs::bsum leaves per K slice; extra_n = 0 without)
 __global__ void splitk_reduce_kernel(const float* __restrict partial, float* __restrict C, int64_t n, int splits, int accumulate,
-                                     const float* __restrict bias, const float* __restrict mask, int relu, int64_t N) {
+                                     const float* __restrict bias, const float* __restrict mask, int relu, int64_t N,
+                                     const float* __restrict extra_partial = nullptr, float* __restrict extra_out = nullptr, int64_t extra_n = 0) {
     int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+    for (int64_t j = i; j < extra_n; j += stride) {
+        float s = extra_out[j];
+        for (int p = 0; p < splits; ++p) s += extra_partial[(int64_t)p * extra_n + j];
+        extra_out[j] = s;
+    }
     for (; i < n; i += stride) {
         float s = accumulate ? C[i] : 0.f;
         int p = 0;

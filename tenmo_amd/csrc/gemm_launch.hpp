@@ -8,11 +8,13 @@
 namespace tenmo {
 
 // One workgroup per tile (grid.y = K slices).  false: no variant for these operand modes.
-bool launch_gemm_256x128(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream);
-bool launch_gemm_128x128(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream);
-bool launch_gemm_64x64(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream);
-bool launch_gemm_128x64(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream);
-bool launch_gemm_64x128(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream);
+// (bsum: also add up the column sums of B, see BsumArgs — both operands with unit stride along M / N only, false otherwise;
+// the same argument of the stream-K launchers below)
+bool launch_gemm_256x128(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream, const BsumArgs* bsum = nullptr);
+bool launch_gemm_128x128(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream, const BsumArgs* bsum = nullptr);
+bool launch_gemm_64x64(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream, const BsumArgs* bsum = nullptr);
+bool launch_gemm_128x64(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream, const BsumArgs* bsum = nullptr);
+bool launch_gemm_64x128(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream, const BsumArgs* bsum = nullptr);
 
 // Two products with the 64x64 tile in one launch (count0 / count1 workgroups).  false: no variant for these operand modes.
 bool launch_gemm_pair_64x64(const GemmArgs& g0, const GemmArgs& g1, unsigned count0, unsigned count1, int amode0, int bmode0, int amode1, int bmode1,
@@ -26,10 +28,14 @@ bool launch_gemm_reduce_64x64(const GemmArgs& g, const BatchReduce& red, unsigne
 
 // Stream-K: `wgs` persistent workgroups, then the fix-up over `tiles` tiles in `fix_parts` parts
 // each (0: no tile is shared, no fix-up).  Vector operand modes only.
-bool launch_streamk_256x128(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);
-bool launch_streamk_128x128(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);
-bool launch_streamk_128x64(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);
-bool launch_streamk_64x64(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream);
+bool launch_streamk_256x128(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream,
+                            const BsumArgs* bsum = nullptr);
+bool launch_streamk_128x128(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream,
+                            const BsumArgs* bsum = nullptr);
+bool launch_streamk_128x64(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream,
+                            const BsumArgs* bsum = nullptr);
+bool launch_streamk_64x64(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles, unsigned fix_parts, int amode, int bmode, hipStream_t stream,
+                            const BsumArgs* bsum = nullptr);
 
 // Short reduction (K up to 64), vector operand modes, plain or accumulating store: persistent workgroups that hold a
 // whole tile's operands in LDS, loaded one tile ahead by wavefronts of their own (gemm_smallk.hip).  `total_tiles` =

@@ -84,6 +84,17 @@ struct GemmArgs {
     BatchDesc batch;
 };
 
+// The column sums of B beside the product (the BSUM instantiations of the kernels; a kernel argument of its own, so that
+// the other instantiations keep their argument layout): out[n] += sum_k B(k, n) — the bias gradient of a Linear layer (the
+// upstream gradient summed over its rows, tenmo/broadcast.mojo:66-88) out of the launch that computes the weight gradient
+// X^T . dY, which streams dY as its B anyway.  One matrix (batch_count == 1); the workgroups of the first tile row do it.
+struct BsumArgs {
+    float* out;      // [N]
+    float* partial;  // one-workgroup-per-tile launch with k_splits > 1: [k_splits][N], the sums of each K slice, added by the
+                     // slice reduction; stream-K launch: [2 * workgroups][BN], the sums over each piece of a shared tile,
+                     // added by the fix-up in the order of the tile's partial sums
+};
+
 // bias, ReLU and ReLU-backward mask on one finished element (i = flat index into the dense C)
 __device__ __forceinline__ float epilogue_value(float v, const float* __restrict bias, const float* __restrict mask, int relu, int64_t i, int64_t col) {
     if (bias) v += bias[col];
@@ -445,12 +456,20 @@ struct TileDest {
     bool fused;      // apply g.bias / g.relu / g.mask (never together with accumulate)
 };
 
+// BSUM kernels: where the sum over a gemm_tile call's K range of B(k, col) goes: out[col - col0] (out null: nowhere)
+struct BsumDest {
+    float* out;
+    int64_t col0;
+    bool add; // += instead of =
+};
+
 // One tile of C over the K range [k_begin, k_end) (k_begin a multiple of GEMM_BK), by the whole
 // workgroup.  The three LDS stages are the caller's; on return every wavefront has left them.
-template <int BM, int BN, int AMODE, int BMODE>
+template <int BM, int BN, int AMODE, int BMODE, bool BSUM = false>
 __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, float* stage1, float* stage2,
                                           int64_t batch, int64_t tile_m, int64_t tile_n, int64_t k_begin, int64_t k_end, const TileDest dst,
-                                          const int64_t a_extra = 0, const int64_t b_extra = 0) { // (element offsets on top of the batch's)
+                                          const int64_t a_extra = 0, const int64_t b_extra = 0, // (element offsets on top of the batch's)
+                                          const BsumDest bsum = BsumDest{nullptr, 0, false}) {
     constexpr int TM = BM / 2, TN = BN / 2;     // wave tile (2x2 waves)
     constexpr int MB = TM / 32, NB = TN / 32;   // 32x32 MFMA blocks per wave tile
     constexpr int A_FLOATS = BM * GEMM_BK;
@@ -482,7 +501,24 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
     TileLoader<BM, AMODE> la;
     TileLoader<BN, BMODE> lb;
 
+    // BSUM: every B fragment that feeds the MFMAs is also added up per lane — a lane always holds the same columns
+    // (block j, column lane & 31; the two halves of the wavefront hold different k), so the sums stay in registers for
+    // the whole K range and are combined once, in the epilogue.  Every wavefront does it (no branch in the K loop; the
+    // vector ALU is idle beside the MFMAs), the ones of the first wave row store.
+    float bs[NB];
+#pragma unroll
+    for (int j = 0; j < NB; ++j) bs[j] = 0.f;
+    auto add_b_fragments = [&](const float (&fb)[NB][4]) {
+        if constexpr (BSUM) {
+#pragma unroll
+            for (int j = 0; j < NB; ++j)
+#pragma unroll
+                for (int s = 0; s < 4; ++s) bs[j] += fb[j][s];
+        }
+    };
+
     auto mfma_chunk = [&](const float (&fa)[MB][4], const float (&fb)[NB][4]) {
+        add_b_fragments(fb);
 #pragma unroll
         for (int s = 0; s < 4; ++s)
 #pragma unroll
@@ -551,6 +587,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
             // to issue, so the loop runs at full rate even with a single wavefront per SIMD
             // (measured at 8192^3: all loads and fetches ahead of the MFMAs 142 TFLOP/s, interleaved 153).
             auto mfma_interleaved = [&](const float (&fa)[MB][4], const float (&fb)[NB][4], auto&& slot) {
+                add_b_fragments(fb);
                 int n = 0;
 #pragma unroll
                 for (int s = 0; s < 4; ++s)
@@ -641,6 +678,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
                 else if (p < PA2 + PB2) load_fragment_part<BN, BMODE, NB>(st + A_FLOATS, wn * TN, kc, lane, fb, p - PA2);
             };
             auto mfma2 = [&](const float (&fa)[MB][4], const float (&fb)[NB][4], auto&& slot) {
+                add_b_fragments(fb);
                 int n = 0;
 #pragma unroll
                 for (int s = 0; s < 4; ++s)
@@ -706,6 +744,7 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
                 else if (p < PA2 + PB2) load_fragment_part<BN, BMODE, NB>(st + A_FLOATS, wn * TN, kc, lane, fb, p - PA2);
             };
             auto mfma2 = [&](const float (&fa)[MB][4], const float (&fb)[NB][4], auto&& slot) {
+                add_b_fragments(fb);
                 int n = 0;
 #pragma unroll
                 for (int s = 0; s < 4; ++s)
@@ -828,6 +867,22 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
             }
         }
     }
+    if constexpr (BSUM) {
+        if (bsum.out != nullptr) { // uniform over the workgroup
+#pragma unroll
+            for (int j = 0; j < NB; ++j) bs[j] += __shfl_xor(bs[j], 32); // the two halves of a wavefront hold different k
+            if (wm == 0 && h == 0) {
+#pragma unroll
+                for (int j = 0; j < NB; ++j) {
+                    const int64_t col = n0 + wn * TN + tile_pos<BMODE, NB>(j, x);
+                    if (col < g.N) {
+                        float* p = bsum.out + (col - bsum.col0);
+                        *p = bsum.add ? *p + bs[j] : bs[j];
+                    }
+                }
+            }
+        }
+    }
     if constexpr (COLSUM) {
         if (colsum) { // uniform over the workgroup; the LDS stages are free: every wave has left the K loop
             float* red = stage0;
@@ -850,8 +905,9 @@ __device__ __forceinline__ void gemm_tile(const GemmArgs& g, float* stage0, floa
 }
 
 // One workgroup per tile (and per K slice when g.k_splits > 1): tile number `pid` (batches included) and K slice `slice`.
-template <int BM, int BN, int AMODE, int BMODE>
-__device__ __forceinline__ void gemm_workgroup(const GemmArgs& g, float* stage0, float* stage1, float* stage2, uint32_t pid, uint32_t slice) {
+template <int BM, int BN, int AMODE, int BMODE, bool BSUM = false>
+__device__ __forceinline__ void gemm_workgroup(const GemmArgs& g, float* stage0, float* stage1, float* stage2, uint32_t pid, uint32_t slice,
+                                               const BsumArgs bsum = BsumArgs{}) {
     const uint32_t tiles = (uint32_t)g.tiles_m * (uint32_t)g.tiles_n; // the grid, batches included, is below 2^31
     uint32_t batch32;
     int64_t tile_m, tile_n;
@@ -881,7 +937,16 @@ __device__ __forceinline__ void gemm_workgroup(const GemmArgs& g, float* stage0,
         dst.base = g.C + batch * g.M * g.N;
         dst.accumulate = g.accumulate != 0; dst.fused = true;
     }
-    gemm_tile<BM, BN, AMODE, BMODE>(g, stage0, stage1, stage2, batch, tile_m, tile_n, k_begin, k_end, dst);
+    if constexpr (BSUM) {
+        BsumDest bd{nullptr, 0, false};
+        if (tile_m == 0 && batch == 0) { // the first tile row sees every element of its columns of B once
+            if (g.k_splits > 1) { bd.out = bsum.partial + (int64_t)slice * g.N; bd.add = false; }
+            else { bd.out = bsum.out; bd.add = true; }
+        }
+        gemm_tile<BM, BN, AMODE, BMODE, true>(g, stage0, stage1, stage2, batch, tile_m, tile_n, k_begin, k_end, dst, 0, 0, bd);
+    } else {
+        gemm_tile<BM, BN, AMODE, BMODE>(g, stage0, stage1, stage2, batch, tile_m, tile_n, k_begin, k_end, dst);
+    }
 }
 
 template <int BM, int BN, int AMODE, int BMODE>
@@ -894,6 +959,16 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_kernel(const GemmAr
     __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
     __shared__ __attribute__((aligned(1024))) float stage2[DIRECT ? STAGE_FLOATS : 4];
     gemm_workgroup<BM, BN, AMODE, BMODE>(g, stage0, stage1, stage2, blockIdx.x, blockIdx.y);
+}
+
+// The same launch with the column sums of B added up beside the product (BsumArgs; vector operand forms).
+template <int BM, int BN, int AMODE, int BMODE>
+__global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_mfma_bsum_kernel(const GemmArgs g, const BsumArgs bsum) {
+    constexpr int STAGE_FLOATS = (BM + BN) * GEMM_BK;
+    __shared__ __attribute__((aligned(1024))) float stage0[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage2[STAGE_FLOATS];
+    gemm_workgroup<BM, BN, AMODE, BMODE, true>(g, stage0, stage1, stage2, blockIdx.x, blockIdx.y, bsum);
 }
 
 // Batch dimensions that a product is SUMMED over (the gradient of a parent that was broadcast along them,
@@ -1008,11 +1083,62 @@ __global__ __launch_bounds__(GEMM_THREADS, (BM * BN <= 128 * 64 ? 4 : 2)) void g
     }
 }
 
+// The same launch with the column sums of B added up beside the product (BsumArgs; vector operand forms; one matrix).  A
+// tile of the first tile row that a workgroup computes whole adds its sums straight onto bsum.out; a piece of a shared tile
+// leaves them in the slot of bsum.partial that matches its slot of sk.partial, for the fix-up.
+template <int BM, int BN, int AMODE, int BMODE>
+__global__ __launch_bounds__(GEMM_THREADS, (BM * BN <= 128 * 64 ? 4 : 2)) void gemm_streamk_bsum_kernel(const GemmArgs g, const StreamKArgs sk, const BsumArgs bsum) {
+    constexpr int STAGE_FLOATS = (BM + BN) * GEMM_BK;
+    __shared__ __attribute__((aligned(1024))) float stage0[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
+    __shared__ __attribute__((aligned(1024))) float stage2[STAGE_FLOATS];
+    const uint32_t tiles = (uint32_t)g.tiles_m * (uint32_t)g.tiles_n;
+    const int64_t w = blockIdx.x;
+    uint32_t whole = blockIdx.x;
+    int64_t it = w * sk.per_wg;
+    const int64_t end = min(sk.total, it + sk.per_wg);
+    for (;;) {
+        uint32_t gt;
+        int64_t k0, k1;
+        if (whole < (uint32_t)sk.dp_tiles) {
+            gt = whole; k0 = 0; k1 = sk.nks;
+            whole += gridDim.x;
+        } else if (it < end) {
+            const int64_t st = it / sk.nks;
+            k0 = it - st * sk.nks;
+            k1 = min(sk.nks, k0 + (end - it));
+            gt = (uint32_t)(sk.dp_tiles + st);
+            it += k1 - k0;
+        } else {
+            break;
+        }
+        int64_t tile_m, tile_n;
+        tile_coords_blocked<BM, BN>(g, gt % tiles, tile_m, tile_n); // (one matrix: the tile id is the tile's number in it)
+        const bool complete = k0 == 0 && k1 == sk.nks;
+        const int64_t slot = 2 * w + (k0 == 0 ? 1 : 0);
+        TileDest dst;
+        if (complete) {
+            dst.base = g.C; dst.ld = g.N; dst.row0 = 0; dst.col0 = 0;
+            dst.accumulate = g.accumulate != 0; dst.fused = true;
+        } else {
+            dst.base = sk.partial + slot * (int64_t)(BM * BN); dst.ld = BN;
+            dst.row0 = tile_m * BM; dst.col0 = tile_n * BN;
+            dst.accumulate = false; dst.fused = false;
+        }
+        BsumDest bd{nullptr, 0, false};
+        if (tile_m == 0) { // the first tile row sees every element of its columns of B once
+            if (complete) { bd.out = bsum.out; bd.add = true; }
+            else { bd.out = bsum.partial + slot * (int64_t)BN; bd.col0 = tile_n * BN; }
+        }
+        gemm_tile<BM, BN, AMODE, BMODE, true>(g, stage0, stage1, stage2, 0, tile_m, tile_n, k0 * GEMM_BK, min(g.K, k1 * GEMM_BK), dst, 0, 0, bd);
+    }
+}
+
 // A tile that was shared between workgroups is the sum of their partial tiles (ascending workgroup
 // order), finished with accumulate / the fused epilogue.  blockIdx.x = shared tile, blockIdx.y = one
 // of gridDim.y equal parts of the tile, so that a launch with few tiles still fills the chip.
 template <int BM, int BN>
-__global__ void streamk_fixup_kernel(const GemmArgs g, const StreamKArgs sk) {
+__global__ void streamk_fixup_kernel(const GemmArgs g, const StreamKArgs sk, const BsumArgs bsum) {
     const int64_t tiles = (int64_t)g.tiles_m * g.tiles_n;
     const int64_t gt = sk.dp_tiles + blockIdx.x;
     const int64_t it0 = (int64_t)blockIdx.x * sk.nks, it1 = it0 + sk.nks;
@@ -1027,6 +1153,16 @@ __global__ void streamk_fixup_kernel(const GemmArgs g, const StreamKArgs sk) {
     // the first contributor's piece starts at the tile's beginning (slot 2w+1) exactly when its run
     // began at or before the tile; every later contributor's piece starts inside the tile (slot 2w)
     const float* __restrict first = sk.partial + (2 * w_first + (w_first * sk.per_wg <= it0 ? 1 : 0)) * (int64_t)(BM * BN);
+    // the column sums of B over the tile's pieces (BSUM launches: a tile of the first tile row), same slots, same order
+    if (bsum.out != nullptr && tile_m == 0 && batch == 0 && blockIdx.y == 0) {
+        for (int c = threadIdx.x; c < BN; c += blockDim.x) {
+            const int64_t col = tile_n * BN + c;
+            if (col >= g.N) continue;
+            float s = bsum.out[col] + bsum.partial[(2 * w_first + (w_first * sk.per_wg <= it0 ? 1 : 0)) * (int64_t)BN + c];
+            for (int64_t w = w_first + 1; w <= w_last; ++w) s += bsum.partial[(2 * w) * (int64_t)BN + c];
+            bsum.out[col] = s;
+        }
+    }
     constexpr int PER_TILE = BM * BN / 4; // float4 positions
     const int part = PER_TILE / gridDim.y;
     for (int q4 = blockIdx.y * part + threadIdx.x; q4 < (int)(blockIdx.y + 1) * part; q4 += blockDim.x) {

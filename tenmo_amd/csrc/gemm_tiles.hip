@@ -13,8 +13,13 @@
 namespace tenmo {
 
 #if !TENMO_TILE_STREAMK
-bool TENMO_NAME(launch_gemm_, TENMO_TILE_BM, TENMO_TILE_BN)(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream) {
+bool TENMO_NAME(launch_gemm_, TENMO_TILE_BM, TENMO_TILE_BN)(const GemmArgs& g, dim3 grid, int amode, int bmode, hipStream_t stream, const BsumArgs* bsum) {
     constexpr int BM = TENMO_TILE_BM, BN = TENMO_TILE_BN;
+    if (bsum != nullptr) { // the column sums of B beside the product: the one operand form the weight gradient of a Linear layer has
+        if (amode != MNMAJOR_VEC || bmode != MNMAJOR_VEC) return false;
+        hipLaunchKernelGGL((gemm_mfma_bsum_kernel<BM, BN, MNMAJOR_VEC, MNMAJOR_VEC>), grid, dim3(GEMM_THREADS), 0, stream, g, *bsum);
+        return true;
+    }
 #define TENMO_CASE(A_, B_)                                                                                     \
     if (amode == A_ && bmode == B_) {                                                                          \
         hipLaunchKernelGGL((gemm_mfma_kernel<BM, BN, A_, B_>), grid, dim3(GEMM_THREADS), 0, stream, g);        \
@@ -35,6 +40,10 @@ bool TENMO_NAME(launch_gemm_reduce_, TENMO_TILE_BM, TENMO_TILE_BN)(const GemmArg
         return true;                                                                                                     \
     }
     TENMO_CASE(KMAJOR_VEC, KMAJOR_VEC) TENMO_CASE(KMAJOR_VEC, MNMAJOR_VEC) TENMO_CASE(MNMAJOR_VEC, KMAJOR_VEC) TENMO_CASE(MNMAJOR_VEC, MNMAJOR_VEC)
+#if TENMO_TILE_BM == 64 // operands without a unit stride (views with steps, overlapping rows): the small tile only
+    TENMO_CASE(KMAJOR_VEC, KMAJOR_GEN) TENMO_CASE(MNMAJOR_VEC, KMAJOR_GEN) TENMO_CASE(KMAJOR_GEN, KMAJOR_VEC) TENMO_CASE(KMAJOR_GEN, MNMAJOR_VEC)
+    TENMO_CASE(KMAJOR_GEN, KMAJOR_GEN)
+#endif
 #undef TENMO_CASE
     return false;
 }
@@ -51,15 +60,19 @@ bool launch_gemm_pair_64x64(const GemmArgs& g0, const GemmArgs& g1, unsigned cou
 #endif
 #else
 bool TENMO_NAME(launch_streamk_, TENMO_TILE_BM, TENMO_TILE_BN)(const GemmArgs& g, const StreamKArgs& sk, unsigned wgs, unsigned tiles,
-                                                              unsigned fix_parts, int amode, int bmode, hipStream_t stream) {
+                                                              unsigned fix_parts, int amode, int bmode, hipStream_t stream, const BsumArgs* bsum) {
     constexpr int BM = TENMO_TILE_BM, BN = TENMO_TILE_BN;
 #define TENMO_CASE(A_, B_)                                                                                               \
     if (amode == A_ && bmode == B_)                                                                                      \
         hipLaunchKernelGGL((gemm_streamk_kernel<BM, BN, A_, B_>), dim3(wgs), dim3(GEMM_THREADS), 0, stream, g, sk);
+    if (bsum != nullptr) {
+        if (amode != MNMAJOR_VEC || bmode != MNMAJOR_VEC) return false;
+        hipLaunchKernelGGL((gemm_streamk_bsum_kernel<BM, BN, MNMAJOR_VEC, MNMAJOR_VEC>), dim3(wgs), dim3(GEMM_THREADS), 0, stream, g, sk, *bsum);
+    } else
     TENMO_CASE(KMAJOR_VEC, KMAJOR_VEC) else TENMO_CASE(KMAJOR_VEC, MNMAJOR_VEC) else TENMO_CASE(MNMAJOR_VEC, KMAJOR_VEC) else TENMO_CASE(MNMAJOR_VEC, MNMAJOR_VEC)
     else return false;
 #undef TENMO_CASE
-    if (fix_parts) hipLaunchKernelGGL((streamk_fixup_kernel<BM, BN>), dim3(tiles, fix_parts), dim3(256), 0, stream, g, sk);
+    if (fix_parts) hipLaunchKernelGGL((streamk_fixup_kernel<BM, BN>), dim3(tiles, fix_parts), dim3(256), 0, stream, g, sk, bsum ? *bsum : BsumArgs{});
     return true;
 }
 #endif

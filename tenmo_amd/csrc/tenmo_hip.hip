@@ -208,6 +208,7 @@ struct Epilogue {
     const int32_t* gather_k = nullptr;
     bool gather_kmajor = false;          // the gathered B is contiguous along k (16-byte loads along k) rather than along n
     float* colsum = nullptr;             // [batch][N]: also write the column sums of the result (needs M <= 128, see GemmArgs)
+    float* bsum = nullptr;               // [N]: += the column sums of B over K (GemmArgs::bsum; see bsum_fits); goes with accumulate
     bool any() const { return bias || mask || relu || colsum; }
 };
 
@@ -220,6 +221,13 @@ void streamk_partition(int64_t tiles, int64_t nks, int64_t wgs, int64_t* whole_r
     if (rest > 0 && rest * nks < 8 * wgs && full > 0) { --full; rest += wgs; }
     *whole_rounds = full;
     *shared = rest;
+}
+
+// What a launch with Epilogue::bsum needs: one matrix, the operand forms of a Linear layer's weight gradient X^T(view) . dY
+// (the only instantiations that add up their B fragments), nothing else fused.
+bool bsum_fits(int64_t a_rs, int64_t a_cs, int64_t b_rs, int64_t b_cs, int64_t M, int64_t N, int64_t K, int64_t batch_count, const Epilogue& ep) {
+    return batch_count == 1 && M > 0 && N > 0 && K > 0 && !ep.any() && !ep.gather_row &&
+           operand_mode(a_rs, a_cs, M, K) == MNMAJOR_VEC && operand_mode(b_cs, b_rs, N, K) == MNMAJOR_VEC;
 }
 
 int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, int64_t b_rs, int64_t b_cs, float* C,
@@ -242,6 +250,11 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     g.bias = ep.bias; g.mask = ep.mask; g.relu = ep.relu; g.bias_rows = ep.bias_rows;
     g.b_gather_row = ep.gather_row; g.b_gather_k = ep.gather_k;
     g.colsum = ep.colsum;
+    BsumArgs bsum_args{};
+    bsum_args.out = ep.bsum;
+    const BsumArgs* const bsum = ep.bsum ? &bsum_args : nullptr;
+    if (ep.bsum && !bsum_fits(a_rs, a_cs, b_rs, b_cs, M, N, K, batch_count, ep))
+        return fail(TENMO_ERR_UNSUPPORTED, "column sums of B beside the product: one matrix, both operands with unit stride along M / N, no other epilogue");
     if (ep.colsum && (M > 128 || accumulate)) return fail(TENMO_ERR_UNSUPPORTED, "column sums in the GEMM store need M <= 128 and no accumulate");
     g.batch = bd;
     g.batch_count = batch_count;
@@ -300,6 +313,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
             // A gathered operand keeps its tile (see above) at that tile's resident workgroups per CU.
             const int gather_tile = M > 64 ? 3 : 2;
             for (int t = ep.gather_row ? gather_tile : 1; t >= 0; --t) {
+                if (ep.bsum && t != 1) continue; // (the column sums of B beside the product: the 128x128 stream-K kernel has the registers for them)
                 const int64_t tiles = ((M + kTiles[t].bm - 1) / kTiles[t].bm) * ((N + kTiles[t].bn - 1) / kTiles[t].bn) * batch_count;
                 const int wpc = ep.gather_row ? kStreamKOccupancy[t] : (t == 0 || tiles >= 2 * (int64_t)S.cus) ? 2 : 1;
                 const int64_t nks = (K + GEMM_BK - 1) / GEMM_BK, wgs = (int64_t)S.cus * wpc;
@@ -358,7 +372,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         const bool a_ok = am == KMAJOR_VEC ? (a_cs == 1 && a_rs >= 0 && a_rs <= (int64_t(1) << 21) && K % 4 == 0)
                                            : (am == MNMAJOR_VEC && a_rs == 1 && a_cs >= 0 && a_cs <= (int64_t(1) << 25) && M % 4 == 0 && M >= 4);
         const bool b_ok = bm == MNMAJOR_VEC && b_cs == 1 && b_rs >= 0 && b_rs <= (int64_t(1) << 25) && N % 4 == 0 && N >= 4;
-        const bool can = batch_count == 1 && !accumulate && K > GEMM_BK && K <= 256 && a_ok && b_ok && !ep.any() && !ep.gather_row && !ep.colsum &&
+        const bool can = batch_count == 1 && !accumulate && K > GEMM_BK && K <= 256 && a_ok && b_ok && !ep.any() && !ep.gather_row && !ep.colsum && !ep.bsum &&
                          N <= (int64_t(1) << 22) && tm <= (int64_t)S.cus * (rbm == 64 ? 2 : 1) / 8; // (worth it with several column blocks per workgroup: for the policy that will choose it once it has been measured)
         if (can) {
             g.tiles_m = (int32_t)tm; g.tiles_n = (int32_t)tn;
@@ -383,7 +397,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         const int pt = S.force_panel == 3 || S.force_panel == 5 ? 64 : 128;
         const bool paired = (S.force_panel == 4 || S.force_panel == 5) && am == KMAJOR_VEC && !accumulate;
         const int64_t tm = (M + pt - 1) / pt, tn = (N + pt - 1) / pt, tiles = tm * tn * batch_count;
-        const bool can = K > GEMM_BK && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum &&
+        const bool can = K > GEMM_BK && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum && !ep.bsum &&
                          N <= (int64_t(1) << 22) && tiles <= 0x7fffffffLL;
         const bool want = S.force_panel > 0 || (S.force_panel < 0 && S.force_tile < 0 && S.force_splitk <= 0 && S.force_streamk <= 0 && S.force_smallk <= 0 &&
                                                  splits == 1 && sk_wpc == 0 && K > 64 && K <= 512 && tiles >= 3 * (int64_t)S.cus);
@@ -412,7 +426,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         // through this kernel faulted — an undeclared SCC clobber of the masked direct load, since fixed (gfx950_asm.hpp) — and
         // the one-step instantiations come back once the fix has been confirmed on a GPU.  Until then the automatic choice
         // is also limited to K % 16 == 0, which never takes the masked load; a ragged K reaches it only through the knob.)
-        const bool can = K > GEMM_BK && K <= 64 && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum &&
+        const bool can = K > GEMM_BK && K <= 64 && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum && !ep.bsum &&
                          N < (int64_t(1) << 29) && tiles64 <= 0x7fffffffLL;
         const bool want = S.force_smallk > 0 || (S.force_smallk < 0 && S.force_tile < 0 && S.force_splitk <= 0 && S.force_streamk <= 0 &&
                                                   splits == 1 && sk_wpc == 0 && tiles64 >= 2048 && K <= 64 && K % GEMM_BK == 0);
@@ -447,18 +461,19 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         const int64_t wgs = whole_rounds > 0 ? want : (sk.total + per - 1) / per;
         if (tiles_total <= 0x7fffffffLL && wgs >= 1) {
             float* ws;
-            if (int rc = workspace((size_t)(2 * wgs) * bmt * bnt * sizeof(float), &ws)) return rc;
+            if (int rc = workspace((size_t)(2 * wgs) * (bmt + (ep.bsum ? 1 : 0)) * bnt * sizeof(float), &ws)) return rc;
             sk.partial = ws;
+            bsum_args.partial = ep.bsum ? ws + (size_t)(2 * wgs) * bmt * bnt : nullptr;
             const bool need_fixup = shared > 0 && per % sk.nks != 0;
             if (S.verbose) fprintf(stderr, "tenmo_hip gemm stream-K: %lld workgroups, %lld whole tiles each, then %lld K steps each of %lld shared tiles of %dx%d\n",
                                    (long long)wgs, (long long)whole_rounds, (long long)per, (long long)shared, bmt, bnt);
             // parts per shared tile in the fix-up: a power of two that brings it to a few workgroups per CU
             unsigned parts = 0;
             if (need_fixup) for (parts = 1; parts < 32 && shared * parts < (int64_t)S.cus * 4; parts *= 2) {}
-            const bool ok = tile == 0   ? launch_streamk_256x128(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream)
-                            : tile == 1 ? launch_streamk_128x128(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream)
-                            : tile == 2 ? launch_streamk_64x64(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream)
-                                        : launch_streamk_128x64(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream);
+            const bool ok = tile == 0   ? launch_streamk_256x128(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream, bsum)
+                            : tile == 1 ? launch_streamk_128x128(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream, bsum)
+                            : tile == 2 ? launch_streamk_64x64(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream, bsum)
+                                        : launch_streamk_128x64(g, sk, (unsigned)wgs, (unsigned)shared, parts, am, bm, S.stream, bsum);
             return ok ? 0 : fail(TENMO_ERR_UNSUPPORTED, "no stream-K variant for operand modes %d/%d", am, bm);
         }
     }
@@ -474,8 +489,9 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     }
     if (splits > 1) {
         float* ws;
-        if (int rc = workspace((size_t)splits * batch_count * M * N * sizeof(float), &ws)) return rc;
+        if (int rc = workspace((size_t)splits * (batch_count * M + (ep.bsum ? 1 : 0)) * N * sizeof(float), &ws)) return rc;
         g.partial = ws;
+        bsum_args.partial = ep.bsum ? ws + (size_t)splits * batch_count * M * N : nullptr;
     }
     g.tiles_m = (int32_t)((M + kTiles[tile].bm - 1) / kTiles[tile].bm);
     g.tiles_n = (int32_t)((N + kTiles[tile].bn - 1) / kTiles[tile].bn);
@@ -483,17 +499,17 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     dim3 grid((unsigned)nb, (unsigned)splits, 1);
     bool ok = false;
     switch (tile) {
-        case 0: ok = launch_gemm_256x128(g, grid, am, bm, S.stream); break;
-        case 1: ok = launch_gemm_128x128(g, grid, am, bm, S.stream); break;
-        case 3: ok = launch_gemm_128x64(g, grid, am, bm, S.stream); break;
-        case 4: ok = launch_gemm_64x128(g, grid, am, bm, S.stream); break;
-        default: ok = launch_gemm_64x64(g, grid, am, bm, S.stream); break;
+        case 0: ok = launch_gemm_256x128(g, grid, am, bm, S.stream, bsum); break;
+        case 1: ok = launch_gemm_128x128(g, grid, am, bm, S.stream, bsum); break;
+        case 3: ok = launch_gemm_128x64(g, grid, am, bm, S.stream, bsum); break;
+        case 4: ok = launch_gemm_64x128(g, grid, am, bm, S.stream, bsum); break;
+        default: ok = launch_gemm_64x64(g, grid, am, bm, S.stream, bsum); break;
     }
     if (!ok) return fail(TENMO_ERR_UNSUPPORTED, "no GEMM variant for operand modes %d/%d", am, bm);
     if (splits > 1) {
         const int64_t n = batch_count * M * N;
         hipLaunchKernelGGL(splitk_reduce_kernel, dim3((unsigned)std::min<int64_t>((n + 255) / 256, 8192)), dim3(256), 0, S.stream,
-                           g.partial, C, n, splits, accumulate, ep.bias, ep.mask, ep.relu, N);
+                           g.partial, C, n, splits, accumulate, ep.bias, ep.mask, ep.relu, N, (const float*)bsum_args.partial, ep.bsum, ep.bsum ? N : (int64_t)0);
     }
     return 0;
 }
@@ -919,7 +935,8 @@ int folded_gradient(const tenmo_view* X, const tenmo_view* Y, const Geometry& g,
     const int64_t M = X->shape[X->rank - 2], K = X->shape[X->rank - 1], N = Y->shape[Y->rank - 1];
     const int64_t x_rs = X->strides[X->rank - 2], x_cs = X->strides[X->rank - 1], y_rs = Y->strides[Y->rank - 2], y_cs = Y->strides[Y->rank - 1];
     const int am = operand_mode(x_rs, x_cs, M, K), bm = operand_mode(y_cs, y_rs, N, K);
-    if (am == KMAJOR_GEN || bm == KMAJOR_GEN || M == 0 || N == 0) return 0;
+    if (M == 0 || N == 0) return 0;
+    const bool generic = am == KMAJOR_GEN || bm == KMAJOR_GEN; // an operand without a unit stride: the 64x64 tile's element-wise loader
     int64_t xs[MAX_BATCH_RANK] = {0}, ys[MAX_BATCH_RANK] = {0};
     batch_strides_of(X, X->rank - 2, g.batch_rank, xs);
     batch_strides_of(Y, Y->rank - 2, g.batch_rank, ys);
@@ -941,7 +958,7 @@ int folded_gradient(const tenmo_view* X, const tenmo_view* Y, const Geometry& g,
     }
     if (red.count <= 1) return 0;
     const int64_t tiles128 = ((M + 127) / 128) * ((N + 127) / 128) * kept_count, tiles64 = ((M + 63) / 64) * ((N + 63) / 64) * kept_count;
-    const bool big = tiles128 >= (int64_t)S.cus;
+    const bool big = tiles128 >= (int64_t)S.cus && !generic;
     if (S.fold_reduce < 0 && !big && tiles64 < (int64_t)S.cus / 2) return 0;
     if (tiles64 > 0x7fffffffLL) return 0;
     a.A = X->data + X->offset; a.B = Y->data + Y->offset; a.C = grad;
@@ -1607,13 +1624,13 @@ int tenmo_hip_vector_matmul_nd(const tenmo_view* v, const tenmo_view* Mx, float*
     return finish(sync);
 }
 
-int tenmo_hip_matmul_backward(const tenmo_view* A, const tenmo_view* B, const float* dC,
-                              float* grad_A, float* grad_B, int32_t sync) {
-    if (int rc = ensure_ready()) return rc;
-    Geometry g;
-    if (int rc = resolve(TENMO_OP_MM, A, B, &g, "tenmo_hip_matmul_backward")) return rc;
-    if (g.batch_count == 0) return 0;
-    if (int rc = need(dC, product(g.oshape, g.orank) > 0 && (grad_A || grad_B), "tenmo_hip_matmul_backward", "upstream gradient")) return rc;
+// The two gradient products of Matmul backward (the body of tenmo_hip_matmul_backward; `g` = resolve(A, B)).
+// grad_b: when not null, the gradient of a bias [N] added to the product (Linear: Matmul, then Adder) is wanted as well —
+// the upstream gradient summed over everything but its last axis.  Where dB runs as ONE product with dC as its right
+// operand (a shared B: always for a Linear weight), the sums come out of that launch (Epilogue::bsum) and *bias_done
+// is set; otherwise the caller streams dC once more.
+static int matmul_backward_impl(const tenmo_view* A, const tenmo_view* B, const float* dC, float* grad_A, float* grad_B, const Geometry& g,
+                                float* grad_b = nullptr, bool* bias_done = nullptr) {
     const tenmo_view dCv = dense_view(dC, g.oshape, g.orank);
     if (grad_A) { // dA = dC . B^T(view)   (tenmo/matmul.mojo:36-38, :116-121)
         const tenmo_view Bt = transposed_last2(B);
@@ -1641,10 +1658,20 @@ int tenmo_hip_matmul_backward(const tenmo_view* A, const tenmo_view* B, const fl
             const int64_t M = A->shape[A->rank - 2], K = A->shape[A->rank - 1], N = B->shape[B->rank - 1];
             BatchDesc none{};
             for (int d = 0; d < MAX_BATCH_RANK; ++d) none.shape[d] = 1;
+            Epilogue ep;
+            if (grad_b && K > 8 && bsum_fits(A->strides[A->rank - 1], A->strides[A->rank - 2], N, 1, K, N, g.batch_count * M, 1, ep)) { ep.bsum = grad_b; *bias_done = true; }
             if (int rc = gemm_dispatch(A->data + A->offset, A->strides[A->rank - 1], A->strides[A->rank - 2], dC, N, 1, grad_B,
-                                       K, N, g.batch_count * M, none, 1, 1)) return rc;
+                                       K, N, g.batch_count * M, none, 1, 1, ep)) return rc;
         } else if (same_batch(g, B, 2)) {
-            if (int rc = matmul_views(&At, &dCv, grad_B, 1, "tenmo_hip_matmul_backward")) return rc;
+            // (one matrix: the weight gradient of a Linear layer under a 2-D input is this product, with dC as its right operand)
+            const int64_t M = A->shape[A->rank - 2], K = A->shape[A->rank - 1], N = B->shape[B->rank - 1];
+            Epilogue ep;
+            if (grad_b && K > 8 && g.batch_count == 1 && bsum_fits(At.strides[At.rank - 2], At.strides[At.rank - 1], N, 1, K, N, M, 1, ep)) {
+                ep.bsum = grad_b; *bias_done = true;
+                BatchDesc none{};
+                for (int d = 0; d < MAX_BATCH_RANK; ++d) none.shape[d] = 1;
+                if (int rc = gemm_dispatch(At.data + At.offset, At.strides[At.rank - 2], At.strides[At.rank - 1], dC, N, 1, grad_B, K, N, M, none, 1, 1, ep)) return rc;
+            } else if (int rc = matmul_views(&At, &dCv, grad_B, 1, "tenmo_hip_matmul_backward")) return rc;
         } else if (const int folded = folded_gradient(&At, &dCv, g, B, grad_B)) {
             if (folded < 0) return folded;
         } else {
@@ -1655,6 +1682,38 @@ int tenmo_hip_matmul_backward(const tenmo_view* A, const tenmo_view* B, const fl
             if (int rc = matmul_views(&At, &dCv, full, 0, "tenmo_hip_matmul_backward")) return rc;
             if (int rc = reduce_to_parent(full, gg, B, 2, grad_B)) return rc;
         }
+    }
+    return 0;
+}
+
+int tenmo_hip_matmul_backward(const tenmo_view* A, const tenmo_view* B, const float* dC,
+                              float* grad_A, float* grad_B, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    Geometry g;
+    if (int rc = resolve(TENMO_OP_MM, A, B, &g, "tenmo_hip_matmul_backward")) return rc;
+    if (g.batch_count == 0) return 0;
+    if (int rc = need(dC, product(g.oshape, g.orank) > 0 && (grad_A || grad_B), "tenmo_hip_matmul_backward", "upstream gradient")) return rc;
+    if (int rc = matmul_backward_impl(A, B, dC, grad_A, grad_B, g)) return rc;
+    return finish(sync);
+}
+
+int tenmo_hip_linear_backward(const tenmo_view* X, const tenmo_view* W, const float* dY,
+                              float* grad_X, float* grad_W, float* grad_bias, int32_t sync) {
+    if (int rc = ensure_ready()) return rc;
+    const char* who = "tenmo_hip_linear_backward";
+    Geometry g;
+    if (int rc = resolve(TENMO_OP_MM, X, W, &g, who)) return rc;
+    if (g.batch_count == 0) return 0;
+    const int64_t total = product(g.oshape, g.orank);
+    if (int rc = need(dY, total > 0 && (grad_X || grad_W || grad_bias), who, "upstream gradient")) return rc;
+    bool bias_done = false;
+    if (int rc = matmul_backward_impl(X, W, dY, grad_X, grad_W, g, grad_W ? grad_bias : nullptr, &bias_done)) return rc;
+    if (grad_bias && !bias_done) {
+        // sum_over_broadcasted_axes for the bias operand of Adder (tenmo/broadcast.mojo:66-88): dY [rows, N] summed over its rows, one streaming pass
+        const int64_t N = g.oshape[g.orank - 1], rows = N > 0 ? total / N : 0;
+        BatchDesc bd{};
+        for (int d = 0; d < MAX_BATCH_RANK; ++d) bd.shape[d] = 1;
+        if (int rc = matvec_dispatch(dY, 1, N, S.one, 0, grad_bias, N, rows, bd, 1, 1)) return rc;
     }
     return finish(sync);
 }

@@ -3,8 +3,9 @@
 ``Linear``        y = x.W + b with W stored [in, out] (tenmo/net.mojo:49-216, :91-97).  For matrix
                   inputs the bias is added in the GEMM store (one launch); for a vector input it
                   is a rank-1 product on the GEMM entry (ones[rows,1] . b[1,out], accumulated).
-                  The bias gradient is the column sum of dY (one streaming pass), so the layer
-                  never leaves ``libtenmo_hip.so``.
+                  The backward of a matrix input is one call (tenmo_hip_linear_backward): dX, dW and
+                  the bias gradient, the latter summed inside the launch that computes dW; a vector
+                  input keeps the separate column sum of dY.  The layer never leaves ``libtenmo_hip.so``.
 ``MLP``           the whole training step of examples/mnist.mojo:150-162 on the device:
                   Linear -> ReLU -> ... -> Linear -> CrossEntropyLoss(mean) -> backward -> SGD(lr).
 ``xavier_uniform``  U(+-sqrt(6/(in+out))) weights, zero bias (tenmo/net.mojo:87-114).
@@ -70,7 +71,22 @@ class Linear:
             ones = torch.ones(rows, dtype=torch.float32, device="cuda")
             check(L.tenmo_hip_gemm_f32(ones.data_ptr(), 0, 1, 1, self.bias.buffer.data_ptr(), self.bias.buffer.offset, self.out_features, 1,
                                        out.buffer.data_ptr(), rows, self.out_features, 1, 0, None, None, None, 1, 1 if sync else 0))
-        if self.training and (out.backward_fn is not None or self.bias.requires_grad):
+        if self.training and xs.rank() >= 2 and (out.backward_fn is not None or self.bias.requires_grad):
+            # Adder backward + Matmul backward in one call of the library: the bias gradient (the upstream gradient summed
+            # over its rows, tenmo/broadcast.mojo:81-87) comes out of the launch that computes the weight gradient
+            x, w, bias = xs, self.weight, self.bias
+
+            def backward_fused(output: Tensor, retain_graph: bool = False):
+                grads = [(p.ensure_gradbox().data_ptr() if p.requires_grad else None) for p in (x, w, bias)]
+                check(L.tenmo_hip_linear_backward(C.byref(x.buffer.c_view()), C.byref(w.buffer.c_view()), output.gradbox.data_ptr(), *grads, 0))
+                if not retain_graph:
+                    output.zero_grad()
+                return [p for p in (x, w, bias) if p.requires_grad]
+
+            out.requires_grad = True
+            out.backward_fn, out.ancestors = None, []
+            out.add_ancestry(backward_fused, x, w, bias)
+        elif self.training and (out.backward_fn is not None or self.bias.requires_grad):
             inner, bias, parents = out.backward_fn, self.bias, list(out.ancestors)
 
             def backward(output: Tensor, retain_graph: bool = False):

@@ -25,7 +25,7 @@ static const any_fn every_symbol[] = {
     (any_fn)tenmo_hip_timer_end, (any_fn)tenmo_hip_clock_probe, (any_fn)tenmo_hip_gemm_f32, (any_fn)tenmo_hip_gemm_epilogue_f32,
     (any_fn)tenmo_hip_mv_f32, (any_fn)tenmo_hip_vm_f32, (any_fn)tenmo_hip_vm_f32_noalloc, (any_fn)tenmo_hip_column_sum_f32, (any_fn)tenmo_hip_dot_f32,
     (any_fn)tenmo_hip_classify_matmul, (any_fn)tenmo_hip_result_shape, (any_fn)tenmo_hip_matmul_nd, (any_fn)tenmo_hip_linear_nd,
-    (any_fn)tenmo_hip_matrix_vector_nd, (any_fn)tenmo_hip_vector_matmul_nd, (any_fn)tenmo_hip_matmul_backward, (any_fn)tenmo_hip_mv_backward,
+    (any_fn)tenmo_hip_matrix_vector_nd, (any_fn)tenmo_hip_vector_matmul_nd, (any_fn)tenmo_hip_matmul_backward, (any_fn)tenmo_hip_linear_backward, (any_fn)tenmo_hip_mv_backward,
     (any_fn)tenmo_hip_vm_backward, (any_fn)tenmo_hip_cross_entropy_forward_f32, (any_fn)tenmo_hip_cross_entropy_backward_f32,
     (any_fn)tenmo_hip_conv2d_forward_f32, (any_fn)tenmo_hip_conv2d_backward_f32, (any_fn)tenmo_hip_sgd_step_f32, (any_fn)cblas_sgemm,
     (any_fn)tenmo_hip_mlp_create, (any_fn)tenmo_hip_mlp_destroy, (any_fn)tenmo_hip_mlp_step, (any_fn)tenmo_hip_mlp_step_graph,
@@ -76,7 +76,7 @@ int main(void) {
     for (int m = 0; m < M; ++m) { y_want[m] = 0.f; for (int k = 0; k < K; ++k) y_want[m] += A[m * K + k] * x[k]; }
     for (int n = 0; n < N; ++n) { z_want[n] = 0.f; for (int k = 0; k < K; ++k) z_want[n] += x[k] * B[k * N + n]; }
 
-    expect(sizeof(every_symbol) / sizeof(every_symbol[0]) == 40, "one table entry per declared function");
+    expect(sizeof(every_symbol) / sizeof(every_symbol[0]) == 41, "one table entry per declared function");
     expect(tenmo_hip_sync() == TENMO_ERR_NOT_INITIALIZED, "calls before init are refused");
     if (tenmo_hip_init(0) != TENMO_OK) { fprintf(stderr, "tenmo_hip_init: %s\n", tenmo_hip_last_error()); return 2; }
     int cus = 0;
@@ -102,6 +102,22 @@ int main(void) {
     int32_t rank = 0;
     expect(tenmo_hip_result_shape(TENMO_OP_MM, &va, &vb, shape, &rank) == M * N && rank == 2 && shape[0] == M && shape[1] == N, "result_shape");
     expect(tenmo_hip_matmul_nd(&va, &vb, dC, 1) == TENMO_OK && same(dC, C_want, M * N, 0.f), "matmul_nd");
+
+    /* the backward of y = A.B + bias from the upstream gradient dY = A.B: grad_A = dY.B^T, grad_B = A^T.dY, grad_bias = column sums of dY,
+     * each added onto what the gradient buffers hold (zeros here) */
+    {
+        float gA_want[M * K], gB_want[K * N], gb_want[N], zeros[M * K + K * N + N];
+        memset(zeros, 0, sizeof(zeros));
+        for (int m = 0; m < M; ++m)
+            for (int k = 0; k < K; ++k) { float s = 0.f; for (int n = 0; n < N; ++n) s += C_want[m * N + n] * B[k * N + n]; gA_want[m * K + k] = s; }
+        for (int k = 0; k < K; ++k)
+            for (int n = 0; n < N; ++n) { float s = 0.f; for (int m = 0; m < M; ++m) s += A[m * K + k] * C_want[m * N + n]; gB_want[k * N + n] = s; }
+        for (int n = 0; n < N; ++n) { gb_want[n] = 0.f; for (int m = 0; m < M; ++m) gb_want[n] += C_want[m * N + n]; }
+        float *gA = to_device(zeros, M * K), *gB = to_device(zeros, K * N), *gb = to_device(zeros, N), *dY = to_device(C_want, M * N);
+        expect(tenmo_hip_linear_backward(&va, &vb, dY, gA, gB, gb, 1) == TENMO_OK, "linear_backward");
+        expect(same(gA, gA_want, M * K, 0.f) && same(gB, gB_want, K * N, 0.f) && same(gb, gb_want, N, 0.f), "linear_backward gradients");
+        hipFree(gA); hipFree(gB); hipFree(gb); hipFree(dY);
+    }
 
     /* y = A.x, z = x.B (with and without allocation), d = x.x */
     expect(tenmo_hip_mv_f32(dA, 0, K, 1, dx, 0, 1, dy, M, K, 0, NULL, NULL, NULL, 0, 1) == TENMO_OK && same(dy, y_want, M, 0.f), "mv");

@@ -16,6 +16,9 @@
 //   CASE = misc:n      dot, column sum ([n/64+1, 64.. ] shapes derived from n), SGD with and without momentum, addresses only
 //   CASE = bwd:M,N,K,a_layout,b_layout,a_batch,b_batch[,knob=value...]   tenmo_hip_matmul_backward of A[a_batch, M, K] . B[b_batch, K, N]
 //     (a batch of 0: no batch dimension; 1: one that broadcasts): both gradients against float64, accumulated onto a start value
+//   CASE = lin:M,N,K,a_layout,n,a_batch,0[,fused=0|1][,knob=value...]   tenmo_hip_linear_backward of X[a_batch, M, K] . W[K, N] + b[N]: the three
+//     gradients against float64; fused=1: the call must take as many kernel launches with the bias gradient as without it (the sums
+//     come out of the weight-gradient launch), fused=0: more
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
@@ -318,19 +321,22 @@ static int run_address_only_case(const std::string& spec) {
     return rc != 0;
 }
 
-static tenmo_view view_of(const float* p, int64_t batch, int64_t rows, int64_t cols, bool transposed) {
+// (generic: row-major storage of twice the width of which every second element is used: no unit stride)
+static tenmo_view view_of(const float* p, int64_t batch, int64_t rows, int64_t cols, bool transposed, bool generic = false) {
     tenmo_view v;
     memset(&v, 0, sizeof(v));
     v.data = p;
     int r = 0;
-    if (batch > 0) { v.shape[r] = batch; v.strides[r] = rows * cols; ++r; }
-    v.shape[r] = rows; v.strides[r] = transposed ? 1 : cols; ++r;
-    v.shape[r] = cols; v.strides[r] = transposed ? rows : 1; ++r;
+    if (batch > 0) { v.shape[r] = batch; v.strides[r] = rows * cols * (generic ? 2 : 1); ++r; }
+    v.shape[r] = rows; v.strides[r] = generic ? 2 * cols : transposed ? 1 : cols; ++r;
+    v.shape[r] = cols; v.strides[r] = generic ? 2 : transposed ? rows : 1; ++r;
     v.rank = r;
     return v;
 }
 
 static int run_backward_case(const std::string& spec) {
+    const bool linear = spec.compare(0, 4, "lin:") == 0;
+    int want_fused = -1;
     std::vector<std::string> f;
     size_t pos = 4;
     while (pos <= spec.size()) {
@@ -341,28 +347,37 @@ static int run_backward_case(const std::string& spec) {
     }
     if (f.size() < 7) { fprintf(stderr, "bad case %s\n", spec.c_str()); return 2; }
     const int64_t M = atoll(f[0].c_str()), N = atoll(f[1].c_str()), K = atoll(f[2].c_str());
-    const bool ta = f[3] == "t", tb = f[4] == "t";
+    const bool ta = f[3] == "t", tb = f[4] == "t", ga = f[3] == "g", gb = f[4] == "g";
     const int64_t ba = atoll(f[5].c_str()), bb = atoll(f[6].c_str());
     std::vector<std::pair<std::string, int>> knobs;
     for (size_t i = 7; i < f.size(); ++i) {
         const size_t eq = f[i].find('=');
-        if (eq != std::string::npos) knobs.push_back({f[i].substr(0, eq), atoi(f[i].c_str() + eq + 1)});
+        if (eq == std::string::npos) continue;
+        if (f[i].substr(0, eq) == "fused") want_fused = atoi(f[i].c_str() + eq + 1);
+        else knobs.push_back({f[i].substr(0, eq), atoi(f[i].c_str() + eq + 1)});
     }
     const int64_t na = ba > 0 ? ba : 1, nb = bb > 0 ? bb : 1, nc = na > nb ? na : nb;
-    const size_t a_n = (size_t)(na * M * K), b_n = (size_t)(nb * K * N), c_n = (size_t)(nc * M * N);
-    float* A = (float*)malloc(a_n * 4); float* B = (float*)malloc(b_n * 4); float* dC = (float*)malloc(c_n * 4);
+    const size_t a_n = (size_t)(na * M * K), b_n = (size_t)(nb * K * N), c_n = (size_t)(nc * M * N); // elements of the views = of the gradients
+    const int64_t a_mat = M * K * (ga ? 2 : 1), b_mat = K * N * (gb ? 2 : 1);                          // storage per matrix
+    const size_t a_store = (size_t)(na * a_mat), b_store = (size_t)(nb * b_mat);
+    float* A = (float*)malloc(a_store * 4); float* B = (float*)malloc(b_store * 4); float* dC = (float*)malloc(c_n * 4);
     float* gA = (float*)malloc(a_n * 4); float* gB = (float*)malloc(b_n * 4);
-    for (size_t i = 0; i < a_n; ++i) { A[i] = next_float(); gA[i] = next_float(); }
-    for (size_t i = 0; i < b_n; ++i) { B[i] = next_float(); gB[i] = next_float(); }
+    float* gbias = (float*)malloc((size_t)N * 4 ? (size_t)N * 4 : 1);
+    std::vector<double> want_bias((size_t)N);
+    for (int64_t n = 0; n < N; ++n) { gbias[n] = next_float(); want_bias[(size_t)n] = gbias[n]; }
+    for (size_t i = 0; i < a_store; ++i) A[i] = next_float();
+    for (size_t i = 0; i < b_store; ++i) B[i] = next_float();
+    for (size_t i = 0; i < a_n; ++i) gA[i] = next_float();
+    for (size_t i = 0; i < b_n; ++i) gB[i] = next_float();
     for (size_t i = 0; i < c_n; ++i) dC[i] = next_float();
-    // storage: A[b] is [M][K] (n) or [K][M] (t); the gradients are dense at the VIEW's shape [.., M, K] / [.., K, N]
-    const int64_t a_rs = ta ? 1 : K, a_cs = ta ? M : 1, b_rs = tb ? 1 : N, b_cs = tb ? K : 1;
+    // storage: A[b] is [M][K] (n), [K][M] (t) or [M][2K] with every second element used (g); the gradients are dense at the VIEW's shape
+    const int64_t a_rs = ga ? 2 * K : ta ? 1 : K, a_cs = ga ? 2 : ta ? M : 1, b_rs = gb ? 2 * N : tb ? 1 : N, b_cs = gb ? 2 : tb ? K : 1;
     std::vector<double> wantA(a_n), wantB(b_n);
     for (size_t i = 0; i < a_n; ++i) wantA[i] = gA[i];
     for (size_t i = 0; i < b_n; ++i) wantB[i] = gB[i];
     for (int64_t c = 0; c < nc; ++c) {
         const int64_t ia = na > 1 ? c : 0, ib = nb > 1 ? c : 0;
-        const float* Ab = A + ia * M * K; const float* Bb = B + ib * K * N; const float* Gb = dC + c * M * N;
+        const float* Ab = A + ia * a_mat; const float* Bb = B + ib * b_mat; const float* Gb = dC + c * M * N;
         for (int64_t m = 0; m < M; ++m)
             for (int64_t k = 0; k < K; ++k) {
                 double s = 0.0;
@@ -375,18 +390,42 @@ static int run_backward_case(const std::string& spec) {
                 for (int64_t m = 0; m < M; ++m) s += (double)Ab[m * a_rs + k * a_cs] * (double)Gb[m * N + n];
                 wantB[(size_t)(ib * K * N + k * N + n)] += s;
             }
+        for (int64_t m = 0; m < M; ++m)
+            for (int64_t n = 0; n < N; ++n) want_bias[(size_t)n] += (double)Gb[m * N + n];
     }
-    replay_register(A, a_n * 4); replay_register(B, b_n * 4); replay_register(dC, c_n * 4); replay_register(gA, a_n * 4); replay_register(gB, b_n * 4);
-    tenmo_view va = view_of(A, ba, M, K, ta), vb = view_of(B, bb, K, N, tb);
+    replay_register(gbias, (size_t)N * 4);
+    replay_register(A, a_store * 4); replay_register(B, b_store * 4); replay_register(dC, c_n * 4); replay_register(gA, a_n * 4); replay_register(gB, b_n * 4);
+    tenmo_view va = view_of(A, ba, M, K, ta, ga), vb = view_of(B, bb, K, N, tb, gb);
     for (auto& kv : knobs) tenmo_hip_set_tuning(kv.first.c_str(), kv.second);
-    const int rc = tenmo_hip_matmul_backward(&va, &vb, dC, gA, gB, 1);
-    for (auto& kv : knobs) tenmo_hip_set_tuning(kv.first.c_str(), -1);
     int bad = 0;
-    double ea = -1, eb = -1;
+    long without_bias = 0;
+    if (linear) { // the same call without the bias gradient, into copies of the gradients: the number of launches to compare with
+        std::vector<float> sA(gA, gA + a_n), sB(gB, gB + b_n);
+        replay_register(sA.data(), a_n * 4); replay_register(sB.data(), b_n * 4);
+        const long before = replay_launch_count();
+        if (tenmo_hip_linear_backward(&va, &vb, dC, sA.data(), sB.data(), nullptr, 1) != 0) bad = 1;
+        without_bias = replay_launch_count() - before;
+        replay_register(sA.data(), 0); replay_register(sB.data(), 0);
+    }
+    const long before = replay_launch_count();
+    const int rc = linear ? tenmo_hip_linear_backward(&va, &vb, dC, gA, gB, gbias, 1) : tenmo_hip_matmul_backward(&va, &vb, dC, gA, gB, 1);
+    const long launches = replay_launch_count() - before;
+    for (auto& kv : knobs) tenmo_hip_set_tuning(kv.first.c_str(), -1);
+    double ea = -1, eb = -1, ebias = -1;
     if (rc != 0) { fprintf(stderr, "%s: error %d: %s\n", spec.c_str(), rc, tenmo_hip_last_error()); bad = 1; }
     else { ea = gradient_error(gA, wantA); eb = gradient_error(gB, wantB); if (!(ea <= 2e-6 && eb <= 2e-6)) bad = 1; }
+    if (linear && rc == 0) {
+        std::vector<float> got(gbias, gbias + N);
+        ebias = gradient_error(got.data(), want_bias);
+        if (!(ebias <= 2e-6)) bad = 1;
+        if (want_fused == 1 && launches != without_bias) bad = 1;
+        if (want_fused == 0 && launches <= without_bias) bad = 1;
+        printf("%s: %ld launches, %ld without the bias gradient; bias gradient error %.3g\n", spec.c_str(), launches, without_bias, ebias);
+    }
     printf("%s: rc %d, relative error %.3g / %.3g%s\n", spec.c_str(), rc, ea, eb, bad ? "  <-- FAILED" : "");
     fflush(stdout);
+    replay_register(gbias, 0);
+    free(gbias);
     replay_register(A, 0); replay_register(B, 0); replay_register(dC, 0); replay_register(gA, 0); replay_register(gB, 0);
     free(A); free(B); free(dC); free(gA); free(gB);
     return bad;
@@ -398,7 +437,7 @@ int main(int argc, char** argv) {
     for (int i = 1; i < argc; ++i) {
         if (!strcmp(argv[i], "late")) { replay_set_late_loads(1); continue; }
         if (!strcmp(argv[i], "early")) { replay_set_late_loads(0); continue; }
-        if (strncmp(argv[i], "bwd:", 4) == 0) bad |= run_backward_case(argv[i]);
+        if (strncmp(argv[i], "bwd:", 4) == 0 || strncmp(argv[i], "lin:", 4) == 0) bad |= run_backward_case(argv[i]);
         else if (strncmp(argv[i], "ce:", 3) == 0 || strncmp(argv[i], "conv:", 5) == 0 || strncmp(argv[i], "misc:", 5) == 0 || strncmp(argv[i], "mlp:", 4) == 0)
             bad |= run_address_only_case(argv[i]);
         else if (strncmp(argv[i], "mv:", 3) == 0) bad |= run_vector_case(argv[i], true);

@@ -187,6 +187,32 @@ def test_gradients_of_broadcast_parents(exe):
             cases.append(f"bwd:300,200,100,{la},{lb},1,3,fold_reduce={fold}")
     run(exe, cases, cus=8)
     run(exe, ["bwd:256,1024,512,n,n,0,4,fold_reduce=1", "bwd:512,256,1024,n,n,1,6"], cus=256, modes=("late",))
+    # an operand without a unit stride under a broadcast: the reducing launch with the element-wise loader
+    generic = []
+    for la, lb in (("g", "n"), ("n", "g"), ("g", "g"), ("g", "t"), ("t", "g")):
+        generic += [f"bwd:70,41,33,{la},{lb},0,5,fold_reduce=1", f"bwd:132,260,48,{la},{lb},3,1,fold_reduce=1", f"bwd:100,68,20,{la},{lb},1,4,fold_reduce=0"]
+    run(exe, generic, cus=8)
+
+
+def test_linear_backward_with_the_bias_gradient_in_the_weight_gradient_launch(exe):
+    """tenmo_hip_linear_backward: the B fragments of the weight-gradient product X^T . dY added up beside the MFMAs
+    (gemm_mfma_bsum_kernel, gemm_streamk_bsum_kernel): every tile, K slices (their sums added by the slice reduction),
+    stream-K (whole tiles onto the result, pieces through the fix-up), whole and ragged tiles, a batched input folded into
+    the reduction; `fused=1` makes the driver check that the call takes no launch more than without the bias gradient.
+    What the fused sum does not take — a transposed-view input, a batch whose rows do not stack — streams dY once more
+    (`fused=0`) and is still right."""
+    cases = []
+    for tile in (0, 1, 2, 3, 4):
+        cases.append(f"lin:300,130,70,n,n,0,0,fused=1,gemm_tile={tile}")
+        cases.append(f"lin:64,256,128,n,n,3,0,fused=1,gemm_tile={tile}")
+    for tile, sk in ((0, 2), (1, 1), (1, 2), (2, 1), (3, 2)):
+        cases.append(f"lin:1000,260,200,n,n,0,0,fused=1,gemm_tile={tile},gemm_streamk={sk}")
+        cases.append(f"lin:2100,132,68,n,n,0,0,fused=1,gemm_tile={tile},gemm_streamk={sk}")
+    for tile, splits in ((0, 3), (1, 4), (2, 2), (3, 8), (4, 5)):
+        cases.append(f"lin:1000,200,260,n,n,0,0,fused=1,gemm_tile={tile},gemm_splitk={splits}")
+    cases += ["lin:515,100,36,n,n,0,0,fused=1", "lin:40,12,4,n,n,0,0", "lin:300,130,70,t,n,0,0,fused=0", "lin:1,70,33,n,n,0,0,fused=1"]
+    run(exe, cases, cus=8)
+    run(exe, ["lin:2048,768,256,n,n,0,0,fused=1", "lin:512,768,768,n,n,4,0,fused=1"], cus=256, modes=("late",), timeout=1200)
 
 
 def test_matrix_vector_kernels(exe):

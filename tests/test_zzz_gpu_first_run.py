@@ -9,6 +9,8 @@ slices joined inside the column kernels' launch, the fused MLP launches, the K-s
 resident-A kernel), last the short-reduction kernel forced onto reductions that are no multiple of 16 — the one path that
 uses the masked direct load (its fault, an undeclared SCC clobber, is fixed; this is the run that confirms it).
 """
+import os
+
 import numpy as np
 import pytest
 
@@ -61,6 +63,38 @@ def test_backward_of_broadcast_parents(T, oracle, fold):
         out.backward(T.Tensor.from_numpy(seed))
         gA, gW = oracle.matmul_backward(sub, w, seed)
         assert rel_fro(W.grad(), gW) <= 2 * RTOL_FRO and rel_fro(A.grad(), gA) <= 2 * RTOL_FRO
+        # operands without a unit stride (every second row and column of their storage) under a broadcast: the reducing
+        # launch takes them through the element-wise loader instead of materialising the batched gradient
+        for sa, sb in (((70, 33), (5, 33, 41)), ((3, 1, 40, 24), (4, 24, 36)), ((4, 50, 32), (32, 68))):
+            a2 = rng.standard_normal(sa[:-2] + (2 * sa[-2], 2 * sa[-1]), dtype=np.float32)
+            b2 = rng.standard_normal(sb[:-2] + (2 * sb[-2], 2 * sb[-1]), dtype=np.float32)
+            av, bv = a2[..., ::2, ::2], b2[..., ::2, ::2]
+            A, B = as_strided_tensor(T, av, requires_grad=True), as_strided_tensor(T, bv, requires_grad=True)
+            out = A.matmul(B)
+            seed = rng.standard_normal(out.shape(), dtype=np.float32)
+            out.backward(T.Tensor.from_numpy(seed), retain_graph=True)
+            out.backward(T.Tensor.from_numpy(seed))
+            gA, gB = oracle.matmul_backward(np.ascontiguousarray(av), np.ascontiguousarray(bv), seed)
+            assert rel_fro(A.grad(), 2 * gA) <= 2 * RTOL_FRO and rel_fro(B.grad(), 2 * gB) <= 2 * RTOL_FRO, (fold, sa, sb)
+        # vector . matrix with the vector shared by the batches (tenmo/vectormatrix.mojo:18-206): its gradient is the sum over
+        # the batches of M_b . dy_b; and matrix . vector likewise (tenmo/matrixvector.mojo:19-201)
+        for vs, ms in (((48,), (5, 48, 70)), ((1, 33), (3, 2, 33, 20)), ((1030,), (2, 1030, 515))):
+            vn = rng.standard_normal(vs, dtype=np.float32)
+            mn = rng.standard_normal(ms, dtype=np.float32)
+            V, M = T.Tensor.from_numpy(vn, True), T.Tensor.from_numpy(mn, True)
+            out = V.matmul(M, mode=T.vm)
+            seed = rng.standard_normal(out.shape(), dtype=np.float32)
+            out.backward(T.Tensor.from_numpy(seed))
+            gv, gm = oracle.vm_backward(vn, mn, seed)
+            assert rel_fro(V.grad(), gv) <= 2 * RTOL_FRO and rel_fro(M.grad(), gm) <= 2 * RTOL_FRO, (fold, vs, ms)
+            assert rel_fro(V.grad(), np.einsum("...kn,...n->...k", mn.astype(np.float64), seed.astype(np.float64)).reshape(-1, vs[-1]).sum(0).reshape(vs)) <= RTOL_FRO
+            mt = np.ascontiguousarray(np.swapaxes(mn, -1, -2))  # [.., n, k] . v[k]
+            V, M = T.Tensor.from_numpy(vn, True), T.Tensor.from_numpy(mt, True)
+            out = M.matmul(V, mode=T.mv)
+            seed = rng.standard_normal(out.shape(), dtype=np.float32)
+            out.backward(T.Tensor.from_numpy(seed))
+            gm, gv = oracle.mv_backward(mt, vn, seed)
+            assert rel_fro(V.grad(), gv) <= 2 * RTOL_FRO and rel_fro(M.grad(), gm) <= 2 * RTOL_FRO, (fold, vs, ms)
     finally:
         L.tenmo_hip_set_tuning(b"fold_reduce", -1)
 
@@ -245,3 +279,76 @@ def test_short_reduction_kernel_layouts_and_k_tails(T, smallk):
                     assert err <= RTOL_FRO, (smallk, bshape, M, N, K, acc, ta, tb, err)
     finally:
         L.tenmo_hip_set_tuning(b"gemm_smallk", -1)
+
+
+def test_linear_backward_sums_the_bias_gradient_in_the_weight_gradient_launch(T, oracle):
+    """tenmo_hip_linear_backward: dX, dW and the bias gradient of x.W + b (tenmo/net.mojo:193-201 = Matmul then Adder; the
+    bias gradient is sum_over_broadcasted_axes of the upstream gradient, tenmo/broadcast.mojo:66-88) against the oracle
+    and fp64, twice in a row (the second call accumulates), for matrix and batched inputs, whole and ragged tiles — with
+    the weight-gradient launch forced through every tile, K slices and stream-K, each of which adds up its dY fragments
+    its own way — and for the forms that take the separate pass over dY instead (a transposed-view input, no dW wanted)."""
+    import ctypes as C
+
+    L, lib = T.lib.load(), T.lib
+    rng = np.random.default_rng(97)
+    knobs = [{}, {"gemm_tile": 0}, {"gemm_tile": 1}, {"gemm_tile": 2}, {"gemm_tile": 3}, {"gemm_tile": 4}, {"gemm_tile": 1, "gemm_splitk": 4},
+             {"gemm_tile": 0, "gemm_splitk": 3}, {"gemm_tile": 1, "gemm_streamk": 1}, {"gemm_tile": 0, "gemm_streamk": 2}, {"gemm_tile": 3, "gemm_streamk": 2},
+             {"gemm_tile": 2, "gemm_streamk": 1}]
+    shapes = [((64, 96), 40), ((300, 130), 70), ((3, 50, 64), 36), ((2, 2, 33, 20), 132), ((1000, 260), 200)]
+    if not os.environ.get("TENMO_TEST_SMALL"):
+        shapes.append(((2048, 768), 1024))
+
+    def run(x, w, dy, xt=None, want=(True, True, True)):
+        """One call through the C ABI on fresh zero gradients, then a second one on top; returns the three gradients."""
+        X = T.Tensor.from_numpy(x if xt is None else xt)
+        Xv = X if xt is None else X.transpose(-1, -2)
+        W, dY = T.Tensor.from_numpy(w), T.Tensor.from_numpy(dy)
+        outs = [T.Tensor.zeros(*a.shape) if on else None for a, on in zip((x, w, np.zeros(w.shape[-1], np.float32)), want)]
+        for _ in range(2):
+            lib.check(L.tenmo_hip_linear_backward(C.byref(Xv.buffer.c_view()), C.byref(W.buffer.c_view()), dY.buffer.data_ptr(),
+                                                  *[(o.buffer.data_ptr() if o is not None else None) for o in outs], 1))
+        return [o.to_numpy() if o is not None else None for o in outs]
+
+    try:
+        for xs, n_out in shapes:
+            x = rng.standard_normal(xs, dtype=np.float32)
+            w = rng.standard_normal((xs[-1], n_out), dtype=np.float32)
+            dy = rng.standard_normal(xs[:-1] + (n_out,), dtype=np.float32)
+            gx, gw = oracle.matmul_backward(x, w, dy)
+            gb = oracle.sum_over_broadcasted_axes(dy, (n_out,))
+            gb64 = dy.astype(np.float64).reshape(-1, n_out).sum(0)
+            assert rel_fro(gb, gb64) <= RTOL_FRO
+            for knob in knobs if len(xs) == 2 or xs == (3, 50, 64) else knobs[:1]:
+                for name, value in knob.items():
+                    L.tenmo_hip_set_tuning(name.encode(), value)
+                try:
+                    dx, dw, db = run(x, w, dy)
+                finally:
+                    for name in knob:
+                        L.tenmo_hip_set_tuning(name.encode(), -1)
+                assert rel_fro(dx, 2 * gx) <= 2 * RTOL_FRO and rel_fro(dw, 2 * gw) <= 2 * RTOL_FRO, (xs, n_out, knob)
+                assert rel_fro(db, 2 * gb64) <= RTOL_FRO and rel_fro(db, 2 * gb.astype(np.float64)) <= 2 * RTOL_FRO, (xs, n_out, knob)
+            # what the fused sum does not take: a transposed-view input, and a call that wants no weight gradient
+            dx, dw, db = run(x, w, dy, xt=np.ascontiguousarray(np.swapaxes(x, -1, -2)))
+            assert rel_fro(dx, 2 * gx) <= 2 * RTOL_FRO and rel_fro(dw, 2 * gw) <= 2 * RTOL_FRO and rel_fro(db, 2 * gb64) <= RTOL_FRO, (xs, n_out)
+            dx, dw, db = run(x, w, dy, want=(True, False, True))
+            assert dw is None and rel_fro(dx, 2 * gx) <= 2 * RTOL_FRO and rel_fro(db, 2 * gb64) <= RTOL_FRO, (xs, n_out)
+            dx, dw, db = run(x, w, dy, want=(False, True, False))
+            assert dx is None and db is None and rel_fro(dw, 2 * gw) <= 2 * RTOL_FRO, (xs, n_out)
+        # through the layer of the host mirror: Linear forward, backward from a seed, gradients of x, W and b
+        from tenmo_amd.net import Linear
+
+        lin = Linear(130, 70, np.random.default_rng(5))
+        x = rng.standard_normal((4, 75, 130), dtype=np.float32)
+        X = T.Tensor.from_numpy(x, True)
+        out = lin(X)
+        seed = rng.standard_normal(out.shape(), dtype=np.float32)
+        out.backward(T.Tensor.from_numpy(seed))
+        w = lin.weight.to_numpy()
+        gx, gw = oracle.matmul_backward(x, w, seed)
+        assert rel_fro(out.to_numpy(), ref_matmul64(x, w) + lin.bias.to_numpy()) <= RTOL_FRO
+        assert rel_fro(X.grad(), gx) <= 2 * RTOL_FRO and rel_fro(lin.weight.grad(), gw) <= 2 * RTOL_FRO
+        assert rel_fro(lin.bias.grad(), seed.astype(np.float64).reshape(-1, 70).sum(0)) <= RTOL_FRO
+    finally:
+        for name in ("gemm_tile", "gemm_splitk", "gemm_streamk"):
+            L.tenmo_hip_set_tuning(name.encode(), -1)
