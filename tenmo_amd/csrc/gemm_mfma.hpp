@@ -998,7 +998,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void gemm_reduce_kernel(const Gemm
     dst.ld = g.N; dst.row0 = 0; dst.col0 = 0;
     dst.base = g.C + batch * g.M * g.N;
     dst.fused = false;
-    for (int64_t r = 0; r < red.count; ++r) {
+    const uint32_t rounds = (uint32_t)red.count; // (below 2^31: it is a factor of the result's batch count)
+    for (uint32_t r = 0; r < rounds; ++r) {
         int64_t a_roff, b_roff;
         batch_offsets(red.dims, r, a_roff, b_roff);
         dst.accumulate = r > 0 || g.accumulate != 0;
@@ -1046,22 +1047,22 @@ __global__ __launch_bounds__(GEMM_THREADS, (BM * BN <= 128 * 64 ? 4 : 2)) void g
     __shared__ __attribute__((aligned(1024))) float stage1[STAGE_FLOATS];
     __shared__ __attribute__((aligned(1024))) float stage2[DIRECT ? STAGE_FLOATS : 4];
     const uint32_t tiles = (uint32_t)g.tiles_m * (uint32_t)g.tiles_n; // tile ids, batches included, are below 2^31
-    const int64_t w = blockIdx.x;
+    // (every count of the schedule is below 2^31 — the host refuses larger ones — and is kept in 32 bits: the persistent
+    // loop's state lives in scalar registers beside the tile function's, which are nearly all in use)
+    const uint32_t w = blockIdx.x, nks = (uint32_t)sk.nks, dp_tiles = (uint32_t)sk.dp_tiles;
     uint32_t whole = blockIdx.x; // next tile of the data-parallel part
-    int64_t it = w * sk.per_wg;
-    const int64_t end = min(sk.total, it + sk.per_wg);
+    uint32_t it = w * (uint32_t)sk.per_wg;
+    const uint32_t end = min((uint32_t)sk.total, it + (uint32_t)sk.per_wg);
     for (;;) { // one call site for gemm_tile: the function is large
-        uint32_t gt;
-        int64_t k0, k1;
-        const bool is_whole = whole < (uint32_t)sk.dp_tiles;
-        if (is_whole) {
-            gt = whole; k0 = 0; k1 = sk.nks;
+        uint32_t gt, k0, k1;
+        if (whole < dp_tiles) {
+            gt = whole; k0 = 0; k1 = nks;
             whole += gridDim.x;
         } else if (it < end) {
-            const int64_t st = it / sk.nks; // shared tile number
-            k0 = it - st * sk.nks;
-            k1 = min(sk.nks, k0 + (end - it));
-            gt = (uint32_t)(sk.dp_tiles + st);
+            const uint32_t st = it / nks; // shared tile number
+            k0 = it - st * nks;
+            k1 = min(nks, k0 + (end - it));
+            gt = dp_tiles + st;
             it += k1 - k0;
         } else {
             break;
@@ -1071,15 +1072,15 @@ __global__ __launch_bounds__(GEMM_THREADS, (BM * BN <= 128 * 64 ? 4 : 2)) void g
         int64_t tile_m, tile_n;
         tile_coords_blocked<BM, BN>(g, gt - batch32 * tiles, tile_m, tile_n); // one numbering for both parts and the fix-up
         TileDest dst;
-        if (k0 == 0 && k1 == sk.nks) {
+        if (k0 == 0 && k1 == nks) {
             dst.base = g.C + batch * g.M * g.N; dst.ld = g.N; dst.row0 = 0; dst.col0 = 0;
             dst.accumulate = g.accumulate != 0; dst.fused = true;
         } else {
-            dst.base = sk.partial + (2 * w + (k0 == 0 ? 1 : 0)) * (int64_t)(BM * BN); dst.ld = BN;
+            dst.base = sk.partial + (uint64_t)(2 * w + (k0 == 0 ? 1 : 0)) * (uint64_t)(BM * BN); dst.ld = BN;
             dst.row0 = tile_m * BM; dst.col0 = tile_n * BN;
             dst.accumulate = false; dst.fused = false;
         }
-        gemm_tile<BM, BN, AMODE, BMODE>(g, stage0, stage1, stage2, batch, tile_m, tile_n, k0 * GEMM_BK, min(g.K, k1 * GEMM_BK), dst);
+        gemm_tile<BM, BN, AMODE, BMODE>(g, stage0, stage1, stage2, batch, tile_m, tile_n, (int64_t)k0 * GEMM_BK, min(g.K, (int64_t)k1 * GEMM_BK), dst);
     }
 }
 

@@ -65,9 +65,13 @@ bool TENMO_NAME(launch_streamk_, TENMO_TILE_BM, TENMO_TILE_BN)(const GemmArgs& g
 #define TENMO_CASE(A_, B_)                                                                                               \
     if (amode == A_ && bmode == B_)                                                                                      \
         hipLaunchKernelGGL((gemm_streamk_kernel<BM, BN, A_, B_>), dim3(wgs), dim3(GEMM_THREADS), 0, stream, g, sk);
-    if (bsum != nullptr) {
+    if (bsum != nullptr) { // (the 128x128 tile only: the others have no registers left for the sums without spilling inside their loops)
+#if TENMO_TILE_BM == 128 && TENMO_TILE_BN == 128
         if (amode != MNMAJOR_VEC || bmode != MNMAJOR_VEC) return false;
         hipLaunchKernelGGL((gemm_streamk_bsum_kernel<BM, BN, MNMAJOR_VEC, MNMAJOR_VEC>), dim3(wgs), dim3(GEMM_THREADS), 0, stream, g, sk, *bsum);
+#else
+        return false;
+#endif
     } else
     TENMO_CASE(KMAJOR_VEC, KMAJOR_VEC) else TENMO_CASE(KMAJOR_VEC, MNMAJOR_VEC) else TENMO_CASE(MNMAJOR_VEC, KMAJOR_VEC) else TENMO_CASE(MNMAJOR_VEC, MNMAJOR_VEC)
     else return false;

@@ -441,6 +441,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
     if (S.force_splitk > 0 && !ep.bias_rows && !ep.colsum) splits = S.force_splitk; // the slice reduction applies the bias by column only
     int streamk = S.force_streamk > 0 && !ep.colsum ? S.force_streamk : 0;
     if (S.force_streamk < 0 && sk_wpc > 0 && S.force_tile < 0 && S.force_splitk <= 0) { streamk = sk_wpc; tile = sk_tile; }
+    if (streamk > 0 && ep.bsum) tile = 1; // the one stream-K kernel that also adds up the column sums of B
     if (streamk > 0 && tile <= 3 && am != KMAJOR_GEN && bm != KMAJOR_GEN && (!ep.gather_row || tile >= 2)) {
         const int bmt = kTiles[tile].bm, bnt = kTiles[tile].bn;
         g.tiles_m = (int32_t)((M + bmt - 1) / bmt);

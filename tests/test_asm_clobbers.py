@@ -228,3 +228,61 @@ def test_generated_isa_has_no_user_of_m0_outside_the_asm_blocks(device_isa):
         assert scan_m0(isa) == [], name
         blocks += isa.count("s_mov_b32 m0,")
     assert blocks > 1000
+
+
+def innermost_loops(text):
+    """(kernel, label, instructions) of every innermost loop: the instructions from a label to a branch back to it that
+    enclose no other backward branch."""
+    loops = []
+    kernels, name, code = [], None, []
+    for line in text.split("\n"):
+        m = re.match(r"^(_Z\S+):", line)
+        if m:
+            if name:
+                kernels.append((name, code))
+            name, code = m.group(1), []
+            continue
+        if name is None:
+            continue
+        m = re.match(r"^(\.LBB\S+):", line)
+        if m:
+            code.append(m.group(1) + ":")
+            continue
+        c = line.split(";")[0].strip()
+        if c and not c.startswith("."):
+            code.append(c)
+    if name:
+        kernels.append((name, code))
+    for name, code in kernels:
+        at = {c[:-1]: i for i, c in enumerate(code) if c.endswith(":")}
+        back = [(at[c.split()[-1]], i) for i, c in enumerate(code) if c.startswith(("s_cbranch", "s_branch")) and at.get(c.split()[-1], i) < i]
+        for lo, hi in back:
+            if not any((l2, h2) != (lo, hi) and lo <= l2 and h2 <= hi for l2, h2 in back):
+                loops.append((name, code[lo][:-1], [c for c in code[lo:hi + 1] if not c.endswith(":")]))
+    return loops
+
+
+@pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")
+def test_no_spilled_register_is_touched_inside_a_k_loop(device_isa):
+    """Some persistent kernels (stream-K, the batch-reducing launch) keep so much state across their tiles that the compiler
+    spills a few registers to scratch memory.  That is harmless as long as the spills sit in the per-tile prologue and
+    epilogue: the loops that issue MFMAs — the K loops, where the time goes — must not read or write scratch memory."""
+    mfma_loops = 0
+    for name, isa in device_isa.items():
+        for kernel, label, body in innermost_loops(isa):
+            if not any(i.startswith("v_mfma") for i in body):
+                continue
+            mfma_loops += 1
+            touched = [i for i in body if i.startswith("scratch_") or i.startswith("buffer_") and "offen" in i and "s[0:3]" in i]
+            assert not touched, (name, kernel, label, touched[:3])
+    assert mfma_loops > 150
+
+
+def test_the_loop_scan_sees_a_spill():
+    bad = "_Zkernel:\n.LBB0_1:\n\tv_mfma_f32_32x32x2_f32 a[0:15], v0, v1, a[0:15]\n\tscratch_load_dword v3, off, off offset:4\n\ts_cbranch_vccnz .LBB0_1\n\ts_endpgm\n"
+    loops = innermost_loops(bad)
+    assert len(loops) == 1 and any(i.startswith("scratch_") for i in loops[0][2])
+    assert innermost_loops(bad.replace("s_cbranch_vccnz .LBB0_1", "s_cbranch_vccnz .LBB0_2")) == []
+    # an outer loop around it is not what is checked: only the inner one counts
+    nested = bad.replace(".LBB0_1:", ".LBB0_0:\n\tscratch_load_dword v9, off, off\n.LBB0_1:").replace("\ts_endpgm", "\ts_cbranch_scc1 .LBB0_0\n\ts_endpgm")
+    assert [l[1] for l in innermost_loops(nested)] == [".LBB0_1"]
