@@ -357,6 +357,21 @@ def test_cross_entropy_oracle_is_pinned(golden, oracle):
         assert abs(grad[i, j] - fd) < 1e-5
 
 
+def test_bias_gradient_oracle_is_pinned(golden, oracle):
+    """sum_over_broadcasted_axes (tenmo/broadcast.mojo:66-88), the gradient of a bias under Adder: the reference's own literals."""
+    case = golden["harness"]["bias_gradient_is_column_sums"]
+    up = np.array(case["upstream"], np.float32)
+    assert np.array_equal(oracle.sum_over_broadcasted_axes(up, (1, 4)), np.array([case["expect"]], np.float32))
+    assert np.array_equal(oracle.sum_over_broadcasted_axes(up, (4,)), np.array(case["expect"], np.float32))
+    case = golden["harness"]["sum_over_broadcasted_axes_of_ones"]
+    got = oracle.sum_over_broadcasted_axes(np.ones(case["shape"], np.float32), tuple(case["target_shape"]))
+    assert got.shape == tuple(case["target_shape"]) and np.array_equal(got.ravel(), np.array(case["expect"], np.float32))
+    # and against numpy on random data, a partial broadcast
+    rng = np.random.default_rng(5)
+    x = rng.standard_normal((3, 4, 5, 6), dtype=np.float32)
+    assert np.allclose(oracle.sum_over_broadcasted_axes(x, (4, 1, 6)), x.astype(np.float64).sum(axis=(0, 2), keepdims=True)[0], rtol=1e-5, atol=1e-6)
+
+
 def test_sgd_oracle_is_pinned(golden, oracle):
     """tests/test_sgd.mojo vectors: plain, weight decay, momentum over three steps."""
     H = golden["harness"]

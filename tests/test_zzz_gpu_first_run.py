@@ -281,6 +281,28 @@ def test_short_reduction_kernel_layouts_and_k_tails(T, smallk):
         L.tenmo_hip_set_tuning(b"gemm_smallk", -1)
 
 
+def test_linear_backward_reference_literal(T, golden):
+    """The reference's own literal for the gradient of a broadcast bias (tests/test_expand.mojo:229-245): whatever the input and the
+    weight, the bias gradient of x.W + b is the upstream gradient summed over its rows — through tenmo_hip_linear_backward (here the
+    three rows take the separate pass: in_features <= 8) and through tenmo_hip_column_sum_f32."""
+    import ctypes as C
+
+    L, lib = T.lib.load(), T.lib
+    case = golden["harness"]["bias_gradient_is_column_sums"]
+    up = np.array(case["upstream"], np.float32)
+    for k in (2, 20):
+        X, W, dY = T.Tensor.from_numpy(np.ones((3, k), np.float32)), T.Tensor.from_numpy(np.ones((k, 4), np.float32)), T.Tensor.from_numpy(up)
+        gb = T.Tensor.zeros(4)
+        gw = T.Tensor.zeros(k, 4)
+        lib.check(L.tenmo_hip_linear_backward(C.byref(X.buffer.c_view()), C.byref(W.buffer.c_view()), dY.buffer.data_ptr(), None, gw.buffer.data_ptr(),
+                                              gb.buffer.data_ptr(), 1))
+        assert np.array_equal(gb.to_numpy(), np.array(case["expect"], np.float32)), k
+        assert np.array_equal(gw.to_numpy(), np.tile(np.array(case["expect"], np.float32), (k, 1))), k  # X = ones: every row of dW is the same sums
+    out, upstream = T.Tensor.zeros(4), T.Tensor.from_numpy(up)
+    lib.check(L.tenmo_hip_column_sum_f32(upstream.buffer.data_ptr(), 0, 4, 3, 4, out.buffer.data_ptr(), 0, 1))
+    assert np.array_equal(out.to_numpy(), np.array(case["expect"], np.float32))
+
+
 def test_linear_backward_sums_the_bias_gradient_in_the_weight_gradient_launch(T, oracle):
     """tenmo_hip_linear_backward: dX, dW and the bias gradient of x.W + b (tenmo/net.mojo:193-201 = Matmul then Adder; the
     bias gradient is sum_over_broadcasted_axes of the upstream gradient, tenmo/broadcast.mojo:66-88) against the oracle
