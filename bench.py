@@ -20,6 +20,13 @@ bytes / 8 TB/s), the fraction of that roof, and the relative Frobenius error of 
 against fp64.  Products whose operands and result would fit the chip's 256 MB memory-side cache are
 timed over several copies of their buffers in rotation, so that every launch reads from HBM.
 `extra` also holds the MLP training step in ms on GPU and CPU and the shader clock under load.
+
+A full run (neither `--no-cpu` nor `--no-extra`) only coordinates in the process started from the command line: the headline,
+the rows and the CPU baseline with the MLP step are measured by three child processes, one after the other, and their
+results are merged into the one line.  A failure in a row then costs that row and the ones behind it, not the headline;
+after a child that died of a signal nothing more is started on the GPU.  A run with `--no-cpu` or `--no-extra` (one thing
+measured, typically under a profiler, which follows one program: `rocprofv3 ... -- python3 bench.py --rows cbow --no-cpu`)
+and any run with `--single-process` measure in the process itself.
 """
 from __future__ import annotations
 
@@ -77,22 +84,108 @@ def main() -> int:
                     help="also time the adjacent operators (cross-entropy, SGD step, convolution) into `extra`; off by default")
     ap.add_argument("--pmc-calibration", action="store_true",
                     help="also run one plain 1 GiB device copy, the known-size kernel against which FETCH_SIZE/WRITE_SIZE are scaled")
+    ap.add_argument("--single-process", action="store_true",
+                    help="measure everything in this process.  A full run (no --no-cpu, no --no-extra) otherwise only coordinates: the "
+                    "headline, the rows and the CPU / MLP leg each run in a child process of their own, so that a failure in an "
+                    "additional measurement cannot take the headline with it")
+    ap.add_argument("--phase", default="", help=argparse.SUPPRESS)            # headline | rows | cpu: what a child process measures
+    ap.add_argument("--worker-launcher", default="", help=argparse.SUPPRESS)  # how to start a child (tests: a wrapper around this file)
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU (the reference has no multi-GPU path and every "
               "configuration fits one MI355X); --gpus %d is not supported" % args.gpus, file=sys.stderr)
         return 2
+    # (a run that leaves out the CPU leg or the rows is a measurement of one thing, typically under a profiler: one process)
+    if not args.single_process and not args.phase and not args.no_cpu and not args.no_extra:
+        return coordinate(args)
+    phases = {args.phase} if args.phase else {"headline", "rows", "cpu"}
+    out, rc = measure(args, phases)
+    print(json.dumps(out), flush=True)
+    return rc
 
+
+def coordinate(args) -> int:
+    """Runs the phases in child processes and prints the one line.  This process never touches the GPU."""
+    import shlex
+    import subprocess
+
+    launcher = shlex.split(args.worker_launcher) if args.worker_launcher else [sys.executable, os.path.abspath(__file__)]
+    passed = [a for a in sys.argv[1:]]
+
+    def child(phase):
+        """(dict printed by the child or None, how it ended)"""
+        proc = subprocess.Popen(launcher + passed + ["--phase", phase], stdout=subprocess.PIPE, text=True, cwd=ROOT)  # stderr passes through
+        last = None
+        partial_rows = []
+        for line in proc.stdout:
+            line = line.strip()
+            if not line.startswith("{"):
+                continue
+            try:
+                obj = json.loads(line)
+            except ValueError:
+                continue
+            if "row_done" in obj:
+                partial_rows.append(obj["row_done"])
+            else:
+                last = obj
+        code = proc.wait()
+        return last, partial_rows, code
+
+    out, _, code = child("headline")
+    if out is None:
+        print("bench.py: the headline measurement ended with status %d and printed no result" % code, file=sys.stderr)
+        return code or 1
+    extra = out.pop("extra", {})
+    gates = out.pop("gates", {})
+    ok = code == 0
+    gpu_alive = True
+    if not args.no_extra:
+        got, partial_rows, code = child("rows")
+        if got is not None:
+            extra.update(got.get("extra", {}))
+            gates.update({k: v for k, v in got.get("gates", {}).items() if k != "max_rel_err_vs_fp64"})
+            gates["max_rel_err_vs_fp64"] = max(gates.get("max_rel_err_vs_fp64", 0.0), got.get("gates", {}).get("max_rel_err_vs_fp64", 0.0))
+        else:  # the child died: keep what it had finished, name where it stopped, start nothing more on the GPU
+            extra["rows"] = partial_rows
+            extra["rows_error"] = "the process measuring the rows ended with status %d after %d rows" % (code, len(partial_rows))
+            gpu_alive = code >= 0 and code not in (124, 134, 137, 139)
+        ok = ok and code == 0 and got is not None
+    if not args.no_cpu:
+        got, _, code = child("cpu" if gpu_alive else "cpu-only")
+        if got is not None:
+            if "cpu_baseline" in got:
+                out["cpu_baseline"] = got["cpu_baseline"]
+            extra.update(got.get("extra", {}))
+            gates.update({k: v for k, v in got.get("gates", {}).items() if k == "mlp_loss_ok"})
+        else:
+            extra["cpu_baseline_error"] = "the process measuring the CPU baseline and the MLP step ended with status %d" % code
+        ok = ok and code == 0 and got is not None
+    if extra:
+        out["extra"] = extra
+    gates["rel_err_ok"] = gates.get("max_rel_err_vs_fp64", 1.0) <= 1e-5
+    gates["measurements_ok"] = ok and not any(k.endswith("_error") for k in extra)
+    out["gates"] = gates
+    print(json.dumps(out), flush=True)
+    return 0 if gates["rel_err_ok"] and gates.get("mlp_loss_ok", True) and gates["measurements_ok"] else 1
+
+
+def measure(args, phases):
+    """The phases in this process: (the result dict, exit status)."""
     import numpy as np
     import torch
 
     from tenmo_amd import _lib
 
+    if phases == {"cpu-only"}:  # (after a GPU failure in another phase: the CPU baseline alone, nothing of this process touches the GPU)
+        return measure_more(args, phases, {}, 0.0, None, _lib, torch, np)
     _lib.init(0)
     L = _lib.load()
     cus = C.c_int()
     name = C.create_string_buffer(128)
     L.tenmo_hip_device_info(C.byref(cus), name, 128)
+    if "headline" not in phases:
+        return measure_more(args, phases, {}, 0.0, L, _lib, torch, np)
 
     if args.pmc_calibration:
         src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
@@ -167,7 +260,14 @@ def main() -> int:
     # the headline so far, on stderr: a run that is cut short in the additional measurements still shows it (stdout carries
     # the one complete line at the end)
     print("bench headline (the complete line follows on stdout): " + json.dumps(out), file=sys.stderr, flush=True)
+    return measure_more(args, phases, out, rel_err, L, _lib, torch, np)
 
+
+def measure_more(args, phases, out, rel_err, L, _lib, torch, np):
+    """The additional measurements (phases "rows" and "cpu") on top of the headline dict `out`."""
+    S = args.size
+    gen = torch.Generator(device="cuda") if phases != {"cpu-only"} else None
+    mhz = C.c_float()
     # The headline line is printed whatever becomes of the additional measurements: an exception in one of them is
     # recorded under its name and the others still run.
     extra = {}
@@ -183,7 +283,7 @@ def main() -> int:
             extra[name + "_error"] = "%s: %s" % (type(e).__name__, e)
             return None
 
-    if not args.no_extra:
+    if not args.no_extra and "rows" in phases:
         only = [s for s in args.rows.split(",") if s]
 
         def rows_under(tune_list):
@@ -192,7 +292,7 @@ def main() -> int:
             for name_, value_ in tuned:
                 _lib.check(L.tenmo_hip_set_tuning(name_.strip().encode(), int(value_)))
             try:
-                return {n.strip(): int(v) for n, v in tuned}, config_rows(L, _lib, torch, only)
+                return {n.strip(): int(v) for n, v in tuned}, config_rows(L, _lib, torch, only, announce=phases == {"rows"})
             finally:
                 for name_, _ in tuned:
                     L.tenmo_hip_set_tuning(name_.strip().encode(), -1 if name_.strip() != "mlp_fused_tail" else 0)
@@ -219,10 +319,15 @@ def main() -> int:
         after = attempt("effective_mhz_after_rows", clock_after_rows)
         if after is not None:
             extra["effective_mhz_after_rows"] = after
-    if args.adjacent:
+    if args.adjacent and "rows" in phases:
         extra.update(attempt("adjacent", lambda: adjacent_operators(L, _lib, torch)) or {})
-    if not args.no_cpu:
+    if not args.no_cpu and ("cpu" in phases or "cpu-only" in phases):
         def cpu_leg():
+            # the same operands as the headline's (the same seeded generator; on the host when the GPU is not to be used any more)
+            if gen is None:
+                host = torch.Generator()
+                host.manual_seed(8192)
+                return cpu_gemm_baseline(torch.randn((S, S), generator=host), torch.randn((S, S), generator=host), S, np)
             gen.manual_seed(8192)
             A = torch.randn((S, S), generator=gen, device="cuda", dtype=torch.float32)
             B = torch.randn((S, S), generator=gen, device="cuda", dtype=torch.float32)
@@ -231,7 +336,7 @@ def main() -> int:
         baseline = attempt("cpu_baseline", cpu_leg)
         if baseline is not None:
             out["cpu_baseline"] = baseline
-        if not args.no_extra:
+        if not args.no_extra and "cpu" in phases:
             extra.update(attempt("mlp_step", lambda: mlp_step_times(_lib, torch, np, args.mlp_fused_tail)) or {})
     if extra:
         out["extra"] = extra
@@ -239,8 +344,7 @@ def main() -> int:
     # run at every one of its steps, and no additional measurement failed
     mlp_ok = extra.get("mlp_max_abs_loss_diff", 0.0) <= MLP_LOSS_TOLERANCE
     out["gates"] = {"max_rel_err_vs_fp64": worst, "rel_err_ok": worst <= 1e-5, "mlp_loss_ok": mlp_ok, "measurements_ok": not failed}
-    print(json.dumps(out), flush=True)
-    return 0 if worst <= 1e-5 and mlp_ok and not failed else 1
+    return out, (0 if worst <= 1e-5 and mlp_ok and not failed else 1)
 
 
 def rel_fro_vs_fp64(torch, got, A, B):
@@ -277,8 +381,9 @@ def hip_time_us(L, _lib, fns, est_us):
     return sorted(groups)[1]
 
 
-def config_rows(L, _lib, torch, only):
-    """One row per product of the benchmark configurations (see the module docstring)."""
+def config_rows(L, _lib, torch, only, announce=False):
+    """One row per product of the benchmark configurations (see the module docstring).  `announce`: print every finished row
+    as a line of its own at once (a child process does: its parent then has the rows that were done if it dies later)."""
     rows = []
     gen = torch.Generator(device="cuda")
 
@@ -303,6 +408,8 @@ def config_rows(L, _lib, torch, only):
                      "tflops": round(flop / us / 1e6, 2), "gbps": round(nbytes / us / 1e3, 1),
                      "bound": "mfma" if t_mfma >= t_hbm else "hbm", "roof_us": round(roof, 2), "frac": round(roof / us, 4),
                      "rel_err_vs_fp64": rel_err, "buffer_copies": copies})
+        if announce:
+            print(json.dumps({"row_done": rows[-1]}), flush=True)
 
     def copies_for(nbytes):
         # enough copies of the buffers that a rotation through them exceeds the memory-side cache twice over

@@ -21,9 +21,34 @@ def _gpu_unavailable_reason():
         import torch
     except ImportError:
         return "torch is not importable"
-    if not torch.cuda.is_available():
+    # (counting devices does not initialise the GPU in this process; torch.cuda.is_available() would, and a process that
+    # has initialised the GPU should not start other programs any more — see early_c_driver_run below)
+    if torch.cuda.device_count() < 1:
         return "no GPU visible to this process"
     return None
+
+
+# The plain-C caller of the header (tests/c_abi_driver.c) is a program of its own.  It is started here, during collection,
+# before anything in this process has touched the GPU, and tests/test_y_c_abi_driver.py asserts on what it printed: on the GPU
+# machines a process that has initialised the GPU must not exec other programs, and whether a forked child of such a process
+# may is not something a test should find out.
+C_DRIVER_RESULT = {}
+
+
+def early_c_driver_run():
+    import subprocess
+
+    exe = os.path.join(ROOT, "tests", "_build", "c_abi_driver")
+    if not os.path.exists(exe):
+        C_DRIVER_RESULT["error"] = exe + " is not built (python __graft_entry__.py)"
+        return
+    env = dict(os.environ)
+    env["LD_LIBRARY_PATH"] = os.path.join(ROOT, "tenmo_amd") + os.pathsep + env.get("LD_LIBRARY_PATH", "")  # the library of THIS tree first
+    try:
+        run = subprocess.run([exe], capture_output=True, text=True, timeout=300, env=env)
+        C_DRIVER_RESULT.update(returncode=run.returncode, stdout=run.stdout, stderr=run.stderr)
+    except (OSError, subprocess.SubprocessError) as e:
+        C_DRIVER_RESULT["error"] = "%s: %s" % (type(e).__name__, e)
 
 
 def pytest_collection_modifyitems(config, items):
@@ -42,6 +67,8 @@ def pytest_collection_modifyitems(config, items):
         skip = pytest.mark.skip(reason="gpu test: " + reason)
         for it in gpu_items:
             it.add_marker(skip)
+    elif any(it.name == "test_driver_runs_on_the_gpu" for it in gpu_items) and not config.pluginmanager.has_plugin("torch_on_host"):
+        early_c_driver_run()
 
 
 @pytest.fixture(scope="session")

@@ -27,9 +27,15 @@ def run_bench(*flags):
     return subprocess.run([sys.executable, "-c", RUNNER] + list(flags), cwd=ROOT, env=env, capture_output=True, text=True, timeout=900)
 
 
-def test_one_json_line_with_every_field():
+@pytest.mark.parametrize("mode", ["children", "single-process"])
+def test_one_json_line_with_every_field(mode):
+    """Both ways of running it: the default (a coordinating process and one child per phase; here the children are started
+    through the same wrapper that puts torch's device on the host) and everything in one process."""
+    import shlex
+
+    how = ["--single-process"] if mode == "single-process" else ["--worker-launcher", " ".join(shlex.quote(a) for a in [sys.executable, "-c", RUNNER])]
     res = run_bench("--size", "256", "--steps", "2", "--warmup", "1", "--rows", "no-such-row", "--mlp-fused-tail", "--clock-probe-rounds", "4",
-                    "--sweep", "gemm_panel=0;gemm_panel=1,gemm_smallk=0")
+                    "--sweep", "gemm_panel=0;gemm_panel=1,gemm_smallk=0", *how)
     lines = [l for l in res.stdout.splitlines() if l.strip()]
     assert res.returncode == 0 and len(lines) == 1, res.stdout[-2000:] + res.stderr[-2000:]
     out = json.loads(lines[0])
@@ -61,3 +67,23 @@ def test_smoke_entry_runs_on_the_replay():
     res = subprocess.run([sys.executable, "-c", "import torch_on_host, __graft_entry__ as g; g.smoke()"], cwd=ROOT, env=env, capture_output=True, text=True,
                          timeout=900)
     assert res.returncode == 0 and "smoke ok" in res.stdout, res.stdout[-2000:] + res.stderr[-2000:]
+
+
+def test_a_dying_row_does_not_take_the_headline_with_it():
+    """The phase that measures the rows dies of a signal after one row (here: a wrapper that kills itself): the line still
+    carries the headline, the row that was finished and where it stopped; the CPU baseline is still measured, but
+    nothing more is started on the GPU (no MLP step), and the exit status says that something went wrong."""
+    import shlex
+
+    dying = ("import sys, os, json, signal\n"
+             "if sys.argv[sys.argv.index('--phase') + 1] == 'rows':\n"
+             "    print(json.dumps({'row_done': {'name': 'only_row', 'us': 1.0, 'frac': 0.5, 'rel_err_vs_fp64': 1e-7}}), flush=True)\n"
+             "    os.kill(os.getpid(), signal.SIGSEGV)\n") + RUNNER
+    res = run_bench("--size", "256", "--steps", "2", "--warmup", "1", "--clock-probe-rounds", "4",
+                    "--worker-launcher", " ".join(shlex.quote(a) for a in [sys.executable, "-c", dying]))
+    lines = [l for l in res.stdout.splitlines() if l.strip()]
+    assert res.returncode != 0 and len(lines) == 1, res.stdout[-2000:] + res.stderr[-2000:]
+    out = json.loads(lines[0])
+    assert out["value"] > 0 and out["roofline"]["frac"] > 0 and out["cpu_baseline"]["value"] > 0
+    assert [r["name"] for r in out["extra"]["rows"]] == ["only_row"] and "status -11" in out["extra"]["rows_error"]
+    assert "mlp_step_ms_gpu" not in out["extra"] and out["gates"]["measurements_ok"] is False
