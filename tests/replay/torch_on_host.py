@@ -73,6 +73,7 @@ def _install():
 
     torch.Tensor.to = to
     torch.cuda.is_available = lambda: True
+    torch.cuda.device_count = lambda: 1
     torch.cuda.current_stream = lambda *a, **k: _Stream()
     torch.cuda.synchronize = lambda *a, **k: None
     torch.cuda.empty_cache = lambda *a, **k: None

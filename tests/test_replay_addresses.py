@@ -36,11 +36,25 @@ def case(M, N, K, la="n", lb="n", batch=0, b_shared=0, acc=0, **knobs):
 
 def run(exe, cases, cus=256, modes=("early", "late"), timeout=600):
     env = dict(os.environ, REPLAY_CUS=str(cus), ASAN_OPTIONS="detect_leaks=0:detect_stack_use_after_return=0")
-    for mode in modes:
-        res = subprocess.run([exe, mode] + cases, capture_output=True, text=True, env=env, timeout=timeout)
-        tail = (res.stdout[-3000:] + "\n" + res.stderr[-6000:]).strip()
-        assert res.returncode == 0, f"mode {mode}, {cus} CUs:\n{tail}"
-        assert res.stdout.count("relative error") == len(cases), tail
+    # the cases are independent: both load models side by side, each over two halves of the list
+    halves = [cases[:(len(cases) + 1) // 2], cases[(len(cases) + 1) // 2:]] if len(cases) > 3 else [cases]
+    jobs = [(mode, part, subprocess.Popen([exe, mode] + part, stdout=subprocess.PIPE, stderr=subprocess.PIPE, text=True, env=env))
+            for mode in modes for part in halves if part]
+    failures = []
+    for mode, part, proc in jobs:
+        try:
+            out, err = proc.communicate(timeout=timeout)
+        except subprocess.TimeoutExpired:
+            proc.kill()
+            out, err = proc.communicate()
+            failures.append(f"mode {mode}, {cus} CUs: no end after {timeout} s\n" + (out[-3000:] + "\n" + err[-3000:]).strip())
+            continue
+        tail = (out[-3000:] + "\n" + err[-6000:]).strip()
+        if proc.returncode != 0:
+            failures.append(f"mode {mode}, {cus} CUs:\n{tail}")
+        elif out.count("relative error") != len(part):
+            failures.append(tail)
+    assert not failures, "\n\n".join(failures)
 
 
 def test_the_checks_bite():

@@ -37,7 +37,7 @@ def run_child(files, extra=()):
     try:
         import xdist  # noqa: F401
 
-        cmd += ["-n", "4"]
+        cmd += ["-n", str(min(8, os.cpu_count() or 1))]
     except ImportError:
         pass
     res = subprocess.run(cmd, cwd=ROOT, env=env, capture_output=True, text=True, timeout=3000)
