@@ -68,7 +68,8 @@ int tenmo_hip_device_info(int* compute_units, char* name, int name_len);
  * 2: 64x64, 3: 128x64, 4: 64x128 workgroup tile; -1 automatic), "gemm_splitk" (number of K slices;
  * -1 automatic), "gemm_streamk" (n > 0: persistent stream-K launch with n workgroups per CU, at most two, for the
  * 256x128 / 128x128 tiles, 0: never, -1 automatic), "gemm_smallk" (the persistent short-reduction kernel, K of 17 up to 64 and a plain
- * or accumulating store: 1 wherever it can run, 0 never, -1 automatic: for results of 2048 and more 64x64 tiles),
+ * or accumulating store: 1 wherever it can run, 3 the same and also for K up to 16 — a path the automatic choice does not take —, 0 never,
+ * -1 automatic: for results of 2048 and more 64x64 tiles and K a multiple of 16),
  * "gemm_panel" (the persistent K-stream kernel with loading wavefronts of its own, 128x128 tiles, K above 16, plain or
  * accumulating store: 1 wherever it can run, 3 the same with 64x64 tiles and a deeper ring, 4 / 5 as 1 / 3 with the loads of two K steps issued together (for a row-major A read
  * in 64-byte pieces from rows far apart; plain store), 0 never, -1 automatic: K of 65 up to 512 and at least

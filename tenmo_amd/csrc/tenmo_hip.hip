@@ -88,7 +88,7 @@ struct State {
     int force_splitk = -1;
     int force_conv_phases = -1; // strided image gradient phase by phase: -1 automatic (large layers), 0 never, 1 always
     int force_streamk = -1;    // -1 automatic, 0 never, n > 0: stream-K with n workgroups per CU
-    int force_smallk = -1;     // -1 automatic, 0 never, 1: the short-reduction kernel wherever it can run
+    int force_smallk = -1;     // -1 automatic, 0 never, 1: the short-reduction kernel wherever it can run (2: without XCD grouping, 3: also for K <= 16)
     int force_resident = 0;    // the resident-A kernel for a few tile rows against a very wide B: 1 with 128x64 tiles, 2 with 64x64, 0 never
     int force_panel = -1;      // -1 automatic, 0 never, 1: the persistent K-stream kernel wherever it can run (2: without XCD grouping, 3: 64x64 tiles, 4 / 5: 128x128 / 64x64 tiles with paired K steps)
     int mlp_fused_tail = 0;    // MLP step: 1 the last two layers, loss, their backward and update in one launch when the shapes fit; 2 also the first layer's weight gradient and update in one; 3 also the first layer's forward in one; 0 neither
@@ -426,7 +426,8 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
         // through this kernel faulted — an undeclared SCC clobber of the masked direct load, since fixed (gfx950_asm.hpp) — and
         // the one-step instantiations come back once the fix has been confirmed on a GPU.  Until then the automatic choice
         // is also limited to K % 16 == 0, which never takes the masked load; a ragged K reaches it only through the knob.)
-        const bool can = K > GEMM_BK && K <= 64 && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum && !ep.bsum &&
+        // (gemm_smallk = 3 forces the kernel onto one-step reductions too: for the checks of exactly that path)
+        const bool can = (K > GEMM_BK || S.force_smallk == 3) && K <= 64 && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum && !ep.bsum &&
                          N < (int64_t(1) << 29) && tiles64 <= 0x7fffffffLL;
         const bool want = S.force_smallk > 0 || (S.force_smallk < 0 && S.force_tile < 0 && S.force_splitk <= 0 && S.force_streamk <= 0 &&
                                                   splits == 1 && sk_wpc == 0 && tiles64 >= 2048 && K <= 64 && K % GEMM_BK == 0);

@@ -317,3 +317,20 @@ def test_one_step_reduction_into_a_large_result(exe):
     cause was an undeclared SCC clobber in an inline-assembly block, which only the generated ISA shows
     (tests/test_asm_clobbers.py).  K <= 16 currently takes the ordinary 64x64 kernel, which is what this replays."""
     run(exe, [case(8192, 8192, 16, "n", "t")], modes=("early",), timeout=1200)
+
+
+def test_short_reduction_kernel_on_one_step_reductions(exe):
+    """K <= 16 through the persistent short-reduction kernel (gemm_smallk = 3; the automatic choice keeps such products on the
+    ordinary kernel): one K step per tile, so a workgroup's loop is all tile turnover — several tiles per workgroup (few
+    modelled CUs), ragged last tile rows and columns, K tails (the masked direct load on every tile), every operand layout,
+    plain and accumulating stores, batches with and without a shared B; and the product that once faulted on a GPU,
+    [8192,16].[16,8192] with B a transposed view, at full size on the real 256 CUs through this kernel."""
+    cases = []
+    for la, lb in LAYOUTS:
+        for (M, N, K) in [(300, 520, 16), (260, 132, 12), (320, 448, 8), (132, 68, 4)]:
+            for acc in (0, 1):
+                cases.append(case(M, N, K, la, lb, acc=acc, gemm_smallk=3, ran="gemm_smallk_kernel"))
+        cases.append(case(200, 264, 16, la, lb, batch=5, gemm_smallk=3, ran="gemm_smallk_kernel"))
+        cases.append(case(200, 264, 12, la, lb, batch=3, b_shared=1, acc=1, gemm_smallk=3, ran="gemm_smallk_kernel"))
+    run(exe, cases, cus=2)
+    run(exe, [case(8192, 8192, 16, "n", "t", gemm_smallk=3, ran="gemm_smallk_kernel", check=0)], modes=("late",), timeout=1800)

@@ -6,8 +6,9 @@ after every other GPU test, so that a first GPU run which goes wrong here has al
 to tests/test_gpu_parity.py once it has passed on a GPU.  In order of collection: the default path first (the batch-
 reducing launch behind the gradients of broadcast parents), then the kernels behind knobs that are off by default (K
 slices joined inside the column kernels' launch, the fused MLP launches, the K-stream kernel's 64x64 and paired forms, the
-resident-A kernel), last the short-reduction kernel forced onto reductions that are no multiple of 16 — the one path that
-uses the masked direct load (its fault, an undeclared SCC clobber, is fixed; this is the run that confirms it).
+resident-A kernel), the Linear backward with the bias gradient summed in the weight-gradient launch, last the short-reduction
+kernel forced onto reductions that are no multiple of 16 and onto one-step reductions (K <= 16) — the paths that use the masked
+direct load (its fault, an undeclared SCC clobber, is fixed; these are the runs that confirm it).
 """
 import os
 
@@ -374,3 +375,47 @@ def test_linear_backward_sums_the_bias_gradient_in_the_weight_gradient_launch(T,
     finally:
         for name in ("gemm_tile", "gemm_splitk", "gemm_streamk"):
             L.tenmo_hip_set_tuning(name.encode(), -1)
+
+
+def test_short_reduction_kernel_on_one_step_reductions(T):
+    """K <= 16 through the persistent short-reduction kernel (gemm_smallk = 3; the automatic choice keeps such products on the
+    ordinary kernel until this has passed on a GPU): several tiles per workgroup, ragged tiles, K tails (the masked direct load
+    on every tile), every operand layout, plain and accumulating stores, batches; last the product after which a GPU run
+    once ended in a memory fault — [8192,16].[16,8192] with B a transposed view (cause: an undeclared SCC clobber in the masked
+    load's asm block, fixed; tests/test_asm_clobbers.py holds the generated code to it).  Against fp64."""
+    import torch
+    L, lib = T.lib.load(), T.lib
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(41)
+    small = bool(os.environ.get("TENMO_TEST_SMALL"))
+    cases = [((), 3072, 3072, 16, 0), ((), 3000, 3100, 12, 1), ((3,), 1024, 2052, 8, 0), ((2,), 2048, 2048, 16, 1), ((), 1028, 4100, 4, 0)]
+    if small:
+        cases = [((), 300, 520, 16, 0), ((), 260, 132, 12, 1), ((3,), 200, 264, 8, 0)]
+    try:
+        L.tenmo_hip_set_tuning(b"gemm_smallk", 3)
+        for bshape, M, N, K, acc in cases:
+            for ta in (False, True):
+                for tb in (False, True):
+                    A = torch.randn((*bshape, *((K, M) if ta else (M, K))), generator=gen, device="cuda")
+                    B = torch.randn((*bshape, *((N, K) if tb else (K, N))), generator=gen, device="cuda")
+                    Cc = torch.randn((*bshape, M, N), generator=gen, device="cuda")
+                    a_rs, a_cs = (1, M) if ta else (K, 1)
+                    b_rs, b_cs = (1, K) if tb else (N, 1)
+                    ref = (A.transpose(-1, -2) if ta else A).double() @ (B.transpose(-1, -2) if tb else B).double() + (Cc.double() if acc else 0)
+                    ab = [A.stride(i) for i in range(len(bshape))]
+                    bb = [B.stride(i) for i in range(len(bshape))]
+                    lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, a_rs, a_cs, B.data_ptr(), 0, b_rs, b_cs, Cc.data_ptr(), M, N, K, len(bshape),
+                                                   lib.i64(bshape), lib.i64(ab), lib.i64(bb), acc, 1))
+                    err = float((Cc.double() - ref).norm() / ref.norm())
+                    assert err <= RTOL_FRO, (bshape, M, N, K, acc, ta, tb, err)
+        if not small:
+            M = N = 8192
+            A = torch.randn((M, 16), generator=gen, device="cuda")
+            Bt = torch.randn((N, 16), generator=gen, device="cuda")
+            Cc = torch.empty((M, N), device="cuda")
+            lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, 16, 1, Bt.data_ptr(), 0, 1, 16, Cc.data_ptr(), M, N, 16, 0, None, None, None, 0, 1))
+            rows = torch.arange(0, M, 61, device="cuda")
+            ref = A[rows].double() @ Bt.double().t()
+            assert float((Cc[rows].double() - ref).norm() / ref.norm()) <= RTOL_FRO
+    finally:
+        L.tenmo_hip_set_tuning(b"gemm_smallk", -1)
