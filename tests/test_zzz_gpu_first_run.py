@@ -249,39 +249,6 @@ def test_resident_left_operand_kernel(T):
         L.tenmo_hip_set_tuning(b"gemm_resident", 0)
 
 
-@pytest.mark.parametrize("smallk", [0, 1])
-def test_short_reduction_kernel_layouts_and_k_tails(T, smallk):
-    """The same kernel over every operand layout (row-major and transposed views of A and of B) and reductions that
-    are no multiple of 16 (zero-filled K tail; a K-major operand then needs K % 4 == 0, other K fall back to the
-    ordinary kernel), whole and ragged tiles, batches, accumulation; against fp64."""
-    import torch
-    L, lib = T.lib.load(), T.lib
-    gen = torch.Generator(device="cuda")
-    gen.manual_seed(29)
-    cases = [((), 64, 64, 16, 0), ((), 128, 192, 100, 0), ((3,), 100, 132, 36, 0), ((2, 3), 256, 68, 64, 1), ((5,), 64, 64, 112, 0),
-             ((2,), 332, 776, 20, 1), ((), 1000, 1000, 7, 0), ((4,), 72, 52, 84, 0), ((), 256, 5000, 100, 0), ((2,), 512, 512, 50, 1),
-             ((9,), 320, 1024, 12, 0), ((), 64, 8192, 104, 0), ((), 130, 70, 33, 0)]
-    try:
-        L.tenmo_hip_set_tuning(b"gemm_smallk", smallk)
-        for bshape, M, N, K, acc in cases:
-            for ta in (False, True):
-                for tb in (False, True):
-                    A = torch.randn((*bshape, *((K, M) if ta else (M, K))), generator=gen, device="cuda")
-                    B = torch.randn((*bshape, *((N, K) if tb else (K, N))), generator=gen, device="cuda")
-                    Cc = torch.randn((*bshape, M, N), generator=gen, device="cuda")
-                    a_rs, a_cs = (1, M) if ta else (K, 1)
-                    b_rs, b_cs = (1, K) if tb else (N, 1)
-                    ref = (A.transpose(-1, -2) if ta else A).double() @ (B.transpose(-1, -2) if tb else B).double() + (Cc.double() if acc else 0)
-                    ab = [A.stride(i) for i in range(len(bshape))]
-                    bb = [B.stride(i) for i in range(len(bshape))]
-                    lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, a_rs, a_cs, B.data_ptr(), 0, b_rs, b_cs, Cc.data_ptr(), M, N, K, len(bshape),
-                                                   lib.i64(bshape), lib.i64(ab), lib.i64(bb), acc, 1))
-                    err = float((Cc.double() - ref).norm() / ref.norm())
-                    assert err <= RTOL_FRO, (smallk, bshape, M, N, K, acc, ta, tb, err)
-    finally:
-        L.tenmo_hip_set_tuning(b"gemm_smallk", -1)
-
-
 def test_linear_backward_reference_literal(T, golden):
     """The reference's own literal for the gradient of a broadcast bias (tests/test_expand.mojo:229-245): whatever the input and the
     weight, the bias gradient of x.W + b is the upstream gradient summed over its rows — through tenmo_hip_linear_backward (here the
@@ -375,6 +342,39 @@ def test_linear_backward_sums_the_bias_gradient_in_the_weight_gradient_launch(T,
     finally:
         for name in ("gemm_tile", "gemm_splitk", "gemm_streamk"):
             L.tenmo_hip_set_tuning(name.encode(), -1)
+
+
+@pytest.mark.parametrize("smallk", [0, 1])
+def test_short_reduction_kernel_layouts_and_k_tails(T, smallk):
+    """The same kernel over every operand layout (row-major and transposed views of A and of B) and reductions that
+    are no multiple of 16 (zero-filled K tail; a K-major operand then needs K % 4 == 0, other K fall back to the
+    ordinary kernel), whole and ragged tiles, batches, accumulation; against fp64."""
+    import torch
+    L, lib = T.lib.load(), T.lib
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(29)
+    cases = [((), 64, 64, 16, 0), ((), 128, 192, 100, 0), ((3,), 100, 132, 36, 0), ((2, 3), 256, 68, 64, 1), ((5,), 64, 64, 112, 0),
+             ((2,), 332, 776, 20, 1), ((), 1000, 1000, 7, 0), ((4,), 72, 52, 84, 0), ((), 256, 5000, 100, 0), ((2,), 512, 512, 50, 1),
+             ((9,), 320, 1024, 12, 0), ((), 64, 8192, 104, 0), ((), 130, 70, 33, 0)]
+    try:
+        L.tenmo_hip_set_tuning(b"gemm_smallk", smallk)
+        for bshape, M, N, K, acc in cases:
+            for ta in (False, True):
+                for tb in (False, True):
+                    A = torch.randn((*bshape, *((K, M) if ta else (M, K))), generator=gen, device="cuda")
+                    B = torch.randn((*bshape, *((N, K) if tb else (K, N))), generator=gen, device="cuda")
+                    Cc = torch.randn((*bshape, M, N), generator=gen, device="cuda")
+                    a_rs, a_cs = (1, M) if ta else (K, 1)
+                    b_rs, b_cs = (1, K) if tb else (N, 1)
+                    ref = (A.transpose(-1, -2) if ta else A).double() @ (B.transpose(-1, -2) if tb else B).double() + (Cc.double() if acc else 0)
+                    ab = [A.stride(i) for i in range(len(bshape))]
+                    bb = [B.stride(i) for i in range(len(bshape))]
+                    lib.check(L.tenmo_hip_gemm_f32(A.data_ptr(), 0, a_rs, a_cs, B.data_ptr(), 0, b_rs, b_cs, Cc.data_ptr(), M, N, K, len(bshape),
+                                                   lib.i64(bshape), lib.i64(ab), lib.i64(bb), acc, 1))
+                    err = float((Cc.double() - ref).norm() / ref.norm())
+                    assert err <= RTOL_FRO, (smallk, bshape, M, N, K, acc, ta, tb, err)
+    finally:
+        L.tenmo_hip_set_tuning(b"gemm_smallk", -1)
 
 
 def test_short_reduction_kernel_on_one_step_reductions(T):
