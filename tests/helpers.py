@@ -145,3 +145,46 @@ def conv_backward_reference64(image, kernel, grad_out, stride, dilation, pads):
     y = torch.nn.functional.conv2d(torch.nn.functional.pad(x, (pads[2], pads[3], pads[0], pads[1])), k, b, stride=stride, dilation=dilation)
     y.backward(torch.from_numpy(grad_out).double())
     return x.grad.numpy(), k.grad.numpy(), b.grad.numpy()
+
+
+def check_golden_extras(case, out, grad_a=None, grad_b=None):
+    """The fixture keys beyond whole-tensor values: a slice of the result or of a gradient at leading indices (the reference asserts
+    one batch of it), and shapes of gradients.  `out`, `grad_a`, `grad_b`: numpy arrays (gradients may be None when not computed)."""
+    if "expect_slice" in case:
+        got = np.asarray(out)[tuple(case["expect_slice"]["index"])]
+        np.testing.assert_allclose(got, np.asarray(case["expect_slice"]["expect"], np.float32), rtol=1e-5, atol=1e-8, err_msg=case["name"])
+    if "grad_A_slice" in case and grad_a is not None:
+        got = np.asarray(grad_a)[tuple(case["grad_A_slice"]["index"])]
+        np.testing.assert_allclose(got, np.asarray(case["grad_A_slice"]["expect"], np.float32), rtol=1e-5, err_msg=case["name"] + " grad_A slice")
+    if "grad_A_shape" in case and grad_a is not None:
+        assert list(np.shape(grad_a)) == case["grad_A_shape"], case["name"]
+    if "grad_B_shape" in case and grad_b is not None:
+        assert list(np.shape(grad_b)) == case["grad_B_shape"], case["name"]
+
+
+GOLDEN_GRADIENT_KEYS = ("grad_A", "grad_B", "base_grad_A", "base_grad_B", "grad_A_slice", "grad_A_shape", "grad_B_shape")
+
+
+def generated_operand(spec):
+    """An operand of a `device_kernel_cases` fixture: the reference builds these with ones / zeros / arange / eye / literal values."""
+    shape = tuple(spec["shape"])
+    kind = spec["gen"]
+    if kind == "ones":
+        return np.ones(shape, np.float32)
+    if kind == "zeros":
+        return np.zeros(shape, np.float32)
+    if kind == "arange":
+        return np.arange(int(np.prod(shape)), dtype=np.float32).reshape(shape)
+    if kind == "eye":
+        return np.eye(shape[0], dtype=np.float32)
+    return np.asarray(spec["values"], np.float32).reshape(shape)
+
+
+def exact_product(op, a, b):
+    """The product in float64 (exact for these small integers): mm broadcasts batches; mv / vm broadcast the vector's batch."""
+    a, b = a.astype(np.float64), b.astype(np.float64)
+    if op == "mm":
+        return a @ b
+    if op == "mv":
+        return (a @ b[..., None])[..., 0]
+    return (a[..., None, :] @ b)[..., 0, :]

@@ -11,7 +11,7 @@ import os
 import numpy as np
 import pytest
 
-from helpers import RTOL_FRO, ce_reference64, numpy_view, ref_matmul64, rel_fro, scatter_to_storage, storage_of, strides_of
+from helpers import GOLDEN_GRADIENT_KEYS, RTOL_FRO, ce_reference64, check_golden_extras, exact_product, generated_operand, numpy_view, ref_matmul64, rel_fro, scatter_to_storage, storage_of, strides_of
 
 pytestmark = pytest.mark.gpu
 
@@ -58,15 +58,20 @@ def as_strided_tensor(T, arr, requires_grad=False):
 def test_golden_forward_and_backward(T, golden):
     mode = {"mm": T.mm, "mv": T.mv, "vm": T.vm, "dot": T.dot}
     for c in golden["cases"]:
-        A = fixture_tensor(T, c["A"], requires_grad=True)
-        B = fixture_tensor(T, c["B"], requires_grad=True)
+        # (a one-element operand of dot is broadcast first, by the reference's Broadcast operator, whose backward is not part of
+        # the matrix-product path: those cases are forward only)
+        grads = not (c["op"] == "dot" and (c["A"]["shape"] == [] or c["B"]["shape"] == []))
+        A = fixture_tensor(T, c["A"], requires_grad=grads)
+        B = fixture_tensor(T, c["B"], requires_grad=grads)
         out = A.matmul(B, mode=mode[c["op"]])
         if "expect" in c:
             np.testing.assert_allclose(out.to_numpy(), np.asarray(c["expect"], np.float32), rtol=1e-5, atol=1e-8, err_msg=c["name"])
         if "expect_shape" in c:
             assert list(out.shape()) == c["expect_shape"], c["name"]
-        if any(k in c for k in ("grad_A", "grad_B", "base_grad_A", "base_grad_B")):
+        check_golden_extras(c, out.to_numpy())
+        if any(k in c for k in GOLDEN_GRADIENT_KEYS):
             out.backward(1.0)  # loss = out.sum(); loss.backward()
+            check_golden_extras(c, out.to_numpy(), A.grad(), B.grad())
             if "grad_A" in c:
                 np.testing.assert_allclose(A.grad(), np.asarray(c["grad_A"], np.float32), rtol=1e-5, err_msg=c["name"] + " grad_A")
             if "grad_B" in c:
@@ -76,6 +81,41 @@ def test_golden_forward_and_backward(T, golden):
                 np.testing.assert_allclose(scatter_to_storage(c["A"], A.grad()), c["base_grad_A"], rtol=1e-5, err_msg=c["name"] + " base_grad_A")
             if "base_grad_B" in c:
                 np.testing.assert_allclose(scatter_to_storage(c["B"], B.grad()), c["base_grad_B"], rtol=1e-5, err_msg=c["name"] + " base_grad_B")
+
+
+def test_reference_device_kernel_cases(T, golden, oracle):
+    """The reference's tests of the launch functions this library replaces (tests/test_gpu.mojo:550-1575) compare the GPU result
+    with the CPU result on these operands; here: the HIP result against the oracle (the restated CPU path), bit for bit where the
+    sums are exact in fp32 (small integers: all of them), and against the values the tests state."""
+    mode = {"mm": T.mm, "mv": T.mv, "vm": T.vm}
+    for c in golden["device_kernel_cases"]["cases"]:
+        a, b = generated_operand(c["A"]), generated_operand(c["B"])
+        out = T.Tensor.from_numpy(a).matmul(T.Tensor.from_numpy(b), mode=mode[c["op"]], track_grad=False).to_numpy()
+        cpu = {"mm": oracle.matmul, "mv": oracle.mv, "vm": oracle.vm}[c["op"]](a, b)
+        assert out.shape == cpu.shape, c["name"]
+        np.testing.assert_array_equal(out, cpu, err_msg=c["name"])
+        np.testing.assert_array_equal(out, exact_product(c["op"], a, b).astype(np.float32), err_msg=c["name"])
+        if "expect" in c:
+            np.testing.assert_array_equal(out, np.asarray(c["expect"], np.float32), err_msg=c["name"])
+
+
+def test_golden_result_shapes(T, golden):
+    """The reference's shape-only tests (random operands there): the broadcast of the batch dimensions, from the library's own
+    shape resolution (tenmo_hip_result_shape), and one of them computed."""
+    import ctypes as C
+
+    L, lib = T.lib.load(), T.lib
+    for c in golden["shape_cases"]:
+        va = lib.make_view(0, 0, c["A_shape"], [1] * len(c["A_shape"]))
+        vb = lib.make_view(0, 0, c["B_shape"], [1] * len(c["B_shape"]))
+        shape, rank = (C.c_int64 * 8)(), C.c_int32()
+        n = L.tenmo_hip_result_shape(lib.OP_MM, C.byref(va), C.byref(vb), shape, C.byref(rank))
+        assert list(shape[:rank.value]) == c["expect_shape"] and n == int(np.prod(c["expect_shape"])), c["name"]
+    c = golden["shape_cases"][1]
+    rng = np.random.default_rng(3)
+    a, b = rng.standard_normal(c["A_shape"], dtype=np.float32), rng.standard_normal(c["B_shape"], dtype=np.float32)
+    out = T.Tensor.from_numpy(a).matmul(T.Tensor.from_numpy(b), track_grad=False)
+    assert list(out.shape()) == c["expect_shape"] and rel_fro(out.to_numpy(), ref_matmul64(a, b)) <= RTOL_FRO
 
 
 def test_closed_forms(T, golden):

@@ -3,7 +3,7 @@ vectors, fp64 brute force, closed forms and algebraic invariants.  Runs without 
 import numpy as np
 import pytest
 
-from helpers import ce_reference64, numpy_view, ref_matmul64, rel_fro, scatter_to_storage, storage_of, strides_of
+from helpers import GOLDEN_GRADIENT_KEYS, ce_reference64, check_golden_extras, exact_product, generated_operand, numpy_view, ref_matmul64, rel_fro, scatter_to_storage, storage_of, strides_of
 
 
 def _view(O, t):
@@ -26,12 +26,29 @@ def test_golden_forward(golden, oracle):
             np.testing.assert_allclose(got, np.asarray(c["expect"], np.float32), rtol=1e-5, atol=1e-8, err_msg=c["name"])
         if "expect_shape" in c:
             assert list(np.shape(got)) == c["expect_shape"], c["name"]
+        check_golden_extras(c, got)
+    for c in golden["shape_cases"]:  # shapes only (random operands in the reference): the broadcast of the batch dimensions
+        assert list(O.result_shape(O.MM, O.View.of(np.zeros(c["A_shape"], np.float32)), O.View.of(np.zeros(c["B_shape"], np.float32)))) == c["expect_shape"], c["name"]
+
+
+def test_reference_device_kernel_cases(golden, oracle):
+    """The operands of the reference's own GPU-launch tests (tests/test_gpu.mojo: CPU result against GPU result): the oracle,
+    which restates that CPU path, against the exact product of these small integers and the values the tests state."""
+    O = oracle
+    for c in golden["device_kernel_cases"]["cases"]:
+        a, b = generated_operand(c["A"]), generated_operand(c["B"])
+        got = {"mm": O.matmul, "mv": O.mv, "vm": O.vm}[c["op"]](a, b)
+        want = exact_product(c["op"], a, b)
+        assert got.shape == want.shape, c["name"]
+        np.testing.assert_array_equal(got, want.astype(np.float32), err_msg=c["name"])
+        if "expect" in c:
+            np.testing.assert_array_equal(got, np.asarray(c["expect"], np.float32), err_msg=c["name"])
 
 
 def test_golden_backward(golden, oracle):
     O = oracle
     for c in golden["cases"]:
-        if not any(k in c for k in ("grad_A", "grad_B", "base_grad_A", "base_grad_B")):
+        if not any(k in c for k in GOLDEN_GRADIENT_KEYS):
             continue
         A, B = _view(O, c["A"]), _view(O, c["B"])
         if c["op"] == "mm":
@@ -39,6 +56,10 @@ def test_golden_backward(golden, oracle):
             gA, gB = O.matmul_backward(A, B, np.ones(shape, np.float32))
         elif c["op"] == "mv":
             gA, gB = O.mv_backward(A, B, np.ones(O.result_shape(O.MV, A, B), np.float32))
+        elif c["op"] == "dot":  # grad_lhs = rhs * g, grad_rhs = lhs * g (tenmo/dotproduct.mojo:13-52) = the backward of lhs[n] . rhs-as-[n, 1]
+            n = c["A"]["shape"][0]
+            gA, gB = O.vm_backward(A, O.View(storage_of(c["B"]), c["B"].get("offset", 0), (n, 1), (strides_of(c["B"])[0], 1)), np.ones((1,), np.float32))
+            gB = gB.reshape(n)
         else:
             gA, gB = O.vm_backward(A, B, np.ones(O.result_shape(O.VM, A, B), np.float32))
         if "grad_A" in c:
@@ -50,6 +71,7 @@ def test_golden_backward(golden, oracle):
             np.testing.assert_allclose(scatter_to_storage(c["A"], gA), c["base_grad_A"], rtol=1e-5, err_msg=c["name"] + " base_grad_A")
         if "base_grad_B" in c:
             np.testing.assert_allclose(scatter_to_storage(c["B"], gB), c["base_grad_B"], rtol=1e-5, err_msg=c["name"] + " base_grad_B")
+        check_golden_extras(c, None, gA, gB)
 
 
 @pytest.mark.parametrize("width", [0, 16, 8, 1])
