@@ -706,17 +706,38 @@ def test_cblas_sgemm(T, golden):
     h = BLASHandle()
     assert h.is_initialized()
     for c in golden["blas"]:
-        A, B = np.asarray(c["A"], np.float32), np.asarray(c["B"], np.float32)
-        if "grad_A" in c:
-            gA, gB = h.matmul_backward(A, B, np.ones((A.shape[0], B.shape[1]), np.float32))
-            np.testing.assert_allclose(gA, c["grad_A"])
-            np.testing.assert_allclose(gB, c["grad_B"])
-            continue
-        out = h.matmul(A, B, c["tA"], c["tB"])
+        if "A_ones" in c:
+            A, B = np.ones(c["A_ones"], np.float32), np.ones(c["B_ones"], np.float32)
+        else:
+            A, B = np.asarray(c["A"], np.float32), np.asarray(c["B"], np.float32)
+        tA, tB = c["tA"], c["tB"]
+        opA, opB = (A.T if tA else A), (B.T if tB else B)
+        out = h.matmul(A, B, tA, tB)
         if "expect" in c:
             np.testing.assert_allclose(out, c["expect"], rtol=1e-5)
-        else:
+        if "expect_00" in c:
             assert abs(out[0, 0] - c["expect_00"]) < 1e-5
+        if "expect_value" in c:
+            assert out.shape == (opA.shape[0], opB.shape[1]) and np.all(out == c["expect_value"])
+        if "grad_A" in c or c.get("equals_native"):
+            gA, gB = h.matmul_backward(A, B, np.ones((opA.shape[0], opB.shape[1]), np.float32), tA, tB)
+        if "grad_A" in c:
+            np.testing.assert_allclose(gA, c["grad_A"])
+            np.testing.assert_allclose(gB, c["grad_B"])
+        if c.get("equals_native"):  # the reference's BLAS-against-native tests: the plugin entry and the device path on transposed views agree
+            At, Bt = T.Tensor.from_numpy(A, True), T.Tensor.from_numpy(B, True)
+            Av, Bv = (At.transpose() if tA else At), (Bt.transpose() if tB else Bt)
+            nat = Av.matmul(Bv)
+            np.testing.assert_array_equal(out, nat.to_numpy())
+            nat.backward(1.0)
+            np.testing.assert_array_equal(gA, Av.grad().T if tA else Av.grad())   # (the gradient of a transposed view has the view's shape)
+            np.testing.assert_array_equal(gB, Bv.grad().T if tB else Bv.grad())
+    rs = np.random.default_rng(59)
+    for m, k, n in golden["blas_shapes"]["cases"]:
+        A, B = rs.standard_normal((m, k), dtype=np.float32), rs.standard_normal((k, n), dtype=np.float32)
+        out = h.matmul(A, B)
+        nat = T.Tensor.from_numpy(A).matmul(T.Tensor.from_numpy(B), track_grad=False).to_numpy()
+        assert rel_fro(out, ref_matmul64(A, B)) <= RTOL_FRO and rel_fro(out, nat) <= RTOL_FRO, (m, k, n)
     assert np.all(h.matmul(np.ones((100, 100), np.float32), np.ones((100, 100), np.float32)) == 100.0)  # tests/test_blas.mojo:216-232
     # four-case backward algebra (tenmo/blashandle.mojo:51-99) against explicit transposes
     rng = np.random.default_rng(53)
