@@ -481,6 +481,29 @@ def config_rows(L, _lib, torch, only, announce=False):
         gemm_row("gpt2_%s_dX" % nm, 4, lambda i, dout=dout: randn((Tk, dout), 420 + i), lambda i, din=din, dout=dout: randn((din, dout), 410 + i, 0.02).t(), (Tk, din))
         gemm_row("gpt2_%s_dW" % nm, 4, lambda i, din=din: randn((Tk, din), 400 + i).t(), lambda i, dout=dout: randn((Tk, dout), 420 + i), (din, dout))
 
+    # ---- config 5: memory-bound products ----
+    n16 = 16384
+    if wanted("mv") or wanted("vm"):
+        W = randn((n16, n16), 500)
+        x = randn((n16,), 501)
+        o = torch.empty((n16,), device="cuda")
+        nbytes = (n16 * n16 + 2 * n16) * 4.0
+        mv = lambda: _lib.check(L.tenmo_hip_mv_f32(W.data_ptr(), 0, n16, 1, x.data_ptr(), 0, 1, o.data_ptr(), n16, n16, 0, None, None, None, 0, 0))
+        vm = lambda: _lib.check(L.tenmo_hip_vm_f32(x.data_ptr(), 0, 1, W.data_ptr(), 0, n16, 1, o.data_ptr(), n16, n16, 0, None, None, None, 0, 0))
+        for nm, fn, ref in (("mv16384", mv, lambda: W.double() @ x.double()), ("vm16384", vm, lambda: x.double() @ W.double())):
+            if not wanted(nm[:2]):
+                continue
+            us = hip_time_us(L, _lib, [fn], 160.0)
+            r = ref()
+            err = float((o.double() - r).norm() / r.norm())
+            finish_row(nm, 5, "[16384x16384] x [16384]", us, 2.0 * n16 * n16, nbytes, err, 1)
+        del W, x, o
+        torch.cuda.empty_cache()
+    gemm_row("skinny_4x768x50257", 5, lambda i: randn((4, 768), 510 + i), lambda i: randn((768, 50257), 520 + i), (4, 50257))
+    gemm_row("cbow_logits", 5, lambda i: randn((256, 100), 530 + i), lambda i: randn((100, 50000), 540 + i), (256, 50000))
+    gemm_row("cbow_At.dC", 5, lambda i: randn((256, 100), 530 + i).t(), lambda i: randn((256, 50000), 550 + i), (100, 50000))
+
+    # ---- last (the one row whose kernels are younger than the others): config 4, the whole backward of a Linear layer ----
     if wanted("gpt2_up_linear_backward"):
         # the whole backward of the MLP-up Linear layer in one call: dX += dY.W^T, dW += X^T.dY, db += column sums of dY
         # (the bias gradient comes out of the dW launch: dY is streamed twice, not three times)
@@ -507,28 +530,6 @@ def config_rows(L, _lib, torch, only, announce=False):
         finish_row("gpt2_up_linear_backward(dX,dW,db)", 4, "[8192x3072].[3072x768] + [768x8192].[8192x3072] + colsum", us, flop, nbytes, max(errs), n)
         del Xs, dYs, gXs, gWs, gbs
         torch.cuda.empty_cache()
-
-    # ---- config 5: memory-bound products ----
-    n16 = 16384
-    if wanted("mv") or wanted("vm"):
-        W = randn((n16, n16), 500)
-        x = randn((n16,), 501)
-        o = torch.empty((n16,), device="cuda")
-        nbytes = (n16 * n16 + 2 * n16) * 4.0
-        mv = lambda: _lib.check(L.tenmo_hip_mv_f32(W.data_ptr(), 0, n16, 1, x.data_ptr(), 0, 1, o.data_ptr(), n16, n16, 0, None, None, None, 0, 0))
-        vm = lambda: _lib.check(L.tenmo_hip_vm_f32(x.data_ptr(), 0, 1, W.data_ptr(), 0, n16, 1, o.data_ptr(), n16, n16, 0, None, None, None, 0, 0))
-        for nm, fn, ref in (("mv16384", mv, lambda: W.double() @ x.double()), ("vm16384", vm, lambda: x.double() @ W.double())):
-            if not wanted(nm[:2]):
-                continue
-            us = hip_time_us(L, _lib, [fn], 160.0)
-            r = ref()
-            err = float((o.double() - r).norm() / r.norm())
-            finish_row(nm, 5, "[16384x16384] x [16384]", us, 2.0 * n16 * n16, nbytes, err, 1)
-        del W, x, o
-        torch.cuda.empty_cache()
-    gemm_row("skinny_4x768x50257", 5, lambda i: randn((4, 768), 510 + i), lambda i: randn((768, 50257), 520 + i), (4, 50257))
-    gemm_row("cbow_logits", 5, lambda i: randn((256, 100), 530 + i), lambda i: randn((100, 50000), 540 + i), (256, 50000))
-    gemm_row("cbow_At.dC", 5, lambda i: randn((256, 100), 530 + i).t(), lambda i: randn((256, 50000), 550 + i), (100, 50000))
     return rows
 
 
