@@ -71,8 +71,7 @@ int tenmo_hip_device_info(int* compute_units, char* name, int name_len);
  * or accumulating store: 1 wherever it can run, 3 the same and also for K up to 16 — a path the automatic choice does not take —, 0 never,
  * -1 automatic: for results of 2048 and more 64x64 tiles and K a multiple of 16),
  * "gemm_panel" (the persistent K-stream kernel with loading wavefronts of its own, 128x128 tiles, K above 16, plain or
- * accumulating store: 1 wherever it can run, 3 the same with 64x64 tiles and a deeper ring, 4 / 5 as 1 / 3 with the loads of two K steps issued together (for a row-major A read
- * in 64-byte pieces from rows far apart; plain store), 0 never, -1 automatic: K of 65 up to 512 and at least
+ * accumulating store: 1 wherever it can run, 3 the same with 64x64 tiles and a deeper ring, 0 never, -1 automatic: K of 65 up to 512 and at least
  * three 128x128 tiles per CU), "gemm_resident" (a left operand of a few tile rows, K of 17 up to 256, against a wide right
  * operand with unit stride along N, one matrix, plain store: persistent workgroups that keep their rows of A in LDS and
  * stream B alone; 1 with 128x64 tiles, 2 with 64x64 tiles, 0 never, the default),

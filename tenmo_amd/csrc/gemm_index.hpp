@@ -149,11 +149,8 @@ TENMO_HD void tile_origin(uint32_t tl, uint32_t tiles_m, uint32_t tiles_n, int c
 //   init_tile(tile)      a tile of the walk begins (loader side)
 //   issue(slot, ks)      start the loads of K step `ks` of the current tile into ring stage `slot`
 //   wait_barrier(ahead)  wait until at most `ahead` issued steps are still in flight, then the workgroup barrier
-// `paired`: the loaders refill two stages behind every second barrier instead of one behind each (the stage freed at the
-// barrier before stays empty for one step): the loads of two consecutive K steps — adjacent 64-byte pieces of every row of a
-// K-major operand — then reach the memory system together instead of a K step's MFMAs apart.
 template <class InitTile, class Issue, class WaitBarrier>
-TENMO_HD void kstream_loader(TileWalk walk, int nk, int np, InitTile&& init_tile, Issue&& issue, WaitBarrier&& wait_barrier, const bool paired = false) {
+TENMO_HD void kstream_loader(TileWalk walk, int nk, int np, InitTile&& init_tile, Issue&& issue, WaitBarrier&& wait_barrier) {
     int ks = 0, slot = 0, issued = 0;
     bool more = true;
     auto next = [&]() {
@@ -168,19 +165,11 @@ TENMO_HD void kstream_loader(TileWalk walk, int nk, int np, InitTile&& init_tile
         }
     };
     init_tile(walk.tile());
-    // (paired: a pair starts at an even step — steps 2j and 2j+1 are the two halves of 128 bytes of a row — so an even ring
-    // starts one step shorter and refills behind the even barriers, an odd one behind the odd barriers)
-    const int ahead_at_start = paired && (np & 1) == 0 ? np - 2 : np - 1;
-    for (int i = 0; i < ahead_at_start && more; ++i) next();
+    for (int i = 0; i < np - 1 && more; ++i) next();
     for (int u = 0; u < issued; ++u) {
         const int ahead = issued - (u + 2);
         wait_barrier(ahead > 0 ? ahead : 0);
-        if (!paired) {
-            if (more) next();
-        } else if ((u & 1) == (np & 1)) {
-            if (more) next();
-            if (more) next();
-        }
+        if (more) next();
     }
 }
 //   barrier()                              the workgroup barrier

@@ -50,9 +50,8 @@ bool launch_gemm_smallk_64x64(const GemmArgs& g, int amode, int bmode, unsigned 
 // `total_tiles` = batches x tiles of the chosen size (g.tiles_m, g.tiles_n set for it).  The caller has checked what the
 // direct loads need (pitches, an MN-major extent divisible by 4, K % 4 == 0 for a K-major operand when K is no multiple
 // of 16) and N <= 2^22.  false: no such variant.
-// (64x64: a ring of eight stages, for long reductions over few tiles; _PAIRED: the loading wavefronts issue two K steps at a
-// time — a K-major A and a plain store only, false otherwise)
-enum PanelTile : int { PANEL_TILE_128x128 = 0, PANEL_TILE_64x64 = 1, PANEL_TILE_128x128_PAIRED = 2, PANEL_TILE_64x64_PAIRED = 3 };
+// (64x64: a ring of eight stages, for long reductions over few tiles)
+enum PanelTile : int { PANEL_TILE_128x128 = 0, PANEL_TILE_64x64 = 1 };
 bool launch_gemm_panel(const GemmArgs& g, int tile, int amode, int bmode, unsigned cus, unsigned total_tiles, bool by_batch, hipStream_t stream);
 
 // A small left operand against a very wide right one (one matrix, K up to 256, B with unit stride along N, plain store):

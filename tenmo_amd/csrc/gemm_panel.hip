@@ -62,8 +62,7 @@ __device__ __forceinline__ void wait_loads_ahead(int units) {
 }
 
 // (the second launch bound is wavefronts per SIMD: a workgroup brings two to each)
-// PAIRED: the loading wavefronts issue two K steps at a time (kstream_loader's `paired`)
-template <int AMODE, int BMODE, int BM, int BN, bool ACC, bool PAIRED = false>
+template <int AMODE, int BMODE, int BM, int BN, bool ACC>
 __global__ __launch_bounds__(PANEL_THREADS, 2 * PANEL_WGS_PER_CU) void gemm_panel_kernel(const GemmArgs g, const PanelArgs pa) {
     constexpr int NP = panel_ring(BM, BN);
     constexpr int TM = BM / 2, TN = BN / 2;   // wave tile (2x2 multiplying wavefronts)
@@ -111,7 +110,7 @@ __global__ __launch_bounds__(PANEL_THREADS, 2 * PANEL_WGS_PER_CU) void gemm_pane
         kstream_loader(walk, nk, NP, init_tile, issue, [&](int ahead) {
             wait_loads_ahead<LPU>(ahead);
             bare_barrier();
-        }, PAIRED);
+        });
         return;
     }
 
@@ -265,7 +264,7 @@ struct PanelLaunch {
     hipStream_t stream;
 };
 
-template <int AMODE, int BMODE, int BM, int BN, bool PAIRED = false>
+template <int AMODE, int BMODE, int BM, int BN>
 void launch_panel(const GemmArgs& g, const PanelLaunch& l) {
     const TileWalkPlan plan = plan_tile_walk(l.total_tiles, (unsigned)g.tiles_m, (unsigned)g.tiles_n, l.cus, PANEL_WGS_PER_CU, l.by_batch);
     PanelArgs pa{};
@@ -273,14 +272,10 @@ void launch_panel(const GemmArgs& g, const PanelLaunch& l) {
     pa.xcds = plan.xcds; pa.chunk = plan.chunk; pa.col_major = plan.col_major;
     pa.nk = (int32_t)((g.K + GEMM_BK - 1) / GEMM_BK);
     pa.k_tail = (int32_t)(g.K - (int64_t)(pa.nk - 1) * GEMM_BK);
-    if constexpr (PAIRED) { // (plain stores only)
-        hipLaunchKernelGGL((gemm_panel_kernel<AMODE, BMODE, BM, BN, false, true>), dim3(plan.grid), dim3(PANEL_THREADS), 0, l.stream, g, pa);
-    } else {
-        if (g.accumulate)
-            hipLaunchKernelGGL((gemm_panel_kernel<AMODE, BMODE, BM, BN, true>), dim3(plan.grid), dim3(PANEL_THREADS), 0, l.stream, g, pa);
-        else
-            hipLaunchKernelGGL((gemm_panel_kernel<AMODE, BMODE, BM, BN, false>), dim3(plan.grid), dim3(PANEL_THREADS), 0, l.stream, g, pa);
-    }
+    if (g.accumulate)
+        hipLaunchKernelGGL((gemm_panel_kernel<AMODE, BMODE, BM, BN, true>), dim3(plan.grid), dim3(PANEL_THREADS), 0, l.stream, g, pa);
+    else
+        hipLaunchKernelGGL((gemm_panel_kernel<AMODE, BMODE, BM, BN, false>), dim3(plan.grid), dim3(PANEL_THREADS), 0, l.stream, g, pa);
 }
 
 template <int BM, int BN>
@@ -298,20 +293,6 @@ bool launch_panel_modes(const GemmArgs& g, int amode, int bmode, const PanelLaun
 bool launch_gemm_panel(const GemmArgs& g, int tile, int amode, int bmode, unsigned cus, unsigned total_tiles, bool by_batch, hipStream_t stream) {
     if (g.K < 1 || total_tiles == 0) return false;
     const PanelLaunch l{cus, total_tiles, by_batch, stream};
-    // two K steps issued together: for a K-major A (whose rows then give 128 adjacent bytes at a time), plain store
-    if (tile == PANEL_TILE_128x128_PAIRED || tile == PANEL_TILE_64x64_PAIRED) {
-        if (amode != KMAJOR_VEC || g.accumulate) return false;
-        if (tile == PANEL_TILE_128x128_PAIRED) {
-            if (bmode == KMAJOR_VEC) launch_panel<KMAJOR_VEC, KMAJOR_VEC, 128, 128, true>(g, l);
-            else if (bmode == MNMAJOR_VEC) launch_panel<KMAJOR_VEC, MNMAJOR_VEC, 128, 128, true>(g, l);
-            else return false;
-        } else {
-            if (bmode == KMAJOR_VEC) launch_panel<KMAJOR_VEC, KMAJOR_VEC, 64, 64, true>(g, l);
-            else if (bmode == MNMAJOR_VEC) launch_panel<KMAJOR_VEC, MNMAJOR_VEC, 64, 64, true>(g, l);
-            else return false;
-        }
-        return true;
-    }
     if (tile == PANEL_TILE_128x128) return launch_panel_modes<128, 128>(g, amode, bmode, l);
     if (tile == PANEL_TILE_64x64) return launch_panel_modes<64, 64>(g, amode, bmode, l);
     return false;

@@ -90,7 +90,7 @@ struct State {
     int force_streamk = -1;    // -1 automatic, 0 never, n > 0: stream-K with n workgroups per CU
     int force_smallk = -1;     // -1 automatic, 0 never, 1: the short-reduction kernel wherever it can run (2: without XCD grouping, 3: also for K <= 16)
     int force_resident = 0;    // the resident-A kernel for a few tile rows against a very wide B: 1 with 128x64 tiles, 2 with 64x64, 0 never
-    int force_panel = -1;      // -1 automatic, 0 never, 1: the persistent K-stream kernel wherever it can run (2: without XCD grouping, 3: 64x64 tiles, 4 / 5: 128x128 / 64x64 tiles with paired K steps)
+    int force_panel = -1;      // -1 automatic, 0 never, 1: the persistent K-stream kernel wherever it can run (2: without XCD grouping, 3: 64x64 tiles)
     int mlp_fused_tail = 0;    // MLP step: 1 the last two layers, loss, their backward and update in one launch when the shapes fit; 2 also the first layer's weight gradient and update in one; 3 also the first layer's forward in one; 0 neither
     int fold_reduce = -1;      // the gradient of a broadcast parent summed inside the GEMM launch: -1 automatic, 0 never, 1 wherever it can
     int verbose = 0;
@@ -392,10 +392,8 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
             if (mode == MNMAJOR_VEC) return row_s == 1 && k_s >= 0 && k_s <= (int64_t(1) << 25) && extent % 4 == 0 && extent >= 4;
             return false;
         };
-        // (3: its 64x64-tile variant, a ring of eight stages, forced: for long reductions over few tiles; 4 / 5: 128x128 / 64x64 tiles with
-        // the loads of two K steps issued together, for a K-major A read in 64-byte pieces from rows far apart)
-        const int pt = S.force_panel == 3 || S.force_panel == 5 ? 64 : 128;
-        const bool paired = (S.force_panel == 4 || S.force_panel == 5) && am == KMAJOR_VEC && !accumulate;
+        // (3: its 64x64-tile variant, a ring of eight stages, forced: for long reductions over few tiles)
+        const int pt = S.force_panel == 3 ? 64 : 128;
         const int64_t tm = (M + pt - 1) / pt, tn = (N + pt - 1) / pt, tiles = tm * tn * batch_count;
         const bool can = K > GEMM_BK && operand_ok(am, a_rs, a_cs, M) && operand_ok(bm, b_cs, b_rs, N) && !ep.any() && !ep.gather_row && !ep.colsum && !ep.bsum &&
                          N <= (int64_t(1) << 22) && tiles <= 0x7fffffffLL;
@@ -405,7 +403,7 @@ int gemm_dispatch(const float* A, int64_t a_rs, int64_t a_cs, const float* B, in
             g.tiles_m = (int32_t)tm; g.tiles_n = (int32_t)tn;
             g.k_splits = 1; g.k_per_split = K; g.partial = nullptr;
             if (S.verbose) fprintf(stderr, "tenmo_hip gemm: K-stream kernel, %lld tiles of %dx%d\n", (long long)tiles, pt, pt);
-            const int which = pt == 64 ? (paired ? PANEL_TILE_64x64_PAIRED : PANEL_TILE_64x64) : (paired ? PANEL_TILE_128x128_PAIRED : PANEL_TILE_128x128);
+            const int which = pt == 64 ? PANEL_TILE_64x64 : PANEL_TILE_128x128;
             if (launch_gemm_panel(g, which, am, bm, (unsigned)S.cus, (unsigned)tiles, S.force_panel != 2, S.stream)) return 0;
         }
     }

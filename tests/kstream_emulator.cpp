@@ -32,7 +32,6 @@ struct EmuProblem {
     int32_t bm, bn, np;             // workgroup tile and ring depth
     uint32_t cus, wgs_per_cu;       // the launch: persistent workgroups per compute unit
     int32_t group_by_xcd;
-    int32_t paired;                 // the loaders issue two K steps at a time (kstream_loader's `paired`)
 };
 
 struct EmuReport {
@@ -121,8 +120,7 @@ void run(const EmuProblem& P, EmuReport& R) {
                     for (int u = 0; u < done; ++u)
                         if (certified_by[u] < 0) certified_by[u] = loader_barriers;
                     ++loader_barriers;
-                },
-                P.paired != 0);
+                });
         }
         R.steps += (int64_t)issues.size();
         CHECK(loader_barriers == (int)issues.size(), "workgroup %u: %d loader barriers for %zu steps", wg, loader_barriers, issues.size());

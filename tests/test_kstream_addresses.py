@@ -25,7 +25,7 @@ class EmuProblem(C.Structure):
     _fields_ = [("M", C.c_int64), ("N", C.c_int64), ("K", C.c_int64), ("a_mn_major", C.c_int32), ("b_mn_major", C.c_int32),
                 ("a_rs", C.c_int64), ("a_cs", C.c_int64), ("b_rs", C.c_int64), ("b_cs", C.c_int64), ("batch", BatchDesc),
                 ("batch_count", C.c_int64), ("bm", C.c_int32), ("bn", C.c_int32), ("np", C.c_int32),
-                ("cus", C.c_uint32), ("wgs_per_cu", C.c_uint32), ("group_by_xcd", C.c_int32), ("paired", C.c_int32)]
+                ("cus", C.c_uint32), ("wgs_per_cu", C.c_uint32), ("group_by_xcd", C.c_int32)]
 
 
 class EmuReport(C.Structure):
@@ -43,7 +43,7 @@ def emu(tmp_path_factory):
     return lib
 
 
-def problem(M, N, K, a_layout, b_layout, batch=(), b_shared=False, a_pad=0, b_pad=0, tile=(128, 128), np_=5, cus=256, wpc=2, group=True, paired=False):
+def problem(M, N, K, a_layout, b_layout, batch=(), b_shared=False, a_pad=0, b_pad=0, tile=(128, 128), np_=5, cus=256, wpc=2, group=True):
     """a_layout / b_layout: 'k' (unit stride along the reduction: row-major A, transposed-view B) or 'mn'."""
     p = EmuProblem()
     p.M, p.N, p.K = M, N, K
@@ -69,7 +69,6 @@ def problem(M, N, K, a_layout, b_layout, batch=(), b_shared=False, a_pad=0, b_pa
         count *= batch[d]
     p.batch_count = count
     p.bm, p.bn, p.np = tile[0], tile[1], np_
-    p.paired = int(paired)
     p.cus, p.wgs_per_cu, p.group_by_xcd = cus, wpc, int(group)
     return p
 
@@ -134,18 +133,6 @@ def test_64x64_tiles_with_a_ring_of_eight(emu, la, lb):
             run(emu, problem(M, N, K, la, lb, tile=(64, 64), np_=8, cus=cus))
     run(emu, problem(256, 384, 64, la, lb, batch=(16,), tile=(64, 64), np_=8, cus=8))
     run(emu, problem(132, 260, 48, la, lb, batch=(9,), b_shared=True, tile=(64, 64), np_=8, cus=16))  # (an MN-major extent must be a multiple of 4)
-
-
-@pytest.mark.parametrize("np_", [4, 5, 7, 8])
-def test_paired_k_steps(emu, np_):
-    """The loaders issue two K steps behind every second barrier (an odd ring behind the odd barriers, an even one behind the
-    even ones, one step shorter at the start): the hand-over must stay safe and complete for streams of one step, fewer
-    steps than the ring, odd and even step counts per tile, and walks of many tiles."""
-    tile = (64, 64) if np_ == 8 else (128, 128)
-    for (M, N, K) in [(128, 128, 16), (128, 128, 32), (128, 256, 48), (512, 512, 80), (300, 520, 100), (256, 384, 1024), (132, 260, 20)]:
-        for cus in (1, 4):
-            run(emu, problem(M, N, K, "k", "mn", tile=tile, np_=np_, cus=cus, paired=True))
-    run(emu, problem(256, 384, 64, "k", "k", batch=(16,), tile=tile, np_=np_, cus=8, paired=True))
 
 
 def test_one_workgroup_per_cu(emu):

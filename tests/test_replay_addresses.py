@@ -139,20 +139,6 @@ def test_k_stream_kernel(exe):
         small.append(case(132, 260, 48, la, lb, batch=9, b_shared=1, acc=1, gemm_panel=3))
     run(exe, small, cus=2)
     run(exe, small[:8] + [case(1024, 1024, 1024, gemm_panel=3)], cus=256, modes=("late",))
-    # two K steps issued at a time (a K-major A, plain store; anything else under these knob values takes the unpaired kernel)
-    paired = []
-    for knob in (4, 5):
-        for lb in ("n", "t"):
-            for (M, N, K) in [(128, 128, 32), (300, 520, 100), (132, 260, 20), (256, 384, 112), (512, 512, 256), (1024, 64, 1024), (128, 256, 48)]:
-                paired.append(case(M, N, K, "n", lb, gemm_panel=knob))
-            paired.append(case(256, 384, 64, "n", lb, batch=16, gemm_panel=knob))
-        paired.append(case(132, 260, 48, "t", "n", gemm_panel=knob))
-        paired.append(case(132, 260, 48, "n", "n", acc=1, gemm_panel=knob))
-    run(exe, paired, cus=2)
-    run(exe, paired[:6] + [case(1024, 64, 1024, "n", "n", batch=12, gemm_panel=5)], cus=256, modes=("late",))
-    # ... and it is the paired instantiation (last template argument) that serves a row-major A, the unpaired one a transposed view
-    run(exe, [case(300, 520, 100, "n", "n", gemm_panel=4, ran="BN; false; true>"), case(300, 520, 100, "n", "t", gemm_panel=5, ran="BN; false; true>"),
-              case(300, 520, 100, "t", "n", gemm_panel=4, ran="BN; false>")], cus=2, modes=("late",))
 
 
 def test_resident_left_operand_kernel(exe):

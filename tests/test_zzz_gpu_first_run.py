@@ -5,7 +5,7 @@ matters, on the generated gfx950 code (tests/test_asm_clobbers.py, tests/test_is
 after every other GPU test, so that a first GPU run which goes wrong here has already recorded the rest; a test moves
 to tests/test_gpu_parity.py once it has passed on a GPU.  In order of collection: the default path first (the batch-
 reducing launch behind the gradients of broadcast parents), then the kernels behind knobs that are off by default (K
-slices joined inside the column kernels' launch, the fused MLP launches, the K-stream kernel's 64x64 and paired forms, the
+slices joined inside the column kernels' launch, the fused MLP launches, the K-stream kernel's 64x64 form, the
 resident-A kernel), the Linear backward with the bias gradient summed in the weight-gradient launch, last the short-reduction
 kernel forced onto reductions that are no multiple of 16 and onto one-step reductions (K <= 16) — the paths that use the masked
 direct load (its fault, an undeclared SCC clobber, is fixed; these are the runs that confirm it).
@@ -206,13 +206,6 @@ def test_kstream_kernel_with_64x64_tiles(T):
     """The same cases through the kernel's 64x64-tile variant (a ring of eight stages; two operand fetches behind an MFMA
     where an operand is MN-major)."""
     _kstream_cases(T, 3)
-
-
-def test_kstream_kernel_with_paired_k_steps(T):
-    """The same cases with the loading wavefronts issuing two K steps at a time (128x128 and 64x64 tiles; the cases with
-    a transposed-view A or an accumulating store take the unpaired kernel)."""
-    _kstream_cases(T, 4)
-    _kstream_cases(T, 5)
 
 
 def test_resident_left_operand_kernel(T):
