@@ -368,6 +368,28 @@ def test_fused_epilogue(T, tile):
         L.tenmo_hip_set_tuning(b"gemm_splitk", -1)
 
 
+def test_relu_epilogue_reference_literals(T, golden):
+    """The ReLU and ReLU-gradient epilogues on the literals of tests/test_relu.mojo: x.I (+ bias) through the GEMM with the
+    ReLU in its store gives the reference's output, ones.I masked by that activation the reference's gradient — exactly
+    (products with an identity matrix are exact), in particular 0 at x = 0."""
+    L, lib = T.lib.load(), T.lib
+    for c in golden["harness"]["relu_literals"]["cases"]:
+        x = np.asarray(c["x"], np.float32)[None, :]
+        n = x.shape[1]
+        bias = np.asarray(c["bias"], np.float32) if "bias" in c else None
+        X, I, one = T.Tensor.from_numpy(x), T.Tensor.from_numpy(np.eye(n, dtype=np.float32)), T.Tensor.from_numpy(np.ones((1, n), np.float32))
+        Bi = T.Tensor.from_numpy(bias) if bias is not None else None
+        h, g = T.Tensor.zeros(1, n), T.Tensor.zeros(1, n)
+        lib.check(L.tenmo_hip_gemm_epilogue_f32(X.buffer.data_ptr(), 0, n, 1, I.buffer.data_ptr(), 0, n, 1, h.buffer.data_ptr(), 1, n, n,
+                                                0, None, None, None, Bi.buffer.data_ptr() if Bi is not None else None, 1, None, 1))
+        want = np.asarray(c["out"], np.float32) if "out" in c else np.maximum(x[0] + (bias if bias is not None else 0), 0)
+        np.testing.assert_array_equal(h.to_numpy()[0], want, err_msg=c["source"])
+        if "grad" in c:
+            lib.check(L.tenmo_hip_gemm_epilogue_f32(one.buffer.data_ptr(), 0, n, 1, I.buffer.data_ptr(), 0, n, 1, g.buffer.data_ptr(), 1, n, n,
+                                                    0, None, None, None, None, 0, h.buffer.data_ptr(), 1))
+            np.testing.assert_array_equal(g.to_numpy()[0], np.asarray(c["grad"], np.float32), err_msg=c["source"])
+
+
 def test_column_sum(T):
     """Bias gradient = column sums of the upstream gradient (tenmo/broadcast.mojo:81-87): small, ragged,
     padded rows, accumulate, and a size that takes the K-sliced streaming path."""

@@ -276,6 +276,31 @@ def test_mlp_harness_pieces(golden, oracle):
         np.testing.assert_allclose(w, s["expect"], rtol=1e-6)
 
 
+def test_relu_and_its_mask_are_pinned(golden, oracle):
+    """The ReLU of the restated step and the mask its backward multiplies by (tenmo/relu.mojo:99-141, :21-46: x > 0, so
+    the gradient at exactly 0 is 0) against the literals of tests/test_relu.mojo: a net [n, n, n] with identity weights
+    computes relu(x + bias) as its logits; the hidden layer's bias gradient is then the output layer's times the mask, and
+    its weight gradient the outer product of x with that."""
+    for c in golden["harness"]["relu_literals"]["cases"]:
+        x = np.asarray(c["x"], np.float32)[None, :]
+        n = x.shape[1]
+        bias = np.asarray(c.get("bias", [0.0] * n), np.float32)
+        eye = np.eye(n, dtype=np.float32)
+        m = oracle.MLP([n, n, n], [eye, eye], [bias, np.zeros(n, np.float32)], 1)
+        if "out" in c:
+            np.testing.assert_array_equal(m.forward(x)[0], np.asarray(c["out"], np.float32), err_msg=c["source"])
+        else:
+            np.testing.assert_array_equal(m.forward(x)[0], np.maximum(x[0] + bias, 0))
+        if "grad" in c:
+            m.step(x, np.zeros(1, np.int32), 0.0)
+            dW1, db1 = m.grads(1)
+            dW0, db0 = m.grads(0)
+            assert np.all(db1 != 0), c["source"]
+            mask = np.asarray(c["grad"], np.float32)
+            np.testing.assert_array_equal(db0, db1 * mask, err_msg=c["source"])
+            np.testing.assert_array_equal(dW0, np.outer(x[0], db1 * mask), err_msg=c["source"])
+
+
 def test_mlp_step_matches_numpy_fp64(oracle):
     """The whole restated step against an independent fp64 numpy implementation."""
     O = oracle
