@@ -264,6 +264,23 @@ def test_linear_backward_reference_literal(T, golden):
     assert np.array_equal(out.to_numpy(), np.array(case["expect"], np.float32))
 
 
+def test_linear_backward_refuses_what_matmul_refuses(T):
+    """Same argument errors as the matmul entry points, before anything is launched: an inner-dimension mismatch is the reference's
+    panic (tenmo/matmul.mojo:226-227), a gradient asked for without an upstream gradient is an invalid argument; a call that asks for
+    no gradient at all is accepted and does nothing."""
+    import ctypes as C
+
+    L = T.lib.load()
+    X, W, bad = T.Tensor.zeros(5, 7), T.Tensor.zeros(7, 3), T.Tensor.zeros(6, 3)
+    g = T.Tensor.from_numpy(np.full(3, 2.0, np.float32))
+    assert L.tenmo_hip_linear_backward(C.byref(X.buffer.c_view()), C.byref(bad.buffer.c_view()), X.buffer.data_ptr(), None, None, g.buffer.data_ptr(), 1) < 0
+    assert b"incompatible" in L.tenmo_hip_last_error() or b"inner" in L.tenmo_hip_last_error()
+    assert L.tenmo_hip_linear_backward(C.byref(X.buffer.c_view()), C.byref(W.buffer.c_view()), None, None, None, g.buffer.data_ptr(), 1) < 0
+    assert b"upstream gradient" in L.tenmo_hip_last_error()
+    assert L.tenmo_hip_linear_backward(C.byref(X.buffer.c_view()), C.byref(W.buffer.c_view()), None, None, None, None, 1) == 0
+    np.testing.assert_array_equal(g.to_numpy(), np.full(3, 2.0, np.float32))
+
+
 def test_linear_backward_sums_the_bias_gradient_in_the_weight_gradient_launch(T, oracle):
     """tenmo_hip_linear_backward: dX, dW and the bias gradient of x.W + b (tenmo/net.mojo:193-201 = Matmul then Adder; the
     bias gradient is sum_over_broadcasted_axes of the upstream gradient, tenmo/broadcast.mojo:66-88) against the oracle
