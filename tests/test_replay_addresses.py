@@ -320,3 +320,13 @@ def test_short_reduction_kernel_on_one_step_reductions(exe):
         cases.append(case(200, 264, 12, la, lb, batch=3, b_shared=1, acc=1, gemm_smallk=3, ran="gemm_smallk_kernel"))
     run(exe, cases, cus=2)
     run(exe, [case(8192, 8192, 16, "n", "t", gemm_smallk=3, ran="gemm_smallk_kernel", check=0)], modes=("late",), timeout=1800)
+
+
+@pytest.mark.skipif(os.environ.get("TENMO_REPLAY_FULL") != "1", reason="a quarter of an hour of CPU time: set TENMO_REPLAY_FULL=1")
+def test_benchmark_shapes_at_full_size_under_the_default_dispatch(exe):
+    """The benchmark's own shapes, whole, at 256 CUs, through whatever kernel the library picks by itself: two GPT-2 Linear products,
+    the up-projection's Linear backward with the bias gradient in the weight-gradient launch, the attention Q.K^T backward (8 of its
+    96 batches), the broadcast-batched backward A[32,512,768].B[1,768,768], both CBOW products and the skinny product."""
+    cases = ["8192,2304,768,n,n,0,0,0", "8192,768,3072,n,n,0,0,0", "lin:8192,3072,768,n,n,0,0,fused=1", "bwd:1024,1024,64,n,t,8,8",
+             "bwd:512,768,768,n,n,32,1", "256,50000,100,n,n,0,0,0", "100,50000,256,t,n,0,0,0", "4,50257,768,n,n,0,0,0"]
+    run(exe, cases, cus=256, modes=("late",), timeout=3000)
