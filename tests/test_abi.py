@@ -100,6 +100,33 @@ def test_missing_library_is_loud(monkeypatch, tmp_path):
         _lib.load()
 
 
+def test_the_product_never_touches_the_oracle():
+    """The oracle is test infrastructure: nothing in the package, the header or the glue names it, the library does not link
+    it, and bench.py imports it only inside the two functions that time / replay the CPU side."""
+    import ast
+    import subprocess
+
+    for top in ("tenmo_amd", "include", "integration"):
+        for folder, _dirs, files in os.walk(os.path.join(ROOT, top)):
+            if "__pycache__" in folder:
+                continue
+            for name in files:
+                if name.endswith((".py", ".hip", ".hpp", ".h", ".mojo")):
+                    assert "oracle" not in open(os.path.join(folder, name)).read().lower(), os.path.join(folder, name)
+    needed = subprocess.run(["readelf", "-d", os.path.join(ROOT, "tenmo_amd", "libtenmo_hip.so")], capture_output=True, text=True).stdout
+    assert "NEEDED" in needed and "oracle" not in needed
+    tree = ast.parse(open(os.path.join(ROOT, "bench.py")).read())
+    importers = set()
+    for fn in ast.walk(tree):
+        if isinstance(fn, (ast.FunctionDef, ast.AsyncFunctionDef)):
+            for node in ast.walk(fn):
+                if isinstance(node, ast.ImportFrom) and (node.module or "").startswith("oracle"):
+                    importers.add(fn.name)
+    assert importers == {"cpu_gemm_baseline", "mlp_step_times"}, importers
+    for node in tree.body:  # and never at module level
+        assert not (isinstance(node, (ast.Import, ast.ImportFrom)) and "oracle" in ast.dump(node))
+
+
 def test_blas_handle_load_failure_is_recorded(tmp_path):
     """tenmo/blashandle.mojo:183-191, :227-228"""
     from tenmo_amd.blashandle import BLASHandle
