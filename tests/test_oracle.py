@@ -115,6 +115,55 @@ def test_padded_row_views(oracle):
     assert info["path"] == 1  # only A padded
 
 
+def test_random_views_against_fp64(oracle):
+    """Property check over what the reference calls a view (tenmo/matmul_cpu.mojo:710-724: offset, strides, dims of size
+    1 read with stride 0): operands cut out of larger storage with steps, offsets, swapped last axes, expanded (stride 0)
+    and broadcast batch dimensions, ranks 2 to 5, extents around the tile and vector edges — against numpy in float64."""
+    from hypothesis import given, settings, strategies as st
+
+    extent = st.sampled_from([1, 2, 3, 5, 8, 15, 16, 17, 31, 33, 64, 65, 70])
+
+    @st.composite
+    def operands(draw):
+        m, k, n = draw(extent), draw(extent), draw(extent)
+        batch = draw(st.lists(st.integers(1, 3), min_size=0, max_size=3))
+        seed = draw(st.integers(0, 2**31 - 1))
+        rng = np.random.default_rng(seed)
+
+        def view(rows, cols, own_batch):
+            step_r, step_c = draw(st.integers(1, 2)), draw(st.integers(1, 3))
+            off_r, off_c = draw(st.integers(0, 2)), draw(st.integers(0, 3))
+            swapped = draw(st.booleans())
+            r, c = (cols, rows) if swapped else (rows, cols)
+            store = rng.standard_normal(tuple(own_batch) + (off_r + r * step_r, off_c + c * step_c + draw(st.integers(0, 2))), dtype=np.float32)
+            v = store[..., off_r:off_r + r * step_r:step_r, off_c:off_c + c * step_c:step_c]
+            return np.swapaxes(v, -1, -2) if swapped else v
+
+        # each operand keeps, drops (size 1) or lacks each batch dimension; a kept size-1 dimension may be expanded with stride 0
+        def own(batch):
+            dims = [d if draw(st.booleans()) else 1 for d in batch]
+            return dims[draw(st.integers(0, len(dims))):]
+
+        a, b = view(m, k, own(batch)), view(k, n, own(batch))
+        if a.ndim > 2 and a.shape[0] == 1 and draw(st.booleans()):
+            a = np.broadcast_to(a, (draw(st.integers(2, 3)),) + a.shape[1:]) if b.ndim < a.ndim or b.shape[len(b.shape) - a.ndim] == 1 else a
+        return a, b
+
+    @settings(max_examples=150, deadline=None, derandomize=True)
+    @given(operands())
+    def check(ab):
+        a, b = ab
+        try:
+            want = np.matmul(a.astype(np.float64), b.astype(np.float64))
+        except ValueError:
+            return  # (the expanded dimension met an incompatible one)
+        got = oracle.matmul(a, b)
+        assert got.shape == want.shape
+        assert rel_fro(got, want) < 2e-6, (a.shape, a.strides, b.shape, b.strides)
+
+    check()
+
+
 def test_tile_table(oracle):
     """tenmo/matmul_cpu.mojo:87-89 and the worked example docs/from-bytes-to-gradients.md:171-177."""
     O = oracle
