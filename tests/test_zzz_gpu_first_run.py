@@ -99,6 +99,49 @@ def test_backward_of_broadcast_parents(T, oracle, fold):
     finally:
         L.tenmo_hip_set_tuning(b"fold_reduce", -1)
 
+def test_randomized_backward_of_views_and_broadcast_parents(T, oracle):
+    """Seeded sweep of Matmul backward (tenmo/matmul.mojo:24-54, :101-137) at the Tensor level: batch shapes of rank 0 to 3 in which
+    each parent keeps, drops or lacks every dimension, operands that are plain, transposed, stepped or offset views of larger
+    storage, ragged and whole tiles, the sum over the broadcast dimensions folded into the launch, materialised, or chosen
+    automatically; gradients against the oracle on dense copies of the same views, twice (the second backward accumulates)."""
+    L = T.lib.load()
+    rng = np.random.default_rng(211)
+
+    def operand(rows, cols, own_batch):
+        kind = rng.choice(["plain", "transposed", "stepped", "offset"])
+        if kind == "plain":
+            return rng.standard_normal(tuple(own_batch) + (rows, cols), dtype=np.float32)
+        if kind == "transposed":
+            return np.swapaxes(rng.standard_normal(tuple(own_batch) + (cols, rows), dtype=np.float32), -1, -2)
+        if kind == "stepped":
+            return rng.standard_normal(tuple(own_batch) + (2 * rows, 2 * cols), dtype=np.float32)[..., ::2, ::2]
+        return rng.standard_normal(tuple(own_batch) + (rows + 3, cols + 4), dtype=np.float32)[..., 2:2 + rows, 4:4 + cols]
+
+    try:
+        for case in range(40):
+            m, k, n = (int(rng.choice([1, 5, 33, 64, 70, 130, 200])) for _ in range(3))
+            batch = [int(rng.integers(2, 5)) for _ in range(int(rng.integers(0, 4)))]
+
+            def own():
+                dims = [d if rng.random() < 0.6 else 1 for d in batch]
+                return dims[int(rng.integers(0, len(dims) + 1)):]
+
+            a, b = operand(m, k, own()), operand(k, n, own())
+            fold = int(rng.choice([-1, 0, 1]))
+            L.tenmo_hip_set_tuning(b"fold_reduce", fold)
+            A, B = as_strided_tensor(T, a, requires_grad=True), as_strided_tensor(T, b, requires_grad=True)
+            out = A.matmul(B)
+            desc = (case, a.shape, a.strides, b.shape, b.strides, fold)
+            assert rel_fro(out.to_numpy(), ref_matmul64(a, b)) <= RTOL_FRO, desc
+            seed = rng.standard_normal(out.shape(), dtype=np.float32)
+            out.backward(T.Tensor.from_numpy(seed), retain_graph=True)
+            out.backward(T.Tensor.from_numpy(seed))
+            gA, gB = oracle.matmul_backward(np.ascontiguousarray(a), np.ascontiguousarray(b), seed)
+            assert A.grad().shape == a.shape and B.grad().shape == b.shape, desc
+            assert rel_fro(A.grad(), 2 * gA) <= 2 * RTOL_FRO and rel_fro(B.grad(), 2 * gB) <= 2 * RTOL_FRO, desc
+    finally:
+        L.tenmo_hip_set_tuning(b"fold_reduce", -1)
+
 
 def test_column_kernels_join_slices_in_the_launch(T):
     """vm, mv on a transposed view, skinny and batched skinny products with the K slices added by the last workgroup of
