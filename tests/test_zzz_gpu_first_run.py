@@ -142,6 +142,52 @@ def test_randomized_backward_of_views_and_broadcast_parents(T, oracle):
     finally:
         L.tenmo_hip_set_tuning(b"fold_reduce", -1)
 
+def test_randomized_mv_vm_backward_of_views(T, oracle):
+    """Seeded sweep of the mv / vm gradients (tenmo/matrixvector.mojo:19-201, tenmo/vectormatrix.mojo:18-206) at the Tensor level:
+    matrices that are plain, transposed, stepped or offset views, vectors with a step, batch shapes in which matrix and vector each
+    keep, drop or lack a dimension (a shared vector's gradient is summed over the batches, a shared matrix's outer products
+    likewise); against the oracle on dense copies, twice."""
+    rng = np.random.default_rng(223)
+
+    def matrix(rows, cols, own_batch):
+        kind = rng.choice(["plain", "transposed", "stepped", "offset"])
+        if kind == "plain":
+            return rng.standard_normal(tuple(own_batch) + (rows, cols), dtype=np.float32)
+        if kind == "transposed":
+            return np.swapaxes(rng.standard_normal(tuple(own_batch) + (cols, rows), dtype=np.float32), -1, -2)
+        if kind == "stepped":
+            return rng.standard_normal(tuple(own_batch) + (2 * rows, 2 * cols), dtype=np.float32)[..., ::2, ::2]
+        return rng.standard_normal(tuple(own_batch) + (rows + 3, cols + 4), dtype=np.float32)[..., 2:2 + rows, 4:4 + cols]
+
+    def vector(n, own_batch):
+        step = int(rng.choice([1, 1, 2]))
+        return rng.standard_normal(tuple(own_batch) + (n * step,), dtype=np.float32)[..., ::step]
+
+    for case in range(40):
+        r, c = (int(rng.choice([1, 4, 33, 64, 130, 515, 1030])) for _ in range(2))
+        batch = [int(rng.integers(2, 5)) for _ in range(int(rng.integers(0, 3)))]
+
+        def own():
+            dims = [d if rng.random() < 0.6 else 1 for d in batch]
+            return dims[int(rng.integers(0, len(dims) + 1)):]
+
+        mn = matrix(r, c, own())
+        as_mv = rng.random() < 0.5
+        vn = vector(c if as_mv else r, own())
+        Mt, vt = as_strided_tensor(T, mn, requires_grad=True), as_strided_tensor(T, vn, requires_grad=True)
+        out = Mt.matmul(vt, mode=T.mv) if as_mv else vt.matmul(Mt, mode=T.vm)
+        desc = (case, "mv" if as_mv else "vm", mn.shape, mn.strides, vn.shape, vn.strides)
+        seed = rng.standard_normal(out.shape(), dtype=np.float32)
+        out.backward(T.Tensor.from_numpy(seed), retain_graph=True)
+        out.backward(T.Tensor.from_numpy(seed))
+        md, vd = np.ascontiguousarray(mn), np.ascontiguousarray(vn)
+        if as_mv:
+            dM, dv = oracle.mv_backward(md, vd, seed)
+        else:
+            dv, dM = oracle.vm_backward(vd, md, seed)
+        assert Mt.grad().shape == mn.shape and vt.grad().shape == vn.shape, desc
+        assert rel_fro(Mt.grad(), 2 * dM) <= 2 * RTOL_FRO and rel_fro(vt.grad(), 2 * dv) <= 2 * RTOL_FRO, desc
+
 
 def test_column_kernels_join_slices_in_the_launch(T):
     """vm, mv on a transposed view, skinny and batched skinny products with the K slices added by the last workgroup of
