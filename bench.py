@@ -73,8 +73,8 @@ def main() -> int:
     ap.add_argument("--no-extra", action="store_true", help="skip the per-configuration rows and the MLP-step measurement")
     ap.add_argument("--clock-probe-rounds", type=int, default=50000, help="length of the shader-clock probe (rounds of four MFMAs per wavefront)")
     ap.add_argument("--mlp-fused-tail", action="store_true",
-                    help="also time the MLP step with its last two layers, loss, backward and update fused into one launch, and with the first layer's "
-                    "gradient and update fused as well (mlp_fused_tail knob 1 and 2)")
+                    help="also time the MLP step with its last two layers, loss, backward and update fused into one launch, with the first layer's "
+                    "gradient and update fused as well, and with the first layer's forward as one launch too (mlp_fused_tail knob 1, 2 and 3)")
     ap.add_argument("--tune", default="", help="comma-separated name=value overrides of the kernel selection (tenmo_hip_set_tuning) for the rows, "
                     "e.g. gemm_panel=1,gemm_smallk=0: the same committed rows under another kernel choice")
     ap.add_argument("--sweep", default="", help="semicolon-separated lists in the form of --tune: the chosen rows (--rows) are timed once more "
