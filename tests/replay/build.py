@@ -89,6 +89,11 @@ def build_gemm_asan() -> str:
     return _build("asan", ASAN, ["replay_gemm_main.cpp"], [], "replay_gemm_asan")
 
 
+def build_gemm_plain() -> str:
+    """replay_gemm_main.cpp without a sanitizer: the producer of launch dumps (REPLAY_DUMP_DIR) for tests/isa/."""
+    return _build("plain", [], ["replay_gemm_main.cpp"], ["-ldl"], "replay_gemm_plain")
+
+
 def build_selftest() -> str:
     """replay_selftest.cpp (deliberately wrong toy kernels) under AddressSanitizer."""
     os.makedirs(OUT, exist_ok=True)

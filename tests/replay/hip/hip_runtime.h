@@ -23,7 +23,10 @@
 #include <cstdint>
 #include <cstring>
 #include <functional>
+#include <tuple>
 #include <type_traits>
+#include <utility>
+#include <vector>
 
 // ---- qualifiers ---------------------------------------------------------------------------------------------------
 #define __host__
@@ -85,7 +88,6 @@ void wg_barrier();               // every live lane of the workgroup arrives
 void complete_loads(int leave);  // this lane's direct loads land until at most `leave` are outstanding
 void check_global(const void* p, size_t bytes, bool write, const char* what);
 void fail(const char* fmt, ...) __attribute__((noreturn));
-void launch(const char* name, dim3 grid, dim3 block, std::function<void()> body);
 
 // v_mfma_f32_32x32x2_f32: lane l brings A[i = l % 32][k = l / 32] and B[k = l / 32][j = l % 32]; it receives, in
 // element e of its 16, D[8 (e / 4) + 4 (l / 32) + e % 4][l % 32]
@@ -252,11 +254,41 @@ hipError_t hipGraphLaunch(hipGraphExec_t e, hipStream_t s);
 template <class T> inline hipError_t hipMalloc(T** p, size_t bytes) { return hipMalloc(reinterpret_cast<void**>(p), bytes); }
 
 namespace replay {
-void enqueue(hipStream_t s, const char* name, dim3 grid, dim3 block, std::function<void()> body);
+// what a real launch would put into the kernel's argument block: the arguments converted to the kernel's parameter types, each at
+// its natural alignment (the layout of these plain structs is the same on the host and on the GPU), and the kernel function itself
+struct KernelArgs {
+    const void* fn = nullptr;
+    std::vector<unsigned char> bytes;
+};
+template <class T, size_t I, class Tuple>
+inline T nth_argument_or_zero(const Tuple& given) {
+    // (a trailing parameter the launch leaves to its default: every such default in the library is a null pointer or 0)
+    if constexpr (I < std::tuple_size_v<Tuple>) return static_cast<T>(std::get<I>(given));
+    else return T{};
+}
+template <class... P, size_t... I, class Tuple>
+inline void pack_each(KernelArgs& k, std::index_sequence<I...>, const Tuple& given) {
+    auto put = [&k](auto value) {
+        using T = decltype(value);
+        const size_t at = (k.bytes.size() + alignof(T) - 1) / alignof(T) * alignof(T);
+        k.bytes.resize(at + sizeof(T));
+        std::memcpy(k.bytes.data() + at, &value, sizeof(T));
+    };
+    (put(nth_argument_or_zero<std::remove_cv_t<P>, I>(given)), ...);
+}
+template <class... P, class... A>
+inline KernelArgs pack_args(void (*fn)(P...), const A&... a) {
+    KernelArgs k;
+    k.fn = reinterpret_cast<const void*>(fn);
+    pack_each<P...>(k, std::index_sequence_for<P...>{}, std::forward_as_tuple(a...));
+    return k;
+}
+void enqueue(hipStream_t s, const char* name, dim3 grid, dim3 block, std::function<void()> body, KernelArgs args);
 }
 // the arguments are evaluated now and copied into the launch, as the real launch copies them into the kernel's argument block
-#define hipLaunchKernelGGL(kernel, grid, block, shmem, stream, ...) \
-    replay::enqueue((stream), #kernel, dim3(grid), dim3(block), replay::bind_kernel([](auto... a) { kernel(a...); }, __VA_ARGS__))
+#define hipLaunchKernelGGL(kernel, grid, block, shmem, stream, ...)                                                                 \
+    replay::enqueue((stream), #kernel, dim3(grid), dim3(block), replay::bind_kernel([](auto... a) { kernel(a...); }, __VA_ARGS__), \
+                    replay::pack_args(kernel, __VA_ARGS__))
 
 namespace replay {
 template <class F, class... Args>

@@ -2,6 +2,7 @@
 // runtime calls the library's host side makes.  Test infrastructure; see the header for what is modelled.
 #include <hip/hip_runtime.h>
 
+#include <dlfcn.h>
 #include <sys/mman.h>
 
 #include <atomic>
@@ -327,9 +328,41 @@ void run_on_pool(const std::function<void()>& job) {
 std::atomic<long> g_launches{0};
 std::string g_last_kernel; // (launches are serialized)
 
-void launch(const char* name, dim3 grid, dim3 block, std::function<void()> body) {
-    ++g_launches;
+// REPLAY_DUMP_DIR: every launch leaves what is needed to run the same launch elsewhere (the emulator of the generated GPU code,
+// tests/isa/): the kernel function (its offset in the file it lives in, for the symbol table), grid and block, the argument block, and
+// every device allocation before and after the launch.
+void dump_memory(const std::string& path) {
+    FILE* f = fopen(path.c_str(), "wb");
+    if (!f) return;
+    std::lock_guard<std::mutex> lock(g_mem_mutex);
+    for (const auto& a : g_allocs) {
+        const uint64_t head[2] = {(uint64_t)a.first, (uint64_t)a.second};
+        fwrite(head, sizeof(head), 1, f);
+        fwrite((const void*)a.first, 1, a.second, f);
+    }
+    fclose(f);
+}
+
+void launch(const char* name, dim3 grid, dim3 block, std::function<void()> body, const KernelArgs& args) {
+    const long index = g_launches++;
     g_last_kernel = name;
+    const char* dump_dir = getenv("REPLAY_DUMP_DIR");
+    char stem[512] = "";
+    if (dump_dir && args.fn) {
+        std::snprintf(stem, sizeof(stem), "%s/launch_%04ld", dump_dir, index);
+        Dl_info info{};
+        dladdr(args.fn, &info);
+        FILE* f = fopen((std::string(stem) + ".txt").c_str(), "w");
+        if (f) {
+            fprintf(f, "kernel %s\nfile %s\noffset %llu\nsymbol %s\ngrid %u %u %u\nblock %u %u %u\nargs ", name, info.dli_fname ? info.dli_fname : "?",
+                    (unsigned long long)((uintptr_t)args.fn - (uintptr_t)info.dli_fbase), info.dli_sname ? info.dli_sname : "?", grid.x, grid.y, grid.z,
+                    block.x, block.y, block.z);
+            for (unsigned char b : args.bytes) fprintf(f, "%02x", b);
+            fprintf(f, "\n");
+            fclose(f);
+        }
+        dump_memory(std::string(stem) + ".before");
+    }
     const int64_t total = (int64_t)grid.x * grid.y * grid.z;
     if ((int64_t)block.x * block.y * block.z > MAX_LANES || total <= 0) fail("launch of %s: bad grid or block", name);
     // what the HIP runtime refuses: more than 65535 workgroups along y or z, 2^32 or more threads along one dimension
@@ -345,6 +378,7 @@ void launch(const char* name, dim3 grid, dim3 block, std::function<void()> body)
             run_workgroup(tl_worker, name, grid, block, bid, body);
         }
     });
+    if (stem[0]) dump_memory(std::string(stem) + ".after");
 }
 
 } // namespace replay
@@ -352,7 +386,7 @@ void launch(const char* name, dim3 grid, dim3 block, std::function<void()> body)
 // ---- runtime API --------------------------------------------------------------------------------------------------
 struct replayStream { bool capturing = false; struct replayGraph* graph = nullptr; };
 struct replayEvent { int dummy; };
-struct LaunchRecord { std::string name; dim3 grid, block; std::function<void()> body; };
+struct LaunchRecord { std::string name; dim3 grid, block; std::function<void()> body; replay::KernelArgs args; };
 struct replayGraph { std::vector<LaunchRecord> nodes; };
 struct replayGraphExec { std::vector<LaunchRecord> nodes; };
 
@@ -362,10 +396,10 @@ replayStream* stream_of(hipStream_t s) { return s ? s : &g_null_stream; }
 } // namespace
 
 namespace replay {
-void enqueue(hipStream_t s, const char* name, dim3 grid, dim3 block, std::function<void()> body) {
+void enqueue(hipStream_t s, const char* name, dim3 grid, dim3 block, std::function<void()> body, KernelArgs args) {
     replayStream* st = stream_of(s);
-    if (st->capturing) { st->graph->nodes.push_back(LaunchRecord{name, grid, block, std::move(body)}); return; }
-    launch(name, grid, block, std::move(body));
+    if (st->capturing) { st->graph->nodes.push_back(LaunchRecord{name, grid, block, std::move(body), std::move(args)}); return; }
+    launch(name, grid, block, std::move(body), args);
 }
 } // namespace replay
 
@@ -401,7 +435,7 @@ hipError_t hipFree(void* p) {
 hipError_t hipMemcpy(void* dst, const void* src, size_t bytes, hipMemcpyKind) { std::memmove(dst, src, bytes); return hipSuccess; }
 hipError_t hipMemcpyAsync(void* dst, const void* src, size_t bytes, hipMemcpyKind, hipStream_t s) {
     replayStream* st = stream_of(s);
-    if (st->capturing) { st->graph->nodes.push_back(LaunchRecord{"memcpy", dim3(0), dim3(0), [=]() { std::memmove(dst, src, bytes); }}); return hipSuccess; }
+    if (st->capturing) { st->graph->nodes.push_back(LaunchRecord{"memcpy", dim3(0), dim3(0), [=]() { std::memmove(dst, src, bytes); }, {}}); return hipSuccess; }
     std::memmove(dst, src, bytes);
     return hipSuccess;
 }
@@ -412,7 +446,7 @@ hipError_t hipMemcpy2DAsync(void* dst, size_t dpitch, const void* src, size_t sp
 hipError_t hipMemset(void* dst, int value, size_t bytes) { std::memset(dst, value, bytes); return hipSuccess; }
 hipError_t hipMemsetAsync(void* dst, int value, size_t bytes, hipStream_t s) {
     replayStream* st = stream_of(s);
-    if (st->capturing) { st->graph->nodes.push_back(LaunchRecord{"memset", dim3(0), dim3(0), [=]() { std::memset(dst, value, bytes); }}); return hipSuccess; }
+    if (st->capturing) { st->graph->nodes.push_back(LaunchRecord{"memset", dim3(0), dim3(0), [=]() { std::memset(dst, value, bytes); }, {}}); return hipSuccess; }
     std::memset(dst, value, bytes);
     return hipSuccess;
 }
@@ -450,7 +484,7 @@ hipError_t hipGraphExecDestroy(hipGraphExec_t e) { delete e; return hipSuccess; 
 hipError_t hipGraphLaunch(hipGraphExec_t e, hipStream_t) {
     for (const LaunchRecord& n : e->nodes) {
         if (n.grid.x == 0) n.body();
-        else replay::launch(n.name.c_str(), n.grid, n.block, n.body);
+        else replay::launch(n.name.c_str(), n.grid, n.block, n.body, n.args);
     }
     return hipSuccess;
 }
