@@ -369,7 +369,7 @@ class Wave:
     def vread(self, o: Operand) -> np.ndarray:
         """32-bit source of a vector instruction as uint32[64]."""
         if o.kind in ("v", "a"):
-            return self.v[self.vindex(o)]
+            return self.v[self.vindex(o)].copy()   # (a copy: the destination may be the same register)
         return np.full(64, self.sread(o) & MASK32, dtype=np.uint32)
 
     def vread64(self, o: Operand, signed_imm=True) -> np.ndarray:
@@ -1530,7 +1530,7 @@ def _ds_read(self, w, i, ndw, offsets):
     active = w.em.copy()
     values = []
     for off in offsets:
-        addr = base + off
+        addr = (base + off) & MASK32   # (32-bit address arithmetic: a negative base with a positive offset is in use)
         _lds_check(w, addr, 4 * ndw, active, "read")
         word = np.where(active, addr // 4, 0)
         for j in range(ndw):
@@ -1585,7 +1585,7 @@ def _ds_write(self, w, i, pieces):
     base = w.vread(i.ops[0]).astype(np.int64)
     active = w.em
     for off, op, ndw in pieces:
-        addr = base + off
+        addr = (base + off) & MASK32
         _lds_check(w, addr, 4 * ndw, active, "write")
         word = (addr // 4)[active]
         vi = w.vindex(op)

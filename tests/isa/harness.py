@@ -149,3 +149,38 @@ def run_launch(d: dict, late=True, program=None, max_steps=50_000_000):
         if len(bad):
             wrong.append((addr, bad))
     return emu, wrong
+
+
+def compile_all(names=None):
+    """Every unit (or the named ones) compiled in parallel; name -> path of its assembly."""
+    from concurrent.futures import ThreadPoolExecutor
+
+    _flags, units = device_units()
+    names = list(names or units)
+    with ThreadPoolExecutor(max_workers=min(len(names), int(os.environ.get("MAX_JOBS", os.cpu_count() or 1)))) as pool:
+        return dict(zip(names, pool.map(compile_unit, names)))
+
+
+def replay_and_emulate(job):
+    """(index, CUs, case of tests/replay/replay_gemm_main.cpp, dump directory) -> (case, [(kernel symbol, instructions, verdict)]):
+    the case runs on the CPU replay, which records its launches, and every launch then runs on the generated code; 'ok' means
+    that every device allocation holds what the replay left there."""
+    import shutil
+
+    index, cus, case, root, exe = job
+    d = os.path.join(root, str(index))
+    shutil.rmtree(d, ignore_errors=True)
+    os.makedirs(d)
+    r = subprocess.run([exe, "early", case], env=dict(os.environ, REPLAY_CUS=str(cus), REPLAY_DUMP_DIR=d), capture_output=True, text=True)
+    if r.returncode != 0:
+        return case, [("-", 0, "the replay failed: " + (r.stdout[-500:] + r.stderr[-500:]))]
+    out = []
+    for launch in launches(d):
+        try:
+            emu, wrong = run_launch(launch)
+            verdict = "ok" if not wrong else "wrong values in " + ", ".join(f"{len(b)} dwords of the buffer at 0x{a:x}" for a, b in wrong)
+            out.append((launch["symbol"], sum(emu.opcode_counts.values()), verdict))
+        except (gfx950.EmulationError, KeyError) as e:
+            out.append((launch["symbol"], 0, "error: " + str(e)[:1500]))
+    shutil.rmtree(d, ignore_errors=True)
+    return case, out

@@ -191,22 +191,15 @@ def device_units():
 
 
 @pytest.fixture(scope="module")
-def device_isa(tmp_path_factory):
-    """name -> gfx950 assembly text of every translation unit (compiled here, in parallel; about a minute)."""
-    from concurrent.futures import ThreadPoolExecutor
+def device_isa():
+    """name -> gfx950 assembly text of every translation unit (compiled in parallel, about a minute; kept under tests/_build/isa and
+    shared with tests/test_isa_emulation.py until a source changes)."""
+    import sys
 
-    flags, units = device_units()
-    out = tmp_path_factory.mktemp("isa")
+    sys.path.insert(0, os.path.join(ROOT, "tests", "isa"))
+    import harness
 
-    def one(unit):
-        name, extra, src = unit
-        path = str(out / (name + ".s"))
-        res = subprocess.run([HIPCC] + flags + extra + ["--cuda-device-only", "-S", os.path.join(CSRC, src), "-o", path], capture_output=True, text=True)
-        assert res.returncode == 0, res.stderr[-3000:]
-        return name, open(path).read()
-
-    with ThreadPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
-        return dict(pool.map(one, units))
+    return {name: open(path).read() for name, path in harness.compile_all().items()}
 
 
 @pytest.mark.skipif(not os.path.exists(HIPCC), reason="no hipcc")

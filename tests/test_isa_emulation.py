@@ -1,0 +1,134 @@
+"""The generated gfx950 code of the kernels, executed on the CPU.
+
+tests/isa/gfx950.py interprets the assembly hipcc emits for the library's translation units; tests/isa/harness.py feeds it the
+launches that the CPU replay records (kernel, grid, argument block, every device allocation before and after).  A case passes
+when the interpreted machine code leaves in memory what the replay of the C++ source left there, with every global and LDS
+access in bounds, results of loads used only after the wait that covers them, and the wait states an asm block owes kept.
+This is the check that sees what the compiler made of the source: the one GPU fault of this code base — a carry parked in SCC
+across an inline-assembly block that overwrote it — is invisible to the source-level replay and is found here (first test).
+No GPU involved.
+"""
+import os
+import shutil
+import subprocess
+import sys
+from concurrent.futures import ProcessPoolExecutor
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+sys.path.insert(0, os.path.join(ROOT, "tests", "replay"))
+sys.path.insert(0, os.path.join(ROOT, "tests", "isa"))
+import build as replay_build  # noqa: E402
+import gfx950  # noqa: E402
+import harness  # noqa: E402
+
+pytestmark = pytest.mark.skipif(not (replay_build.available() and os.path.exists(harness.HIPCC)), reason="needs the host clang++ and hipcc")
+
+
+@pytest.fixture(scope="module")
+def exe():
+    return replay_build.build_gemm_plain()
+
+
+@pytest.fixture(scope="module")
+def isa():
+    return harness.compile_all()
+
+
+def record(exe, case, cus, where):
+    shutil.rmtree(where, ignore_errors=True)
+    os.makedirs(where)
+    res = subprocess.run([exe, "early", case], env=dict(os.environ, REPLAY_CUS=str(cus), REPLAY_DUMP_DIR=str(where)), capture_output=True, text=True)
+    assert res.returncode == 0, res.stdout[-2000:] + res.stderr[-2000:]
+    return harness.launches(str(where))
+
+
+def modified_unit(tmp_path, unit, old, new):
+    """The unit's assembly with one piece of text of gfx950_asm.hpp changed (a copy of the sources; the library's stay as they are)."""
+    src = tmp_path / "csrc"
+    shutil.copytree(harness.CSRC, src)
+    text = (src / "gfx950_asm.hpp").read_text()
+    assert old in text
+    (src / "gfx950_asm.hpp").write_text(text.replace(old, new))
+    return gfx950.parse_program(open(harness.compile_unit(unit, csrc=str(src), out_dir=str(tmp_path / "isa"))).read())
+
+
+def test_the_fault_of_the_masked_load_is_found_without_the_fix_and_gone_with_it(exe, isa, tmp_path):
+    """The short-reduction kernel on a one-step reduction with several tiles per workgroup — the launch that faulted on the GPU.  Built
+    without "scc" in the clobber list of the masked direct load, the interpreted code computes a load address 4 GiB above its operand
+    in the loop over further tiles (s_and_b64 inside the block sets SCC, the s_addc_u32 the compiler scheduled behind the block adds
+    it into the high half); built as the library has it, every access is in bounds and the result is the replay's."""
+    launch = record(exe, "260,132,12,n,t,0,0,0,gemm_smallk=3", 1, tmp_path / "dump")[0]
+    assert "gemm_smallk_kernel" in launch["symbol"]
+    emu, wrong = harness.run_launch(launch)
+    assert not wrong and emu.opcode_counts["global_load_lds_dwordx4"] > 0
+    unfixed = modified_unit(tmp_path, "gemm_smallk", ': "memory", "vcc", "scc");', ': "memory", "vcc");')
+    with pytest.raises(gfx950.EmulationError) as e:
+        harness.run_launch(launch, program=unfixed)
+    assert "direct load to LDS" in str(e.value) and "lies outside every buffer" in str(e.value)
+    operands = [(base, len(data)) for base, data in launch["before"]]
+    address = int(str(e.value).split(" at 0x")[1].split()[0], 16)
+    assert any(base <= address - (1 << 32) < base + size for base, size in operands), "the access is exactly 4 GiB above an operand"
+
+
+def test_wait_states_owed_by_the_asm_blocks_are_checked(exe, isa, tmp_path):
+    """Without the s_nop of the direct-load block, M0 is written in the instruction before the load that reads it: the interpreter
+    counts wait states and says so (the chip needs one; with the vector-written scalar base, five)."""
+    launch = record(exe, "70,130,48,n,n,0,0,0,gemm_tile=2", 2, tmp_path / "dump")[0]
+    bare = modified_unit(tmp_path, "gemm_64x64_0", "s_mov_b32 m0, %0\\n\\ts_nop 3\\n\\tglobal_load_lds_dwordx4", "s_mov_b32 m0, %0\\n\\tglobal_load_lds_dwordx4")
+    with pytest.raises(gfx950.EmulationError, match="wait states after M0 was written"):
+        harness.run_launch(launch, program=bare)
+
+
+def test_a_wait_that_is_too_lenient_gives_wrong_numbers(exe, isa, tmp_path):
+    """Loads return late in the interpreter: with every vmcnt wait of the kernel relaxed to 63 the tiles in LDS are stale and the
+    product is wrong — which is what makes a passing run evidence for the waits the kernels and the compiler placed."""
+    launch = record(exe, "70,130,48,n,n,0,0,0,gemm_tile=2", 2, tmp_path / "dump")[0]
+    program = gfx950.parse_program(open(isa["gemm_64x64_0"]).read())
+    assert not harness.run_launch(launch, program=program)[1]
+    for ins in program[launch["symbol"]].instructions:
+        if ins.op == "s_waitcnt" and ins.mods["vm"] is not None:
+            ins.mods["vm"] = 63
+    assert harness.run_launch(launch, program=program)[1]
+
+
+# (CUs, case): every kernel family of the library, through the entry points, at sizes the interpreter finishes in seconds
+CASES = [
+    # the five tiles of the ordinary kernel: operand layouts (n row-major, t transposed view, g every second element), K tails, batches, accumulate
+    (2, "70,130,40,n,n,0,0,0"), (2, "70,132,40,t,n,0,0,0,gemm_tile=2"), (2, "70,130,40,n,t,0,0,1,gemm_tile=2"), (2, "72,130,40,t,t,0,0,0,gemm_tile=2"),
+    (2, "70,130,40,g,g,0,0,0,gemm_tile=2"), (2, "130,260,48,n,n,0,0,0,gemm_tile=1"), (2, "128,128,40,n,n,0,0,0,gemm_tile=1"), (2, "260,132,36,t,n,0,0,0,gemm_tile=0"),
+    (2, "130,68,36,n,t,2,0,0,gemm_tile=3"), (2, "68,130,36,n,n,3,1,0,gemm_tile=4"), (2, "64,64,8,n,n,0,0,0,gemm_tile=2"),
+    # K slices + their reduction, stream-K + fix-up
+    (2, "70,130,200,n,n,0,0,0,gemm_tile=2,gemm_splitk=3"), (4, "300,260,64,n,n,0,0,0,gemm_tile=1,gemm_streamk=1"),
+    # the persistent kernels: short reduction (several steps, K tails; one step), K-stream (both tiles), resident A (both tiles)
+    (1, "260,132,40,n,t,0,0,0,gemm_smallk=1"), (1, "132,260,20,t,n,2,0,1,gemm_smallk=1"), (2, "132,68,56,t,t,0,0,0,gemm_smallk=1"),
+    (1, "130,260,16,n,t,0,0,0,gemm_smallk=3"), (1, "300,520,8,t,n,2,0,0,gemm_smallk=3"), (1, "132,68,4,t,t,0,0,1,gemm_smallk=3"),
+    (2, "300,260,100,n,n,0,0,0,gemm_panel=1"), (2, "132,260,36,t,n,2,1,1,gemm_panel=1"), (2, "132,260,100,n,t,0,0,0,gemm_panel=3"),
+    (2, "128,2052,32,n,n,0,0,0,gemm_resident=1"), (2, "36,1000,112,t,n,0,0,0,gemm_resident=2"),
+    # Matmul backward: plain, broadcast parents through the batch-reducing launch (vector and element-wise loaders)
+    (2, "bwd:64,48,32,n,n,3,1"), (4, "bwd:70,41,33,n,n,0,5,fold_reduce=1"), (4, "bwd:66,130,20,t,n,3,1,fold_reduce=1"), (4, "bwd:40,36,24,g,g,1,4,fold_reduce=1"),
+    # Linear backward with the bias gradient in the weight-gradient launch: whole K, K slices, stream-K
+    (2, "lin:300,130,70,n,n,0,0,fused=1,gemm_tile=1"), (2, "lin:300,130,70,n,n,0,0,fused=1,gemm_tile=0"),
+    (4, "lin:1000,260,200,n,n,0,0,fused=1,gemm_tile=1,gemm_streamk=1"), (2, "lin:1000,200,260,n,n,0,0,fused=1,gemm_tile=2,gemm_splitk=3"),
+    # matrix-vector, vector-matrix (slices joined in the launch and by a launch of their own), skinny products, dot / column sum / SGD
+    (2, "mv:515,1030,n,0,1,0"), (2, "mv:70,300,t,3,0,1"), (2, "vm:1030,515,n,0,1,0,join=1"), (2, "vm:300,4099,n,3,0,1"), (2, "vm:300,515,n,-3,0,0"),
+    (2, "4,2052,768,n,n,0,0,0"), (2, "3,2051,300,t,n,0,0,1"), (2, "misc:1000"),
+    # the adjacent operators and the MLP step op by op and in three launches
+    (2, "ce:33,1000,0,0"), (2, "ce:5,50257,1,10"), (2, "ce:64,10,0,0"), (2, "conv:2,3,12,11,8,3,3,1,1"), (2, "conv:2,4,15,14,6,3,2,2,1"),
+    (2, "mlp:64,784,128,32,10,0"), (2, "mlp:37,257,77,33,7,3"),
+]
+
+
+def test_every_kernel_family_on_the_generated_code(exe, isa, tmp_path):
+    jobs = [(n, cus, case, str(tmp_path), exe) for n, (cus, case) in enumerate(CASES)]
+    failures, kernels, instructions = [], set(), 0
+    with ProcessPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+        for case, launches in pool.map(harness.replay_and_emulate, jobs):
+            for symbol, count, verdict in launches:
+                kernels.add(symbol)
+                instructions += count
+                if verdict != "ok":
+                    failures.append(f"{case}: {symbol}: {verdict}")
+    assert not failures, "\n".join(failures)
+    assert len(kernels) >= 60 and instructions > 3_000_000, (len(kernels), instructions)
