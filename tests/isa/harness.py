@@ -78,10 +78,10 @@ def symbol_at(path: str, offset: int) -> str:
         loads = subprocess.run(["readelf", "-lW", path], capture_output=True, text=True, check=True).stdout
         first = min(int(m.group(1), 16) for m in re.finditer(r"^\s*LOAD\s+0x[0-9a-f]+\s+0x([0-9a-f]+)", loads, re.M))
         table = {}
-        for line in subprocess.run(["nm", "--defined-only", path], capture_output=True, text=True, check=True).stdout.splitlines():
-            parts = line.split()
-            if len(parts) == 3 and parts[1] in "tTwW":
-                table[int(parts[0], 16) - first] = parts[2]
+        for line in subprocess.run(["readelf", "-sW", path], capture_output=True, text=True, check=True).stdout.splitlines():
+            parts = line.split()   # Num: Value Size Type Bind Vis Ndx Name
+            if len(parts) == 8 and parts[3] == "FUNC" and parts[6] != "UND":
+                table[int(parts[1], 16) - first] = parts[7]
         _symbols[path] = table
     return _symbols[path][offset]
 

@@ -14,6 +14,8 @@
 //   CASE = conv:N,C_in,H_pad,W_pad,C_out,KH,KW,stride,dilation    convolution forward and backward (all three gradients), addresses only
 //   CASE = mlp:batch,d0,d1,d2,d3,fused    two training steps of a 3-layer MLP (tenmo_hip_mlp_step), addresses only
 //   CASE = misc:n      dot, column sum ([n/64+1, 64.. ] shapes derived from n), SGD with and without momentum, addresses only
+//   CASE = vbw:m,k,matrix_batch,vector_batch,generic    matrix . vector and vector . matrix through the view-level entry points, each with its
+//     backward (outer-product and vector gradients), addresses only
 //   CASE = bwd:M,N,K,a_layout,b_layout,a_batch,b_batch[,knob=value...]   tenmo_hip_matmul_backward of A[a_batch, M, K] . B[b_batch, K, N]
 //     (a batch of 0: no batch dimension; 1: one that broadcasts): both gradients against float64, accumulated onto a start value
 //   CASE = lin:M,N,K,a_layout,n,a_batch,0[,fused=0|1][,knob=value...]   tenmo_hip_linear_backward of X[a_batch, M, K] . W[K, N] + b[N]: the three
@@ -334,6 +336,43 @@ static tenmo_view view_of(const float* p, int64_t batch, int64_t rows, int64_t c
     return v;
 }
 
+// mv and vm with their gradients through the view-level entry points, addresses only (the parity tests check the numbers):
+// vbw:m,k,matrix_batch,vector_batch,generic   M[matrix_batch, m, k] (generic: every second element of its storage), v[vector_batch, k]
+// (a batch of 0: no batch dimension); then the same matrix as [k', n] = [m, k] under u[vector_batch, m]
+static int run_vector_backward_case(const std::string& spec) {
+    const std::vector<int64_t> a = numbers_of(spec, 4);
+    if (a.size() < 5) return 2;
+    const int64_t m = a[0], k = a[1], bm = a[2], bv = a[3];
+    const bool generic = a[4] != 0;
+    const int64_t nm = bm > 0 ? bm : 1, nv = bv > 0 ? bv : 1, nb = nm > nv ? nm : nv;
+    float* Mx = exact_block((size_t)(nm * m * k * (generic ? 4 : 1)));
+    float* v = exact_block((size_t)(nv * k)); float* u = exact_block((size_t)(nv * m));
+    float* out_mv = exact_block((size_t)(nb * m), false); float* out_vm = exact_block((size_t)(nb * k), false);
+    float* dy_mv = exact_block((size_t)(nb * m)); float* dy_vm = exact_block((size_t)(nb * k));
+    float* gM = exact_block((size_t)(nm * m * k)); float* gv = exact_block((size_t)(nv * k)); float* gu = exact_block((size_t)(nv * m));
+    tenmo_view vM = view_of(Mx, bm, m, k, false, generic);
+    tenmo_view vv, vu;
+    memset(&vv, 0, sizeof(vv));
+    vv.data = v;
+    int r = 0;
+    if (bv > 0) { vv.shape[r] = bv; vv.strides[r] = k; ++r; }
+    vv.shape[r] = k; vv.strides[r] = 1; ++r;
+    vv.rank = r;
+    vu = vv;
+    vu.data = u;
+    vu.shape[r - 1] = m;
+    if (bv > 0) vu.strides[0] = m;
+    int rc = tenmo_hip_matrix_vector_nd(&vM, &vv, out_mv, 1);
+    if (rc == 0) rc = tenmo_hip_mv_backward(&vM, &vv, dy_mv, gM, gv, 1);
+    if (rc == 0) rc = tenmo_hip_vector_matmul_nd(&vu, &vM, out_vm, 1);
+    if (rc == 0) rc = tenmo_hip_vm_backward(&vu, &vM, dy_vm, gu, gM, 1);
+    if (rc != 0) fprintf(stderr, "%s: error %d: %s\n", spec.c_str(), rc, tenmo_hip_last_error());
+    printf("%s: rc %d, relative error n/a\n", spec.c_str(), rc);
+    fflush(stdout);
+    drop_block(Mx); drop_block(v); drop_block(u); drop_block(out_mv); drop_block(out_vm); drop_block(dy_mv); drop_block(dy_vm); drop_block(gM); drop_block(gv); drop_block(gu);
+    return rc != 0;
+}
+
 static int run_backward_case(const std::string& spec) {
     const bool linear = spec.compare(0, 4, "lin:") == 0;
     int want_fused = -1;
@@ -440,6 +479,7 @@ int main(int argc, char** argv) {
         if (strncmp(argv[i], "bwd:", 4) == 0 || strncmp(argv[i], "lin:", 4) == 0) bad |= run_backward_case(argv[i]);
         else if (strncmp(argv[i], "ce:", 3) == 0 || strncmp(argv[i], "conv:", 5) == 0 || strncmp(argv[i], "misc:", 5) == 0 || strncmp(argv[i], "mlp:", 4) == 0)
             bad |= run_address_only_case(argv[i]);
+        else if (strncmp(argv[i], "vbw:", 4) == 0) bad |= run_vector_backward_case(argv[i]);
         else if (strncmp(argv[i], "mv:", 3) == 0) bad |= run_vector_case(argv[i], true);
         else if (strncmp(argv[i], "vm:", 3) == 0) bad |= run_vector_case(argv[i], false);
         else bad |= run_case(argv[i]);
