@@ -273,18 +273,20 @@ SCALAR_WRITERS_BY_VALU = ("v_readfirstlane_b32", "v_readlane_b32")
 class Wave:
     def __init__(self, emu, kernel: Kernel, wg, wave_index: int, lanes_alive: int):
         self.emu, self.k, self.wg, self.index = emu, kernel, wg, wave_index
-        self.s = [0] * 128
-        self.v = np.zeros((512, 64), dtype=np.uint32)
-        self.vcc = 0
+        # nothing is zero that the hardware does not promise to be: registers, LDS and scratch start with a pattern that is a NaN as a
+        # float and far outside every buffer as an address, so that a value used before it is written cannot pass for a right one
+        self.s = [0xDEADBEEF] * 128
+        self.v = np.full((512, 64), 0xFFFFDEAD, dtype=np.uint32)
+        self.vcc = 0xAAAAAAAAAAAAAAAA
         self.exec = (1 << lanes_alive) - 1 if lanes_alive < 64 else MASK64
         self.em = self._mask_array(self.exec)
-        self.m0 = 0
-        self.scc = 0
+        self.m0 = 0xDEADBEEF
+        self.scc = 1
         self.pc = 0
         self.done = False
         self.vm_queue = []      # vector memory operations in flight: callables that complete them (None: nothing to do)
         self.lgkm_queue = []    # (is_scalar_load, completion)
-        self.scratch = np.zeros((64, max(4, kernel.desc.get("private_segment_fixed_size", 0) + 64)), dtype=np.uint8)
+        self.scratch = np.full((64, max(4, kernel.desc.get("private_segment_fixed_size", 0) + 64)), 0xFF, dtype=np.uint8)
         self.steps = 0
         self.clock = 0                       # issue slots, counting the wait states of s_nop
         self.sgpr_written_by_valu = {}       # sgpr index -> clock of the vector instruction that wrote it
@@ -455,7 +457,7 @@ class Wave:
 class Workgroup:
     def __init__(self, bid, lds_bytes):
         self.bid = bid
-        self.lds = np.zeros(max(lds_bytes, 4), dtype=np.uint8)
+        self.lds = np.full(max(lds_bytes, 4), 0xFF, dtype=np.uint8)   # (LDS is not cleared between workgroups on the chip)
         self.lds32 = self.lds.view(np.uint32)
         self.lds_bytes = lds_bytes
 
@@ -477,8 +479,10 @@ def _sext_imm(o: Operand, bits: int) -> int:
 
 
 class Emulator:
-    def __init__(self, program: dict, memory: Memory, late=True, check_hazards=True):
-        self.program, self.mem, self.late, self.check_hazards = program, memory, late, check_hazards
+    def __init__(self, program: dict, memory: Memory, late=True, check_hazards=True, reverse=False):
+        """reverse: workgroups of the grid and the wavefronts of a workgroup take their turns in descending instead of ascending order
+        (a result must not depend on either: what one wavefront hands to another goes through a barrier)."""
+        self.program, self.mem, self.late, self.check_hazards, self.reverse = program, memory, late, check_hazards, reverse
         self.kernarg_base = 0x7F00_0000_0000
         self.instruction_count = 0
         self.opcode_counts = {}
@@ -516,10 +520,9 @@ class Emulator:
         self.mem.map(self.kernarg_base, kbuf)
         try:
             threads = block[0] * block[1] * block[2]
-            for bz in range(grid[2]):
-                for by in range(grid[1]):
-                    for bx in range(grid[0]):
-                        self.run_workgroup(k, (bx, by, bz), block, threads, max_steps)
+            ids = [(bx, by, bz) for bz in range(grid[2]) for by in range(grid[1]) for bx in range(grid[0])]
+            for bid in (reversed(ids) if self.reverse else ids):
+                self.run_workgroup(k, bid, block, threads, max_steps)
         finally:
             self.mem.bases.pop()
             self.mem.buffers.pop()
@@ -563,7 +566,7 @@ class Emulator:
             running = [w for w in waves if not w.done]
             if not running:
                 break
-            for w in running:
+            for w in (reversed(running) if self.reverse else running):
                 self.run_until_barrier(w, max_steps)
             # (a wave that ended no longer takes part)
 

@@ -133,7 +133,7 @@ def differences(got: np.ndarray, want: np.ndarray, rtol=2e-6):
     return bad[~close]
 
 
-def run_launch(d: dict, late=True, program=None, max_steps=50_000_000):
+def run_launch(d: dict, late=True, program=None, max_steps=50_000_000, reverse=False):
     """Executes the recorded launch on the generated code; returns (emulator, list of (address, differing dword indices))."""
     prog = program or program_of(unit_of_symbol(d["symbol"]))
     if d["symbol"] not in prog:
@@ -141,7 +141,7 @@ def run_launch(d: dict, late=True, program=None, max_steps=50_000_000):
     mem = gfx950.Memory()
     for addr, data in d["before"]:
         mem.map(addr, data.copy())
-    emu = gfx950.Emulator(prog, mem, late=late)
+    emu = gfx950.Emulator(prog, mem, late=late, reverse=reverse)
     emu.launch(d["symbol"], d["grid"], d["block"], d["args"], max_steps=max_steps)
     wrong = []
     for (addr, want), got in zip(d["after"], mem.buffers):
@@ -167,7 +167,8 @@ def replay_and_emulate(job):
     that every device allocation holds what the replay left there."""
     import shutil
 
-    index, cus, case, root, exe = job
+    index, cus, case, root, exe = job[:5]
+    reverse = bool(job[5]) if len(job) > 5 else False
     d = os.path.join(root, str(index))
     shutil.rmtree(d, ignore_errors=True)
     os.makedirs(d)
@@ -177,7 +178,7 @@ def replay_and_emulate(job):
     out = []
     for launch in launches(d):
         try:
-            emu, wrong = run_launch(launch)
+            emu, wrong = run_launch(launch, reverse=reverse)
             verdict = "ok" if not wrong else "wrong values in " + ", ".join(f"{len(b)} dwords of the buffer at 0x{a:x}" for a, b in wrong)
             out.append((launch["symbol"], sum(emu.opcode_counts.values()), verdict))
         except (gfx950.EmulationError, KeyError) as e:

@@ -46,6 +46,7 @@ def record(exe, case, cus, where):
 
 def modified_unit(tmp_path, unit, old, new):
     """The unit's assembly with one piece of text of gfx950_asm.hpp changed (a copy of the sources; the library's stay as they are)."""
+    os.makedirs(tmp_path, exist_ok=True)
     src = tmp_path / "csrc"
     shutil.copytree(harness.CSRC, src)
     text = (src / "gfx950_asm.hpp").read_text()
@@ -73,12 +74,18 @@ def test_the_fault_of_the_masked_load_is_found_without_the_fix_and_gone_with_it(
 
 
 def test_wait_states_owed_by_the_asm_blocks_are_checked(exe, isa, tmp_path):
-    """Without the s_nop of the direct-load block, M0 is written in the instruction before the load that reads it: the interpreter
-    counts wait states and says so (the chip needs one; with the vector-written scalar base, five)."""
+    """The interpreter counts wait states.  Without the s_nop of the direct-load block, M0 is written in the instruction before the
+    load that reads it (the chip needs one wait state); with `s_nop 0` in its place that is satisfied, but the load's scalar base,
+    which the compiler takes out of a v_readfirstlane right before the block, is then read 3 wait states after a vector instruction
+    wrote it where the chip needs 5 — the hazard the block's `s_nop 3` is there for."""
     launch = record(exe, "70,130,48,n,n,0,0,0,gemm_tile=2", 2, tmp_path / "dump")[0]
-    bare = modified_unit(tmp_path, "gemm_64x64_0", "s_mov_b32 m0, %0\\n\\ts_nop 3\\n\\tglobal_load_lds_dwordx4", "s_mov_b32 m0, %0\\n\\tglobal_load_lds_dwordx4")
+    block = "s_mov_b32 m0, %0\\n\\ts_nop 3\\n\\tglobal_load_lds_dwordx4"
+    bare = modified_unit(tmp_path / "bare", "gemm_64x64_0", block, block.replace("\\ts_nop 3\\n", ""))
     with pytest.raises(gfx950.EmulationError, match="wait states after M0 was written"):
         harness.run_launch(launch, program=bare)
+    short = modified_unit(tmp_path / "short", "gemm_64x64_0", block, block.replace("s_nop 3", "s_nop 0"))
+    with pytest.raises(gfx950.EmulationError, match="3 wait states after a vector instruction wrote it"):
+        harness.run_launch(launch, program=short)
 
 
 def test_a_wait_that_is_too_lenient_gives_wrong_numbers(exe, isa, tmp_path):
@@ -122,8 +129,11 @@ CASES = [
 ]
 
 
-def test_every_kernel_family_on_the_generated_code(exe, isa, tmp_path):
-    jobs = [(n, cus, case, str(tmp_path), exe) for n, (cus, case) in enumerate(CASES)]
+@pytest.mark.parametrize("reverse", [False, True], ids=["ascending", "descending"])
+def test_every_kernel_family_on_the_generated_code(exe, isa, tmp_path, reverse):
+    """Registers, LDS and scratch start as garbage (NaN as floats, far out of bounds as addresses); the workgroups of a grid and the
+    wavefronts of a workgroup take their turns in ascending order and, second run, in descending order — the results are the same."""
+    jobs = [(n, cus, case, str(tmp_path), exe, reverse) for n, (cus, case) in enumerate(CASES)]
     failures, kernels, instructions = [], set(), 0
     with ProcessPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
         for case, launches in pool.map(harness.replay_and_emulate, jobs):
