@@ -17,7 +17,8 @@
 //   CASE = vbw:m,k,matrix_batch,vector_batch,generic    matrix . vector and vector . matrix through the view-level entry points, each with its
 //     backward (outer-product and vector gradients), addresses only
 //   CASE = bwd:M,N,K,a_layout,b_layout,a_batch,b_batch[,knob=value...]   tenmo_hip_matmul_backward of A[a_batch, M, K] . B[b_batch, K, N]
-//     (a batch of 0: no batch dimension; 1: one that broadcasts): both gradients against float64, accumulated onto a start value
+//     (a batch of 0: no batch dimension; 1: one that broadcasts; skip=1: A's matrices lie two matrices apart): both gradients against float64,
+//     accumulated onto a start value
 //   CASE = lin:M,N,K,a_layout,n,a_batch,0[,fused=0|1][,knob=value...]   tenmo_hip_linear_backward of X[a_batch, M, K] . W[K, N] + b[N]: the three
 //     gradients against float64; fused=1: the call must take as many kernel launches with the bias gradient as without it (the sums
 //     come out of the weight-gradient launch), fused=0: more
@@ -376,6 +377,7 @@ static int run_vector_backward_case(const std::string& spec) {
 static int run_backward_case(const std::string& spec) {
     const bool linear = spec.compare(0, 4, "lin:") == 0;
     int want_fused = -1;
+    int64_t a_skip = 1; // skip=1: A's matrices are every second one of its storage (their rows do not stack into one taller matrix)
     std::vector<std::string> f;
     size_t pos = 4;
     while (pos <= spec.size()) {
@@ -393,11 +395,12 @@ static int run_backward_case(const std::string& spec) {
         const size_t eq = f[i].find('=');
         if (eq == std::string::npos) continue;
         if (f[i].substr(0, eq) == "fused") want_fused = atoi(f[i].c_str() + eq + 1);
+        else if (f[i].substr(0, eq) == "skip") a_skip = atoi(f[i].c_str() + eq + 1) > 0 ? 2 : 1;
         else knobs.push_back({f[i].substr(0, eq), atoi(f[i].c_str() + eq + 1)});
     }
     const int64_t na = ba > 0 ? ba : 1, nb = bb > 0 ? bb : 1, nc = na > nb ? na : nb;
     const size_t a_n = (size_t)(na * M * K), b_n = (size_t)(nb * K * N), c_n = (size_t)(nc * M * N); // elements of the views = of the gradients
-    const int64_t a_mat = M * K * (ga ? 2 : 1), b_mat = K * N * (gb ? 2 : 1);                          // storage per matrix
+    const int64_t a_mat = M * K * (ga ? 2 : 1) * a_skip, b_mat = K * N * (gb ? 2 : 1);                 // storage per matrix (of A: distance between matrices)
     const size_t a_store = (size_t)(na * a_mat), b_store = (size_t)(nb * b_mat);
     float* A = (float*)malloc(a_store * 4); float* B = (float*)malloc(b_store * 4); float* dC = (float*)malloc(c_n * 4);
     float* gA = (float*)malloc(a_n * 4); float* gB = (float*)malloc(b_n * 4);
@@ -435,6 +438,7 @@ static int run_backward_case(const std::string& spec) {
     replay_register(gbias, (size_t)N * 4);
     replay_register(A, a_store * 4); replay_register(B, b_store * 4); replay_register(dC, c_n * 4); replay_register(gA, a_n * 4); replay_register(gB, b_n * 4);
     tenmo_view va = view_of(A, ba, M, K, ta, ga), vb = view_of(B, bb, K, N, tb, gb);
+    if (ba > 0) va.strides[0] = a_mat;
     for (auto& kv : knobs) tenmo_hip_set_tuning(kv.first.c_str(), kv.second);
     int bad = 0;
     long without_bias = 0;

@@ -9,6 +9,7 @@ across an inline-assembly block that overwrote it — is invisible to the source
 No GPU involved.
 """
 import os
+import re
 import shutil
 import subprocess
 import sys
@@ -129,11 +130,57 @@ CASES = [
 ]
 
 
+def sweep_of_instantiations():
+    """One case for every instantiation of the matrix-product kernels: the compiler allocates registers and schedules each of them
+    on its own (the masked-load fault lived in some instantiations of one kernel and not in others), so each one is run."""
+    a_layout = {0: "n", 1: "t", 2: "g"}   # operand mode of A (K-major rows, MN-major = transposed view, element-wise) -> layout of the case
+    b_layout = {0: "t", 1: "n", 2: "g"}
+    cases = []
+    dims = {0: (260, 132, 40), 1: (132, 132, 40), 2: (68, 132, 24), 3: (132, 68, 24), 4: (68, 132, 24)}
+    for tile in range(5):                 # the ordinary kernel: every tile x every pair of operand modes
+        for am in range(3):
+            for bm in range(3):
+                M, N, K = dims[tile]
+                cases.append((2, f"{M},{N},{K},{a_layout[am]},{b_layout[bm]},0,0,{(am + bm) % 2},gemm_tile={tile}"))
+    for tile in range(4):                 # stream-K with a fix-up: every tile x the vector modes
+        for am in range(2):
+            for bm in range(2):
+                M, N = {0: (700, 128), 1: (380, 128), 2: (190, 64), 3: (380, 64)}[tile]
+                cases.append((2, f"{M},{N},80,{a_layout[am]},{b_layout[bm]},0,0,0,gemm_tile={tile},gemm_streamk=1"))
+    for am in range(2):                   # short reduction: modes x K steps (1 .. 4, each with a K tail) x accumulate
+        for bm in range(2):
+            for steps, K in ((1, 12), (2, 20), (3, 48), (4, 56)):
+                for acc in (0, 1):
+                    cases.append((1, f"132,196,{K},{a_layout[am]},{b_layout[bm]},0,0,{acc},gemm_smallk={3 if steps == 1 else 1}"))
+    for am in range(2):                   # K-stream: modes x tile x accumulate
+        for bm in range(2):
+            for knob in (1, 3):
+                for acc in (0, 1):
+                    cases.append((2, f"132,260,36,{a_layout[am]},{b_layout[bm]},0,0,{acc},gemm_panel={knob}"))
+    for am in range(2):                   # resident A: mode of A x tile height x K range
+        for knob in (1, 2):
+            for K in (36, 132):
+                cases.append((16, f"128,1028,{K},{a_layout[am]},n,0,0,0,gemm_resident={knob},ran=gemm_resident_kernel"))
+    for la in "ntg":                      # the batch-reducing launch: layouts x which parent is shared x tile
+        for lb in "ntg":
+            cases.append((4, f"bwd:40,36,24,{la},{lb},1,4,fold_reduce=1"))
+            cases.append((4, f"bwd:40,36,24,{la},{lb},4,1,fold_reduce=1,skip=1"))
+    for la in "nt":
+        for lb in "nt":
+            cases.append((1, f"bwd:132,132,24,{la},{lb},1,3,fold_reduce=1"))
+            cases.append((1, f"bwd:132,132,24,{la},{lb},3,1,fold_reduce=1,skip=1"))
+    for tile in range(5):                 # the bias gradient in the weight-gradient launch: every tile
+        cases.append((2, f"lin:300,132,68,n,n,0,0,fused=1,gemm_tile={tile}"))
+    return cases
+
+
 @pytest.mark.parametrize("reverse", [False, True], ids=["ascending", "descending"])
 def test_every_kernel_family_on_the_generated_code(exe, isa, tmp_path, reverse):
     """Registers, LDS and scratch start as garbage (NaN as floats, far out of bounds as addresses); the workgroups of a grid and the
-    wavefronts of a workgroup take their turns in ascending order and, second run, in descending order — the results are the same."""
-    jobs = [(n, cus, case, str(tmp_path), exe, reverse) for n, (cus, case) in enumerate(CASES)]
+    wavefronts of a workgroup take their turns in ascending order and, second run, in descending order — the results are the same.
+    The ascending run adds the sweep over every instantiation of the matrix-product kernels."""
+    cases = CASES + ([] if reverse else sweep_of_instantiations())
+    jobs = [(n, cus, case, str(tmp_path), exe, reverse) for n, (cus, case) in enumerate(cases)]
     failures, kernels, instructions = [], set(), 0
     with ProcessPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
         for case, launches in pool.map(harness.replay_and_emulate, jobs):
@@ -144,3 +191,13 @@ def test_every_kernel_family_on_the_generated_code(exe, isa, tmp_path, reverse):
                     failures.append(f"{case}: {symbol}: {verdict}")
     assert not failures, "\n".join(failures)
     assert len(kernels) >= 70 and instructions > 5_000_000, (len(kernels), instructions)
+    if not reverse:   # every instantiation of the matrix-product units has run (the rest live in tenmo_hip.hip: no assembly blocks there)
+        units = harness.device_units()[1]
+        not_run = [name for unit in units if unit != "tenmo_hip" for name in harness.program_of(unit) if name not in kernels]
+        # (instantiated but out of reach of Matmul backward: the left operand of a folded dA and the right one of a folded dB are the dense
+        # upstream gradient, so the batch-reducing launch never sees an MN-major or element-wise left operand beside a K-major or
+        # element-wise right one)
+        unreachable = re.compile(r"gemm_reduce_kernelILi\d+ELi\d+ELi[12]ELi[02]E")
+        assert not [name for name in not_run if not unreachable.search(name)], not_run
+        assert len(not_run) <= 5
+        assert len(kernels) >= 170
