@@ -90,11 +90,16 @@ def read_memory(path: str):
     out = []
     data = open(path, "rb").read()
     at = 0
-    while at < len(data):
-        addr, size = np.frombuffer(data[at:at + 16], dtype=np.uint64)
-        at += 16
-        out.append((int(addr), np.frombuffer(data[at:at + int(size)], dtype=np.uint8).copy()))
-        at += int(size)
+    while at < len(data):   # per allocation: address, size, number of pages that are not all zeros; then (offset, page) each
+        addr, size, pages = (int(x) for x in np.frombuffer(data[at:at + 24], dtype=np.uint64))
+        at += 24
+        buf = np.zeros(size, dtype=np.uint8)
+        for _ in range(pages):
+            off = int(np.frombuffer(data[at:at + 8], dtype=np.uint64)[0])
+            n = min(4096, size - off)
+            buf[off:off + n] = np.frombuffer(data[at + 8:at + 8 + n], dtype=np.uint8)
+            at += 8 + n
+        out.append((addr, buf))
     return out
 
 

@@ -10,6 +10,7 @@
 #include <cstdarg>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <map>
 #include <mutex>
 #include <string>
@@ -331,16 +332,32 @@ std::string g_last_kernel; // (launches are serialized)
 // REPLAY_DUMP_DIR: every launch leaves what is needed to run the same launch elsewhere (the emulator of the generated GPU code,
 // tests/isa/): the kernel function (its offset in the file it lives in, for the symbol table), grid and block, the argument block, and
 // every device allocation before and after the launch.
-void dump_memory(const std::string& path) {
+// (pages of zeros are left out: the library's workspace is tens of megabytes of which a launch touches little; and the whole
+// process writes at most REPLAY_DUMP_LIMIT_MB, 4096 by default, after which it records no further launch)
+std::atomic<uint64_t> g_dumped{0};
+bool dump_memory(const std::string& path) {
+    static const uint64_t limit = (uint64_t)(getenv("REPLAY_DUMP_LIMIT_MB") ? atoll(getenv("REPLAY_DUMP_LIMIT_MB")) : 4096) << 20;
+    if (g_dumped.load() > limit) return false;
     FILE* f = fopen(path.c_str(), "wb");
-    if (!f) return;
+    if (!f) return false;
+    constexpr size_t PAGE = 4096;
+    static const unsigned char zeros[PAGE] = {0};
     std::lock_guard<std::mutex> lock(g_mem_mutex);
     for (const auto& a : g_allocs) {
-        const uint64_t head[2] = {(uint64_t)a.first, (uint64_t)a.second};
+        const unsigned char* base = (const unsigned char*)a.first;
+        std::vector<uint64_t> pages;
+        for (size_t off = 0; off < a.second; off += PAGE)
+            if (std::memcmp(base + off, zeros, std::min(PAGE, a.second - off)) != 0) pages.push_back(off);
+        const uint64_t head[3] = {(uint64_t)a.first, (uint64_t)a.second, (uint64_t)pages.size()};
         fwrite(head, sizeof(head), 1, f);
-        fwrite((const void*)a.first, 1, a.second, f);
+        for (uint64_t off : pages) {
+            fwrite(&off, sizeof(off), 1, f);
+            fwrite(base + off, 1, std::min(PAGE, a.second - (size_t)off), f);
+        }
+        g_dumped += sizeof(head) + pages.size() * (PAGE + 8);
     }
     fclose(f);
+    return true;
 }
 
 void launch(const char* name, dim3 grid, dim3 block, std::function<void()> body, const KernelArgs& args) {
@@ -361,7 +378,7 @@ void launch(const char* name, dim3 grid, dim3 block, std::function<void()> body,
             fprintf(f, "\n");
             fclose(f);
         }
-        dump_memory(std::string(stem) + ".before");
+        if (!dump_memory(std::string(stem) + ".before")) { remove((std::string(stem) + ".txt").c_str()); stem[0] = 0; }
     }
     const int64_t total = (int64_t)grid.x * grid.y * grid.z;
     if ((int64_t)block.x * block.y * block.z > MAX_LANES || total <= 0) fail("launch of %s: bad grid or block", name);
