@@ -122,10 +122,12 @@ CASES = [
     # matrix-vector, vector-matrix (slices joined in the launch and by a launch of their own), skinny products, dot / column sum / SGD
     (2, "mv:515,1030,n,0,1,0"), (2, "mv:70,300,t,3,0,1"), (2, "vm:1030,515,n,0,1,0,join=1"), (2, "vm:300,4099,n,3,0,1"), (2, "vm:300,515,n,-3,0,0"),
     (2, "4,2052,768,n,n,0,0,0"), (2, "3,2051,300,t,n,0,0,1"), (2, "misc:1000"), (2, "misc:4096"),
+    (2, "2,2052,300,n,n,0,0,0"), (2, "2,2052,300,n,n,0,0,0,cols_join=1"), (2, "2,2051,300,n,n,0,0,0"), (2, "3,2052,300,n,n,0,0,0,cols_join=1"),
+    (2, "5,2052,300,n,n,0,0,0"), (2, "5,2052,300,n,n,0,0,0,cols_join=1"), (2, "5,2051,300,n,n,0,0,0"), (2, "mv:3,5000,n,0,0,0"),
     # mv / vm through the view-level entries with their gradients: stacked, shared and element-wise (every second element) matrices
     (2, "vbw:70,33,3,0,0"), (2, "vbw:40,36,0,4,1"), (2, "vbw:64,128,2,2,0"),
     # the adjacent operators and the MLP step op by op and in three launches
-    (2, "ce:33,1000,0,0"), (2, "ce:5,50257,1,10"), (2, "ce:64,10,0,0"), (2, "ce:37,9001,0,5"), (2, "conv:2,3,12,11,8,3,3,1,1"), (2, "conv:2,4,15,14,6,3,2,2,1"),
+    (2, "ce:33,1000,0,0"), (2, "ce:5,50257,1,10"), (2, "ce:64,10,0,0"), (2, "ce:37,9001,0,5"), (2, "ce:9,64,1,10"), (2, "ce:9,2048,0,0"), (2, "ce:9,4096,1,10"), (2, "ce:3,16384,0,0"), (2, "conv:2,3,12,11,8,3,3,1,1"), (2, "conv:2,4,15,14,6,3,2,2,1"),
     (2, "mlp:64,784,128,32,10,0"), (2, "mlp:37,257,77,33,7,3"),
 ]
 
