@@ -139,11 +139,13 @@ def sweep_of_instantiations():
     b_layout = {0: "t", 1: "n", 2: "g"}
     cases = []
     dims = {0: (260, 132, 40), 1: (132, 132, 40), 2: (68, 132, 24), 3: (132, 68, 24), 4: (68, 132, 24)}
+    whole = {0: (512, 128), 1: (256, 128), 2: (128, 64), 3: (256, 64), 4: (128, 128)}
     for tile in range(5):                 # the ordinary kernel: every tile x every pair of operand modes
         for am in range(3):
             for bm in range(3):
                 M, N, K = dims[tile]
                 cases.append((2, f"{M},{N},{K},{a_layout[am]},{b_layout[bm]},0,0,{(am + bm) % 2},gemm_tile={tile}"))
+                cases.append((2, f"{whole[tile][0]},{whole[tile][1]},32,{a_layout[am]},{b_layout[bm]},0,0,0,gemm_tile={tile}"))   # whole tiles, whole K steps
     for tile in range(4):                 # stream-K with a fix-up: every tile x the vector modes
         for am in range(2):
             for bm in range(2):
@@ -154,11 +156,13 @@ def sweep_of_instantiations():
             for steps, K in ((1, 12), (2, 20), (3, 48), (4, 56)):
                 for acc in (0, 1):
                     cases.append((1, f"132,196,{K},{a_layout[am]},{b_layout[bm]},0,0,{acc},gemm_smallk={3 if steps == 1 else 1}"))
+                    cases.append((1, f"128,192,{16 * steps},{a_layout[am]},{b_layout[bm]},0,0,{acc},gemm_smallk={3 if steps == 1 else 1}"))
     for am in range(2):                   # K-stream: modes x tile x accumulate
         for bm in range(2):
             for knob in (1, 3):
                 for acc in (0, 1):
                     cases.append((2, f"132,260,36,{a_layout[am]},{b_layout[bm]},0,0,{acc},gemm_panel={knob}"))
+                    cases.append((2, f"256,256,48,{a_layout[am]},{b_layout[bm]},0,0,{acc},gemm_panel={knob}"))
     for am in range(2):                   # resident A: mode of A x tile height x K range
         for knob in (1, 2):
             for K in (36, 132):
