@@ -138,16 +138,35 @@ def differences(got: np.ndarray, want: np.ndarray, rtol=2e-6):
     return bad[~close]
 
 
-def run_launch(d: dict, late=True, program=None, max_steps=50_000_000, reverse=False):
-    """Executes the recorded launch on the generated code; returns (emulator, list of (address, differing dword indices))."""
+def across_4gib(buffers, args: bytes):
+    """New addresses for the buffers, each placed so that a multiple of 4 GiB falls into its middle (keeping its alignment within a page),
+    and the argument block with every pointer into a buffer moved along.  Host allocations never lie like that; device allocations can,
+    and then every 64-bit address computation of the kernel has to carry."""
+    placed, moved = [], bytearray(args)
+    for n, (addr, data) in enumerate(buffers):
+        half = (len(data) // 2) // 4096 * 4096
+        placed.append(((n + 2) << 34) + (1 << 32) - half - (4096 if len(data) > 4096 and half == 0 else 0) + addr % 4096)
+    for off in range(0, len(args) - 7, 8):
+        value = int.from_bytes(args[off:off + 8], "little")
+        for (addr, data), new in zip(buffers, placed):
+            if addr <= value <= addr + len(data) and value > 0xFFFF:
+                moved[off:off + 8] = (value - addr + new).to_bytes(8, "little")
+                break
+    return placed, bytes(moved)
+
+
+def run_launch(d: dict, late=True, program=None, max_steps=50_000_000, reverse=False, relocate=False):
+    """Executes the recorded launch on the generated code; returns (emulator, list of (address, differing dword indices)).
+    relocate: with the buffers moved across 4 GiB boundaries (see across_4gib)."""
     prog = program or program_of(unit_of_symbol(d["symbol"]))
     if d["symbol"] not in prog:
         raise KeyError(f"{d['symbol']} is not in the unit {unit_of_symbol(d['symbol'])}")
     mem = gfx950.Memory()
-    for addr, data in d["before"]:
-        mem.map(addr, data.copy())
+    bases, args = ([addr for addr, _ in d["before"]], d["args"]) if not relocate else across_4gib(d["before"], d["args"])
+    for base, (_addr, data) in zip(bases, d["before"]):
+        mem.map(base, data.copy())
     emu = gfx950.Emulator(prog, mem, late=late, reverse=reverse)
-    emu.launch(d["symbol"], d["grid"], d["block"], d["args"], max_steps=max_steps)
+    emu.launch(d["symbol"], d["grid"], d["block"], args, max_steps=max_steps)
     wrong = []
     for (addr, want), got in zip(d["after"], mem.buffers):
         bad = differences(got, want)
@@ -174,6 +193,7 @@ def replay_and_emulate(job):
 
     index, cus, case, root, exe = job[:5]
     reverse = bool(job[5]) if len(job) > 5 else False
+    relocate = bool(job[6]) if len(job) > 6 else False
     d = os.path.join(root, str(index))
     shutil.rmtree(d, ignore_errors=True)
     os.makedirs(d)
@@ -183,7 +203,7 @@ def replay_and_emulate(job):
     out = []
     for launch in launches(d):
         try:
-            emu, wrong = run_launch(launch, reverse=reverse)
+            emu, wrong = run_launch(launch, reverse=reverse, relocate=relocate)
             verdict = "ok" if not wrong else "wrong values in " + ", ".join(f"{len(b)} dwords of the buffer at 0x{a:x}" for a, b in wrong)
             out.append((launch["symbol"], sum(emu.opcode_counts.values()), verdict))
         except (gfx950.EmulationError, KeyError) as e:
