@@ -374,7 +374,7 @@ class Wave:
             return self.v[self.vindex(o)].copy()   # (a copy: the destination may be the same register)
         return np.full(64, self.sread(o) & MASK32, dtype=np.uint32)
 
-    def vread64(self, o: Operand, signed_imm=True) -> np.ndarray:
+    def vread64(self, o: Operand) -> np.ndarray:
         if o.kind in ("v", "a"):
             i = self.vindex(o)
             return self.v[i].astype(np.uint64) | (self.v[i + 1].astype(np.uint64) << np.uint64(32))
@@ -472,10 +472,6 @@ def _s32(x: int) -> int:
 def _s64(x: int) -> int:
     x &= MASK64
     return x - (1 << 64) if x & (1 << 63) else x
-
-
-def _sext_imm(o: Operand, bits: int) -> int:
-    return o.value
 
 
 class Emulator:
@@ -1052,13 +1048,7 @@ class Emulator:
         w.vwrite(i.ops[0], w.vread(i.ops[1]))
 
     def op_v_mov_b64(self, w, i):
-        src = i.ops[1]
-        if src.kind == "imm":
-            v = src.value
-            value = np.full(64, (v if v <= 64 or v > MASK32 else v) & MASK64, dtype=np.uint64)
-        else:
-            value = w.vread64(src)
-        w.vwrite64(i.ops[0], value)
+        w.vwrite64(i.ops[0], w.vread64(i.ops[1]))
 
     def op_v_accvgpr_read_b32(self, w, i):
         w.vwrite(i.ops[0], w.vread(i.ops[1]))
@@ -1251,10 +1241,7 @@ class Emulator:
             a, b = w.fread(i.ops[1]).view(np.uint32), w.fread(i.ops[2]).view(np.uint32)
         w.vwrite(i.ops[0], np.where(sel, b, a))
 
-    # carries
-    def _carry_out(self, i):
-        return i.ops[1]
-
+    # carries (vdst, carry-out, a, b[, carry-in])
     def op_v_add_co_u32(self, w, i):
         a, b = w.vread(i.ops[2]).astype(np.uint64), w.vread(i.ops[3]).astype(np.uint64)
         r = a + b
@@ -1726,10 +1713,10 @@ def _global_atomic(self, w, i, f):
     addr = _global_address(w, ops[0], ops[2], i)
     data = w.vread(ops[1])
     old = np.zeros(64, dtype=np.uint32)
-    for lane in np.nonzero(w.em)[0]:
+    for lane in np.nonzero(w.em)[0]:   # (lane after lane: lanes may name the same address)
         cur = np.frombuffer(self.mem.read(int(addr[lane]), 4, f"global atomic (lane {lane})"), dtype=np.uint32)[0]
         old[lane] = cur
-        self.mem.write(int(addr[lane]), np.asarray(f(cur, data[lane])).astype(np.uint32).tobytes() if not isinstance(f(cur, data[lane]), bytes) else f(cur, data[lane]))
+        self.mem.write(int(addr[lane]), np.uint32(f(cur, data[lane])).tobytes())
     active = w.em.copy()
     if returns:
         vi = w.vindex(i.ops[0])
