@@ -90,10 +90,10 @@ def read_memory(path: str):
     out = []
     data = open(path, "rb").read()
     at = 0
-    while at < len(data):   # per allocation: address, size, number of pages that are not all zeros; then (offset, page) each
-        addr, size, pages = (int(x) for x in np.frombuffer(data[at:at + 24], dtype=np.uint64))
-        at += 24
-        buf = np.zeros(size, dtype=np.uint8)
+    while at < len(data):   # per allocation: address, size, number of pages written out, the byte every other page is full of; then (offset, page) each
+        addr, size, pages, background = (int(x) for x in np.frombuffer(data[at:at + 32], dtype=np.uint64))
+        at += 32
+        buf = np.full(size, background, dtype=np.uint8)
         for _ in range(pages):
             off = int(np.frombuffer(data[at:at + 8], dtype=np.uint64)[0])
             n = min(4096, size - off)

@@ -332,7 +332,7 @@ std::string g_last_kernel; // (launches are serialized)
 // REPLAY_DUMP_DIR: every launch leaves what is needed to run the same launch elsewhere (the emulator of the generated GPU code,
 // tests/isa/): the kernel function (its offset in the file it lives in, for the symbol table), grid and block, the argument block, and
 // every device allocation before and after the launch.
-// (pages of zeros are left out: the library's workspace is tens of megabytes of which a launch touches little; and the whole
+// (pages that are all 0x00 or all 0xFF are left out: the library's workspace is tens of megabytes of which a launch touches little; and the whole
 // process writes at most REPLAY_DUMP_LIMIT_MB, 4096 by default, after which it records no further launch)
 std::atomic<uint64_t> g_dumped{0};
 bool dump_memory(const std::string& path) {
@@ -341,14 +341,23 @@ bool dump_memory(const std::string& path) {
     FILE* f = fopen(path.c_str(), "wb");
     if (!f) return false;
     constexpr size_t PAGE = 4096;
-    static const unsigned char zeros[PAGE] = {0};
+    static unsigned char fill[2][PAGE];
+    std::memset(fill[0], 0x00, PAGE);
+    std::memset(fill[1], 0xFF, PAGE); // (what hipMalloc leaves in an allocation here)
     std::lock_guard<std::mutex> lock(g_mem_mutex);
     for (const auto& a : g_allocs) {
         const unsigned char* base = (const unsigned char*)a.first;
-        std::vector<uint64_t> pages;
-        for (size_t off = 0; off < a.second; off += PAGE)
-            if (std::memcmp(base + off, zeros, std::min(PAGE, a.second - off)) != 0) pages.push_back(off);
-        const uint64_t head[3] = {(uint64_t)a.first, (uint64_t)a.second, (uint64_t)pages.size()};
+        // pages that are all 0x00 or all 0xFF are not written: whichever kind there is more of is the allocation's background
+        std::vector<uint64_t> plain[2], pages;
+        for (size_t off = 0; off < a.second; off += PAGE) {
+            const size_t n = std::min(PAGE, a.second - off);
+            if (std::memcmp(base + off, fill[0], n) == 0) plain[0].push_back(off);
+            else if (std::memcmp(base + off, fill[1], n) == 0) plain[1].push_back(off);
+            else pages.push_back(off);
+        }
+        const int background = plain[1].size() > plain[0].size() ? 1 : 0;
+        pages.insert(pages.end(), plain[1 - background].begin(), plain[1 - background].end());
+        const uint64_t head[4] = {(uint64_t)a.first, (uint64_t)a.second, (uint64_t)pages.size(), background ? 0xFFull : 0ull};
         fwrite(head, sizeof(head), 1, f);
         for (uint64_t off : pages) {
             fwrite(&off, sizeof(off), 1, f);
@@ -435,6 +444,7 @@ hipError_t hipGetDeviceProperties(hipDeviceProp_t* p, int) {
 hipError_t hipMalloc(void** p, size_t bytes) {
     void* q = nullptr;
     if (posix_memalign(&q, 256, bytes ? bytes : 1) != 0) return hipErrorOutOfMemory;
+    std::memset(q, 0xFF, bytes); // device memory comes with whatever was there: NaNs here, so that nothing can lean on fresh pages being zero
     std::lock_guard<std::mutex> lock(replay::g_mem_mutex);
     replay::g_allocs[(uintptr_t)q] = bytes;
     *p = q;
