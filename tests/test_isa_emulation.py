@@ -208,3 +208,18 @@ def test_every_kernel_family_on_the_generated_code(exe, isa, tmp_path, reverse):
         assert not [name for name in not_run if not unreachable.search(name)], not_run
         assert len(not_run) <= 5
         assert len(kernels) >= 170
+
+
+@pytest.mark.skipif(os.environ.get("TENMO_REPLAY_FULL") != "1", reason="ten minutes of CPU time: set TENMO_REPLAY_FULL=1")
+def test_the_default_dispatch_at_medium_sizes(exe, isa, tmp_path):
+    """What the library picks by itself on 8 to 16 modelled CUs, at sizes where the persistent kernels walk many tiles: a 1024 x 1024 x 256
+    product, attention-shaped batches, both CBOW shapes at a tenth of the vocabulary, Linear backward with the fused bias gradient, the
+    broadcast-batched backward, the skinny product at its real width, mv and vm at 4096 squared."""
+    cases = [(16, "1024,1024,256,n,n,0,0,0"), (16, "512,512,64,n,t,4,0,0"), (16, "256,5000,100,n,n,0,0,0"), (16, "100,5000,256,t,n,0,0,0"),
+             (16, "lin:2048,768,256,n,n,0,0,fused=1"), (16, "bwd:512,768,768,n,n,4,1"), (8, "4,50257,768,n,n,0,0,0"), (8, "mv:4096,4096,n,0,0,0"),
+             (8, "vm:4096,4096,n,0,0,0")]
+    failures = []
+    with ProcessPoolExecutor(max_workers=min(8, os.cpu_count() or 1)) as pool:
+        for case, launches in pool.map(harness.replay_and_emulate, [(n, cus, case, str(tmp_path), exe) for n, (cus, case) in enumerate(cases)]):
+            failures += [f"{case}: {symbol}: {verdict}" for symbol, _count, verdict in launches if verdict != "ok"]
+    assert not failures, "\n".join(failures)
