@@ -184,3 +184,15 @@ def test_wait_states_before_a_vector_memory_instruction_reading_a_fresh_scalar()
 def test_an_unknown_instruction_stops_the_run():
     with pytest.raises(gfx950.EmulationError, match="no model of instruction v_frobnicate_b32"):
         run("v_frobnicate_b32 v1, v2")
+
+
+def test_relocation_across_4gib_moves_the_pointers_along():
+    import harness
+
+    buffers = [(0x5000_1230, np.zeros(100_000, np.uint8)), (0x7F00_0000_0100, np.zeros(64, np.uint8))]
+    args = struct.pack("<QqQQ", 0x5000_1230 + 4000, 12345, 0x7F00_0000_0100, 0x5000_1230 + 100_000)   # a pointer, a number, a pointer, one past the end
+    placed, moved = harness.across_4gib(buffers, args)
+    p0, number, p1, end = struct.unpack("<QqQQ", moved)
+    assert number == 12345 and p0 == placed[0] + 4000 and p1 == placed[1] and end == placed[0] + 100_000
+    assert placed[0] % 4096 == 0x230 and placed[0] >> 32 != (placed[0] + 100_000) >> 32   # same alignment within a page; the boundary lies inside
+    assert placed[1] % 4096 == 0x100
