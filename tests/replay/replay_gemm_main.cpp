@@ -10,7 +10,8 @@
 //     a case may carry check=0: do not compute the float64 product (large shapes: the addresses are the point)
 //   CASE = mv:m,k,layout,batch,pad,accumulate   out[m] = Mx[m,k] . v[k]; layout n (rows of k, pitch k + pad) or t (a transposed view of [k][m + pad])
 //   CASE = vm:k,n,layout,batch,pad,accumulate[,entry=noalloc]   out[n] = v[k] . Mx[k,n]; the matrix shared by every batch when batch < 0
-//   CASE = ce:M,C,target_is_int64,label_smoothing_percent    cross-entropy forward (all outputs) and backward (mean), addresses only
+//   CASE = ce:M,C,target_is_int64,label_smoothing_percent[,unaligned]    cross-entropy forward (all outputs) and backward (mean), addresses only
+//     (unaligned 1 / 2 / 3: the softmax, also the gradient, also the logits begin one float into their blocks)
 //   CASE = conv:N,C_in,H_pad,W_pad,C_out,KH,KW,stride,dilation    convolution forward and backward (all three gradients), addresses only
 //   CASE = mlp:batch,d0,d1,d2,d3,fused    two training steps of a 3-layer MLP (tenmo_hip_mlp_step), addresses only
 //   CASE = misc:n      dot, column sum ([n/64+1, 64.. ] shapes derived from n), SGD with and without momentum, addresses only
@@ -260,13 +261,19 @@ static int run_address_only_case(const std::string& spec) {
             const int64_t t = (m % 7 == 3) ? -100 : (m * 31) % C;
             if (i64) ((int64_t*)target)[m] = t; else ((int32_t*)target)[m] = (int32_t)t;
         }
-        float* softmax = exact_block((size_t)(M * C), false); float* per = exact_block((size_t)M, false); float* sum = exact_block(1, false);
-        int32_t* valid = (int32_t*)exact_block(1, false); float* up = exact_block(1); float* grad = exact_block((size_t)(M * C));
+        // a fifth number: softmax (1), softmax and gradient (2) or all three arrays (3) begin one float into their blocks: no 16-byte alignment
+        const int64_t shift = a.size() > 4 ? a[4] : 0;
+        float* logits_block = shift >= 3 ? exact_block((size_t)(M * C) + 1) : nullptr;
+        if (logits_block) { drop_block(logits); logits = logits_block + 1; }
+        float* softmax_block = exact_block((size_t)(M * C) + (shift >= 1), false); float* per = exact_block((size_t)M, false); float* sum = exact_block(1, false);
+        int32_t* valid = (int32_t*)exact_block(1, false); float* up = exact_block(1); float* grad_block = exact_block((size_t)(M * C) + (shift >= 2));
+        float* softmax = softmax_block + (shift >= 1); float* grad = grad_block + (shift >= 2);
         rc = tenmo_hip_cross_entropy_forward_f32(logits, target, i64, M, C, -100, ls, softmax, per, sum, valid, 1);
         if (rc == 0) rc = tenmo_hip_cross_entropy_forward_f32(logits, target, i64, M, C, -100, ls, nullptr, per, sum, valid, 1);
         if (rc == 0) rc = tenmo_hip_cross_entropy_backward_f32(softmax, target, i64, up, M, C, -100, ls, 2, valid[0], grad, 0, 1);
         if (rc == 0) rc = tenmo_hip_cross_entropy_backward_f32(softmax, target, i64, up, M, C, -100, ls, 1, valid[0], grad, 1, 1);
-        drop_block(logits); drop_block(target); drop_block(softmax); drop_block(per); drop_block(sum); drop_block(valid); drop_block(up); drop_block(grad);
+        if (logits_block) drop_block(logits_block); else drop_block(logits);
+        drop_block(target); drop_block(softmax_block); drop_block(per); drop_block(sum); drop_block(valid); drop_block(up); drop_block(grad_block);
     } else if (spec.compare(0, 5, "conv:") == 0) {
         const std::vector<int64_t> a = numbers_of(spec, 5);
         if (a.size() < 9) return 2;
@@ -313,6 +320,7 @@ static int run_address_only_case(const std::string& spec) {
         float* vel = exact_block((size_t)n);
         if (rc == 0) rc = tenmo_hip_sgd_step_f32(x, y, nullptr, n, 0.01f, 0.f, 0.f, 1);
         if (rc == 0) rc = tenmo_hip_sgd_step_f32(x, y, vel, n, 0.01f, 0.9f, 1e-4f, 1);
+        if (rc == 0 && n > 1) rc = tenmo_hip_sgd_step_f32(x + 1, y, vel, n - 1, 0.01f, 0.9f, 1e-4f, 1); // (parameters that are not 16-byte aligned)
         const int64_t rows = n / 64 + 1, cols = 64 + n % 61;
         float* G = exact_block((size_t)(rows * cols)); float* cs = exact_block((size_t)cols);
         if (rc == 0) rc = tenmo_hip_column_sum_f32(G, 0, cols, rows, cols, cs, 1, 1);
