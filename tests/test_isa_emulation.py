@@ -128,6 +128,7 @@ CASES = [
     (2, "vbw:70,33,3,0,0"), (2, "vbw:40,36,0,4,1"), (2, "vbw:64,128,2,2,0"),
     # the adjacent operators and the MLP step op by op and in three launches
     (2, "ce:33,1000,0,0"), (2, "ce:5,50257,1,10"), (2, "ce:64,10,0,0"), (2, "ce:37,9001,0,5"), (2, "ce:9,64,1,10"), (2, "ce:9,2048,0,0"), (2, "ce:9,4096,1,10"), (2, "ce:3,16384,0,0"),
+    (2, "ce:9,1999,1,0"), (2, "ce:9,2047,1,0"), (2, "ce:9,4095,0,0"), (2, "ce:5,8191,1,0"), (2, "ce:3,16383,1,0"), (2, "ce:3,32767,0,0"), (2, "ce:3,32767,1,0"),
     (2, "ce:9,1000,0,0,1"), (2, "ce:9,1000,1,10,2"), (2, "ce:9,1001,0,0,3"), (2, "ce:3,70001,1,0,3"),   # arrays that are not 16-byte aligned (2, "conv:2,3,12,11,8,3,3,1,1"), (2, "conv:2,4,15,14,6,3,2,2,1"),
     (2, "mlp:64,784,128,32,10,0"), (2, "mlp:37,257,77,33,7,3"), (2, "mlp:300,40,24,16,10,0"),
 ]
